@@ -1,0 +1,15 @@
+"""MI355X-native OPT incremental-decoding forward path (drop-in for metaseq's
+TransformerDecoder.forward / SequenceGenerator on one gfx950 GPU)."""
+from .config import OPTConfig, opt_config
+from .dictionary import Dictionary
+from .kv_cache import KVCache
+from .sequence_generator import SequenceGenerator
+from .synthetic import random_prompts, random_state_dict
+from .transformer_decoder import ModelParallelTransformerDecoder, TransformerDecoder
+from .transformer_lm import TransformerLanguageModel
+
+__all__ = [
+    "OPTConfig", "opt_config", "Dictionary", "KVCache", "SequenceGenerator", "random_prompts",
+    "random_state_dict", "TransformerDecoder", "ModelParallelTransformerDecoder",
+    "TransformerLanguageModel",
+]

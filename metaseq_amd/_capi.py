@@ -1,0 +1,84 @@
+"""ctypes binding of libmetaseq_amd.so (the C ABI declared in include/metaseq_amd.h).
+
+There is no fallback: if the library is missing or a call fails, an exception is raised.
+Shape / argument errors surface as ValueError, capacity overruns as ValueError, HIP
+failures as RuntimeError (the reference's serving loop treats a RuntimeError from
+``generate`` as a device fault and restarts the worker, metaseq/cli/interactive_hosted.py:161-171).
+"""
+import ctypes
+import os
+from ctypes import c_char_p, c_float, c_int, c_int32, c_int64, c_size_t, c_uint, c_void_p
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "csrc", "libmetaseq_amd.so")
+
+MSA_EPI_RELU = 1
+
+_P = c_void_p
+
+# name -> argtypes, in the order of include/metaseq_amd.h
+SIGNATURES = {
+    "msa_layernorm_f16": [_P, _P, _P, _P, c_int64, c_int, c_float, _P],
+    "msa_embed_f16": [_P, c_int64, c_int, c_int, c_int, _P, c_int, _P, c_int, c_int, c_int, _P, _P,
+                      _P, _P],
+    "msa_linear_f16": [_P, _P, _P, _P, _P, c_int64, c_int, c_int, c_uint, _P, c_size_t, _P],
+    "msa_linear_w8a16": [_P, _P, _P, _P, _P, _P, c_int64, c_int, c_int, c_uint, _P, c_size_t, _P],
+    "msa_qkv_proj_f16": [_P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
+                         _P, c_size_t, _P],
+    "msa_qkv_proj_w8a16": [_P, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int,
+                           c_int, _P, c_size_t, _P],
+    "msa_attention_f16": [_P, _P, _P, _P, c_int64, _P, c_int, c_int, c_int, c_int, c_int, c_int,
+                          _P],
+    "msa_greedy_select_f16": [_P, c_int64, c_int, c_int, c_float, _P, c_int, _P, c_int, _P, c_int,
+                              c_int, _P, c_int64, _P, c_int64, _P],
+    "msa_target_logprob_f16": [_P, c_int64, c_int64, c_int, c_float, _P, _P, _P],
+}
+OTHER_SYMBOLS = ["msa_last_error", "msa_version", "msa_linear_workspace_bytes"]
+
+_lib = None
+
+
+def load():
+    """Loads the shared library once; raises if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(
+            "metaseq_amd: %s is missing - build it with `python -m metaseq_amd.csrc.build` "
+            "(there is no non-HIP fallback)" % LIB_PATH)
+    lib = ctypes.CDLL(LIB_PATH)
+    for name, args in SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.argtypes = args
+        fn.restype = c_int
+    lib.msa_last_error.argtypes = []
+    lib.msa_last_error.restype = c_char_p
+    lib.msa_version.argtypes = []
+    lib.msa_version.restype = c_int
+    lib.msa_linear_workspace_bytes.argtypes = [c_int64, c_int, c_int]
+    lib.msa_linear_workspace_bytes.restype = c_size_t
+    _lib = lib
+    return lib
+
+
+def check(rc, lib=None):
+    if rc == 0:
+        return
+    lib = lib or load()
+    msg = lib.msa_last_error().decode("utf-8", "replace")
+    if rc == -3:
+        raise RuntimeError("metaseq_amd HIP failure: " + msg)
+    raise ValueError("metaseq_amd: " + msg)
+
+
+def ptr(t):
+    """Device pointer of a torch tensor (or NULL for None)."""
+    return None if t is None else t.data_ptr()
+
+
+def stream_ptr():
+    """hipStream_t of torch's current stream, so kernels order with torch's own work."""
+    import torch
+
+    return torch.cuda.current_stream().cuda_stream

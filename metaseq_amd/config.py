@@ -1,0 +1,58 @@
+"""Flat model configuration with the attribute names the reference's decoder reads from
+its args namespace (metaseq/models/transformer_decoder.py:73-117,
+metaseq/modules/transformer_decoder_layer.py:44-98), and the OPT size table
+(metaseq/launcher/opt_job_constants.py:32-45)."""
+from dataclasses import dataclass, replace
+
+
+@dataclass
+class OPTConfig:
+    decoder_layers: int
+    decoder_embed_dim: int
+    decoder_attention_heads: int
+    decoder_ffn_embed_dim: int = 0
+    vocab_size: int = 50272  # 50265 tokenizer entries padded to a multiple of 8
+    max_target_positions: int = 2048
+    padding_idx: int = 1
+    eos_idx: int = 2
+    activation_fn: str = "relu"
+    share_decoder_input_output_embed: bool = True
+    decoder_learned_pos: bool = True
+    no_scale_embedding: bool = True
+    quantize_int8: bool = False  # int8 weight-only for qkv / out_proj / fc1 / fc2
+
+    def __post_init__(self):
+        if not self.decoder_ffn_embed_dim:
+            self.decoder_ffn_embed_dim = 4 * self.decoder_embed_dim
+        if self.decoder_embed_dim % self.decoder_attention_heads:
+            raise ValueError("decoder_embed_dim must be divisible by decoder_attention_heads")
+        if self.activation_fn != "relu":
+            raise NotImplementedError("only --activation-fn relu (OPT) is implemented")
+        if not (self.share_decoder_input_output_embed and self.decoder_learned_pos
+                and self.no_scale_embedding):
+            raise NotImplementedError(
+                "only the OPT setup (tied embeddings, learned positions, no embedding scale) "
+                "is implemented")
+
+    @property
+    def head_dim(self):
+        return self.decoder_embed_dim // self.decoder_attention_heads
+
+
+# name -> (layers, embed dim, heads)
+_OPT_SIZES = {
+    "125m": (12, 768, 12),
+    "350m": (24, 1024, 16),
+    "1.3b": (24, 2048, 32),
+    "2.7b": (32, 2560, 32),
+    "6.7b": (32, 4096, 32),
+    "13b": (40, 5120, 40),
+    "30b": (48, 7168, 56),
+    "66b": (64, 9216, 72),
+    "175b": (96, 12288, 96),
+}
+
+
+def opt_config(name: str, **overrides) -> OPTConfig:
+    layers, dim, heads = _OPT_SIZES[name.lower()]
+    return replace(OPTConfig(layers, dim, heads), **overrides)

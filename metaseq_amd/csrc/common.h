@@ -1,0 +1,75 @@
+// Shared helpers for the gfx950 kernels: vector types, wave64 reductions, error plumbing.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#include "../../include/metaseq_amd.h"
+
+typedef _Float16 half_t;
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef float float16_t __attribute__((ext_vector_type(16)));
+
+#define MSA_WAVE 64
+
+void msa_set_error(const char* fmt, ...);
+
+#define MSA_REQUIRE(cond, code, ...) \
+  do {                               \
+    if (!(cond)) {                   \
+      msa_set_error(__VA_ARGS__);    \
+      return (code);                 \
+    }                                \
+  } while (0)
+
+#define MSA_CHECK_LAUNCH(name)                                              \
+  do {                                                                      \
+    hipError_t e_ = hipGetLastError();                                      \
+    if (e_ != hipSuccess) {                                                 \
+      msa_set_error("%s: launch failed: %s", name, hipGetErrorString(e_));  \
+      return MSA_ERR_HIP;                                                   \
+    }                                                                       \
+  } while (0)
+
+// round-to-nearest-even fp32 -> fp16 -> fp32 (a "materialise in fp16" point)
+__device__ __forceinline__ float round_h(float v) { return (float)(half_t)v; }
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, MSA_WAVE);
+  return v;
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, MSA_WAVE));
+  return v;
+}
+
+// Block-wide reductions for blocks of up to 16 waves; `red` is >= 16 floats of LDS.
+// All threads receive the result.  Contains barriers: call from uniform control flow.
+__device__ __forceinline__ float block_sum(float v, float* red) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = (blockDim.x + 63) >> 6;
+  v = wave_sum(v);
+  __syncthreads();
+  if (lane == 0) red[wave] = v;
+  __syncthreads();
+  float t = 0.f;
+  for (int i = 0; i < nw; ++i) t += red[i];
+  return t;
+}
+
+__device__ __forceinline__ float block_max(float v, float* red) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = (blockDim.x + 63) >> 6;
+  v = wave_max(v);
+  __syncthreads();
+  if (lane == 0) red[wave] = v;
+  __syncthreads();
+  float t = red[0];
+  for (int i = 1; i < nw; ++i) t = fmaxf(t, red[i]);
+  return t;
+}

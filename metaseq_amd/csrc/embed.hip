@@ -1,0 +1,123 @@
+// Token + learned-position embedding.  Positions follow the reference's make_positions:
+// pads keep pad_idx, every other token gets pad_idx + (number of non-pad tokens up to and
+// including it).  Only the last T_out columns are embedded (T_out = 1 for a decode step).
+#include "common.h"
+
+namespace {
+
+constexpr int EMB_THREADS = 256;
+
+// number of non-pad tokens in row[0 .. upto) ; all threads get the result
+__device__ __forceinline__ int count_nonpad(const int64_t* row, int upto, int pad, float* red) {
+  int c = 0;
+  for (int i = threadIdx.x; i < upto; i += blockDim.x) c += (row[i] != pad);
+  // counts are < 2^24 so the float reduction is exact
+  return (int)block_sum((float)c, red);
+}
+
+__device__ __forceinline__ void gather_row(const half_t* __restrict__ E,
+                                           const half_t* __restrict__ P, int64_t tok, int pos,
+                                           half_t* __restrict__ out, int D) {
+  const half_t* e = E + tok * (int64_t)D;
+  const half_t* p = P + (int64_t)pos * D;
+  for (int i = threadIdx.x; i < (D >> 3); i += blockDim.x) {
+    const half8_t a = *reinterpret_cast<const half8_t*>(e + (i << 3));
+    const half8_t b = *reinterpret_cast<const half8_t*>(p + (i << 3));
+    half8_t o;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) o[k] = (half_t)((float)a[k] + (float)b[k]);
+    *reinterpret_cast<half8_t*>(out + (i << 3)) = o;
+  }
+}
+
+__device__ __forceinline__ void clamp_ids(int64_t& tok, int& pos, int V, int n_pos_rows,
+                                          int32_t* status) {
+  if (tok < 0 || tok >= V || pos >= n_pos_rows) {
+    if (status && threadIdx.x == 0) *status = 1;
+    tok = tok < 0 ? 0 : (tok >= V ? V - 1 : tok);
+    pos = pos >= n_pos_rows ? n_pos_rows - 1 : pos;
+  }
+}
+
+// decode step: one block per batch row, last token only
+__global__ __launch_bounds__(EMB_THREADS) void embed_last_kernel(
+    const int64_t* __restrict__ tokens, int64_t tok_stride, int n, const half_t* __restrict__ E,
+    int V, const half_t* __restrict__ P, int n_pos_rows, int pad, int D, half_t* __restrict__ x,
+    int64_t* __restrict__ positions_out, int32_t* status) {
+  __shared__ float red[16];
+  const int b = blockIdx.x;
+  const int64_t* row = tokens + b * tok_stride;
+  int64_t tok = row[n - 1];
+  int pos = pad;
+  const int cnt = count_nonpad(row, n, pad, red);
+  if (tok != pad) pos = pad + cnt;
+  clamp_ids(tok, pos, V, n_pos_rows, status);
+  if (positions_out && threadIdx.x == 0) positions_out[b] = pos;
+  gather_row(E, P, tok, pos, x + (int64_t)b * D, D);
+}
+
+// prefill: positions for the last T_out columns of every row (one block per row)
+__global__ __launch_bounds__(EMB_THREADS) void positions_kernel(
+    const int64_t* __restrict__ tokens, int64_t tok_stride, int n, int T_out, int pad,
+    int64_t* __restrict__ positions_out) {
+  __shared__ int seg[EMB_THREADS];
+  const int b = blockIdx.x;
+  const int64_t* row = tokens + b * tok_stride;
+  const int per = (n + EMB_THREADS - 1) / EMB_THREADS;
+  const int lo = threadIdx.x * per, hi = min(n, lo + per);
+  int c = 0;
+  for (int i = lo; i < hi; ++i) c += (row[i] != pad);
+  seg[threadIdx.x] = c;
+  __syncthreads();
+  int run = 0;
+  for (int i = 0; i < (int)threadIdx.x; ++i) run += seg[i];
+  const int first = n - T_out;
+  for (int i = lo; i < hi; ++i) {
+    const bool np = row[i] != pad;
+    run += np;
+    if (i >= first) positions_out[(int64_t)b * T_out + (i - first)] = np ? pad + run : pad;
+  }
+}
+
+__global__ __launch_bounds__(EMB_THREADS) void embed_rows_kernel(
+    const int64_t* __restrict__ tokens, int64_t tok_stride, int n, int T_out,
+    const half_t* __restrict__ E, int V, const half_t* __restrict__ P, int n_pos_rows, int D,
+    half_t* __restrict__ x, const int64_t* __restrict__ positions, int32_t* status) {
+  const int64_t r = blockIdx.x;  // b * T_out + j
+  const int b = (int)(r / T_out), j = (int)(r % T_out);
+  int64_t tok = tokens[b * tok_stride + (n - T_out + j)];
+  int pos = (int)positions[r];
+  clamp_ids(tok, pos, V, n_pos_rows, status);
+  gather_row(E, P, tok, pos, x + r * D, D);
+}
+
+}  // namespace
+
+extern "C" int msa_embed_f16(const int64_t* tokens, int64_t tok_stride, int B, int n, int T_out,
+                             const void* E, int V, const void* P, int n_pos_rows, int pad_idx,
+                             int D, void* x, int64_t* positions_out, int32_t* status_dev,
+                             void* stream) {
+  MSA_REQUIRE(tokens && E && P && x, MSA_ERR_INVALID_ARG, "msa_embed_f16: null pointer");
+  MSA_REQUIRE(B > 0 && n > 0 && T_out > 0 && T_out <= n && tok_stride >= n, MSA_ERR_INVALID_ARG,
+              "msa_embed_f16: bad shape B=%d n=%d T_out=%d stride=%lld", B, n, T_out,
+              (long long)tok_stride);
+  MSA_REQUIRE(D > 0 && D % 8 == 0 && V > 0 && n_pos_rows > pad_idx && pad_idx >= 0,
+              MSA_ERR_INVALID_ARG, "msa_embed_f16: bad sizes D=%d V=%d n_pos_rows=%d pad=%d", D, V,
+              n_pos_rows, pad_idx);
+  hipStream_t s = (hipStream_t)stream;
+  if (T_out == 1) {
+    hipLaunchKernelGGL(embed_last_kernel, dim3(B), dim3(EMB_THREADS), 0, s, tokens, tok_stride, n,
+                       (const half_t*)E, V, (const half_t*)P, n_pos_rows, pad_idx, D, (half_t*)x,
+                       positions_out, status_dev);
+  } else {
+    MSA_REQUIRE(positions_out, MSA_ERR_INVALID_ARG,
+                "msa_embed_f16: positions_out is required when T_out > 1");
+    hipLaunchKernelGGL(positions_kernel, dim3(B), dim3(EMB_THREADS), 0, s, tokens, tok_stride, n,
+                       T_out, pad_idx, positions_out);
+    hipLaunchKernelGGL(embed_rows_kernel, dim3((unsigned)((int64_t)B * T_out)), dim3(EMB_THREADS),
+                       0, s, tokens, tok_stride, n, T_out, (const half_t*)E, V, (const half_t*)P,
+                       n_pos_rows, D, (half_t*)x, positions_out, status_dev);
+  }
+  MSA_CHECK_LAUNCH("msa_embed_f16");
+  return MSA_OK;
+}

@@ -1,0 +1,168 @@
+// Per-row vocabulary reductions of the greedy generation loop: fp32 log-sum-exp over fp16
+// logits, masked arg-max with lowest-index tie-break, and target log-probability gather.
+// One workgroup per logits row; the row (V * 2 bytes) is read twice from cache/HBM.
+#include <math.h>
+
+#include "common.h"
+
+namespace {
+
+constexpr int SM_THREADS = 1024;
+
+struct RowStats {
+  float max;  // max of z = logit / temperature over the whole row
+  float lse;  // log(sum(exp(z - max)))   (so log_softmax(z) = z - max - lse)
+};
+
+__device__ __forceinline__ RowStats row_logsumexp(const half_t* __restrict__ row, int V,
+                                                  float temp, bool scale, float* red) {
+  float mx = -INFINITY;
+  bool nan = false;
+  for (int i = threadIdx.x; i < V; i += blockDim.x) {
+    float z = (float)row[i];
+    if (scale) z = z / temp;
+    nan |= (z != z);
+    mx = fmaxf(mx, z);
+  }
+  mx = block_max(mx, red);
+  const float any_nan = block_max(nan ? 1.f : 0.f, red);
+  float s = 0.f;
+  for (int i = threadIdx.x; i < V; i += blockDim.x) {
+    float z = (float)row[i];
+    if (scale) z = z / temp;
+    s += expf(z - mx);
+  }
+  s = block_sum(s, red);
+  RowStats r;
+  r.max = mx;
+  r.lse = any_nan > 0.f ? NAN : logf(s);
+  return r;
+}
+
+struct IdList {
+  int32_t n;
+  int32_t id[16];
+};
+
+__global__ __launch_bounds__(SM_THREADS) void greedy_select_kernel(
+    const half_t* __restrict__ logits, int64_t ld, int V, float temperature, bool scale,
+    IdList banned, IdList stop, uint8_t* __restrict__ finished, int force_eos_all, int eos,
+    int64_t* __restrict__ tok, int64_t tok_stride, float* __restrict__ score,
+    int64_t score_stride) {
+  __shared__ float red[16];
+  __shared__ float wbest[16];
+  __shared__ int widx[16];
+  const int b = blockIdx.x;
+  const half_t* row = logits + (int64_t)b * ld;
+  const RowStats st = row_logsumexp(row, V, temperature, scale, red);
+  const bool dead = st.lse != st.lse;  // a NaN anywhere turns every log-prob into -inf
+  const bool only_eos = force_eos_all || (finished && finished[b]);
+
+  float best = -INFINITY;
+  int bidx = 0x7fffffff;
+  for (int i = threadIdx.x; i < V; i += blockDim.x) {
+    float z = (float)row[i];
+    if (scale) z = z / temperature;
+    float lp = dead ? -INFINITY : (z - st.max) - st.lse;
+    for (int j = 0; j < banned.n; ++j)
+      if (banned.id[j] == i) lp = -INFINITY;
+    if (only_eos && i != eos) lp = -INFINITY;
+    if (lp > best || (lp == best && i < bidx)) {
+      best = lp;
+      bidx = i;
+    }
+  }
+  // wave then block arg-max; ties resolve to the lowest index
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    const float ob = __shfl_xor(best, o, MSA_WAVE);
+    const int oi = __shfl_xor(bidx, o, MSA_WAVE);
+    if (ob > best || (ob == best && oi < bidx)) {
+      best = ob;
+      bidx = oi;
+    }
+  }
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  if (lane == 0) {
+    wbest[wave] = best;
+    widx[wave] = bidx;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < (int)(blockDim.x >> 6); ++w)
+      if (wbest[w] > best || (wbest[w] == best && widx[w] < bidx)) {
+        best = wbest[w];
+        bidx = widx[w];
+      }
+    tok[b * tok_stride] = bidx;
+    score[b * score_stride] = best;
+    if (finished) {
+      bool f = bidx == eos;
+      for (int j = 0; j < stop.n; ++j) f |= (stop.id[j] == bidx);
+      if (f) finished[b] = 1;
+    }
+  }
+}
+
+__global__ __launch_bounds__(SM_THREADS) void target_logprob_kernel(
+    const half_t* __restrict__ logits, int64_t ld, int V, float temperature, bool scale,
+    const int64_t* __restrict__ target, float* __restrict__ out) {
+  __shared__ float red[16];
+  const int64_t r = blockIdx.x;
+  const half_t* row = logits + r * ld;
+  const RowStats st = row_logsumexp(row, V, temperature, scale, red);
+  if (threadIdx.x == 0) {
+    int64_t t = target[r];
+    t = t < 0 ? 0 : (t >= V ? V - 1 : t);
+    float z = (float)row[t];
+    if (scale) z = z / temperature;
+    out[r] = (z - st.max) - st.lse;
+  }
+}
+
+}  // namespace
+
+extern "C" int msa_greedy_select_f16(const void* logits, int64_t ld_logits, int B, int V,
+                                     float temperature, const int32_t* banned_host, int n_banned,
+                                     const int32_t* stop_host, int n_stop, uint8_t* finished,
+                                     int force_eos_all, int eos_idx, int64_t* tok,
+                                     int64_t tok_stride, float* score, int64_t score_stride,
+                                     void* stream) {
+  MSA_REQUIRE(logits && tok && score, MSA_ERR_INVALID_ARG, "msa_greedy_select_f16: null pointer");
+  MSA_REQUIRE(B > 0 && V > 0 && ld_logits >= V, MSA_ERR_INVALID_ARG,
+              "msa_greedy_select_f16: bad shape B=%d V=%d ld=%lld", B, V, (long long)ld_logits);
+  MSA_REQUIRE(n_banned >= 0 && n_banned <= 16 && (n_banned == 0 || banned_host),
+              MSA_ERR_INVALID_ARG, "msa_greedy_select_f16: n_banned=%d (0..16)", n_banned);
+  MSA_REQUIRE(n_stop >= 0 && n_stop <= 16 && (n_stop == 0 || stop_host), MSA_ERR_INVALID_ARG,
+              "msa_greedy_select_f16: n_stop=%d (0..16)", n_stop);
+  MSA_REQUIRE(eos_idx >= 0 && eos_idx < V, MSA_ERR_INVALID_ARG,
+              "msa_greedy_select_f16: eos_idx=%d outside the vocabulary", eos_idx);
+  MSA_REQUIRE(temperature >= 0.f, MSA_ERR_INVALID_ARG, "msa_greedy_select_f16: temperature < 0");
+  const bool scale = temperature > 0.f && temperature != 1.0f;
+  IdList banned{}, stop{};
+  banned.n = n_banned;
+  for (int i = 0; i < n_banned; ++i) banned.id[i] = banned_host[i];
+  stop.n = n_stop;
+  for (int i = 0; i < n_stop; ++i) stop.id[i] = stop_host[i];
+  hipLaunchKernelGGL(greedy_select_kernel, dim3(B), dim3(SM_THREADS), 0, (hipStream_t)stream,
+                     (const half_t*)logits, ld_logits, V, temperature, scale, banned, stop,
+                     finished, force_eos_all, eos_idx, tok, tok_stride, score, score_stride);
+  MSA_CHECK_LAUNCH("msa_greedy_select_f16");
+  return MSA_OK;
+}
+
+extern "C" int msa_target_logprob_f16(const void* logits, int64_t ld_logits, int64_t rows, int V,
+                                      float temperature, const int64_t* target, float* out,
+                                      void* stream) {
+  MSA_REQUIRE(logits && target && out, MSA_ERR_INVALID_ARG, "msa_target_logprob_f16: null pointer");
+  MSA_REQUIRE(rows >= 0 && rows < (1ll << 31) && V > 0 && ld_logits >= V, MSA_ERR_INVALID_ARG,
+              "msa_target_logprob_f16: bad shape rows=%lld V=%d ld=%lld", (long long)rows, V,
+              (long long)ld_logits);
+  if (rows == 0) return MSA_OK;
+  const bool scale = temperature > 0.f && temperature != 1.0f;
+  hipLaunchKernelGGL(target_logprob_kernel, dim3((unsigned)rows), dim3(SM_THREADS), 0,
+                     (hipStream_t)stream, (const half_t*)logits, ld_logits, V, temperature, scale,
+                     target, out);
+  MSA_CHECK_LAUNCH("msa_target_logprob_f16");
+  return MSA_OK;
+}

@@ -1,0 +1,45 @@
+"""Preallocated contiguous per-layer KV cache.
+
+The reference grows its cache by ``torch.cat`` every step and every layer
+(metaseq/modules/multihead_attention.py:449-479), re-copying the whole history.  Here each
+layer owns one fp16 tensor ``[2, B, H, S_cap, hd]`` (K then V) that the QKV kernel appends to
+in place; ``length`` counts the valid positions.  The object lives inside the caller-owned
+``incremental_state`` dict, as the reference's per-module buffers do
+(metaseq/incremental_decoding_utils.py:30-69), and is freed with it.
+"""
+import torch
+
+
+class KVCache:
+    def __init__(self, n_layers, batch, heads, head_dim, capacity, device):
+        self.n_layers, self.batch, self.heads, self.head_dim = n_layers, batch, heads, head_dim
+        self.capacity = int(capacity)
+        self.length = 0
+        self.device = device
+        self.has_pads = False
+        self.layers = [
+            torch.empty(2, batch, heads, self.capacity, head_dim, dtype=torch.float16,
+                        device=device)
+            for _ in range(n_layers)
+        ]
+
+    def k(self, i):
+        return self.layers[i][0]
+
+    def v(self, i):
+        return self.layers[i][1]
+
+    def grow(self, new_capacity):
+        """Reallocates every layer to ``new_capacity`` positions, keeping the valid prefix."""
+        new_capacity = int(new_capacity)
+        if new_capacity <= self.capacity:
+            return
+        for i, old in enumerate(self.layers):
+            new = torch.empty(2, self.batch, self.heads, new_capacity, self.head_dim,
+                              dtype=torch.float16, device=self.device)
+            new[:, :, :, :self.length].copy_(old[:, :, :, :self.length])
+            self.layers[i] = new
+        self.capacity = new_capacity
+
+    def bytes(self):
+        return sum(t.numel() * 2 for t in self.layers)

@@ -1,0 +1,206 @@
+"""Greedy generation loop with the constructor, call signature and return value of the
+reference's ``SequenceGenerator`` (metaseq/sequence_generator.py:26-534).
+
+The reference makes ~6 full-vocabulary fp32 passes and two device-to-host syncs per step; here
+one kernel per step does log-sum-exp, masking, arg-max, token/score write-back and the
+finished-row update on the device, and the host only syncs once end-of-sequence becomes
+possible (step >= min_len).
+
+Implemented: beam_size replicas, min_len / max_len_b, stop tokens, temperature, prompt
+scoring, ``need_logprobs``.  Not implemented (raise): top-p / factual-nucleus sampling and
+repetition penalties.
+"""
+import ctypes
+from typing import Dict, List, Optional
+
+import torch
+from torch import nn
+
+from . import _capi
+from ._capi import check, ptr
+
+
+class SequenceGenerator(nn.Module):
+    def __init__(self, models, tgt_dict, beam_size: int = 1, max_len_a: int = 0,
+                 max_len_b: int = 200, min_len: int = 1, temperature: float = 1.0,
+                 need_logprobs: bool = False, stop: Optional[List[int]] = None,
+                 topp: float = -1, profile=False, omega_bound: float = 0.3,
+                 lambda_decay: float = -1, alpha_presence: float = 0.0,
+                 alpha_frequency: float = 0.0, alpha_presence_src: float = 0.0,
+                 alpha_frequency_src: float = 0.0, alpha_src_penalty_end_idx: int = -1):
+        super().__init__()
+        self.model = models[0] if isinstance(models, (list, tuple)) else models
+        self.tgt_dict = tgt_dict
+        self.pad = tgt_dict.pad()
+        self.unk = tgt_dict.unk()
+        self.eos = tgt_dict.eos()
+        self.vocab_size = len(tgt_dict)
+        self.beam_size = min(beam_size, self.vocab_size - 1)
+        self.max_len_a = max_len_a
+        self.max_len_b = max_len_b
+        self.min_len = min_len
+        self.need_logprobs = need_logprobs
+        self.stop = list(stop) if stop is not None else []
+        if topp is None:
+            topp = 0.0
+        self.sampling_topp = max(0, topp)
+        self.temperature = temperature
+        assert temperature >= 0, "--temperature must be >=0"
+        if not (self.temperature == 0.0 or self.sampling_topp == 0.0):
+            raise NotImplementedError("top-p sampling is not implemented; use topp <= 0 (greedy)")
+        if lambda_decay > 0:
+            raise NotImplementedError("factual-nucleus sampling is not implemented")
+        if max(alpha_presence, alpha_frequency, alpha_presence_src, alpha_frequency_src) > 0:
+            raise NotImplementedError("repetition penalties are not implemented")
+        if len(self.stop) > 14:
+            raise ValueError("at most 14 stop tokens are supported")
+        self.model.eval()
+        self.profile = profile
+
+    def cuda(self):
+        self.model.cuda()
+        return self
+
+    @torch.no_grad()
+    def forward(self, sample, prefix_tokens=None, bos_token=None):
+        return self._generate(sample, prefix_tokens, bos_token=bos_token)
+
+    @torch.no_grad()
+    def generate(self, models, sample, **kwargs):
+        return self._generate(sample, **kwargs)
+
+    # ------------------------------------------------------------------
+    def _select(self, lib, logits2d, step, min_len, max_len, finished, tokens, scores):
+        """Fused log-softmax + masks + arg-max + bookkeeping for one step
+        (metaseq/sequence_generator.py:272-308)."""
+        banned = [self.pad]
+        if step < min_len:
+            banned += [self.eos] + self.stop
+        B, V = logits2d.shape
+        arr = (ctypes.c_int32 * len(banned))(*banned)
+        stop = (ctypes.c_int32 * max(1, len(self.stop)))(*self.stop)
+        tok = tokens[:, step]
+        sc = scores[:, step]
+        check(lib.msa_greedy_select_f16(
+            ptr(logits2d), logits2d.stride(0), B, V, float(self.temperature), arr, len(banned),
+            stop, len(self.stop), ptr(finished), int(step >= max_len - 1), self.eos,
+            ptr(tok), tokens.stride(0), ptr(sc), scores.stride(0), _capi.stream_ptr()))
+
+    def _generate(self, sample: Dict[str, Dict[str, torch.Tensor]], prefix_tokens=None,
+                  bos_token=None):
+        lib = _capi.load()
+        incremental_states: Dict = {}
+        net_input = sample["net_input"]
+        if "src_tokens" not in net_input:
+            raise Exception("expected src_tokens in net input")
+        src_tokens = net_input["src_tokens"]
+        if not src_tokens.is_cuda:
+            raise RuntimeError("metaseq_amd: src_tokens must live on the GPU")
+        src_lengths = (src_tokens.ne(self.eos) & src_tokens.ne(self.pad)).long().sum(dim=1)
+        bsz, src_len = src_tokens.size()[:2]
+        beam_size = self.beam_size
+        dev = src_tokens.device
+
+        max_len = int(min(self.model.max_decoder_positions(), self.max_len_b or 1e99))
+        min_len = min(max_len, self.min_len or 0)
+        assert min_len <= max_len, "min_len cannot be larger than max_len, please adjust these!"
+        start_step = src_tokens.shape[1]
+        if start_step > max_len:
+            raise ValueError("prompt length %d exceeds max_len %d" % (start_step, max_len))
+        BB = bsz * beam_size
+
+        scores = torch.zeros(BB, max_len, device=dev, dtype=torch.float32)
+        tokens = torch.full((BB, max_len), self.pad, device=dev, dtype=torch.long)
+        tokens[:, :start_step] = src_tokens.repeat_interleave(beam_size, 0)
+        rep_lengths = src_lengths.repeat_interleave(beam_size, 0)
+        all_lprobs = None
+        if self.need_logprobs:
+            all_lprobs = torch.zeros(BB, max_len, self.vocab_size, device=dev,
+                                     dtype=torch.float32)
+
+        decoder = self.model.decoder
+        old_cap = getattr(decoder, "kv_cache_capacity", None)
+        decoder.kv_cache_capacity = max_len
+        try:
+            # ---- prefill over all forced tokens (:223-230) ----
+            logits = self.model(tokens[:, :start_step], incremental_state=incremental_states)[0]
+            T, V = logits.shape[1], logits.shape[2]
+            flat = logits.view(BB * T, V)
+            stream = _capi.stream_ptr()
+            # log-prob of every prompt token given its prefix (:252-258)
+            if start_step > 1:
+                target = torch.zeros(BB, T, dtype=torch.long, device=dev)
+                target[:, :-1] = tokens[:, 1:start_step]
+                lp = torch.empty(BB, T, dtype=torch.float32, device=dev)
+                check(lib.msa_target_logprob_f16(ptr(flat), flat.stride(0), BB * T, V,
+                                                 float(self.temperature), ptr(target), ptr(lp),
+                                                 stream))
+                scores[:, 1:start_step] = lp[:, :-1]
+            # scores after each row's own prompt are reset (:262-266)
+            col = torch.arange(max_len, device=dev).unsqueeze(0)
+            scores.masked_fill_(col > rep_lengths.unsqueeze(1), 0.0)
+            if all_lprobs is not None:
+                full = self.model.get_normalized_probs(self._tempered(logits), log_probs=True)
+                all_lprobs[:, 1:start_step] = full[:, :-1]
+                del full
+            # the row that predicts each sample's first free token (:262-267)
+            if int(rep_lengths.max()) >= T:
+                # the reference indexes lprobs[i, prompt_len] out of range in this case: every
+                # prompt needs a leading eos (or trailing pads)
+                raise IndexError("prompt without eos/pad: row prompt_len is outside the prefill")
+            rows = torch.arange(BB, device=dev) * T + rep_lengths
+            step_logits = flat.index_select(0, rows)
+            del logits, flat
+
+            finished = torch.zeros(BB, dtype=torch.uint8, device=dev)
+            for step in range(start_step, max_len):
+                if all_lprobs is not None:
+                    all_lprobs[:, step] = self._masked_lprobs(step_logits, step, min_len, max_len,
+                                                              finished)
+                self._select(lib, step_logits, step, min_len, max_len, finished, tokens, scores)
+                # rows can only finish once eos / stop tokens are allowed or forced
+                if (step >= min_len or step >= max_len - 1) and bool(finished.all()):
+                    break
+                if step + 1 >= max_len:
+                    break
+                out = decoder(tokens[:, :step + 1], incremental_state=incremental_states)[0]
+                step_logits = out.view(BB, V)
+        finally:
+            decoder.kv_cache_capacity = old_cap
+
+        # highest cumulative score first within each sample's replicas (:325-333)
+        beamscores = scores.view(bsz, beam_size, -1).cumsum(dim=-1)[:, :, -1]
+        indices = beamscores.sort(dim=-1, descending=True).indices
+        sorted_indices = (indices + beam_size * torch.arange(bsz, device=dev).unsqueeze(1)).view(-1)
+        tokens = tokens[sorted_indices]
+        scores = scores[sorted_indices]
+        retval = {"tokens": tokens.view(bsz, beam_size, -1),
+                  "scores": scores.view(bsz, beam_size, -1)}
+        if all_lprobs is not None:
+            retval["distributions"] = all_lprobs[sorted_indices].view(bsz, beam_size, -1,
+                                                                      self.vocab_size)
+        return retval
+
+    # ---- slow path used only with need_logprobs ----
+    def _tempered(self, logits):
+        x = logits.float()
+        if self.temperature > 0 and self.temperature != 1.0:
+            x = x / self.temperature
+        return x
+
+    def _masked_lprobs(self, step_logits, step, min_len, max_len, finished):
+        import math
+        lprobs = self.model.get_normalized_probs(self._tempered(step_logits), log_probs=True)
+        if step < min_len:
+            lprobs[:, self.eos] = -math.inf
+            for t in self.stop:
+                lprobs[:, t] = -math.inf
+        lprobs[lprobs != lprobs] = -math.inf
+        lprobs[:, self.pad] = -math.inf
+        if step >= max_len - 1:
+            lprobs[:, :self.eos] = -math.inf
+            lprobs[:, self.eos + 1:] = -math.inf
+        fin = finished.bool()
+        lprobs[fin, :self.eos] = -math.inf
+        lprobs[fin, self.eos + 1:] = -math.inf
+        return lprobs

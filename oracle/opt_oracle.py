@@ -1,0 +1,334 @@
+"""CPU restatement of metaseq's OPT incremental-decoding forward and greedy loop.
+
+TEST INFRASTRUCTURE ONLY.  Nothing in the shipped package imports this file; it is
+the checker that the parity tests, the smoke test and the benchmark's CPU-baseline
+leg compare the HIP path against.  It is written from the reference's sources (cited
+per function, paths relative to the metaseq tree) in plain PyTorch ops and runs on
+any torch device.
+
+Two arithmetic modes, selected by ``dtype``:
+
+* ``torch.float32`` - everything in fp32.
+* ``torch.float16`` - "rounding faithful": every tensor the reference materialises
+  in fp16 is rounded to fp16 here at the same point (after each matmul, after each
+  separate bias add, after ``q *= scaling``, after the softmax cast-back, after each
+  residual add, after each LayerNorm), while the arithmetic between two rounding
+  points runs in fp32, which is what the BLAS / softmax / LayerNorm kernels behind
+  the reference's torch calls do (fp32 accumulation, one rounding on output).
+
+How each function is pinned (tests/test_oracle_*.py):
+
+* ``make_positions``           - the reference's own known-answer table
+                                 (cpu_tests/test_utils.py:55-93), committed as
+                                 tests/golden/make_positions.json.
+* ``layer_norm``               - closed form in float64 numpy; constant-row and
+                                 affine special cases.
+* ``attention`` (prefill and   - brute-force python loops on tiny inputs and
+  incremental)                   ``F.scaled_dot_product_attention(is_causal=True)``;
+                                 invariant: incremental logits at step t equal the
+                                 last row of a full forward on tokens[:t+1].
+* whole decoder, K|V|Q order,  - Hugging Face ``OPTForCausalLM`` built from a config
+  position offset, pad mask      object with the same weights mapped in (the
+                                 relation the reference's own
+                                 gpu_tests/test_hf_compatibility.py:128-155 asserts).
+* ``greedy_generate``          - scripted-logit fake decoders with hand-derived
+                                 expected token/score tables (the idea of the
+                                 reference's tests/utils.py:420-465).
+* ``quantize_int8``            - parity unpinned by the reference (its int8
+                                 quantiser lives in FasterTransformer and no
+                                 reference test touches it); pinned by the closed
+                                 form stated in the function and brute force.
+"""
+
+import math
+import uuid
+from dataclasses import dataclass
+from typing import Dict, List, Optional
+
+import torch
+import torch.nn.functional as F
+
+
+@dataclass
+class OracleConfig:
+    """Attribute names follow the reference's args namespace
+    (metaseq/models/transformer_decoder.py:73-117)."""
+
+    decoder_layers: int
+    decoder_embed_dim: int
+    decoder_attention_heads: int
+    decoder_ffn_embed_dim: int
+    vocab_size: int
+    max_target_positions: int = 2048
+    padding_idx: int = 1
+    eos_idx: int = 2
+
+    @property
+    def head_dim(self) -> int:
+        return self.decoder_embed_dim // self.decoder_attention_heads
+
+
+def make_positions(tokens: torch.Tensor, padding_idx: int) -> torch.Tensor:
+    """metaseq/utils.py:83-93: non-pad symbols get cumsum(non-pad) + padding_idx,
+    pads get padding_idx."""
+    mask = tokens.ne(padding_idx).int()
+    return (torch.cumsum(mask, dim=1).type_as(mask) * mask).long() + padding_idx
+
+
+def layer_norm(x, gamma, beta, eps=1e-5):
+    """metaseq/modules/layer_norm.py:28-33 (torch.nn.LayerNorm / apex
+    cuApplyLayerNorm, apex/layer_norm_cuda_kernel.cu:441-455): statistics in fp32,
+    biased variance, y = gamma * (x - mean) * rsqrt(var + eps) + beta."""
+    x = x.float()
+    mean = x.mean(dim=-1, keepdim=True)
+    var = ((x - mean) ** 2).mean(dim=-1, keepdim=True)
+    return (x - mean) * torch.rsqrt(var + eps) * gamma.float() + beta.float()
+
+
+def quantize_int8(w: torch.Tensor):
+    """Symmetric per-output-channel weight-only int8 (the benchmark's definition; the
+    reference delegates this to FasterTransformer, scripts/convert_metaseq_ft.py:99-133).
+
+    w [out, in] -> (q int8 [out, in], scale fp16 [out]) with
+    scale_j = fp16(max_i |w_ji| / 127), q = clamp(rint(w / scale_j), -127, 127),
+    dequantised weight = fp16(q * scale_j).
+    """
+    wf = w.float()
+    scale = (wf.abs().amax(dim=1) / 127.0).to(torch.float16)
+    s = scale.float().clamp_min(1e-30).unsqueeze(1)
+    q = torch.clamp(torch.round(wf / s), -127, 127).to(torch.int8)
+    return q, scale
+
+
+def dequantize_int8(q: torch.Tensor, scale: torch.Tensor) -> torch.Tensor:
+    return (q.float() * scale.float().unsqueeze(1)).to(torch.float16)
+
+
+def linear(x, w, b, r):
+    """mpu/layers.py:290-292: output = matmul(x, W.t()), then output = output + bias as a
+    separate op; ``r`` is the rounding applied where the reference materialises a tensor."""
+    y = r(x @ w.t())
+    if b is not None:
+        y = r(y + b)
+    return y
+
+
+class OracleDecoder:
+    """Restates ModelParallelTransformerDecoder.forward at tensor-parallel size 1
+    (metaseq/models/transformer_decoder.py:494-537) with the inference branch of
+    ModelParallelMultiheadAttention (metaseq/modules/multihead_attention.py:428-556).
+
+    ``state_dict`` uses the reference's parameter names
+    (metaseq/scripts/convert_metaseq_ft.py:74-90): decoder.embed_tokens.weight,
+    decoder.embed_positions.weight, decoder.layers.{i}.self_attn_layer_norm.*,
+    decoder.layers.{i}.self_attn.qkv_proj.* (rows K | V | Q),
+    decoder.layers.{i}.self_attn.out_proj.*, decoder.layers.{i}.final_layer_norm.*,
+    decoder.layers.{i}.fc1.*, decoder.layers.{i}.fc2.*, decoder.layer_norm.*.
+    """
+
+    def __init__(self, cfg: OracleConfig, state_dict: Dict[str, torch.Tensor],
+                 dtype=torch.float32, device="cpu"):
+        self.cfg = cfg
+        self.dtype = dtype
+        self.device = torch.device(device)
+        # weights are held as fp32 copies of values already rounded to `dtype`
+        self.w = {
+            k: v.detach().to(self.device).to(dtype).float()
+            for k, v in state_dict.items()
+            if v.is_floating_point()
+        }
+        self.layer_ids = [str(uuid.uuid4()) for _ in range(cfg.decoder_layers)]
+
+    # -- rounding point --------------------------------------------------
+    def _r(self, t: torch.Tensor) -> torch.Tensor:
+        if self.dtype == torch.float32:
+            return t
+        return t.to(self.dtype).float()
+
+    def max_positions(self) -> int:
+        # transformer_decoder.py:430-434 with learned_positional_embedding.py:25-28
+        return min(
+            self.cfg.max_target_positions,
+            self.w["decoder.embed_positions.weight"].shape[0] - self.cfg.padding_idx - 1,
+        )
+
+    # -- linear: matmul -> round -> (+ bias -> round) ----------------------
+    def _linear(self, x, wname, bname=None):
+        return linear(x, self.w[wname], self.w[bname] if bname is not None else None, self._r)
+
+    def attention_core(self, q, k, v, B, attn_mask=None, key_padding_mask=None):
+        """multihead_attention.py:492-543 on q [B*H, T, hd] (already scaled) and
+        k, v [B*H, S, hd]: scores, additive causal mask, key padding mask, fp32 softmax cast
+        back to the activation dtype, weighted sum of values."""
+        BH, T, _ = q.shape
+        H, S = BH // B, k.shape[1]
+        s = self._r(torch.bmm(q, k.transpose(1, 2)))  # :492
+        if attn_mask is not None:
+            s = s + attn_mask.unsqueeze(0)  # :516-518
+        if key_padding_mask is not None:  # :520-531
+            assert key_padding_mask.shape == (B, S)
+            s = s.view(B, H, T, S).masked_fill(
+                key_padding_mask.unsqueeze(1).unsqueeze(2).to(torch.bool), float("-inf")
+            ).view(BH, T, S)
+        pr = self._r(F.softmax(s, dim=-1, dtype=torch.float32))  # :533-534
+        return self._r(torch.bmm(pr, v))  # :543
+
+    def _attention(self, i, x, incremental_state, attn_mask, key_padding_mask):
+        """multihead_attention.py:278-556, inference branch. x is [T, B, D]."""
+        cfg = self.cfg
+        T, B, D = x.shape
+        H, hd = cfg.decoder_attention_heads, cfg.head_dim
+        p = f"decoder.layers.{i}.self_attn."
+        kvq = self._linear(x, p + "qkv_proj.weight", p + "qkv_proj.bias")
+        k, v, q = kvq.split(D, dim=-1)  # :316-319, thirds are K | V | Q
+        q = self._r(q * (hd ** -0.5))  # :429
+        q = q.contiguous().view(T, B * H, hd).transpose(0, 1)  # :431-435
+        k = k.contiguous().view(-1, B * H, hd).transpose(0, 1)
+        v = v.contiguous().view(-1, B * H, hd).transpose(0, 1)
+        if incremental_state is not None:
+            key = self.layer_ids[i] + ".attn_state"
+            saved = incremental_state.get(key, {})
+            if "prev_key" in saved:  # :451-467
+                k = torch.cat([saved["prev_key"].view(B * H, -1, hd), k], dim=1)
+                v = torch.cat([saved["prev_value"].view(B * H, -1, hd), v], dim=1)
+            saved["prev_key"] = k.view(B, H, -1, hd)
+            saved["prev_value"] = v.view(B, H, -1, hd)
+            saved["prev_key_padding_mask"] = key_padding_mask
+            incremental_state[key] = saved
+        o = self.attention_core(q, k, v, B, attn_mask, key_padding_mask)
+        o = o.transpose(0, 1).contiguous().view(T, B, D)  # :552
+        return self._linear(o, p + "out_proj.weight", None), self.w[p + "out_proj.bias"]
+
+    def _layer(self, i, x, incremental_state, attn_mask, key_padding_mask):
+        """transformer_decoder_layer.py:233-284 (pre-LN, ReLU FFN)."""
+        p = f"decoder.layers.{i}."
+        residual = x
+        h = self._r(layer_norm(x, self.w[p + "self_attn_layer_norm.weight"],
+                               self.w[p + "self_attn_layer_norm.bias"]))
+        a, a_bias = self._attention(i, h, incremental_state, attn_mask, key_padding_mask)
+        a = self._r(a + a_bias)  # :222-223
+        x = self._r(a + residual)  # :230
+        residual = x
+        h = self._r(layer_norm(x, self.w[p + "final_layer_norm.weight"],
+                               self.w[p + "final_layer_norm.bias"]))
+        u = F.relu(self._linear(h, p + "fc1.weight", p + "fc1.bias"))  # feedforward.py:21
+        z = self._linear(u, p + "fc2.weight", p + "fc2.bias")
+        return self._r(residual + z)  # :283
+
+    def extract_features(self, prev_output_tokens, incremental_state=None,
+                         self_attn_padding_mask=None):
+        """transformer_decoder.py:348-396 with forward_embedding :263-346."""
+        cfg = self.cfg
+        tokens = prev_output_tokens.to(self.device)
+        if self_attn_padding_mask is None and bool(tokens.eq(cfg.padding_idx).any()):
+            self_attn_padding_mask = tokens.eq(cfg.padding_idx)  # :357-361
+        positions = make_positions(tokens, cfg.padding_idx)
+        pos_emb = F.embedding(positions, self.w["decoder.embed_positions.weight"])
+        if incremental_state:  # non-empty dict == decode step (:324-327)
+            tokens = tokens[:, -1:]
+            pos_emb = pos_emb[:, -1:]
+        emb = F.embedding(tokens, self.w["decoder.embed_tokens.weight"])
+        x = self._r(emb + pos_emb)  # embed_scale == 1.0 (:89, :329-335)
+        x = x.transpose(0, 1).contiguous()  # [T, B, D] (:341)
+        T = x.shape[0]
+        if not incremental_state:  # :371-374
+            attn_mask = torch.triu(
+                torch.full((T, T), float("-inf"), device=self.device), 1)
+        else:
+            attn_mask = None
+        inner_states: List = [{"tok": emb, "pos": pos_emb, "emb": x}]
+        for i in range(cfg.decoder_layers):
+            x = self._layer(i, x, incremental_state, attn_mask, self_attn_padding_mask)
+        inner_states.append(x)
+        x = self._r(layer_norm(x, self.w["decoder.layer_norm.weight"],
+                               self.w["decoder.layer_norm.bias"]))  # :392-393
+        return x, {"inner_states": inner_states}
+
+    def output_layer(self, features):
+        """transformer_decoder.py:398-428: tied projection, no bias."""
+        return self._r(features @ self.w["decoder.embed_tokens.weight"].t())
+
+    def forward(self, prev_output_tokens, incremental_state=None, features_only=False,
+                self_attn_padding_mask=None):
+        x, extra = self.extract_features(prev_output_tokens, incremental_state,
+                                         self_attn_padding_mask)
+        if not features_only:
+            x = self.output_layer(x)
+        return x.transpose(0, 1).contiguous(), extra  # :536
+
+    __call__ = forward
+
+
+def greedy_generate(decoder, src_tokens: torch.Tensor, max_len_b: int, min_len: int = 1,
+                    pad: int = 1, eos: int = 2, stop: Optional[List[int]] = None,
+                    temperature: float = 1.0, max_positions: Optional[int] = None,
+                    return_step_logits: bool = False):
+    """SequenceGenerator._generate at beam 1 with greedy selection
+    (metaseq/sequence_generator.py:142-344; buffers :368-371; greedy :413-415).
+
+    ``decoder(tokens, incremental_state=dict)`` must return ``(logits[B, T, V], extra)``.
+    Returns {"tokens": [B, 1, max_len], "scores": [B, 1, max_len]} and, on request, the
+    list of logits tensors seen by the loop (prefill logits first).
+    """
+    stop = stop or []
+    incremental_state: Dict = {}
+    device = src_tokens.device
+    src_lengths = (src_tokens.ne(eos) & src_tokens.ne(pad)).long().sum(dim=1)  # :164-166
+    bsz = src_tokens.shape[0]
+    if max_positions is None:
+        max_positions = decoder.max_positions()
+    max_len = int(min(max_positions, max_len_b or 1e99))  # :182
+    min_len = min(max_len, min_len or 0)
+    assert min_len <= max_len
+    scores = torch.zeros(bsz, max_len, device=device).float()  # :368-371
+    tokens = torch.full((bsz, max_len), pad, dtype=torch.long, device=device)
+    start_step = src_tokens.shape[1]
+    tokens[:, :start_step] = src_tokens
+    step_logits = []
+    logits = decoder(tokens[:, :start_step], incremental_state=incremental_state)[0]
+    if return_step_logits:
+        step_logits.append(logits.clone())
+    preds = logits.float()
+    if temperature > 0 and temperature != 1.0:
+        preds = preds / temperature
+    lprobs = F.log_softmax(preds, dim=-1, dtype=torch.float32)  # :240
+    prompt_tokens = tokens[:, 1:start_step].unsqueeze(-1)
+    scores[:, 1:start_step] = torch.gather(lprobs, -1, prompt_tokens).squeeze(-1)  # :255-258
+    cut = []
+    for i in range(bsz):  # :262-267
+        prompt_len = int(src_lengths[i])
+        scores[i, prompt_len + 1:] = 0.0
+        cut.append(lprobs[i:i + 1, prompt_len])
+    lprobs = torch.cat(cut, dim=0)
+    eos_mask = torch.zeros(bsz, dtype=torch.bool, device=device)
+    for step in range(start_step, max_len):  # :271
+        if step < min_len:
+            lprobs[:, eos] = -math.inf
+            for t in stop:
+                lprobs[:, t] = -math.inf
+        lprobs[lprobs != lprobs] = -math.inf
+        lprobs[:, pad] = -math.inf
+        if step >= max_len - 1:  # :282-284
+            lprobs[:, :eos] = -math.inf
+            lprobs[:, eos + 1:] = -math.inf
+        lprobs[eos_mask, :eos] = -math.inf  # :292-293
+        lprobs[eos_mask, eos + 1:] = -math.inf
+        next_scores, next_toks = lprobs.max(dim=-1)  # :413-415
+        tokens[:, step] = next_toks
+        scores[:, step] = next_scores
+        eos_mask |= next_toks == eos
+        for t in stop:
+            eos_mask |= next_toks == t
+        if bool(torch.all(eos_mask)):
+            break
+        logits = decoder(tokens[:, :step + 1], incremental_state=incremental_state)[0]
+        if return_step_logits:
+            step_logits.append(logits.clone())
+        preds = logits.float()
+        if temperature > 0 and temperature != 1.0:
+            preds = preds / temperature
+        lprobs = F.log_softmax(preds, dim=-1, dtype=torch.float32)[:, -1, :]
+    out = {"tokens": tokens.view(bsz, 1, -1), "scores": scores.view(bsz, 1, -1)}
+    if return_step_logits:
+        out["step_logits"] = step_logits
+    return out

@@ -1,0 +1,64 @@
+"""CPU-side checks of the boundary: the shared library loads, exports every symbol the header
+declares, and the Python binding's signature table matches the header."""
+import ctypes
+import os
+import re
+
+import pytest
+
+from metaseq_amd import _capi
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "metaseq_amd.h")
+
+
+def _declared():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    decls = {}
+    for m in re.finditer(r"\b(msa_\w+)\s*\(([^;{]*?)\)\s*;", text, flags=re.S):
+        args = [a.strip() for a in m.group(2).split(",") if a.strip() and a.strip() != "void"]
+        decls[m.group(1)] = args
+    return decls
+
+
+def test_library_exports_every_declared_symbol():
+    if not os.path.exists(_capi.LIB_PATH):
+        from metaseq_amd.csrc.build import build
+        build(force=True, verbose=False)
+    lib = ctypes.CDLL(_capi.LIB_PATH)
+    decls = _declared()
+    assert len(decls) >= 12
+    for name in decls:
+        assert hasattr(lib, name), name
+
+
+def test_binding_table_matches_header_arity():
+    decls = _declared()
+    for name, argtypes in _capi.SIGNATURES.items():
+        assert name in decls, name
+        assert len(argtypes) == len(decls[name]), (name, len(argtypes), decls[name])
+    for name in decls:
+        assert name in _capi.SIGNATURES or name in _capi.OTHER_SYMBOLS, name
+
+
+def test_loader_reports_version_and_fails_loudly_without_library(monkeypatch, tmp_path):
+    lib = _capi.load()
+    assert lib.msa_version() >= 1
+    monkeypatch.setattr(_capi, "_lib", None)
+    monkeypatch.setattr(_capi, "LIB_PATH", str(tmp_path / "missing.so"))
+    with pytest.raises(RuntimeError, match="no non-HIP fallback"):
+        _capi.load()
+
+
+def test_argument_validation_needs_no_gpu():
+    """Entry points reject bad arguments before touching the device."""
+    lib = _capi.load()
+    assert lib.msa_layernorm_f16(None, None, None, None, 1, 64, 1e-5, None) == -1
+    assert b"null pointer" in lib.msa_last_error()
+    one = ctypes.c_void_p(16)
+    assert lib.msa_linear_f16(one, one, None, None, one, 4, 8, 40, 0, None, 0, None) == -1
+    assert b"multiple of 32" in lib.msa_last_error()
+    assert lib.msa_attention_f16(one, one, one, None, 0, one, 1, 1, 64, 2, 9, 10, None) == -2
+    with pytest.raises(ValueError):
+        _capi.check(-2, lib)

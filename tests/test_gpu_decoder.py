@@ -1,0 +1,194 @@
+"""End-to-end parity of the HIP decoder and generator against the oracle on identical seeded
+weights and token ids.
+
+Tolerances are the benchmark's: fp16 logits within max-abs 2e-2 and mean-abs 2e-3 of the
+reference forward, and identical greedy tokens over the first 32 generated tokens."""
+import pytest
+import torch
+
+from metaseq_amd import (Dictionary, OPTConfig, SequenceGenerator, TransformerLanguageModel,
+                         opt_config, random_prompts, random_state_dict)
+from oracle.opt_oracle import greedy_generate
+from tests.common import make_oracle, tiny_cfg
+from tests.scripted import CASES, ScriptedDecoder
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+MAX_ABS, MEAN_ABS = 2e-2, 2e-3
+
+
+def check_logits(got, want, what):
+    got, want = got.float().cpu(), want.float().cpu()
+    assert got.shape == want.shape, (what, got.shape, want.shape)
+    d = (got - want).abs()
+    print("%s: max-abs %.3e mean-abs %.3e" % (what, float(d.max()), float(d.mean())), flush=True)
+    assert float(d.max()) <= MAX_ABS, what
+    assert float(d.mean()) <= MEAN_ABS, what
+
+
+def build(cfg, seed=1234, int8=False):
+    sd = random_state_dict(cfg, seed=seed, dtype=torch.float16)
+    model = TransformerLanguageModel.build_model(cfg, sd, device=DEV)
+    if int8:
+        model.decoder.quantize_int8_()
+        sd = {k: v.cpu() for k, v in model.decoder.dequantized_state_dict().items()}
+    return model, sd
+
+
+def run_generate(model, cfg, src, max_len_b, min_len):
+    gen = SequenceGenerator([model], Dictionary(cfg.vocab_size), beam_size=1,
+                            max_len_b=max_len_b, min_len=min_len)
+    return gen.generate([model], {"net_input": {"src_tokens": src.to(DEV)}})
+
+
+@pytest.mark.parametrize("dim,heads", [(128, 2), (256, 2)])  # head_dim 64 and 128
+@pytest.mark.parametrize("padded", [False, True])
+@pytest.mark.parametrize("int8", [False, True])
+def test_tiny_forward_matches_oracle(dim, heads, padded, int8):
+    print("tiny", dim, heads, padded, int8, flush=True)
+    cfg = tiny_cfg(layers=2, dim=dim, heads=heads, vocab=128, max_pos=64)
+    model, sd = build(cfg, seed=7, int8=int8)
+    oracle = make_oracle(cfg, sd, torch.float16)
+    toks = random_prompts(cfg, 3, 20, seed=5)
+    if padded:
+        toks[1, 15:] = 1
+        toks[2, 9:] = 1
+    P = 12
+    inc_o, inc_h = {}, {}
+    want = oracle(toks[:, :P], incremental_state=inc_o)[0]
+    got = model(toks[:, :P].to(DEV), incremental_state=inc_h)[0]
+    assert inc_h, "the caller's dict must become non-empty after the prefill"
+    valid = toks[:, :P].ne(1)
+    check_logits(got.cpu()[valid], want[valid], "prefill")
+    for t in range(P, 21):
+        want = oracle(toks[:, :t + 1], incremental_state=inc_o)[0]
+        got = model.decoder(toks[:, :t + 1].to(DEV), incremental_state=inc_h)[0]
+        assert got.shape == (3, 1, cfg.vocab_size)
+        v = toks[:, t].ne(1)
+        check_logits(got.cpu()[v], want[v], "step %d" % t)
+
+
+def test_incremental_equals_full_recompute_on_device():
+    """Size-independent property: the logits of decode step t equal the last row of a fresh
+    prefill over tokens[:t+1] (same kernels except attention T=1 vs T>1 and skinny vs tiled
+    GEMM, so equality is to rounding)."""
+    cfg = opt_config("125m", max_target_positions=256)
+    model, _ = build(cfg, seed=3)
+    toks = random_prompts(cfg, 4, 80, seed=8).to(DEV)
+    inc = {}
+    model(toks[:, :70], incremental_state=inc)
+    for t in range(70, 81):
+        step = model.decoder(toks[:, :t + 1], incremental_state=inc)[0]
+        full = model(toks[:, :t + 1])[0][:, -1:]
+        check_logits(step, full, "incremental vs full t=%d" % t)
+
+
+def test_forward_is_deterministic():
+    cfg = opt_config("125m", max_target_positions=128)
+    model, _ = build(cfg, seed=4)
+    toks = random_prompts(cfg, 8, 40, seed=2).to(DEV)
+    outs = []
+    for _ in range(2):
+        inc = {}
+        a = model(toks[:, :32], incremental_state=inc)[0]
+        b = model.decoder(toks[:, :33], incremental_state=inc)[0]
+        outs.append((a.clone(), b.clone()))
+    assert torch.equal(outs[0][0], outs[1][0]) and torch.equal(outs[0][1], outs[1][1])
+
+
+@pytest.mark.parametrize("int8", [False, True])
+def test_config1_opt125m_greedy_matches_oracle(int8):
+    """BASELINE config 1: OPT-125m shape, batch 1, EOS + 32 random ids, greedy 32 tokens."""
+    cfg = opt_config("125m")
+    model, sd = build(cfg, seed=1234, int8=int8)
+    src = random_prompts(cfg, 1, 32, seed=4321)
+    G = 32
+    max_len_b = src.shape[1] + G + 1
+    oracle = make_oracle(cfg, sd, torch.float16)
+    want = greedy_generate(oracle, src, max_len_b=max_len_b, min_len=max_len_b - 1,
+                           return_step_logits=True)
+    got = run_generate(model, cfg, src, max_len_b, max_len_b - 1)
+    wt, gt = want["tokens"][0, 0], got["tokens"][0, 0].cpu()
+    print("oracle tokens", wt.tolist(), "\nhip    tokens", gt.tolist(), flush=True)
+    assert torch.equal(gt, wt), "greedy tokens diverge at %s" % (
+        (gt != wt).nonzero()[:1].tolist())
+    assert torch.allclose(got["scores"][0, 0].cpu(), want["scores"][0, 0], atol=5e-2)
+    # teacher-forced logits along the same token path
+    inc = {}
+    toks = wt.unsqueeze(0).to(DEV)
+    n0 = src.shape[1]
+    check_logits(model(toks[:, :n0], incremental_state=inc)[0], want["step_logits"][0], "prefill")
+    for i, t in enumerate(range(n0, n0 + G)):
+        got_l = model.decoder(toks[:, :t + 1], incremental_state=inc)[0]
+        check_logits(got_l, want["step_logits"][i + 1], "step %d" % t)
+    # and the fp32 oracle stays within the same tolerance of the fp16 path
+    o32 = make_oracle(cfg, sd, torch.float32)
+    check_logits(model(toks[:, :n0])[0], o32(src)[0], "prefill vs fp32 oracle")
+
+
+def test_batch4_padded_generation_matches_oracle():
+    cfg = opt_config("125m", max_target_positions=128)
+    model, sd = build(cfg, seed=99)
+    src = random_prompts(cfg, 4, 24, seed=17)
+    src[1, 20:] = 1
+    src[3, 11:] = 1
+    oracle = make_oracle(cfg, sd, torch.float16)
+    max_len_b = src.shape[1] + 17
+    want = greedy_generate(oracle, src, max_len_b=max_len_b, min_len=max_len_b - 1)
+    got = run_generate(model, cfg, src, max_len_b, max_len_b - 1)
+    assert torch.equal(got["tokens"].cpu(), want["tokens"])
+    assert torch.allclose(got["scores"].cpu(), want["scores"], atol=5e-2)
+
+
+@pytest.mark.parametrize("name", sorted(CASES))
+def test_generator_scripted_known_answers(name):
+    """The product generator's bookkeeping (fused select kernel, finished rows, stop tokens,
+    forced eos, padded rows, early exit) against the hand-derived tables."""
+    c = CASES[name]
+    dec = ScriptedDecoder(c["script"], vocab=6, device=DEV, dtype=torch.float16)
+    gen = SequenceGenerator([dec], Dictionary(6), max_len_b=c["max_len_b"], min_len=c["min_len"],
+                            stop=c["stop"])
+    out = gen.generate([dec], {"net_input": {"src_tokens": torch.tensor(c["src"], device=DEV)}})
+    assert out["tokens"][:, 0].cpu().tolist() == c["tokens"]
+    assert torch.allclose(out["scores"][:, 0].cpu(), torch.tensor(c["scores"]), atol=2e-3)
+    assert dec.calls == c["calls"]
+
+
+def test_need_logprobs_and_beam_replicas():
+    cfg = tiny_cfg(layers=1, dim=128, heads=2, vocab=64, max_pos=32)
+    model, sd = build(cfg, seed=5)
+    src = random_prompts(cfg, 2, 5, seed=3)
+    gen = SequenceGenerator([model], Dictionary(cfg.vocab_size), beam_size=2, max_len_b=10,
+                            min_len=9, need_logprobs=True)
+    out = gen.generate([model], {"net_input": {"src_tokens": src.to(DEV)}})
+    assert out["tokens"].shape == (2, 2, 10) and out["distributions"].shape == (2, 2, 10, 64)
+    assert torch.equal(out["tokens"][:, 0], out["tokens"][:, 1])  # replicas of a greedy run
+    oracle = make_oracle(cfg, sd, torch.float16)
+    want = greedy_generate(oracle, src, max_len_b=10, min_len=9)
+    assert torch.equal(out["tokens"][:, 0].cpu(), want["tokens"][:, 0])
+
+
+def test_errors_are_loud():
+    cfg = tiny_cfg(layers=1, dim=128, heads=2, vocab=64, max_pos=16)
+    model, _ = build(cfg, seed=5)
+    with pytest.raises(RuntimeError):
+        model(torch.tensor([[2, 5, 6]]))  # CPU tensor: no CPU path exists
+    with pytest.raises(ValueError):
+        model(torch.full((1, 40), 5, device=DEV))  # longer than the learned positions
+    inc = {}
+    model(torch.tensor([[2, 5, 6]], device=DEV), incremental_state=inc)
+    with pytest.raises(AssertionError):
+        model.decoder(torch.tensor([[2, 5, 6, 7, 8]], device=DEV), incremental_state=inc)
+    with pytest.raises(NotImplementedError):
+        SequenceGenerator([model], Dictionary(64), topp=0.9)
+    with pytest.raises(IndexError):
+        SequenceGenerator([model], Dictionary(64), max_len_b=8).generate(
+            [model], {"net_input": {"src_tokens": torch.tensor([[5, 6, 7]], device=DEV)}})
+
+
+def test_state_dict_uses_reference_names():
+    cfg = tiny_cfg(layers=1, dim=128, heads=2, vocab=64, max_pos=16)
+    model, sd = build(cfg, seed=5)
+    keys = set(model.state_dict().keys())
+    assert keys == set(sd.keys())
+    assert tuple(model.state_dict()["decoder.layers.0.self_attn.qkv_proj.weight"].shape) == (384, 128)

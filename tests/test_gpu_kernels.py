@@ -1,0 +1,310 @@
+"""Per-kernel parity through the C ABI: every entry point of libmetaseq_amd.so against the
+oracle's restatement of the same reference op on identical seeded inputs.
+
+Tolerance: both sides accumulate in fp32 and round to fp16 at the same points, so results
+may differ only where a different fp32 summation order straddles an fp16 rounding boundary:
+at most 1 fp16 ulp on a small fraction of elements (integer outputs: bit-exact)."""
+import ctypes
+import sys
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import opt_oracle as O
+from tests.fp16util import assert_fp16_close
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda"
+
+
+def r16(t):
+    return t.to(torch.float16).float()
+
+
+@pytest.fixture(scope="module")
+def lib():
+    from metaseq_amd import _capi
+    return _capi.load()
+
+
+def P(t):
+    return None if t is None else t.data_ptr()
+
+
+def ok(rc, lib):
+    assert rc == 0, lib.msa_last_error().decode()
+
+
+def rnd(*shape, seed=0, std=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(*shape, generator=g) * std).half()
+
+
+@pytest.mark.parametrize("rows,D", [(1, 64), (32, 768), (7, 2048), (32, 4096), (33, 7168),
+                                    (32, 9216), (300, 1024)])
+def test_layernorm(lib, rows, D):
+    print("layernorm", rows, D, flush=True)
+    x = rnd(rows, D, seed=1)
+    g = (1 + rnd(D, seed=2, std=0.1).float()).half()
+    b = rnd(D, seed=3, std=0.1)
+    want = O.layer_norm(x, g, b).half()
+    y = torch.empty(rows, D, dtype=torch.float16, device=DEV)
+    ok(lib.msa_layernorm_f16(P(x.to(DEV)), P(g.to(DEV)), P(b.to(DEV)), P(y), rows, D, 1e-5, None),
+       lib)
+    torch.cuda.synchronize()
+    assert_fp16_close(y, want, what="layernorm")
+
+
+def test_layernorm_rejects_bad_dim(lib):
+    x = torch.zeros(4, 12, dtype=torch.float16, device=DEV)
+    assert lib.msa_layernorm_f16(P(x), P(x), P(x), P(x), 4, 12, 1e-5, None) == -1
+    assert b"multiple of 8" in lib.msa_last_error()
+
+
+@pytest.mark.parametrize("T_out", [1, 9])
+def test_embed_positions_and_sum(lib, T_out):
+    print("embed", T_out, flush=True)
+    V, D, n, B, pad = 50, 64, 9, 4, 1
+    E, Ptab = rnd(V, D, seed=4), rnd(n + 8, D, seed=5)
+    g = torch.Generator().manual_seed(6)
+    toks = torch.randint(4, V, (B, 12), generator=g)
+    toks[:, 0] = 2
+    toks[1, 3:5] = pad
+    toks[2, 6:9] = pad        # right padded row (last token is pad)
+    toks[3, 0:2] = pad        # left padded row
+    view = toks[:, :n]        # strided view, as the generator passes tokens[:, :step + 1]
+    pos = O.make_positions(view, pad)
+    want_pos = pos[:, n - T_out:]
+    want = r16(F.embedding(view[:, n - T_out:], E.float()) + F.embedding(want_pos, Ptab.float()))
+    td = toks.to(DEV)
+    x = torch.empty(B * T_out, D, dtype=torch.float16, device=DEV)
+    po = torch.empty(B, T_out, dtype=torch.long, device=DEV)
+    st = torch.zeros(1, dtype=torch.int32, device=DEV)
+    ok(lib.msa_embed_f16(P(td), td.stride(0), B, n, T_out, P(E.to(DEV)), V, P(Ptab.to(DEV)),
+                         Ptab.shape[0], pad, D, P(x), P(po), P(st), None), lib)
+    torch.cuda.synchronize()
+    assert torch.equal(po.cpu(), want_pos)
+    assert torch.equal(x.cpu().float().view(B, T_out, D), want)
+    assert int(st) == 0
+
+
+def test_embed_flags_out_of_range_ids(lib):
+    V, D = 20, 64
+    E, Ptab = rnd(V, D), rnd(6, D)
+    toks = torch.tensor([[2, 5, 25]], device=DEV)
+    x = torch.empty(1, D, dtype=torch.float16, device=DEV)
+    st = torch.zeros(1, dtype=torch.int32, device=DEV)
+    ok(lib.msa_embed_f16(P(toks), 3, 1, 3, 1, P(E.to(DEV)), V, P(Ptab.to(DEV)), 6, 1, D, P(x),
+                         None, P(st), None), lib)
+    torch.cuda.synchronize()
+    assert int(st) == 1
+
+
+LINEAR_SHAPES = [
+    # M, N, K
+    (1, 96, 64), (8, 768, 768), (32, 3072, 768), (32, 768, 3072), (33, 2048, 2048),
+    (64, 4096, 4096), (17, 50272, 768), (65, 768, 768), (200, 2304, 768), (513, 4096, 1024),
+    (129, 1000, 96),
+]
+
+
+@pytest.mark.parametrize("M,N,K", LINEAR_SHAPES)
+@pytest.mark.parametrize("epi", ["plain", "bias", "bias_relu", "bias_res"])
+def test_linear_f16(lib, M, N, K, epi):
+    print("linear", M, N, K, epi, flush=True)
+    x, W = rnd(M, K, seed=7), rnd(N, K, seed=8, std=0.05)
+    b = rnd(N, seed=9, std=0.1) if epi != "plain" else None
+    res = rnd(M, N, seed=10) if epi == "bias_res" else None
+    want = O.linear(x.float(), W.float(), None if b is None else b.float(), r16)
+    if epi == "bias_relu":
+        want = F.relu(want)
+    if res is not None:
+        want = r16(want + res.float())
+    y = torch.full((M, N), float("nan"), dtype=torch.float16, device=DEV)
+    dres = None if res is None else res.to(DEV)
+    ok(lib.msa_linear_f16(P(x.to(DEV)), P(W.to(DEV)), P(None if b is None else b.to(DEV)),
+                          P(dres), P(y), M, N, K, 1 if epi == "bias_relu" else 0, None, 0, None),
+       lib)
+    torch.cuda.synchronize()
+    assert_fp16_close(y, want.half(), what="linear %s" % epi)
+
+
+def test_linear_in_place_residual(lib):
+    M, N, K = 32, 768, 3072
+    x, W, b, res = rnd(M, K, seed=1), rnd(N, K, seed=2, std=0.05), rnd(N, seed=3), rnd(M, N, seed=4)
+    want = r16(O.linear(x.float(), W.float(), b.float(), r16) + res.float())
+    y = res.to(DEV).clone()
+    ok(lib.msa_linear_f16(P(x.to(DEV)), P(W.to(DEV)), P(b.to(DEV)), P(y), P(y), M, N, K, 0, None,
+                          0, None), lib)
+    torch.cuda.synchronize()
+    assert_fp16_close(y, want.half(), what="in-place residual")
+
+
+def test_linear_rejects_bad_shapes(lib):
+    x = torch.zeros(4, 40, dtype=torch.float16, device=DEV)
+    assert lib.msa_linear_f16(P(x), P(x), None, None, P(x), 4, 8, 40, 0, None, 0, None) == -1
+    assert lib.msa_linear_f16(None, P(x), None, None, P(x), 4, 8, 32, 0, None, 0, None) == -1
+    assert lib.msa_linear_f16(P(x), P(x), None, None, P(x), 4, 8, 32, 8, None, 0, None) == -1
+
+
+@pytest.mark.parametrize("M,N,K", [(8, 768, 768), (64, 3072, 768), (32, 768, 3072),
+                                   (200, 2304, 768)])
+def test_linear_w8a16(lib, M, N, K):
+    print("w8a16", M, N, K, flush=True)
+    x, W, b = rnd(M, K, seed=7), rnd(N, K, seed=8, std=0.02), rnd(N, seed=9, std=0.1)
+    q, s = O.quantize_int8(W)
+    Wd = O.dequantize_int8(q, s)
+    want = O.linear(x.float(), Wd.float(), b.float(), r16)
+    y = torch.empty(M, N, dtype=torch.float16, device=DEV)
+    ok(lib.msa_linear_w8a16(P(x.to(DEV)), P(q.to(DEV)), P(s.to(DEV)), P(b.to(DEV)), None, P(y), M,
+                            N, K, 0, None, 0, None), lib)
+    torch.cuda.synchronize()
+    assert_fp16_close(y, want.half(), what="w8a16")
+
+
+@pytest.mark.parametrize("B,T,H,hd,S0", [(3, 1, 2, 64, 5), (2, 7, 4, 128, 0), (32, 1, 12, 64, 40),
+                                         (2, 70, 2, 64, 0)])
+@pytest.mark.parametrize("w8", [False, True])
+def test_qkv_proj_scatter(lib, B, T, H, hd, S0, w8):
+    print("qkv", B, T, H, hd, S0, w8, flush=True)
+    D = H * hd
+    S_cap = S0 + T + 3
+    x, W, b = rnd(B * T, D, seed=1), rnd(3 * D, D, seed=2, std=0.05), rnd(3 * D, seed=3, std=0.1)
+    if w8:
+        qw, sc = O.quantize_int8(W)
+        Wuse = O.dequantize_int8(qw, sc)
+    else:
+        Wuse = W
+    kvq = O.linear(x.float(), Wuse.float(), b.float(), r16)
+    k, v, q = kvq.split(D, dim=-1)
+    q = r16(q * (hd ** -0.5))
+    Kc = torch.zeros(B, H, S_cap, hd, dtype=torch.float16, device=DEV)
+    Vc = torch.zeros_like(Kc)
+    qo = torch.empty(B * T, D, dtype=torch.float16, device=DEV)
+    if w8:
+        ok(lib.msa_qkv_proj_w8a16(P(x.to(DEV)), P(qw.to(DEV)), P(sc.to(DEV)), P(b.to(DEV)), P(qo),
+                                  P(Kc), P(Vc), B, T, H, hd, S0, S_cap, D, None, 0, None), lib)
+    else:
+        ok(lib.msa_qkv_proj_f16(P(x.to(DEV)), P(W.to(DEV)), P(b.to(DEV)), P(qo), P(Kc), P(Vc), B,
+                                T, H, hd, S0, S_cap, D, None, 0, None), lib)
+    torch.cuda.synchronize()
+    assert_fp16_close(qo, q.half(), what="q")
+    want_k = k.view(B, T, H, hd).permute(0, 2, 1, 3)
+    want_v = v.view(B, T, H, hd).permute(0, 2, 1, 3)
+    assert_fp16_close(Kc[:, :, S0:S0 + T], want_k.half(), what="K cache")
+    assert_fp16_close(Vc[:, :, S0:S0 + T], want_v.half(), what="V cache")
+    # nothing outside the appended slice was touched
+    assert float(Kc[:, :, :S0].abs().sum()) == 0 and float(Kc[:, :, S0 + T:].abs().sum()) == 0
+
+
+def test_qkv_proj_capacity_error(lib):
+    x = torch.zeros(2, 128, dtype=torch.float16, device=DEV)
+    rc = lib.msa_qkv_proj_f16(P(x), P(x), P(x), P(x), P(x), P(x), 2, 1, 2, 64, 10, 10, 128, None,
+                              0, None)
+    assert rc == -2 and b"capacity" in lib.msa_last_error()
+
+
+def _oracle_core(dtype=torch.float16):
+    cfg = O.OracleConfig(1, 64, 1, 64, 8)
+    return O.OracleDecoder(cfg, {}, dtype=dtype)
+
+
+@pytest.mark.parametrize("B,H,hd,T,S0,masked", [
+    (2, 2, 64, 1, 0, False), (3, 2, 64, 1, 37, False), (2, 3, 128, 1, 300, True),
+    (32, 12, 64, 1, 65, False), (2, 2, 128, 9, 0, False), (2, 2, 64, 33, 0, True),
+    (1, 4, 128, 130, 0, False), (8, 32, 64, 1, 513, False), (2, 2, 64, 5, 11, False),
+])
+def test_attention(lib, B, H, hd, T, S0, masked):
+    print("attention", B, H, hd, T, S0, masked, flush=True)
+    D, S = H * hd, S0 + T
+    S_cap = S + 5
+    q = rnd(B * T, D, seed=1, std=0.3)
+    Kc = rnd(B, H, S_cap, hd, seed=2)
+    Vc = rnd(B, H, S_cap, hd, seed=3)
+    mask = None
+    if masked:
+        mask = torch.zeros(B, S, dtype=torch.bool)
+        mask[0, 1:3] = True
+        mask[B - 1, S // 2] = True
+    core = _oracle_core()
+    qq = q.float().view(B, T, H, hd).permute(0, 2, 1, 3).reshape(B * H, T, hd)
+    kk = Kc[:, :, :S].float().reshape(B * H, S, hd)
+    vv = Vc[:, :, :S].float().reshape(B * H, S, hd)
+    causal = torch.full((T, S), float("-inf")).triu(S0 + 1)  # query t sees keys 0..S0+t
+    want = core.attention_core(qq, kk, vv, B, causal, mask)
+    want = want.view(B, H, T, hd).permute(0, 2, 1, 3).reshape(B * T, D)
+    out = torch.empty(B * T, D, dtype=torch.float16, device=DEV)
+    dm = None if mask is None else mask.to(torch.uint8).to(DEV)
+    ok(lib.msa_attention_f16(P(q.to(DEV)), P(Kc.to(DEV)), P(Vc.to(DEV)), P(dm),
+                             0 if dm is None else dm.stride(0), P(out), B, H, hd, T, S0, S_cap,
+                             None), lib)
+    torch.cuda.synchronize()
+    assert_fp16_close(out, want.half(), max_frac=2e-2, what="attention")
+
+
+def test_attention_rejects(lib):
+    x = torch.zeros(64, 96, dtype=torch.float16, device=DEV)
+    assert lib.msa_attention_f16(P(x), P(x), P(x), None, 0, P(x), 1, 1, 96, 1, 0, 4, None) == -1
+    assert lib.msa_attention_f16(P(x), P(x), P(x), None, 0, P(x), 1, 1, 64, 1, 4, 4, None) == -2
+
+
+def _select(lib, logits, temperature=1.0, banned=(), stop=(), finished=None, force=0, eos=2):
+    B, V = logits.shape
+    tok = torch.zeros(B, 3, dtype=torch.long, device=DEV)
+    sc = torch.zeros(B, 3, dtype=torch.float32, device=DEV)
+    ba = (ctypes.c_int32 * max(1, len(banned)))(*banned)
+    sa = (ctypes.c_int32 * max(1, len(stop)))(*stop)
+    ok(lib.msa_greedy_select_f16(P(logits), logits.stride(0), B, V, temperature, ba, len(banned),
+                                 sa, len(stop), P(finished), force, eos, P(tok[:, 1]), 3,
+                                 P(sc[:, 1]), 3, None), lib)
+    torch.cuda.synchronize()
+    assert float(tok[:, 0].abs().sum()) == 0 and float(tok[:, 2].abs().sum()) == 0
+    return tok[:, 1].cpu(), sc[:, 1].cpu()
+
+
+@pytest.mark.parametrize("temperature", [1.0, 0.7])
+def test_greedy_select_matches_reference_passes(lib, temperature):
+    B, V = 5, 50272
+    logits = rnd(B, V, seed=3, std=1.3)
+    logits[1, 777] = logits[1].max() + 1       # clear winner
+    logits[2, 1] = 30.0                        # pad would win: must never be selected
+    logits[3, 100] = logits[3, 4000] = 20.0    # exact tie -> lowest index
+    logits[4, 2] = 25.0                        # eos wins but is banned below
+    lp = torch.log_softmax(logits.float() / temperature, -1)
+    lp[:, 1] = float("-inf")
+    lp[:, 2] = float("-inf")
+    want_s, want_t = lp.max(-1)
+    tok, sc = _select(lib, logits.to(DEV), temperature, banned=[1, 2])
+    assert torch.equal(tok, want_t)
+    assert torch.allclose(sc, want_s, atol=2e-5)
+    assert tok[3] == 100
+
+
+def test_greedy_select_finished_force_stop_nan(lib):
+    B, V = 4, 1000
+    logits = rnd(B, V, seed=5)
+    logits[3, 5] = float("nan")
+    fin = torch.tensor([1, 0, 0, 0], dtype=torch.uint8, device=DEV)
+    logits[1, 77] = 50.0   # row 1 picks the stop token 77
+    tok, sc = _select(lib, logits.to(DEV), banned=[1], stop=[77], finished=fin)
+    lp = torch.log_softmax(logits.float(), -1)
+    assert tok[0] == 2 and abs(float(sc[0]) - float(lp[0, 2])) < 2e-5   # finished row: eos only
+    assert tok[1] == 77
+    assert tok[3] == 0 and sc[3] == float("-inf")                         # NaN row: all -inf
+    assert fin.cpu().tolist() == [1, 1, 0, 0]
+    tok, sc = _select(lib, logits.to(DEV), banned=[1], force=1)
+    assert tok[:3].tolist() == [2, 2, 2]
+
+
+def test_target_logprob(lib):
+    R, V = 37, 50272
+    logits = rnd(R, V, seed=9, std=1.2)
+    tgt = torch.randint(0, V, (R,), generator=torch.Generator().manual_seed(1))
+    want = torch.log_softmax(logits.float(), -1).gather(1, tgt[:, None])[:, 0]
+    out = torch.empty(R, dtype=torch.float32, device=DEV)
+    d = logits.to(DEV)
+    ok(lib.msa_target_logprob_f16(P(d), d.stride(0), R, V, 1.0, P(tgt.to(DEV)), P(out), None), lib)
+    torch.cuda.synchronize()
+    assert torch.allclose(out.cpu(), want, atol=2e-5)
