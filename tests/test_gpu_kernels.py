@@ -29,8 +29,28 @@ def lib():
     return _capi.load()
 
 
+_KEEP = []
+
+
 def P(t):
     return None if t is None else t.data_ptr()
+
+
+def G(t):
+    """Device copy that stays alive until the end of the test (a temporary's memory would be
+    recycled by the caching allocator before the kernel reads it)."""
+    if t is None:
+        return None
+    d = t.to(DEV)
+    _KEEP.append(d)
+    return d
+
+
+@pytest.fixture(autouse=True)
+def _drop_keepalive():
+    yield
+    torch.cuda.synchronize()
+    _KEEP.clear()
 
 
 def ok(rc, lib):
@@ -51,7 +71,7 @@ def test_layernorm(lib, rows, D):
     b = rnd(D, seed=3, std=0.1)
     want = O.layer_norm(x, g, b).half()
     y = torch.empty(rows, D, dtype=torch.float16, device=DEV)
-    ok(lib.msa_layernorm_f16(P(x.to(DEV)), P(g.to(DEV)), P(b.to(DEV)), P(y), rows, D, 1e-5, None),
+    ok(lib.msa_layernorm_f16(P(G(x)), P(G(g)), P(G(b)), P(y), rows, D, 1e-5, None),
        lib)
     torch.cuda.synchronize()
     assert_fp16_close(y, want, what="layernorm")
@@ -82,7 +102,7 @@ def test_embed_positions_and_sum(lib, T_out):
     x = torch.empty(B * T_out, D, dtype=torch.float16, device=DEV)
     po = torch.empty(B, T_out, dtype=torch.long, device=DEV)
     st = torch.zeros(1, dtype=torch.int32, device=DEV)
-    ok(lib.msa_embed_f16(P(td), td.stride(0), B, n, T_out, P(E.to(DEV)), V, P(Ptab.to(DEV)),
+    ok(lib.msa_embed_f16(P(td), td.stride(0), B, n, T_out, P(G(E)), V, P(G(Ptab)),
                          Ptab.shape[0], pad, D, P(x), P(po), P(st), None), lib)
     torch.cuda.synchronize()
     assert torch.equal(po.cpu(), want_pos)
@@ -96,7 +116,7 @@ def test_embed_flags_out_of_range_ids(lib):
     toks = torch.tensor([[2, 5, 25]], device=DEV)
     x = torch.empty(1, D, dtype=torch.float16, device=DEV)
     st = torch.zeros(1, dtype=torch.int32, device=DEV)
-    ok(lib.msa_embed_f16(P(toks), 3, 1, 3, 1, P(E.to(DEV)), V, P(Ptab.to(DEV)), 6, 1, D, P(x),
+    ok(lib.msa_embed_f16(P(toks), 3, 1, 3, 1, P(G(E)), V, P(G(Ptab)), 6, 1, D, P(x),
                          None, P(st), None), lib)
     torch.cuda.synchronize()
     assert int(st) == 1
@@ -124,11 +144,14 @@ def test_linear_f16(lib, M, N, K, epi):
         want = r16(want + res.float())
     y = torch.full((M, N), float("nan"), dtype=torch.float16, device=DEV)
     dres = None if res is None else res.to(DEV)
-    ok(lib.msa_linear_f16(P(x.to(DEV)), P(W.to(DEV)), P(None if b is None else b.to(DEV)),
+    ok(lib.msa_linear_f16(P(G(x)), P(G(W)), P(G(b)),
                           P(dres), P(y), M, N, K, 1 if epi == "bias_relu" else 0, None, 0, None),
        lib)
     torch.cuda.synchronize()
-    assert_fp16_close(y, want.half(), what="linear %s" % epi)
+    # with a second rounding point (bias / residual add) a 1-ulp difference of the intermediate
+    # survives at the intermediate's magnitude even where the final value cancels to ~0
+    atol = 2e-5 if epi == "plain" else float(want.abs().max()) * 2 ** -10
+    assert_fp16_close(y, want.half(), atol=atol, what="linear %s" % epi)
 
 
 def test_linear_in_place_residual(lib):
@@ -136,10 +159,11 @@ def test_linear_in_place_residual(lib):
     x, W, b, res = rnd(M, K, seed=1), rnd(N, K, seed=2, std=0.05), rnd(N, seed=3), rnd(M, N, seed=4)
     want = r16(O.linear(x.float(), W.float(), b.float(), r16) + res.float())
     y = res.to(DEV).clone()
-    ok(lib.msa_linear_f16(P(x.to(DEV)), P(W.to(DEV)), P(b.to(DEV)), P(y), P(y), M, N, K, 0, None,
+    ok(lib.msa_linear_f16(P(G(x)), P(G(W)), P(G(b)), P(y), P(y), M, N, K, 0, None,
                           0, None), lib)
     torch.cuda.synchronize()
-    assert_fp16_close(y, want.half(), what="in-place residual")
+    assert_fp16_close(y, want.half(), atol=float(want.abs().max()) * 2 ** -10,
+                      what="in-place residual")
 
 
 def test_linear_rejects_bad_shapes(lib):
@@ -158,10 +182,10 @@ def test_linear_w8a16(lib, M, N, K):
     Wd = O.dequantize_int8(q, s)
     want = O.linear(x.float(), Wd.float(), b.float(), r16)
     y = torch.empty(M, N, dtype=torch.float16, device=DEV)
-    ok(lib.msa_linear_w8a16(P(x.to(DEV)), P(q.to(DEV)), P(s.to(DEV)), P(b.to(DEV)), None, P(y), M,
+    ok(lib.msa_linear_w8a16(P(G(x)), P(G(q)), P(G(s)), P(G(b)), None, P(y), M,
                             N, K, 0, None, 0, None), lib)
     torch.cuda.synchronize()
-    assert_fp16_close(y, want.half(), what="w8a16")
+    assert_fp16_close(y, want.half(), atol=float(want.abs().max()) * 2 ** -10, what="w8a16")
 
 
 @pytest.mark.parametrize("B,T,H,hd,S0", [(3, 1, 2, 64, 5), (2, 7, 4, 128, 0), (32, 1, 12, 64, 40),
@@ -184,17 +208,18 @@ def test_qkv_proj_scatter(lib, B, T, H, hd, S0, w8):
     Vc = torch.zeros_like(Kc)
     qo = torch.empty(B * T, D, dtype=torch.float16, device=DEV)
     if w8:
-        ok(lib.msa_qkv_proj_w8a16(P(x.to(DEV)), P(qw.to(DEV)), P(sc.to(DEV)), P(b.to(DEV)), P(qo),
+        ok(lib.msa_qkv_proj_w8a16(P(G(x)), P(G(qw)), P(G(sc)), P(G(b)), P(qo),
                                   P(Kc), P(Vc), B, T, H, hd, S0, S_cap, D, None, 0, None), lib)
     else:
-        ok(lib.msa_qkv_proj_f16(P(x.to(DEV)), P(W.to(DEV)), P(b.to(DEV)), P(qo), P(Kc), P(Vc), B,
+        ok(lib.msa_qkv_proj_f16(P(G(x)), P(G(W)), P(G(b)), P(qo), P(Kc), P(Vc), B,
                                 T, H, hd, S0, S_cap, D, None, 0, None), lib)
     torch.cuda.synchronize()
-    assert_fp16_close(qo, q.half(), what="q")
+    atol = float(kvq.abs().max()) * 2 ** -10
+    assert_fp16_close(qo, q.half(), atol=atol, what="q")
     want_k = k.view(B, T, H, hd).permute(0, 2, 1, 3)
     want_v = v.view(B, T, H, hd).permute(0, 2, 1, 3)
-    assert_fp16_close(Kc[:, :, S0:S0 + T], want_k.half(), what="K cache")
-    assert_fp16_close(Vc[:, :, S0:S0 + T], want_v.half(), what="V cache")
+    assert_fp16_close(Kc[:, :, S0:S0 + T], want_k.half(), atol=atol, what="K cache")
+    assert_fp16_close(Vc[:, :, S0:S0 + T], want_v.half(), atol=atol, what="V cache")
     # nothing outside the appended slice was touched
     assert float(Kc[:, :, :S0].abs().sum()) == 0 and float(Kc[:, :, S0 + T:].abs().sum()) == 0
 
@@ -237,11 +262,14 @@ def test_attention(lib, B, H, hd, T, S0, masked):
     want = want.view(B, H, T, hd).permute(0, 2, 1, 3).reshape(B * T, D)
     out = torch.empty(B * T, D, dtype=torch.float16, device=DEV)
     dm = None if mask is None else mask.to(torch.uint8).to(DEV)
-    ok(lib.msa_attention_f16(P(q.to(DEV)), P(Kc.to(DEV)), P(Vc.to(DEV)), P(dm),
+    ok(lib.msa_attention_f16(P(G(q)), P(G(Kc)), P(G(Vc)), P(dm),
                              0 if dm is None else dm.stride(0), P(out), B, H, hd, T, S0, S_cap,
                              None), lib)
     torch.cuda.synchronize()
-    assert_fp16_close(out, want.half(), max_frac=2e-2, what="attention")
+    # scores and probabilities are intermediate fp16 roundings: a 1-ulp flip of one of them
+    # moves the output by up to one ulp of the largest output
+    assert_fp16_close(out, want.half(), max_frac=2e-2, atol=float(want.abs().max()) * 2 ** -10,
+                      what="attention")
 
 
 def test_attention_rejects(lib):
@@ -305,6 +333,6 @@ def test_target_logprob(lib):
     want = torch.log_softmax(logits.float(), -1).gather(1, tgt[:, None])[:, 0]
     out = torch.empty(R, dtype=torch.float32, device=DEV)
     d = logits.to(DEV)
-    ok(lib.msa_target_logprob_f16(P(d), d.stride(0), R, V, 1.0, P(tgt.to(DEV)), P(out), None), lib)
+    ok(lib.msa_target_logprob_f16(P(d), d.stride(0), R, V, 1.0, P(G(tgt)), P(out), None), lib)
     torch.cuda.synchronize()
     assert torch.allclose(out.cpu(), want, atol=2e-5)
