@@ -202,7 +202,7 @@ def main():
         for i in range(cfg.decoder_layers):
             _capi.check(lib.msa_attention_f16(q.data_ptr(), cache.k(i).data_ptr(),
                                               cache.v(i).data_ptr(), None, 0, o.data_ptr(), B, H,
-                                              hd, 1, S_probe - 1, cache.capacity, stream))
+                                              hd, 1, S_probe - 1, cache.capacity, 0, stream))
     attn_all_layers()
     torch.cuda.synchronize()
     a0, a1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)

@@ -32,18 +32,52 @@ typedef enum {
   MSA_ERR_HIP = -3          /* a HIP runtime call or kernel launch failed  */
 } msa_status;
 
-/* epilogue flags for msa_linear_f16 / msa_linear_w8a16 */
-#define MSA_EPI_RELU 1u /* y = max(y, 0) after the bias add                       */
+/* flags */
+#define MSA_EPI_RELU 1u   /* y = max(y, 0) after the bias add                                  */
+#define MSA_IN_PACKED 2u  /* the input activation is in the packed layout (M <= 64, see below) */
+#define MSA_OUT_PACKED 4u /* write the output activation in the packed layout (M <= 64)        */
 
 const char* msa_last_error(void);
 int msa_version(void);
 
+/* ---- memory layouts --------------------------------------------------------------------------
+ * Weights are consumed in a TILE-PACKED layout: the 16 x 32 block of W[N,K] that one
+ * v_mfma_f32_16x16x32_f16 reads as its A operand is one contiguous KB in lane order, and the
+ * blocks of a 16-row tile follow each other along K, so a wave instruction reads a whole KB and
+ * a tile's K sweep is one linear HBM stream.
+ *   fp16: block (t = n/16, ks = k/32) at half offset (t*K/32 + ks)*512; lane l = 16*((k%32)/8) +
+ *         n%16 owns halves 8l..8l+7 = W[n][8*(k/8) .. +7].                N % 16 == 0, K % 32 == 0.
+ *   int8: block (t, ks8 = k/64) at byte offset (t*K/64 + ks8)*1024; lane l = 16g + r owns 16 bytes:
+ *         0..7 = W[16t+r][64ks8 + 8g ..+7], 8..15 = W[16t+r][64ks8 + 32 + 8g ..+7].   K % 64 == 0.
+ * The pack / unpack calls convert from / to row-major [N,K] (src != dst).
+ * Activations of at most 64 rows may be PACKED the same way (the MFMA B operand in lane order):
+ * with MB = ceil(M/16), element (m,k) sits at half offset
+ *   ((k/32*MB + m/16)*64 + 16*((k%32)/8) + m%16)*8 + k%8;   the buffer holds MB*16*K halves.
+ * No reference counterpart: the reference keeps torch's row-major tensors
+ * (metaseq/modules/megatron/mpu/layers.py:290). */
+int msa_pack_weight_f16(const void* src, void* dst, int N, int K, void* stream);
+int msa_unpack_weight_f16(const void* src, void* dst, int N, int K, void* stream);
+int msa_pack_weight_i8(const int8_t* src, int8_t* dst, int N, int K, void* stream);
+int msa_unpack_weight_i8(const int8_t* src, int8_t* dst, int N, int K, void* stream);
+
 /* Pre-LN LayerNorm forward: y[r,:] = round(gamma * (x[r,:] - mean) * rsqrt(var + eps) + beta),
- * mean / biased variance in fp32.  D % 8 == 0, D <= 16384.
+ * mean / biased variance in fp32.  D % 8 == 0, D <= 16384.  flags: MSA_OUT_PACKED.
  * Replaces metaseq/modules/layer_norm.py:28-33 -> apex cuApplyLayerNorm
  * (metaseq/modules/apex/layer_norm_cuda_kernel.cu:441-455, host :868-893). */
 int msa_layernorm_f16(const void* x, const void* gamma, const void* beta, void* y,
-                      int64_t rows, int D, float eps, void* stream);
+                      int64_t rows, int D, float eps, unsigned flags, void* stream);
+
+/* Tail of a split-K linear layer fused with the LayerNorm that follows it:
+ *   x[r,:] = round(round(round(sum_{s<S} part[s][r,:]) + bias) + x[r,:])          (in place)
+ *   y[r,:] = LayerNorm(x[r,:]; gamma, beta)      (skipped when gamma, beta and y are all NULL)
+ * part is fp32 [S, rows, D] as written by msa_linear_partial_*.  flags: MSA_OUT_PACKED (y).
+ * Replaces the bias and residual adds of metaseq/modules/transformer_decoder_layer.py:222-230
+ * (attention block) and :283 with metaseq/modules/megatron/mpu/layers.py:669-671 (fc2 bias),
+ * followed by the LayerNorm at :275, the next layer's :264 or the final one at
+ * metaseq/models/transformer_decoder.py:392-393. */
+int msa_residual_layernorm_f16(const float* part, int S, const void* bias, void* x,
+                               const void* gamma, const void* beta, void* y, int64_t rows, int D,
+                               float eps, unsigned flags, void* stream);
 
 /* Token + learned-position embedding for the last `T_out` columns of tokens[B, n]:
  *   pos(b,t) = pad_idx                      if tokens[b,t] == pad_idx
@@ -60,58 +94,65 @@ int msa_embed_f16(const int64_t* tokens, int64_t tok_stride, int B, int n, int T
                   const void* E, int V, const void* P, int n_pos_rows, int pad_idx, int D,
                   void* x, int64_t* positions_out, int32_t* status_dev, void* stream);
 
-/* y[M,N] = epilogue(x[M,K] . W[N,K]^T):
+/* y[M,N] = epilogue(x[M,K] . W[N,K]^T) with W tile-packed:
  *   t = round(acc); if bias: t = round(t + bias[n]); if RELU: t = max(t,0);
  *   if residual: t = round(t + residual[m,n]);  y[m,n] = t.
- * K % 32 == 0, N % 8 == 0.  M <= 64 selects the weight-streaming kernel (HBM bound),
- * larger M the LDS-tiled MFMA kernel.  `workspace` (fp32, >= msa_linear_workspace_bytes)
- * is used for split-K partial sums and tile counters and must be zero on first use; the
- * kernels leave the counter region zero again.
+ * N % 16 == 0, K % 32 == 0.  With MSA_IN_PACKED (M <= 64) the HBM-bound weight-streaming kernel
+ * runs; otherwise the LDS-tiled MFMA kernel (any M, row-major x).  residual is row-major and may
+ * alias a row-major y.  flags: MSA_EPI_RELU | MSA_IN_PACKED | MSA_OUT_PACKED.
  * Replaces LinearWithGradAccumulationAndAsyncCommunication.forward
- * (metaseq/modules/megatron/mpu/layers.py:290-292) as used by qkv_proj
- * (metaseq/modules/multihead_attention.py:316), out_proj (:553, bias and residual added in
+ * (metaseq/modules/megatron/mpu/layers.py:290-292) as used by out_proj
+ * (metaseq/modules/multihead_attention.py:553, bias and residual added in
  * metaseq/modules/transformer_decoder_layer.py:222-230), fc1/fc2
  * (metaseq/modules/feedforward.py:19-22; residual transformer_decoder_layer.py:283) and the
  * tied vocabulary projection (metaseq/models/transformer_decoder.py:413-420). */
-int msa_linear_f16(const void* x, const void* W, const void* bias, const void* residual,
-                   void* y, int64_t M, int N, int K, unsigned flags, void* workspace,
-                   size_t workspace_bytes, void* stream);
+int msa_linear_f16(const void* x, const void* Wp, const void* bias, const void* residual,
+                   void* y, int64_t M, int N, int K, unsigned flags, void* stream);
 
-/* Same contract with int8 weights Wq[N,K] and per-output-channel fp16 scales[N]:
+/* Same contract with tile-packed int8 weights Wq and per-output-channel fp16 scales[N]:
  * the product uses the dequantised weight round(Wq[n,k] * scales[n]) (formed in registers).
- * No reference counterpart: the reference hands int8 serving to FasterTransformer
+ * K % 64 == 0.  No reference counterpart: the reference hands int8 serving to FasterTransformer
  * (metaseq/scripts/convert_metaseq_ft.py:99-133); semantics are the benchmark's definition. */
 int msa_linear_w8a16(const void* x, const int8_t* Wq, const void* scales, const void* bias,
                      const void* residual, void* y, int64_t M, int N, int K, unsigned flags,
-                     void* workspace, size_t workspace_bytes, void* stream);
+                     void* stream);
 
-size_t msa_linear_workspace_bytes(int64_t M, int N, int K);
+/* Split-K form for the decode step (1 <= M <= 64, MSA_IN_PACKED required): K is cut into S
+ * ranges and part[s][m][n] (fp32, [S, M, N]) receives the exact fp32 partial sums of range s;
+ * the consumer adds them in slice order (msa_residual_layernorm_f16).  Used where N alone gives
+ * the chip too few weight tiles (out_proj, fc2).  msa_linear_default_splits suggests S. */
+int msa_linear_partial_f16(const void* x, const void* Wp, float* part, int64_t M, int N, int K,
+                           int S, unsigned flags, void* stream);
+int msa_linear_partial_w8a16(const void* x, const int8_t* Wq, const void* scales, float* part,
+                             int64_t M, int N, int K, int S, unsigned flags, void* stream);
+int msa_linear_default_splits(int64_t M, int N, int K);
 
 /* Fused QKV projection: kvq = round(round(x . Wqkv^T) + bqkv) with rows of Wqkv ordered
  * K | V | Q; then for row m = b*T + t and head h:
  *   Kcache[b,h,S0+t,:] = k,  Vcache[b,h,S0+t,:] = v,  q_out[m, h*hd:(h+1)*hd] = round(q * hd^-0.5).
- * Caches are [B, H, S_cap, hd] fp16.  Same size rules as msa_linear_f16 with N = 3*H*hd.
+ * Caches are [B, H, S_cap, hd] fp16, q_out row-major.  Same size rules as msa_linear_f16 with
+ * N = 3*H*hd.  flags: MSA_IN_PACKED.
  * Replaces metaseq/modules/multihead_attention.py:316-319 (projection + split), :429
  * (q scaling) and :449-479 (cache growth by torch.cat, here an in-place append). */
 int msa_qkv_proj_f16(const void* x, const void* Wqkv, const void* bqkv, void* q_out,
                      void* Kcache, void* Vcache, int B, int T, int H, int hd, int S0, int S_cap,
-                     int K, void* workspace, size_t workspace_bytes, void* stream);
+                     int K, unsigned flags, void* stream);
 int msa_qkv_proj_w8a16(const void* x, const int8_t* Wq, const void* scales, const void* bqkv,
                        void* q_out, void* Kcache, void* Vcache, int B, int T, int H, int hd,
-                       int S0, int S_cap, int K, void* workspace, size_t workspace_bytes,
-                       void* stream);
+                       int S0, int S_cap, int K, unsigned flags, void* stream);
 
 /* Causal attention of T new queries (already scaled, q[B*T, H*hd]) over the cache, whose
  * positions 0 .. S0+T-1 are valid: query t sees keys 0 .. S0+t.
  *   s = round(q . k);  s = -inf where key_pad_mask[b, key] != 0;
  *   p = round(softmax_fp32(s));  out[b*T+t, h*hd:(h+1)*hd] = round(sum_key p * v).
  * key_pad_mask (optional) is uint8 [B, mask_stride].  hd in {64, 128}.  T == 1 is the
- * bandwidth-bound decode kernel; T > 1 the prefill kernel.
+ * bandwidth-bound decode kernel; T > 1 the prefill kernel.  q is row-major; flags:
+ * MSA_OUT_PACKED (T == 1, B <= 64).
  * Replaces metaseq/modules/multihead_attention.py:492 (bmm q k^T), :516-531 (causal and
  * padding masks), :533-534 (fp32 softmax, cast back), :543-552 (bmm p v, transpose). */
 int msa_attention_f16(const void* q, const void* Kcache, const void* Vcache,
                       const uint8_t* key_pad_mask, int64_t mask_stride, void* out, int B, int H,
-                      int hd, int T, int S0, int S_cap, void* stream);
+                      int hd, int T, int S0, int S_cap, unsigned flags, void* stream);
 
 /* One step of greedy selection over fp16 logits[B, V] (row stride ld_logits), with the
  * generator's bookkeeping fused in:

@@ -13,27 +13,38 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "csrc", "libmetaseq_amd.so")
 
 MSA_EPI_RELU = 1
+MSA_IN_PACKED = 2
+MSA_OUT_PACKED = 4
 
 _P = c_void_p
 
 # name -> argtypes, in the order of include/metaseq_amd.h
 SIGNATURES = {
-    "msa_layernorm_f16": [_P, _P, _P, _P, c_int64, c_int, c_float, _P],
+    "msa_pack_weight_f16": [_P, _P, c_int, c_int, _P],
+    "msa_unpack_weight_f16": [_P, _P, c_int, c_int, _P],
+    "msa_pack_weight_i8": [_P, _P, c_int, c_int, _P],
+    "msa_unpack_weight_i8": [_P, _P, c_int, c_int, _P],
+    "msa_layernorm_f16": [_P, _P, _P, _P, c_int64, c_int, c_float, c_uint, _P],
+    "msa_residual_layernorm_f16": [_P, c_int, _P, _P, _P, _P, _P, c_int64, c_int, c_float, c_uint,
+                                   _P],
     "msa_embed_f16": [_P, c_int64, c_int, c_int, c_int, _P, c_int, _P, c_int, c_int, c_int, _P, _P,
                       _P, _P],
-    "msa_linear_f16": [_P, _P, _P, _P, _P, c_int64, c_int, c_int, c_uint, _P, c_size_t, _P],
-    "msa_linear_w8a16": [_P, _P, _P, _P, _P, _P, c_int64, c_int, c_int, c_uint, _P, c_size_t, _P],
+    "msa_linear_f16": [_P, _P, _P, _P, _P, c_int64, c_int, c_int, c_uint, _P],
+    "msa_linear_w8a16": [_P, _P, _P, _P, _P, _P, c_int64, c_int, c_int, c_uint, _P],
+    "msa_linear_partial_f16": [_P, _P, _P, c_int64, c_int, c_int, c_int, c_uint, _P],
+    "msa_linear_partial_w8a16": [_P, _P, _P, _P, c_int64, c_int, c_int, c_int, c_uint, _P],
+    "msa_linear_default_splits": [c_int64, c_int, c_int],
     "msa_qkv_proj_f16": [_P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
-                         _P, c_size_t, _P],
+                         c_uint, _P],
     "msa_qkv_proj_w8a16": [_P, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int,
-                           c_int, _P, c_size_t, _P],
+                           c_int, c_uint, _P],
     "msa_attention_f16": [_P, _P, _P, _P, c_int64, _P, c_int, c_int, c_int, c_int, c_int, c_int,
-                          _P],
+                          c_uint, _P],
     "msa_greedy_select_f16": [_P, c_int64, c_int, c_int, c_float, _P, c_int, _P, c_int, _P, c_int,
                               c_int, _P, c_int64, _P, c_int64, _P],
     "msa_target_logprob_f16": [_P, c_int64, c_int64, c_int, c_float, _P, _P, _P],
 }
-OTHER_SYMBOLS = ["msa_last_error", "msa_version", "msa_linear_workspace_bytes"]
+OTHER_SYMBOLS = ["msa_last_error", "msa_version"]
 
 _lib = None
 
@@ -56,8 +67,6 @@ def load():
     lib.msa_last_error.restype = c_char_p
     lib.msa_version.argtypes = []
     lib.msa_version.restype = c_int
-    lib.msa_linear_workspace_bytes.argtypes = [c_int64, c_int, c_int]
-    lib.msa_linear_workspace_bytes.restype = c_size_t
     _lib = lib
     return lib
 

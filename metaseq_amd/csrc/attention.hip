@@ -16,7 +16,8 @@ template <int HD>
 __global__ void attention_kernel(const half_t* __restrict__ q, const half_t* __restrict__ Kc,
                                  const half_t* __restrict__ Vc,
                                  const uint8_t* __restrict__ key_pad_mask, int64_t mask_stride,
-                                 half_t* __restrict__ out, int H, int T, int S0, int S_cap) {
+                                 half_t* __restrict__ out, int H, int T, int S0, int S_cap,
+                                 int out_mb) {
   constexpr int LPR = HD / 8;    // lanes per key row (16 bytes each)
   constexpr int RPW = 64 / LPR;  // key rows per wave instruction
   extern __shared__ float smem[];
@@ -126,7 +127,10 @@ __global__ void attention_kernel(const half_t* __restrict__ q, const half_t* __r
   for (int d = threadIdx.x; d < HD; d += blockDim.x) {
     float s = 0.f;
     for (int w = 0; w < nw; ++w) s += oacc[w][d];
-    out[((int64_t)b * T + t) * D + h * HD + d] = (half_t)s;
+    if (out_mb > 0)  // packed activation layout of the decode GEMMs (T == 1: row = b)
+      out[packed_act_offset(b, h * HD + d, out_mb)] = (half_t)s;
+    else
+      out[((int64_t)b * T + t) * D + h * HD + d] = (half_t)s;
   }
 }
 
@@ -134,7 +138,8 @@ __global__ void attention_kernel(const half_t* __restrict__ q, const half_t* __r
 
 extern "C" int msa_attention_f16(const void* q, const void* Kcache, const void* Vcache,
                                  const uint8_t* key_pad_mask, int64_t mask_stride, void* out, int B,
-                                 int H, int hd, int T, int S0, int S_cap, void* stream) {
+                                 int H, int hd, int T, int S0, int S_cap, unsigned flags,
+                                 void* stream) {
   MSA_REQUIRE(q && Kcache && Vcache && out, MSA_ERR_INVALID_ARG, "msa_attention_f16: null pointer");
   MSA_REQUIRE(B > 0 && H > 0 && T > 0 && S0 >= 0, MSA_ERR_INVALID_ARG,
               "msa_attention_f16: bad shape B=%d H=%d T=%d S0=%d", B, H, T, S0);
@@ -148,6 +153,11 @@ extern "C" int msa_attention_f16(const void* q, const void* Kcache, const void* 
               "msa_attention_f16: mask_stride %lld shorter than %d keys", (long long)mask_stride,
               S0 + T);
   MSA_REQUIRE(T <= 65535, MSA_ERR_INVALID_ARG, "msa_attention_f16: T=%d too large", T);
+  MSA_REQUIRE((flags & ~MSA_OUT_PACKED) == 0, MSA_ERR_INVALID_ARG,
+              "msa_attention_f16: unsupported flags 0x%x", flags);
+  MSA_REQUIRE(!(flags & MSA_OUT_PACKED) || (T == 1 && B <= 64), MSA_ERR_INVALID_ARG,
+              "msa_attention_f16: packed output needs T == 1 and B <= 64 (T=%d B=%d)", T, B);
+  const int out_mb = (flags & MSA_OUT_PACKED) ? (B + 15) / 16 : 0;
   const int64_t BH = (int64_t)B * H;
   // few (b,h) pairs: spend more waves on each so the chip still fills
   const int threads = (T == 1 && BH < 512) ? 1024 : 256;
@@ -157,11 +167,11 @@ extern "C" int msa_attention_f16(const void* q, const void* Kcache, const void* 
   if (hd == 64)
     hipLaunchKernelGGL(attention_kernel<64>, grid, dim3(threads), lds, s, (const half_t*)q,
                        (const half_t*)Kcache, (const half_t*)Vcache, key_pad_mask, mask_stride,
-                       (half_t*)out, H, T, S0, S_cap);
+                       (half_t*)out, H, T, S0, S_cap, out_mb);
   else
     hipLaunchKernelGGL(attention_kernel<128>, grid, dim3(threads), lds, s, (const half_t*)q,
                        (const half_t*)Kcache, (const half_t*)Vcache, key_pad_mask, mask_stride,
-                       (half_t*)out, H, T, S0, S_cap);
+                       (half_t*)out, H, T, S0, S_cap, out_mb);
   MSA_CHECK_LAUNCH("msa_attention_f16");
   return MSA_OK;
 }

@@ -35,6 +35,14 @@ void msa_set_error(const char* fmt, ...);
     }                                                                       \
   } while (0)
 
+// Packed activation layout for M <= 64 rows (the B operand of v_mfma_f32_16x16x32_f16, stored
+// in lane order): element (m, k) of a [M, K] activation with MB = ceil(M/16) row blocks lives
+// at half offset ((k/32 * MB + m/16) * 64 + 16*((k%32)/8) + m%16) * 8 + k%8.
+__host__ __device__ __forceinline__ int64_t packed_act_offset(int m, int k, int MB) {
+  return ((((int64_t)(k >> 5) * MB + (m >> 4)) * 64 + (((k & 31) >> 3) << 4) + (m & 15)) << 3) +
+         (k & 7);
+}
+
 // round-to-nearest-even fp32 -> fp16 -> fp32 (a "materialise in fp16" point)
 __device__ __forceinline__ float round_h(float v) { return (float)(half_t)v; }
 

@@ -1,15 +1,22 @@
 // y[M,N] = epilogue(x[M,K] . W[N,K]^T) on fp16 MFMA with fp32 accumulation.
 //
-// Two kernels behind one entry point:
-//   * skinny (M <= 64, the decode step): HBM-bound weight streaming.  A workgroup owns 16
-//     rows of W; its 4 waves take interleaved 32-wide K steps, load W straight from HBM into
-//     MFMA A-operand registers (16 bytes per lane, 64 contiguous bytes per row per
-//     instruction), multiply against the M activation rows (B operand) and reduce across
-//     waves through LDS in a fixed order, so results are run-to-run deterministic.
-//   * tiled (any M, the prefill): 128x128x32 LDS double-buffered tiles, 4 waves of 64x64,
-//     32x32x16 MFMA.
-// Both share one epilogue that reproduces the reference's fp16 rounding points, and a QKV
-// mode that scatters K/V into the per-layer cache and scales Q.
+// Weights live in HBM in a tile-packed layout (see pack kernels below): the 16 x 32 block of
+// W that one v_mfma_f32_16x16x32_f16 consumes as its A operand is one contiguous KB, stored in
+// the order the 64 lanes read it, and the blocks of one 16-row tile follow each other along K.
+// A wave instruction therefore reads one whole KB and a tile's K sweep is one linear stream.
+//
+// Two kernels:
+//   * stream (M <= 64, the decode step): HBM-bound.  A workgroup of 8 waves owns a contiguous
+//     range of 16-row tiles (and, with split-K, one K range); it walks the tiles 4 at a time,
+//     the waves taking interleaved K steps.  Activations come in the matching packed fragment
+//     layout from L2 and every activation fragment is reused for 4 weight tiles.  Fragments
+//     are double buffered several steps deep and the prefetch runs across tile-group
+//     boundaries, so the memory pipe never drains while a finished group is reduced across
+//     the waves through LDS (fixed order: results are run-to-run deterministic).
+//   * tiled (any M, the prefill): 128 x 128 x 32 LDS double-buffered tiles, 4 waves of 64 x 64,
+//     v_mfma_f32_32x32x16_f16.
+// Both share one epilogue that reproduces the reference's fp16 rounding points, and a QKV mode
+// that scatters K/V into the per-layer cache and scales Q.
 #include <math.h>
 
 #include "common.h"
@@ -24,6 +31,7 @@ struct Epilogue {
   half_t* y;
   int N;
   unsigned flags;
+  int out_mb;  // > 0: y is written in the packed activation layout with this many 16-row blocks
   // MODE_QKV
   half_t* q_out;
   half_t* Kc;
@@ -56,7 +64,10 @@ __device__ __forceinline__ void epilogue4(const Epilogue& e, int64_t m, int n, f
     half4_t o;
 #pragma unroll
     for (int i = 0; i < 4; ++i) o[i] = (half_t)t[i];
-    *reinterpret_cast<half4_t*>(e.y + m * e.N + n) = o;
+    if (e.out_mb > 0)
+      *reinterpret_cast<half4_t*>(e.y + packed_act_offset((int)m, n, e.out_mb)) = o;
+    else
+      *reinterpret_cast<half4_t*>(e.y + m * e.N + n) = o;
   } else {
     const int D = e.H * e.hd;
     const int part = n / D, c = n - part * D;  // 0 = K, 1 = V, 2 = Q
@@ -77,106 +88,222 @@ __device__ __forceinline__ void epilogue4(const Epilogue& e, int64_t m, int n, f
   }
 }
 
-// ---- int8 -> fp16 dequantisation in registers --------------------------------------
-// 8 int8 (two dwords) times an fp16 per-row scale -> 8 fp16, each round(q * scale).
+__device__ __forceinline__ half8_t zero8() { return half8_t{0, 0, 0, 0, 0, 0, 0, 0}; }
+
+// 8 int8 (two dwords) times an fp16 per-row scale -> 8 fp16, each round(q * scale)
 __device__ __forceinline__ half8_t dequant8(uint32_t lo, uint32_t hi, half_t scale) {
   half8_t r;
   const uint32_t w[2] = {lo, hi};
+  const float s = (float)scale;
 #pragma unroll
   for (int j = 0; j < 2; ++j) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int q = (int)(int8_t)((w[j] >> (8 * i)) & 0xff);
-      r[j * 4 + i] = (half_t)((float)q * (float)scale);
+      r[j * 4 + i] = (half_t)((float)q * s);
     }
   }
   return r;
 }
 
-// ---- skinny kernel --------------------------------------------------------------------
-constexpr int SK_THREADS = 256;
-constexpr int SK_WAVES = 4;
-constexpr int SK_ROWS = 16;  // W rows per workgroup
-constexpr int SK_U = 4;      // K steps in flight per wave
+// ---- weight packing ---------------------------------------------------------------------
+// fp16: block (tile t = n/16, step ks = k/32) at halves ((t * K/32 + ks) * 512); inside the block
+// lane l = 16*((k%32)/8) + n%16 owns halves l*8 .. l*8+7 = W[n][8*(k/8) .. +7].
+// int8: block (t, ks8 = k/64) at bytes ((t * K/64 + ks8) * 1024); lane l = 16*g + r owns 16 bytes:
+// bytes 0..7 = W[16t+r][64*ks8 + 8g .. +7] and bytes 8..15 = W[16t+r][64*ks8 + 32 + 8g .. +7],
+// i.e. the A fragments of the two 32-wide steps the block covers.
+__global__ __launch_bounds__(256) void pack_f16_kernel(const half_t* __restrict__ src,
+                                                       half_t* __restrict__ dst, int N, int K,
+                                                       bool unpack) {
+  const int64_t piece = (int64_t)blockIdx.x * 256 + threadIdx.x;  // one 16-byte piece
+  const int nks = K >> 5;
+  if (piece >= (int64_t)N * K / 8) return;
+  const int lane = (int)(piece & 63);
+  const int64_t blk = piece >> 6;
+  const int ks = (int)(blk % nks), t = (int)(blk / nks);
+  const int64_t rm = ((int64_t)t * 16 + (lane & 15)) * K + ks * 32 + (lane >> 4) * 8;
+  if (unpack)
+    *reinterpret_cast<half8_t*>(dst + rm) = *reinterpret_cast<const half8_t*>(src + piece * 8);
+  else
+    *reinterpret_cast<half8_t*>(dst + piece * 8) = *reinterpret_cast<const half8_t*>(src + rm);
+}
+
+__global__ __launch_bounds__(256) void pack_i8_kernel(const int8_t* __restrict__ src,
+                                                      int8_t* __restrict__ dst, int N, int K,
+                                                      bool unpack) {
+  const int64_t piece = (int64_t)blockIdx.x * 256 + threadIdx.x;  // one 8-byte piece
+  const int nks8 = K >> 6;
+  if (piece >= (int64_t)N * K / 8) return;
+  const int half = (int)(piece & 1), lane = (int)((piece >> 1) & 63);
+  const int64_t blk = piece >> 7;
+  const int ks8 = (int)(blk % nks8), t = (int)(blk / nks8);
+  const int64_t rm = ((int64_t)t * 16 + (lane & 15)) * K + ks8 * 64 + half * 32 + (lane >> 4) * 8;
+  if (unpack)
+    *reinterpret_cast<uint2*>(dst + rm) = *reinterpret_cast<const uint2*>(src + piece * 8);
+  else
+    *reinterpret_cast<uint2*>(dst + piece * 8) = *reinterpret_cast<const uint2*>(src + rm);
+}
+
+// ---- stream kernel (M <= 64) --------------------------------------------------------------
+// MFMA fragments: lane l supplies 8 consecutive K elements (offset 8*(l>>4)) of row (l&15) of
+// its operand; A rows are output features n, B rows are activation rows m.  The accumulator
+// of lane l holds m = l&15 and n = 4*(l>>4) .. +3.
+constexpr int ST_KG = 8;  // waves per workgroup = interleaved K lanes
+constexpr int ST_NT = 4;  // weight tiles sharing one activation fragment
 
 template <int MB, bool W8, int MODE>
-__global__ __launch_bounds__(SK_THREADS) void linear_skinny_kernel(
-    const half_t* __restrict__ x, const void* __restrict__ Wv, const half_t* __restrict__ scales,
-    int M, int N, int K, Epilogue epi) {
-  __shared__ float4_t part[SK_WAVES][MB][64];
+__global__ __launch_bounds__(ST_KG * 64) void linear_stream_kernel(
+    const half_t* __restrict__ xp, const void* __restrict__ Wp, const half_t* __restrict__ scales,
+    float* __restrict__ part, int M, int N, int K, int tiles_per_wg, int ks_per_split,
+    Epilogue epi) {
+  constexpr int KG = ST_KG, NT = ST_NT;
+  // K steps (32 wide) buffered per stage; an int8 block covers two steps
+  constexpr int U = MB <= 2 ? 4 : 2;
+  constexpr int UA = W8 ? U / 2 : U;  // weight loads per stage and tile
+  __shared__ float4_t red[KG][NT * MB][64];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int r = lane & 15, g = lane >> 4;
-  const int n0 = blockIdx.x * SK_ROWS;
-  const int nks = K >> 5;  // 32-wide K steps
+  const int ntiles = N >> 4;
+  const int nks = K >> 5;  // 32-wide steps in a row
+  const int tile_begin = blockIdx.x * tiles_per_wg;
+  const int tile_end = min(ntiles, tile_begin + tiles_per_wg);
+  const int ks_begin = blockIdx.y * ks_per_split;
+  const int ks_end = min(nks, ks_begin + ks_per_split);
+  if (tile_begin >= tile_end || ks_begin >= ks_end) return;
+  const int ngroups = (tile_end - tile_begin + NT - 1) / NT;
+  const int nstages = (ks_end - ks_begin + KG * U - 1) / (KG * U);
+  const int total = ngroups * nstages;
 
-  const half_t* xrow[MB];
+  struct Stage {
+    half8_t a[UA][NT];  // fp16: one A fragment; int8: 16 raw bytes = two A fragments
+    half8_t b[U][MB];
+  };
+  Stage s0, s1;
+  auto load = [&](Stage& s, int idx) {
+    const int grp = idx / nstages, st = idx - grp * nstages;
+    const int t0 = tile_begin + grp * NT;
 #pragma unroll
-  for (int mb = 0; mb < MB; ++mb) {
-    int m = mb * 16 + r;
-    if (m >= M) m = M - 1;  // rows past M are computed on valid memory and discarded
-    xrow[mb] = x + (int64_t)m * K + g * 8;
-  }
-  float4_t acc[MB];
+    for (int u = 0; u < UA; ++u) {
+      // first 32-wide step covered by this load (wave-uniform)
+      const int ks = W8 ? ks_begin + 2 * (wave + KG * (st * UA + u))
+                        : ks_begin + wave + KG * (st * U + u);
+      const bool kv = idx < total && ks < ks_end;
 #pragma unroll
-  for (int mb = 0; mb < MB; ++mb) acc[mb] = float4_t{0.f, 0.f, 0.f, 0.f};
-
-  if (!W8) {
-    const half_t* wrow = (const half_t*)Wv + (int64_t)(n0 + r) * K + g * 8;
-    int ks = wave;
-    for (; ks + SK_WAVES * (SK_U - 1) < nks; ks += SK_WAVES * SK_U) {
-      half8_t a[SK_U], b[SK_U][MB];
-#pragma unroll
-      for (int u = 0; u < SK_U; ++u) {
-        const int k = (ks + SK_WAVES * u) << 5;
-        a[u] = *reinterpret_cast<const half8_t*>(wrow + k);
-#pragma unroll
-        for (int mb = 0; mb < MB; ++mb) b[u][mb] = *reinterpret_cast<const half8_t*>(xrow[mb] + k);
+      for (int j = 0; j < NT; ++j) {
+        if (kv && t0 + j < tile_end) {
+          const int64_t blk = W8 ? (int64_t)(t0 + j) * (nks >> 1) + (ks >> 1)
+                                 : (int64_t)(t0 + j) * nks + ks;
+          s.a[u][j] = __builtin_nontemporal_load(
+              reinterpret_cast<const half8_t*>((const half_t*)Wp + blk * 512 + lane * 8));
+        } else {
+          s.a[u][j] = zero8();
+        }
       }
 #pragma unroll
-      for (int u = 0; u < SK_U; ++u)
+      for (int h = 0; h < (W8 ? 2 : 1); ++h) {
 #pragma unroll
-        for (int mb = 0; mb < MB; ++mb)
-          acc[mb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[u], b[u][mb], acc[mb], 0, 0, 0);
-    }
-    for (; ks < nks; ks += SK_WAVES) {
-      const int k = ks << 5;
-      const half8_t a = *reinterpret_cast<const half8_t*>(wrow + k);
-#pragma unroll
-      for (int mb = 0; mb < MB; ++mb) {
-        const half8_t b = *reinterpret_cast<const half8_t*>(xrow[mb] + k);
-        acc[mb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, acc[mb], 0, 0, 0);
+        for (int mb = 0; mb < MB; ++mb) {
+          const int kk = ks + h;
+          if (kv && kk < ks_end)
+            s.b[W8 ? 2 * u + h : u][mb] = *reinterpret_cast<const half8_t*>(
+                xp + (((int64_t)kk * MB + mb) * 64 + lane) * 8);
+          else
+            s.b[W8 ? 2 * u + h : u][mb] = zero8();
+        }
       }
     }
-  } else {
-    // int8 weights: one 8-byte load per lane per K step, dequantised in registers
-    const int8_t* wrow = (const int8_t*)Wv + (int64_t)(n0 + r) * K + g * 8;
-    const half_t sc = scales[n0 + r];
-    for (int ks = wave; ks < nks; ks += SK_WAVES) {
-      const int k = ks << 5;
-      const uint2 w = *reinterpret_cast<const uint2*>(wrow + k);
-      const half8_t a = dequant8(w.x, w.y, sc);
+  };
+  float4_t acc[NT][MB];
+  auto clear = [&]() {
 #pragma unroll
-      for (int mb = 0; mb < MB; ++mb) {
-        const half8_t b = *reinterpret_cast<const half8_t*>(xrow[mb] + k);
-        acc[mb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, acc[mb], 0, 0, 0);
+    for (int j = 0; j < NT; ++j)
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb) acc[j][mb] = float4_t{0.f, 0.f, 0.f, 0.f};
+  };
+  auto mma = [&](Stage& s, int idx) {
+    half_t sc[NT];
+    if (W8) {
+      const int grp = idx / nstages;
+      const int t0 = tile_begin + grp * NT;
+#pragma unroll
+      for (int j = 0; j < NT; ++j)
+        sc[j] = (t0 + j < tile_end) ? scales[(t0 + j) * 16 + (lane & 15)] : (half_t)0;
+    }
+#pragma unroll
+    for (int u = 0; u < UA; ++u)
+#pragma unroll
+      for (int j = 0; j < NT; ++j) {
+        if (!W8) {
+#pragma unroll
+          for (int mb = 0; mb < MB; ++mb)
+            acc[j][mb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(s.a[u][j], s.b[u][mb], acc[j][mb],
+                                                                0, 0, 0);
+        } else {
+          typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+          const u4 raw = __builtin_bit_cast(u4, s.a[u][j]);
+          const half8_t f0 = dequant8(raw[0], raw[1], sc[j]);
+          const half8_t f1 = dequant8(raw[2], raw[3], sc[j]);
+#pragma unroll
+          for (int mb = 0; mb < MB; ++mb) {
+            acc[j][mb] =
+                __builtin_amdgcn_mfma_f32_16x16x32_f16(f0, s.b[2 * u][mb], acc[j][mb], 0, 0, 0);
+            acc[j][mb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(f1, s.b[2 * u + 1][mb],
+                                                                acc[j][mb], 0, 0, 0);
+          }
+        }
       }
+  };
+  auto finish = [&](int idx) {  // after the last stage of a tile group
+    const int grp = idx / nstages;
+    const int t0 = tile_begin + grp * NT;
+#pragma unroll
+    for (int j = 0; j < NT; ++j)
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb) red[wave][j * MB + mb][lane] = acc[j][mb];
+    __syncthreads();
+    for (int e = threadIdx.x; e < NT * MB * 64; e += KG * 64) {
+      const int jm = e >> 6, l = e & 63;
+      const int j = jm / MB, mb = jm - j * MB;
+      float4_t sum = red[0][jm][l];
+#pragma unroll
+      for (int w = 1; w < KG; ++w) sum += red[w][jm][l];
+      const int m = mb * 16 + (l & 15);
+      const int n = (t0 + j) * 16 + ((l >> 4) << 2);
+      if (m < M && t0 + j < tile_end) {
+        if (part)
+          *reinterpret_cast<float4_t*>(part + ((int64_t)blockIdx.y * M + m) * N + n) = sum;
+        else
+          epilogue4<MODE>(epi, m, n, sum);
+      }
+    }
+    __syncthreads();
+    clear();
+  };
+  clear();
+  load(s0, 0);
+  for (int idx = 0; idx < total; idx += 2) {
+    load(s1, idx + 1);
+    mma(s0, idx);
+    if ((idx + 1) % nstages == 0) finish(idx);
+    load(s0, idx + 2);
+    if (idx + 1 < total) {
+      mma(s1, idx + 1);
+      if ((idx + 2) % nstages == 0) finish(idx + 1);
     }
   }
+}
 
-#pragma unroll
-  for (int mb = 0; mb < MB; ++mb) part[wave][mb][lane] = acc[mb];
-  __syncthreads();
-  for (int idx = threadIdx.x; idx < MB * 64; idx += SK_THREADS) {
-    const int mb = idx >> 6, l = idx & 63;
-    float4_t s = part[0][mb][l];
-#pragma unroll
-    for (int w = 1; w < SK_WAVES; ++w) s += part[w][mb][l];
-    // MFMA 16x16 output: lane l holds column (l & 15) of B = activation row m, and rows
-    // 4*(l >> 4) .. +3 of A = output features n.
-    const int m = mb * 16 + (l & 15);
-    const int n = n0 + ((l >> 4) << 2);
-    if (m < M) epilogue4<MODE>(epi, m, n, s);
-  }
+// sums split-K partials part[s][m][n] in slice order and applies the epilogue
+template <int MODE>
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ part, int S,
+                                                            int M, int N, Epilogue epi) {
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;  // one float4 of one row
+  const int nq = N >> 2;
+  if (idx >= (int64_t)M * nq) return;
+  const int m = (int)(idx / nq), n = (int)(idx % nq) << 2;
+  float4_t s = *reinterpret_cast<const float4_t*>(part + (int64_t)m * N + n);
+  for (int i = 1; i < S; ++i)
+    s += *reinterpret_cast<const float4_t*>(part + ((int64_t)i * M + m) * N + n);
+  epilogue4<MODE>(epi, m, n, s);
 }
 
 // ---- tiled kernel ---------------------------------------------------------------------
@@ -184,7 +311,7 @@ constexpr int TL_BM = 128, TL_BN = 128, TL_BK = 32, TL_LD = TL_BK + 8, TL_THREAD
 
 template <bool W8, int MODE>
 __global__ __launch_bounds__(TL_THREADS) void linear_tiled_kernel(
-    const half_t* __restrict__ x, const void* __restrict__ Wv, const half_t* __restrict__ scales,
+    const half_t* __restrict__ x, const void* __restrict__ Wp, const half_t* __restrict__ scales,
     int64_t M, int N, int K, Epilogue epi) {
   __shared__ __attribute__((aligned(16))) half_t lx[2][TL_BM * TL_LD];
   __shared__ __attribute__((aligned(16))) half_t lw[2][TL_BN * TL_LD];
@@ -194,14 +321,18 @@ __global__ __launch_bounds__(TL_THREADS) void linear_tiled_kernel(
   const int64_t m0 = (int64_t)blockIdx.y * TL_BM;
   const int n0 = blockIdx.x * TL_BN;
   const int nkt = K / TL_BK;
+  const int nks = K >> 5;
 
-  // staging: each thread moves two 16-byte chunks of each operand tile
-  int srow[2], scol[2];
+  // staging: each thread moves two 16-byte pieces of each operand tile.  x: piece c covers row
+  // c/4, columns 8*(c%4); W: piece c is lane c%64 of the packed block of row tile c/64.
+  int xrow[2], xcol[2], wrow[2], wcol[2];
 #pragma unroll
   for (int i = 0; i < 2; ++i) {
     const int c = tid + TL_THREADS * i;
-    srow[i] = c >> 2;
-    scol[i] = (c & 3) << 3;
+    xrow[i] = c >> 2;
+    xcol[i] = (c & 3) << 3;
+    wrow[i] = (c >> 6) * 16 + (c & 15);
+    wcol[i] = ((c >> 4) & 3) << 3;
   }
   half8_t rx[2], rw[2];
 
@@ -209,31 +340,34 @@ __global__ __launch_bounds__(TL_THREADS) void linear_tiled_kernel(
     const int k0 = kt * TL_BK;
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
-      const int64_t m = m0 + srow[i];
+      const int64_t m = m0 + xrow[i];
       if (m < M)
-        rx[i] = *reinterpret_cast<const half8_t*>(x + m * K + k0 + scol[i]);
+        rx[i] = *reinterpret_cast<const half8_t*>(x + m * K + k0 + xcol[i]);
       else
-        rx[i] = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
-      const int n = n0 + srow[i];
+        rx[i] = zero8();
+      const int n = n0 + wrow[i];
       if (n < N) {
+        const int c = tid + TL_THREADS * i;
         if (!W8) {
-          rw[i] = *reinterpret_cast<const half8_t*>((const half_t*)Wv + (int64_t)n * K + k0 +
-                                                    scol[i]);
+          rw[i] = *reinterpret_cast<const half8_t*>((const half_t*)Wp +
+                                                    ((int64_t)(n >> 4) * nks + kt) * 512 +
+                                                    (c & 63) * 8);
         } else {
-          const uint2 w =
-              *reinterpret_cast<const uint2*>((const int8_t*)Wv + (int64_t)n * K + k0 + scol[i]);
+          const uint2 w = *reinterpret_cast<const uint2*>(
+              (const int8_t*)Wp + ((int64_t)(n >> 4) * (nks >> 1) + (kt >> 1)) * 1024 +
+              (c & 63) * 16 + (kt & 1) * 8);
           rw[i] = dequant8(w.x, w.y, scales[n]);
         }
       } else {
-        rw[i] = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
+        rw[i] = zero8();
       }
     }
   };
   auto store_tile = [&](int buf) {
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
-      *reinterpret_cast<half8_t*>(&lx[buf][srow[i] * TL_LD + scol[i]]) = rx[i];
-      *reinterpret_cast<half8_t*>(&lw[buf][srow[i] * TL_LD + scol[i]]) = rw[i];
+      *reinterpret_cast<half8_t*>(&lx[buf][xrow[i] * TL_LD + xcol[i]]) = rx[i];
+      *reinterpret_cast<half8_t*>(&lw[buf][wrow[i] * TL_LD + wcol[i]]) = rw[i];
     }
   };
 
@@ -291,39 +425,68 @@ __global__ __launch_bounds__(TL_THREADS) void linear_tiled_kernel(
     }
 }
 
-template <bool W8, int MODE>
-int launch_linear(const void* x, const void* W, const void* scales, int64_t M, int N, int K,
-                  const Epilogue& epi, hipStream_t s) {
-  if (M <= 64 && N % SK_ROWS == 0) {
-    const dim3 grid(N / SK_ROWS), block(SK_THREADS);
-    const int MB = (int)((M + 15) / 16);
-#define MSA_SK(mb)                                                                              \
-  hipLaunchKernelGGL((linear_skinny_kernel<mb, W8, MODE>), grid, block, 0, s, (const half_t*)x, \
-                     W, (const half_t*)scales, (int)M, N, K, epi)
-    switch (MB) {
-      case 1: MSA_SK(1); break;
-      case 2: MSA_SK(2); break;
-      case 3: MSA_SK(3); break;
-      default: MSA_SK(4); break;
-    }
-#undef MSA_SK
-  } else {
-    const dim3 grid((N + TL_BN - 1) / TL_BN, (unsigned)((M + TL_BM - 1) / TL_BM));
-    hipLaunchKernelGGL((linear_tiled_kernel<W8, MODE>), grid, dim3(TL_THREADS), 0, s,
-                       (const half_t*)x, W, (const half_t*)scales, M, N, K, epi);
+// ---- host side ------------------------------------------------------------------------------
+int g_num_cus = 0;
+int num_cus() {
+  if (g_num_cus == 0) {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
+        n <= 0)
+      n = 256;
+    g_num_cus = n;
   }
-  return MSA_OK;
+  return g_num_cus;
+}
+
+template <int MB, bool W8, int MODE>
+void launch_stream_mb(const void* xp, const void* W, const void* scales, float* part, int S, int M,
+                      int N, int K, const Epilogue& epi, hipStream_t s) {
+  const int ntiles = N / 16, nks = K / 32;
+  int G = num_cus() / S;
+  if (G < 1) G = 1;
+  int tiles_per_wg = (ntiles + G - 1) / G;
+  const int gx = (ntiles + tiles_per_wg - 1) / tiles_per_wg;
+  int ks_per_split = (nks + S - 1) / S;
+  if (W8) ks_per_split = (ks_per_split + 1) & ~1;  // int8 blocks cover two steps
+  hipLaunchKernelGGL((linear_stream_kernel<MB, W8, MODE>), dim3(gx, S), dim3(ST_KG * 64), 0, s,
+                     (const half_t*)xp, W, (const half_t*)scales, part, M, N, K, tiles_per_wg,
+                     ks_per_split, epi);
+}
+
+template <bool W8, int MODE>
+void launch_stream(const void* xp, const void* W, const void* scales, float* part, int S, int M,
+                   int N, int K, const Epilogue& epi, hipStream_t s) {
+  switch ((M + 15) / 16) {
+    case 1: launch_stream_mb<1, W8, MODE>(xp, W, scales, part, S, M, N, K, epi, s); break;
+    case 2: launch_stream_mb<2, W8, MODE>(xp, W, scales, part, S, M, N, K, epi, s); break;
+    case 3: launch_stream_mb<3, W8, MODE>(xp, W, scales, part, S, M, N, K, epi, s); break;
+    default: launch_stream_mb<4, W8, MODE>(xp, W, scales, part, S, M, N, K, epi, s); break;
+  }
+}
+
+template <bool W8, int MODE>
+void launch_tiled(const void* x, const void* W, const void* scales, int64_t M, int N, int K,
+                  const Epilogue& epi, hipStream_t s) {
+  const dim3 grid((N + TL_BN - 1) / TL_BN, (unsigned)((M + TL_BM - 1) / TL_BM));
+  hipLaunchKernelGGL((linear_tiled_kernel<W8, MODE>), grid, dim3(TL_THREADS), 0, s,
+                     (const half_t*)x, W, (const half_t*)scales, M, N, K, epi);
 }
 
 int check_linear_args(const char* name, const void* x, const void* W, const void* y, int64_t M,
-                      int N, int K) {
+                      int N, int K, bool w8, unsigned flags, unsigned allowed) {
   MSA_REQUIRE(x && W && y, MSA_ERR_INVALID_ARG, "%s: null pointer", name);
   MSA_REQUIRE(M >= 0 && M < (1ll << 31) && N > 0 && K > 0, MSA_ERR_INVALID_ARG,
               "%s: bad shape M=%lld N=%d K=%d", name, (long long)M, N, K);
-  MSA_REQUIRE(K % 32 == 0 && N % 8 == 0, MSA_ERR_INVALID_ARG,
-              "%s: K=%d must be a multiple of 32 and N=%d a multiple of 8", name, K, N);
+  MSA_REQUIRE(K % (w8 ? 64 : 32) == 0 && N % 16 == 0, MSA_ERR_INVALID_ARG,
+              "%s: K=%d must be a multiple of %d and N=%d a multiple of 16", name, K, w8 ? 64 : 32,
+              N);
   MSA_REQUIRE((M + TL_BM - 1) / TL_BM <= 65535, MSA_ERR_INVALID_ARG, "%s: M=%lld too large", name,
               (long long)M);
+  MSA_REQUIRE((flags & ~allowed) == 0, MSA_ERR_INVALID_ARG, "%s: unsupported flags 0x%x", name,
+              flags);
+  MSA_REQUIRE(!(flags & (MSA_IN_PACKED | MSA_OUT_PACKED)) || M <= 64, MSA_ERR_INVALID_ARG,
+              "%s: packed activations exist only for M <= 64 (M=%lld)", name, (long long)M);
   return MSA_OK;
 }
 
@@ -331,19 +494,40 @@ template <bool W8>
 int linear_entry(const char* name, const void* x, const void* W, const void* scales,
                  const void* bias, const void* residual, void* y, int64_t M, int N, int K,
                  unsigned flags, void* stream) {
-  int rc = check_linear_args(name, x, W, y, M, N, K);
+  int rc = check_linear_args(name, x, W, y, M, N, K, W8, flags,
+                             MSA_EPI_RELU | MSA_IN_PACKED | MSA_OUT_PACKED);
   if (rc) return rc;
   MSA_REQUIRE(!W8 || scales, MSA_ERR_INVALID_ARG, "%s: null scales", name);
-  MSA_REQUIRE((flags & ~MSA_EPI_RELU) == 0, MSA_ERR_INVALID_ARG, "%s: unknown flags 0x%x", name,
-              flags);
+  MSA_REQUIRE(!((flags & MSA_OUT_PACKED) && residual && residual == y), MSA_ERR_INVALID_ARG,
+              "%s: a packed output cannot alias the row-major residual", name);
   if (M == 0) return MSA_OK;
   Epilogue e{};
   e.bias = (const half_t*)bias;
   e.residual = (const half_t*)residual;
   e.y = (half_t*)y;
   e.N = N;
-  e.flags = flags;
-  launch_linear<W8, MODE_PLAIN>(x, W, scales, M, N, K, e, (hipStream_t)stream);
+  e.flags = flags & MSA_EPI_RELU;
+  e.out_mb = (flags & MSA_OUT_PACKED) ? (int)((M + 15) / 16) : 0;
+  if (flags & MSA_IN_PACKED)
+    launch_stream<W8, MODE_PLAIN>(x, W, scales, nullptr, 1, (int)M, N, K, e, (hipStream_t)stream);
+  else
+    launch_tiled<W8, MODE_PLAIN>(x, W, scales, M, N, K, e, (hipStream_t)stream);
+  MSA_CHECK_LAUNCH(name);
+  return MSA_OK;
+}
+
+template <bool W8>
+int partial_entry(const char* name, const void* x, const void* W, const void* scales, float* part,
+                  int64_t M, int N, int K, int S, unsigned flags, void* stream) {
+  int rc = check_linear_args(name, x, W, part, M, N, K, W8, flags, MSA_IN_PACKED);
+  if (rc) return rc;
+  MSA_REQUIRE(!W8 || scales, MSA_ERR_INVALID_ARG, "%s: null scales", name);
+  MSA_REQUIRE((flags & MSA_IN_PACKED) && M >= 1 && M <= 64, MSA_ERR_INVALID_ARG,
+              "%s: needs packed activations and 1 <= M <= 64 (M=%lld)", name, (long long)M);
+  MSA_REQUIRE(S >= 1 && S <= K / (W8 ? 64 : 32), MSA_ERR_INVALID_ARG,
+              "%s: S=%d outside 1..%d", name, S, K / (W8 ? 64 : 32));
+  Epilogue e{};
+  launch_stream<W8, MODE_PLAIN>(x, W, scales, part, S, (int)M, N, K, e, (hipStream_t)stream);
   MSA_CHECK_LAUNCH(name);
   return MSA_OK;
 }
@@ -351,7 +535,7 @@ int linear_entry(const char* name, const void* x, const void* W, const void* sca
 template <bool W8>
 int qkv_entry(const char* name, const void* x, const void* W, const void* scales, const void* bqkv,
               void* q_out, void* Kc, void* Vc, int B, int T, int H, int hd, int S0, int S_cap,
-              int K, void* stream) {
+              int K, unsigned flags, void* stream) {
   MSA_REQUIRE(q_out && Kc && Vc, MSA_ERR_INVALID_ARG, "%s: null pointer", name);
   MSA_REQUIRE(B > 0 && T > 0 && H > 0 && hd > 0 && hd % 8 == 0 && S0 >= 0, MSA_ERR_INVALID_ARG,
               "%s: bad shape B=%d T=%d H=%d hd=%d S0=%d", name, B, T, H, hd, S0);
@@ -359,7 +543,7 @@ int qkv_entry(const char* name, const void* x, const void* W, const void* scales
               "%s: S0 + T = %d exceeds the cache capacity %d", name, S0 + T, S_cap);
   const int64_t M = (int64_t)B * T;
   const int N = 3 * H * hd;
-  int rc = check_linear_args(name, x, W, q_out, M, N, K);
+  int rc = check_linear_args(name, x, W, q_out, M, N, K, W8, flags, MSA_IN_PACKED);
   if (rc) return rc;
   MSA_REQUIRE(!W8 || scales, MSA_ERR_INVALID_ARG, "%s: null scales", name);
   Epilogue e{};
@@ -374,40 +558,93 @@ int qkv_entry(const char* name, const void* x, const void* W, const void* scales
   e.S0 = S0;
   e.S_cap = S_cap;
   e.qscale = (float)pow((double)hd, -0.5);  // the reference's head_dim ** -0.5, cast to fp32
-  launch_linear<W8, MODE_QKV>(x, W, scales, M, N, K, e, (hipStream_t)stream);
+  if (flags & MSA_IN_PACKED)
+    launch_stream<W8, MODE_QKV>(x, W, scales, nullptr, 1, (int)M, N, K, e, (hipStream_t)stream);
+  else
+    launch_tiled<W8, MODE_QKV>(x, W, scales, M, N, K, e, (hipStream_t)stream);
+  MSA_CHECK_LAUNCH(name);
+  return MSA_OK;
+}
+
+int pack_entry(const char* name, const void* src, void* dst, int N, int K, bool i8, bool unpack,
+               void* stream) {
+  MSA_REQUIRE(src && dst && src != dst, MSA_ERR_INVALID_ARG, "%s: null or aliased pointers", name);
+  MSA_REQUIRE(N > 0 && K > 0 && N % 16 == 0 && K % (i8 ? 64 : 32) == 0, MSA_ERR_INVALID_ARG,
+              "%s: N=%d must be a multiple of 16 and K=%d of %d", name, N, K, i8 ? 64 : 32);
+  const int64_t pieces = (int64_t)N * K / 8;
+  const dim3 grid((unsigned)((pieces + 255) / 256));
+  if (i8)
+    hipLaunchKernelGGL(pack_i8_kernel, grid, dim3(256), 0, (hipStream_t)stream, (const int8_t*)src,
+                       (int8_t*)dst, N, K, unpack);
+  else
+    hipLaunchKernelGGL(pack_f16_kernel, grid, dim3(256), 0, (hipStream_t)stream,
+                       (const half_t*)src, (half_t*)dst, N, K, unpack);
   MSA_CHECK_LAUNCH(name);
   return MSA_OK;
 }
 
 }  // namespace
 
-extern "C" size_t msa_linear_workspace_bytes(int64_t, int, int) { return 0; }
+extern "C" int msa_pack_weight_f16(const void* src, void* dst, int N, int K, void* stream) {
+  return pack_entry("msa_pack_weight_f16", src, dst, N, K, false, false, stream);
+}
+extern "C" int msa_unpack_weight_f16(const void* src, void* dst, int N, int K, void* stream) {
+  return pack_entry("msa_unpack_weight_f16", src, dst, N, K, false, true, stream);
+}
+extern "C" int msa_pack_weight_i8(const int8_t* src, int8_t* dst, int N, int K, void* stream) {
+  return pack_entry("msa_pack_weight_i8", src, dst, N, K, true, false, stream);
+}
+extern "C" int msa_unpack_weight_i8(const int8_t* src, int8_t* dst, int N, int K, void* stream) {
+  return pack_entry("msa_unpack_weight_i8", src, dst, N, K, true, true, stream);
+}
 
-extern "C" int msa_linear_f16(const void* x, const void* W, const void* bias, const void* residual,
-                              void* y, int64_t M, int N, int K, unsigned flags, void*, size_t,
-                              void* stream) {
-  return linear_entry<false>("msa_linear_f16", x, W, nullptr, bias, residual, y, M, N, K, flags,
+extern "C" int msa_linear_default_splits(int64_t M, int N, int K) {
+  // split K only where one split leaves most compute units without a tile group
+  if (M > 64 || N % 16 || K % 64) return 1;
+  const int groups = (N / 16 + ST_NT - 1) / ST_NT;
+  int S = 1;
+  while (S < 8 && groups * S * 2 <= num_cus() && K / 32 / (S * 2) >= ST_KG * 2) S *= 2;
+  return S;
+}
+
+extern "C" int msa_linear_f16(const void* x, const void* Wp, const void* bias,
+                              const void* residual, void* y, int64_t M, int N, int K,
+                              unsigned flags, void* stream) {
+  return linear_entry<false>("msa_linear_f16", x, Wp, nullptr, bias, residual, y, M, N, K, flags,
                              stream);
 }
 
 extern "C" int msa_linear_w8a16(const void* x, const int8_t* Wq, const void* scales,
                                 const void* bias, const void* residual, void* y, int64_t M, int N,
-                                int K, unsigned flags, void*, size_t, void* stream) {
+                                int K, unsigned flags, void* stream) {
   return linear_entry<true>("msa_linear_w8a16", x, Wq, scales, bias, residual, y, M, N, K, flags,
                             stream);
 }
 
+extern "C" int msa_linear_partial_f16(const void* x, const void* Wp, float* part, int64_t M, int N,
+                                      int K, int S, unsigned flags, void* stream) {
+  return partial_entry<false>("msa_linear_partial_f16", x, Wp, nullptr, part, M, N, K, S, flags,
+                              stream);
+}
+
+extern "C" int msa_linear_partial_w8a16(const void* x, const int8_t* Wq, const void* scales,
+                                        float* part, int64_t M, int N, int K, int S,
+                                        unsigned flags, void* stream) {
+  return partial_entry<true>("msa_linear_partial_w8a16", x, Wq, scales, part, M, N, K, S, flags,
+                             stream);
+}
+
 extern "C" int msa_qkv_proj_f16(const void* x, const void* Wqkv, const void* bqkv, void* q_out,
                                 void* Kcache, void* Vcache, int B, int T, int H, int hd, int S0,
-                                int S_cap, int K, void*, size_t, void* stream) {
+                                int S_cap, int K, unsigned flags, void* stream) {
   return qkv_entry<false>("msa_qkv_proj_f16", x, Wqkv, nullptr, bqkv, q_out, Kcache, Vcache, B, T,
-                          H, hd, S0, S_cap, K, stream);
+                          H, hd, S0, S_cap, K, flags, stream);
 }
 
 extern "C" int msa_qkv_proj_w8a16(const void* x, const int8_t* Wq, const void* scales,
                                   const void* bqkv, void* q_out, void* Kcache, void* Vcache, int B,
-                                  int T, int H, int hd, int S0, int S_cap, int K, void*, size_t,
+                                  int T, int H, int hd, int S0, int S_cap, int K, unsigned flags,
                                   void* stream) {
   return qkv_entry<true>("msa_qkv_proj_w8a16", x, Wq, scales, bqkv, q_out, Kcache, Vcache, B, T, H,
-                         hd, S0, S_cap, K, stream);
+                         hd, S0, S_cap, K, flags, stream);
 }

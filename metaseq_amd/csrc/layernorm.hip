@@ -1,6 +1,8 @@
-// Pre-LN LayerNorm forward, fp16 in / fp16 out, fp32 statistics.
-// One workgroup per row; the row lives in registers between the two reduction passes, so
-// HBM traffic is exactly one read and one write of the row plus gamma/beta.
+// Pre-LN LayerNorm forward, fp16 in / fp16 out, fp32 statistics, optionally fused with the
+// tail of the preceding split-K linear layer (sum of fp32 partials, bias add, residual add),
+// and optionally writing the packed activation layout the decode GEMMs read.
+// One workgroup per row; the row lives in registers between the reduction passes, so HBM
+// traffic is one read and one write of the row plus gamma/beta.
 #include "common.h"
 
 namespace {
@@ -9,12 +11,11 @@ constexpr int LN_THREADS = 256;
 constexpr int LN_MAX_CHUNKS = 8;  // 8 halves per chunk per thread -> D <= 256*8*8 = 16384
 
 __global__ __launch_bounds__(LN_THREADS) void layernorm_f16_kernel(
-    const half_t* __restrict__ x, const half_t* __restrict__ gamma,
-    const half_t* __restrict__ beta, half_t* __restrict__ y, int D, float eps) {
+    const half_t* x, const float* __restrict__ part, int S,
+    const half_t* __restrict__ bias, half_t* x_out, const half_t* __restrict__ gamma,
+    const half_t* __restrict__ beta, half_t* __restrict__ y, int M, int D, float eps, int out_mb) {
   __shared__ float red[16];
-  const int64_t row = blockIdx.x;
-  const half_t* xr = x + row * D;
-  half_t* yr = y + row * D;
+  const int row = blockIdx.x;
   const int nchunk = D >> 3;  // 16-byte chunks in the row
 
   half8_t v[LN_MAX_CHUNKS];
@@ -23,11 +24,34 @@ __global__ __launch_bounds__(LN_THREADS) void layernorm_f16_kernel(
   for (int c = 0; c < LN_MAX_CHUNKS; ++c) {
     const int idx = threadIdx.x + c * LN_THREADS;
     if (idx < nchunk) {
-      v[c] = *reinterpret_cast<const half8_t*>(xr + (idx << 3));
+      if (part) {
+        // x_out = round(round(round(sum_s part) + bias) + x): the fp16 rounding points of
+        // "linear, + bias, + residual" in the reference layer
+        const float* p = part + (int64_t)row * D + (idx << 3);
+        float4_t a0 = *reinterpret_cast<const float4_t*>(p);
+        float4_t a1 = *reinterpret_cast<const float4_t*>(p + 4);
+        for (int i = 1; i < S; ++i) {
+          const float* q = p + (int64_t)i * M * D;
+          a0 += *reinterpret_cast<const float4_t*>(q);
+          a1 += *reinterpret_cast<const float4_t*>(q + 4);
+        }
+        const half8_t b = *reinterpret_cast<const half8_t*>(bias + (idx << 3));
+        const half8_t r = *reinterpret_cast<const half8_t*>(x + (int64_t)row * D + (idx << 3));
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          float t = round_h(i < 4 ? a0[i] : a1[i - 4]);
+          t = round_h(t + (float)b[i]);
+          v[c][i] = (half_t)(t + (float)r[i]);
+        }
+        *reinterpret_cast<half8_t*>(x_out + (int64_t)row * D + (idx << 3)) = v[c];
+      } else {
+        v[c] = *reinterpret_cast<const half8_t*>(x + (int64_t)row * D + (idx << 3));
+      }
 #pragma unroll
       for (int i = 0; i < 8; ++i) s += (float)v[c][i];
     }
   }
+  if (!gamma) return;
   const float mean = block_sum(s, red) / (float)D;
   float q = 0.f;
 #pragma unroll
@@ -53,25 +77,61 @@ __global__ __launch_bounds__(LN_THREADS) void layernorm_f16_kernel(
 #pragma unroll
       for (int i = 0; i < 8; ++i)
         o[i] = (half_t)(((float)v[c][i] - mean) * rstd * (float)g[i] + (float)b[i]);
-      *reinterpret_cast<half8_t*>(yr + (idx << 3)) = o;
+      half_t* dst = out_mb > 0 ? y + packed_act_offset(row, idx << 3, out_mb)
+                               : y + (int64_t)row * D + (idx << 3);
+      *reinterpret_cast<half8_t*>(dst) = o;
     }
   }
+}
+
+int check(const char* name, int64_t rows, int D, unsigned flags) {
+  MSA_REQUIRE(rows >= 0 && rows <= 0x7fffffff, MSA_ERR_INVALID_ARG, "%s: rows=%lld out of range",
+              name, (long long)rows);
+  MSA_REQUIRE(D > 0 && D % 8 == 0 && D <= LN_THREADS * 8 * LN_MAX_CHUNKS, MSA_ERR_INVALID_ARG,
+              "%s: D=%d must be a multiple of 8 and <= %d", name, D,
+              LN_THREADS * 8 * LN_MAX_CHUNKS);
+  MSA_REQUIRE((flags & ~MSA_OUT_PACKED) == 0, MSA_ERR_INVALID_ARG, "%s: unsupported flags 0x%x",
+              name, flags);
+  MSA_REQUIRE(!(flags & MSA_OUT_PACKED) || (rows <= 64 && D % 32 == 0), MSA_ERR_INVALID_ARG,
+              "%s: packed output needs rows <= 64 and D %% 32 == 0 (rows=%lld D=%d)", name,
+              (long long)rows, D);
+  return MSA_OK;
 }
 
 }  // namespace
 
 extern "C" int msa_layernorm_f16(const void* x, const void* gamma, const void* beta, void* y,
-                                 int64_t rows, int D, float eps, void* stream) {
+                                 int64_t rows, int D, float eps, unsigned flags, void* stream) {
   MSA_REQUIRE(x && gamma && beta && y, MSA_ERR_INVALID_ARG, "msa_layernorm_f16: null pointer");
-  MSA_REQUIRE(rows >= 0 && rows <= 0x7fffffff, MSA_ERR_INVALID_ARG,
-              "msa_layernorm_f16: rows=%lld out of range", (long long)rows);
-  MSA_REQUIRE(D > 0 && D % 8 == 0 && D <= LN_THREADS * 8 * LN_MAX_CHUNKS, MSA_ERR_INVALID_ARG,
-              "msa_layernorm_f16: D=%d must be a multiple of 8 and <= %d", D,
-              LN_THREADS * 8 * LN_MAX_CHUNKS);
+  int rc = check("msa_layernorm_f16", rows, D, flags);
+  if (rc) return rc;
   if (rows == 0) return MSA_OK;
+  const int out_mb = (flags & MSA_OUT_PACKED) ? (int)((rows + 15) / 16) : 0;
   hipLaunchKernelGGL(layernorm_f16_kernel, dim3((unsigned)rows), dim3(LN_THREADS), 0,
-                     (hipStream_t)stream, (const half_t*)x, (const half_t*)gamma,
-                     (const half_t*)beta, (half_t*)y, D, eps);
+                     (hipStream_t)stream, (const half_t*)x, (const float*)nullptr, 0,
+                     (const half_t*)nullptr, (half_t*)nullptr, (const half_t*)gamma,
+                     (const half_t*)beta, (half_t*)y, (int)rows, D, eps, out_mb);
   MSA_CHECK_LAUNCH("msa_layernorm_f16");
+  return MSA_OK;
+}
+
+extern "C" int msa_residual_layernorm_f16(const float* part, int S, const void* bias, void* x,
+                                          const void* gamma, const void* beta, void* y,
+                                          int64_t rows, int D, float eps, unsigned flags,
+                                          void* stream) {
+  MSA_REQUIRE(part && bias && x, MSA_ERR_INVALID_ARG, "msa_residual_layernorm_f16: null pointer");
+  MSA_REQUIRE(S >= 1, MSA_ERR_INVALID_ARG, "msa_residual_layernorm_f16: S=%d", S);
+  MSA_REQUIRE((gamma == nullptr) == (beta == nullptr) && (gamma == nullptr) == (y == nullptr),
+              MSA_ERR_INVALID_ARG,
+              "msa_residual_layernorm_f16: gamma, beta and y must be given together");
+  int rc = check("msa_residual_layernorm_f16", rows, D, flags);
+  if (rc) return rc;
+  if (rows == 0) return MSA_OK;
+  const int out_mb = (flags & MSA_OUT_PACKED) ? (int)((rows + 15) / 16) : 0;
+  hipLaunchKernelGGL(layernorm_f16_kernel, dim3((unsigned)rows), dim3(LN_THREADS), 0,
+                     (hipStream_t)stream, (const half_t*)x, part, S, (const half_t*)bias,
+                     (half_t*)x, (const half_t*)gamma, (const half_t*)beta, (half_t*)y, (int)rows,
+                     D, eps, out_mb);
+  MSA_CHECK_LAUNCH("msa_residual_layernorm_f16");
   return MSA_OK;
 }

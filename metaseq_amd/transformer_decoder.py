@@ -14,45 +14,85 @@ import torch
 from torch import nn
 
 from . import _capi
-from ._capi import MSA_EPI_RELU, check, ptr
+from ._capi import MSA_EPI_RELU, MSA_IN_PACKED, MSA_OUT_PACKED, check, ptr
 from .config import OPTConfig
 from .kv_cache import KVCache
 
 
 class _Affine(nn.Module):
-    """weight + bias holder (Linear or LayerNorm parameters under the reference's names)."""
+    """weight + bias holder (Linear or LayerNorm parameters under the reference's names).
 
-    def __init__(self, w_shape, b_shape):
+    For a linear layer, ``prepare_`` converts ``weight`` in place to the tile-packed layout the
+    kernels stream (same shape and bytes, permuted), or to packed int8 + fp16 scales."""
+
+    def __init__(self, w_shape, b_shape, device=None):
         super().__init__()
-        self.weight = nn.Parameter(torch.zeros(w_shape, dtype=torch.float16), requires_grad=False)
-        self.bias = nn.Parameter(torch.zeros(b_shape, dtype=torch.float16), requires_grad=False)
-        # int8 weight-only form, filled by TransformerDecoder.quantize_int8_()
-        self.qweight: Optional[torch.Tensor] = None
+        self.weight = nn.Parameter(torch.zeros(w_shape, dtype=torch.float16, device=device),
+                                   requires_grad=False)
+        self.bias = nn.Parameter(torch.zeros(b_shape, dtype=torch.float16, device=device),
+                                 requires_grad=False)
+        self.packed = False
+        self.qweight: Optional[torch.Tensor] = None  # tile-packed int8
         self.scales: Optional[torch.Tensor] = None
+        self.shape = tuple(w_shape)
+
+    def prepare_(self, lib, int8=False):
+        if self.packed or self.qweight is not None:
+            return
+        N, K = self.shape
+        w = self.weight.data
+        if int8:
+            wf = w.float()
+            scales = (wf.abs().amax(dim=1) / 127.0).to(torch.float16)
+            s = scales.float().clamp_min(1e-30).unsqueeze(1)
+            q = torch.clamp(torch.round(wf / s), -127, 127).to(torch.int8).contiguous()
+            del wf
+            qp = torch.empty_like(q)
+            check(lib.msa_pack_weight_i8(ptr(q), ptr(qp), N, K, _capi.stream_ptr()))
+            self.qweight, self.scales = qp, scales.contiguous()
+            self.weight.data = torch.empty(0, dtype=torch.float16, device=w.device)
+        else:
+            wp = torch.empty_like(w)
+            check(lib.msa_pack_weight_f16(ptr(w), ptr(wp), N, K, _capi.stream_ptr()))
+            self.weight.data = wp
+            self.packed = True
+
+    def row_major_weight(self, lib):
+        """fp16 [N, K] row-major weight (for int8: the dequantised round(q * scale))."""
+        N, K = self.shape
+        if self.qweight is not None:
+            q = torch.empty_like(self.qweight)
+            check(lib.msa_unpack_weight_i8(ptr(self.qweight), ptr(q), N, K, _capi.stream_ptr()))
+            return (q.float() * self.scales.float().unsqueeze(1)).to(torch.float16)
+        if not self.packed:
+            return self.weight.data
+        w = torch.empty_like(self.weight.data)
+        check(lib.msa_unpack_weight_f16(ptr(self.weight.data), ptr(w), N, K, _capi.stream_ptr()))
+        return w
 
 
 class _Table(nn.Module):
-    def __init__(self, rows, dim):
+    def __init__(self, rows, dim, device=None):
         super().__init__()
-        self.weight = nn.Parameter(torch.zeros(rows, dim, dtype=torch.float16),
+        self.weight = nn.Parameter(torch.zeros(rows, dim, dtype=torch.float16, device=device),
                                    requires_grad=False)
 
 
 class _SelfAttention(nn.Module):
-    def __init__(self, D):
+    def __init__(self, D, device=None):
         super().__init__()
-        self.qkv_proj = _Affine((3 * D, D), (3 * D,))  # rows K | V | Q
-        self.out_proj = _Affine((D, D), (D,))
+        self.qkv_proj = _Affine((3 * D, D), (3 * D,), device)  # rows K | V | Q
+        self.out_proj = _Affine((D, D), (D,), device)
 
 
 class _DecoderLayer(nn.Module):
-    def __init__(self, D, F):
+    def __init__(self, D, F, device=None):
         super().__init__()
-        self.self_attn_layer_norm = _Affine((D,), (D,))
-        self.self_attn = _SelfAttention(D)
-        self.final_layer_norm = _Affine((D,), (D,))
-        self.fc1 = _Affine((F, D), (F,))
-        self.fc2 = _Affine((D, F), (D,))
+        self.self_attn_layer_norm = _Affine((D,), (D,), device)
+        self.self_attn = _SelfAttention(D, device)
+        self.final_layer_norm = _Affine((D,), (D,), device)
+        self.fc1 = _Affine((F, D), (F,), device)
+        self.fc2 = _Affine((D, F), (D,), device)
 
 
 class TransformerDecoder(nn.Module):
@@ -74,60 +114,87 @@ class TransformerDecoder(nn.Module):
         self.share_input_output_embed = True
         self.embed_scale = 1.0
         self.register_buffer("version", torch.tensor([3.0]))
-        self.embed_tokens = _Table(cfg.vocab_size, D)
-        self.embed_positions = _Table(cfg.max_target_positions + cfg.padding_idx + 1, D)
-        self.layers = nn.ModuleList([_DecoderLayer(D, F) for _ in range(cfg.decoder_layers)])
-        self.layer_norm = _Affine((D,), (D,))
+        self.embed_tokens = _Table(cfg.vocab_size, D, device)
+        self.embed_positions = _Table(cfg.max_target_positions + cfg.padding_idx + 1, D, device)
+        self.layers = nn.ModuleList([_DecoderLayer(D, F, device)
+                                     for _ in range(cfg.decoder_layers)])
+        self.layer_norm = _Affine((D,), (D,), device)
         self.inference = True
         self.return_inner_states = False
         # capacity (positions) of the KV cache the next prefill allocates; None = grow on demand
         self.kv_cache_capacity: Optional[int] = None
         self._state_key = str(uuid.uuid4()) + ".kv_cache"
         self._lib = None
+        self._lm_head: Optional[torch.Tensor] = None  # tile-packed copy of the tied embedding
+        self.to(device)
         if state_dict is not None:
             self.load_state_dict(state_dict)
-        self.to(device)
-        if cfg.quantize_int8:
-            self.quantize_int8_()
 
     # ------------------------------------------------------------------ weights
+    def _linears(self):
+        for i, layer in enumerate(self.layers):
+            yield f"layers.{i}.self_attn.qkv_proj", layer.self_attn.qkv_proj
+            yield f"layers.{i}.self_attn.out_proj", layer.self_attn.out_proj
+            yield f"layers.{i}.fc1", layer.fc1
+            yield f"layers.{i}.fc2", layer.fc2
+
     def load_state_dict(self, state_dict, strict=True, **kw):
         sd = dict(state_dict)
         # accept a model-level dict ("decoder." prefix) and the tied duplicate key
         if any(k.startswith("decoder.") for k in sd):
             sd = {k[len("decoder."):]: v for k, v in sd.items() if k.startswith("decoder.")}
         sd.pop("output_projection.weight", None)
+        for _, lin in self._linears():  # back to plain row-major parameters before loading
+            if lin.packed or lin.qweight is not None:
+                lin.weight.data = torch.empty(lin.shape, dtype=torch.float16,
+                                              device=lin.bias.device)
+                lin.packed, lin.qweight, lin.scales = False, None, None
+        self._lm_head = None
         return super().load_state_dict(sd, strict=strict, **kw)
 
+    def state_dict(self, *args, **kwargs):
+        """Reference-layout (row-major, fp16) state dict; quantised matrices come back as their
+        dequantised values round(q * scale)."""
+        sd = super().state_dict(*args, **kwargs)
+        prefix = kwargs.get("prefix", args[1] if len(args) > 1 else "")
+        if self._lib is not None:
+            for name, lin in self._linears():
+                if lin.packed or lin.qweight is not None:
+                    sd[prefix + name + ".weight"] = lin.row_major_weight(self._lib)
+        return sd
+
+    def prepare_(self):
+        """Packs every linear weight for the kernels (idempotent); with ``cfg.quantize_int8`` the
+        four per-layer matrices become symmetric per-output-channel int8 first:
+        scale_j = fp16(max_i |W_ji| / 127), q = clamp(rint(W / scale_j), -127, 127) - the
+        matrices the reference quantises for serving
+        (metaseq/scripts/convert_metaseq_ft.py:118-129)."""
+        lib = self._lib or _capi.load()
+        self._lib = lib
+        if not self.embed_tokens.weight.is_cuda:
+            raise RuntimeError("metaseq_amd: the model must live on the GPU (no CPU path exists)")
+        for _, lin in self._linears():
+            lin.prepare_(lib, int8=self.cfg.quantize_int8)
+        if self._lm_head is None:
+            e = self.embed_tokens.weight.data
+            self._lm_head = torch.empty_like(e)
+            check(lib.msa_pack_weight_f16(ptr(e), ptr(self._lm_head), e.shape[0], e.shape[1],
+                                          _capi.stream_ptr()))
+        return lib
+
     def quantize_int8_(self):
-        """Symmetric per-output-channel int8 for qkv / out_proj / fc1 / fc2 (the matrices the
-        reference quantises for serving, metaseq/scripts/convert_metaseq_ft.py:118-129):
-        scale_j = fp16(max_i |W_ji| / 127), q = clamp(rint(W / scale_j), -127, 127).  The fp16
-        matrices are released."""
-        for layer in self.layers:
-            for lin in (layer.self_attn.qkv_proj, layer.self_attn.out_proj, layer.fc1, layer.fc2):
-                w = lin.weight.data.float()
-                scales = (w.abs().amax(dim=1) / 127.0).to(torch.float16)
-                s = scales.float().clamp_min(1e-30).unsqueeze(1)
-                lin.qweight = torch.clamp(torch.round(w / s), -127, 127).to(torch.int8).contiguous()
-                lin.scales = scales.contiguous()
-                lin.weight.data = torch.empty(0, dtype=torch.float16, device=w.device)
-                del w
         self.cfg.quantize_int8 = True
+        for _, lin in self._linears():
+            if lin.packed:
+                raise RuntimeError("quantize_int8_() must be called before the first forward")
+        self.prepare_()
         return self
 
     def dequantized_state_dict(self):
         """Reference-named fp16 weights with quantised matrices replaced by round(q * scale):
         what a reference model must be loaded with to be compared against the int8 path."""
-        sd = {"decoder." + k: v for k, v in self.state_dict().items()}
-        for i, layer in enumerate(self.layers):
-            for name, lin in (("self_attn.qkv_proj", layer.self_attn.qkv_proj),
-                              ("self_attn.out_proj", layer.self_attn.out_proj),
-                              ("fc1", layer.fc1), ("fc2", layer.fc2)):
-                if lin.qweight is not None:
-                    sd[f"decoder.layers.{i}.{name}.weight"] = (
-                        lin.qweight.float() * lin.scales.float().unsqueeze(1)).to(torch.float16)
-        return sd
+        self.prepare_()
+        return {"decoder." + k: v for k, v in self.state_dict().items()}
 
     # ------------------------------------------------------------------ reference API
     def max_positions(self):
@@ -156,30 +223,46 @@ class TransformerDecoder(nn.Module):
 
     # ------------------------------------------------------------------ kernels
     def _linear(self, lib, stream, x, lin, M, N, K, bias=True, residual=None, relu=False,
-                out=None):
+                out=None, flags=0):
         y = out if out is not None else torch.empty(M, N, dtype=torch.float16, device=x.device)
-        flags = MSA_EPI_RELU if relu else 0
+        flags |= MSA_EPI_RELU if relu else 0
         b = lin.bias if bias else None
         if lin.qweight is not None:
             check(lib.msa_linear_w8a16(ptr(x), ptr(lin.qweight), ptr(lin.scales), ptr(b),
-                                       ptr(residual), ptr(y), M, N, K, flags, None, 0, stream))
+                                       ptr(residual), ptr(y), M, N, K, flags, stream))
         else:
             check(lib.msa_linear_f16(ptr(x), ptr(lin.weight), ptr(b), ptr(residual), ptr(y), M, N,
-                                     K, flags, None, 0, stream))
+                                     K, flags, stream))
         return y
 
-    def _layernorm(self, lib, stream, x, ln, rows, D, out=None):
-        y = out if out is not None else torch.empty_like(x)
-        check(lib.msa_layernorm_f16(ptr(x), ptr(ln.weight), ptr(ln.bias), ptr(y), rows, D, 1e-5,
-                                    stream))
-        return y
+    def _linear_partial(self, lib, stream, x, lin, part, M, N, K, S):
+        if lin.qweight is not None:
+            check(lib.msa_linear_partial_w8a16(ptr(x), ptr(lin.qweight), ptr(lin.scales),
+                                               ptr(part), M, N, K, S, MSA_IN_PACKED, stream))
+        else:
+            check(lib.msa_linear_partial_f16(ptr(x), ptr(lin.weight), ptr(part), M, N, K, S,
+                                             MSA_IN_PACKED, stream))
+
+    def _qkv(self, lib, stream, h, qkv, q, kc, vc, B, T, H, hd, S0, cap, D, flags):
+        if qkv.qweight is not None:
+            check(lib.msa_qkv_proj_w8a16(ptr(h), ptr(qkv.qweight), ptr(qkv.scales), ptr(qkv.bias),
+                                         ptr(q), ptr(kc), ptr(vc), B, T, H, hd, S0, cap, D, flags,
+                                         stream))
+        else:
+            check(lib.msa_qkv_proj_f16(ptr(h), ptr(qkv.weight), ptr(qkv.bias), ptr(q), ptr(kc),
+                                       ptr(vc), B, T, H, hd, S0, cap, D, flags, stream))
+
+    def _layernorm(self, lib, stream, x, ln, rows, D, out, flags=0):
+        check(lib.msa_layernorm_f16(ptr(x), ptr(ln.weight), ptr(ln.bias), ptr(out), rows, D, 1e-5,
+                                    flags, stream))
+        return out
 
     # ------------------------------------------------------------------ forward
-    def extract_features(self, prev_output_tokens, incremental_state=None,
-                         token_embeddings=None, self_attn_padding_mask=None):
-        """Embedding, L pre-LN layers and the final LayerNorm
-        (metaseq/models/transformer_decoder.py:348-396).  Returns features ``[B, T, D]``
-        (the reference returns the same values as ``[T, B, D]``)."""
+    def _forward_features(self, prev_output_tokens, incremental_state, token_embeddings,
+                          self_attn_padding_mask, want_packed):
+        """Embedding, L pre-LN layers and the final LayerNorm.  Returns (features, packed,
+        extra): features are ``[B, T, D]`` row-major, or - for a decode step of at most 64 rows
+        when ``want_packed`` - the packed activation buffer the vocabulary projection reads."""
         cfg = self.cfg
         if token_embeddings is not None:
             raise NotImplementedError("precomputed token_embeddings are not supported")
@@ -192,8 +275,7 @@ class TransformerDecoder(nn.Module):
             tokens = tokens.long()
         if tokens.stride(1) != 1:
             tokens = tokens.contiguous()
-        lib = self._lib or _capi.load()
-        self._lib = lib
+        lib = self.prepare_()
         stream = _capi.stream_ptr()
         dev = tokens.device
         B, n = tokens.shape
@@ -251,64 +333,125 @@ class TransformerDecoder(nn.Module):
         inner_states = [{"tok": None, "pos": positions, "emb": None}]
         if self.return_inner_states:
             inner_states[0]["emb"] = x.view(B, T, D).transpose(0, 1).clone()
-
-        h = torch.empty_like(x)
-        q = torch.empty_like(x)
-        o = torch.empty_like(x)
-        u = torch.empty(M, F, dtype=torch.float16, device=dev)
         mask_stride = mask.stride(0) if mask is not None else 0
-        for i, layer in enumerate(self.layers):
-            self._layernorm(lib, stream, x, layer.self_attn_layer_norm, M, D, out=h)
-            qkv = layer.self_attn.qkv_proj
-            kc, vc = cache.k(i), cache.v(i)
-            if qkv.qweight is not None:
-                check(lib.msa_qkv_proj_w8a16(ptr(h), ptr(qkv.qweight), ptr(qkv.scales),
-                                             ptr(qkv.bias), ptr(q), ptr(kc), ptr(vc), B, T, H, hd,
-                                             S0, cache.capacity, D, None, 0, stream))
+        q = torch.empty(M, D, dtype=torch.float16, device=dev)
+
+        if T == 1 and M <= 64:
+            # ---- decode step: packed activations, weight-streaming kernels, split-K tails
+            # fused into the LayerNorm that follows ----
+            MP = ((M + 15) // 16) * 16
+            h = torch.empty(MP * D, dtype=torch.float16, device=dev)
+            o = torch.empty(MP * D, dtype=torch.float16, device=dev)
+            u = torch.empty(MP * F, dtype=torch.float16, device=dev)
+            S_o = lib.msa_linear_default_splits(M, D, D)
+            S_f = lib.msa_linear_default_splits(M, D, F)
+            part = torch.empty(max(S_o, S_f) * M * D, dtype=torch.float32, device=dev)
+            IN, OUT = MSA_IN_PACKED, MSA_OUT_PACKED
+            self._layernorm(lib, stream, x, self.layers[0].self_attn_layer_norm, M, D, h, OUT)
+            for i, layer in enumerate(self.layers):
+                kc, vc = cache.k(i), cache.v(i)
+                self._qkv(lib, stream, h, layer.self_attn.qkv_proj, q, kc, vc, B, 1, H, hd, S0,
+                          cache.capacity, D, IN)
+                check(lib.msa_attention_f16(ptr(q), ptr(kc), ptr(vc), ptr(mask), mask_stride,
+                                            ptr(o), B, H, hd, 1, S0, cache.capacity, OUT, stream))
+                op = layer.self_attn.out_proj
+                self._linear_partial(lib, stream, o, op, part, M, D, D, S_o)
+                ln = layer.final_layer_norm
+                check(lib.msa_residual_layernorm_f16(ptr(part), S_o, ptr(op.bias), ptr(x),
+                                                     ptr(ln.weight), ptr(ln.bias), ptr(h), M, D,
+                                                     1e-5, OUT, stream))
+                self._linear(lib, stream, h, layer.fc1, M, F, D, relu=True, out=u,
+                             flags=IN | OUT)
+                self._linear_partial(lib, stream, u, layer.fc2, part, M, D, F, S_f)
+                last = i + 1 == L
+                ln = self.layer_norm if last else self.layers[i + 1].self_attn_layer_norm
+                if last and self.return_inner_states:
+                    check(lib.msa_residual_layernorm_f16(ptr(part), S_f, ptr(layer.fc2.bias),
+                                                         ptr(x), None, None, None, M, D, 1e-5, 0,
+                                                         stream))
+                    inner_states.append(x.view(B, T, D).transpose(0, 1).clone())
+                    out_flags = OUT if want_packed else 0
+                    feat = h if want_packed else torch.empty(M, D, dtype=torch.float16,
+                                                             device=dev)
+                    self._layernorm(lib, stream, x, ln, M, D, feat, out_flags)
+                elif last and not want_packed:
+                    feat = torch.empty(M, D, dtype=torch.float16, device=dev)
+                    check(lib.msa_residual_layernorm_f16(ptr(part), S_f, ptr(layer.fc2.bias),
+                                                         ptr(x), ptr(ln.weight), ptr(ln.bias),
+                                                         ptr(feat), M, D, 1e-5, 0, stream))
+                else:
+                    feat = h
+                    check(lib.msa_residual_layernorm_f16(ptr(part), S_f, ptr(layer.fc2.bias),
+                                                         ptr(x), ptr(ln.weight), ptr(ln.bias),
+                                                         ptr(h), M, D, 1e-5, OUT, stream))
+            if not self.return_inner_states:
+                inner_states.append(None)
+            packed = want_packed
+            features = feat if packed else feat.view(B, T, D)
+        else:
+            # ---- prefill (or a decode batch above 64 rows): row-major activations, tiled MFMA
+            # kernels ----
+            h = torch.empty_like(x)
+            o = torch.empty_like(x)
+            u = torch.empty(M, F, dtype=torch.float16, device=dev)
+            for i, layer in enumerate(self.layers):
+                self._layernorm(lib, stream, x, layer.self_attn_layer_norm, M, D, h)
+                kc, vc = cache.k(i), cache.v(i)
+                self._qkv(lib, stream, h, layer.self_attn.qkv_proj, q, kc, vc, B, T, H, hd, S0,
+                          cache.capacity, D, 0)
+                check(lib.msa_attention_f16(ptr(q), ptr(kc), ptr(vc), ptr(mask), mask_stride,
+                                            ptr(o), B, H, hd, T, S0, cache.capacity, 0, stream))
+                # x = round(round(o Wo^T + bo) + x)   (transformer_decoder_layer.py:222-230)
+                self._linear(lib, stream, o, layer.self_attn.out_proj, M, D, D, residual=x, out=x)
+                self._layernorm(lib, stream, x, layer.final_layer_norm, M, D, h)
+                self._linear(lib, stream, h, layer.fc1, M, F, D, relu=True, out=u)
+                self._linear(lib, stream, u, layer.fc2, M, D, F, residual=x, out=x)
+            if self.return_inner_states:
+                inner_states.append(x.view(B, T, D).transpose(0, 1).clone())
             else:
-                check(lib.msa_qkv_proj_f16(ptr(h), ptr(qkv.weight), ptr(qkv.bias), ptr(q),
-                                           ptr(kc), ptr(vc), B, T, H, hd, S0, cache.capacity, D,
-                                           None, 0, stream))
-            check(lib.msa_attention_f16(ptr(q), ptr(kc), ptr(vc), ptr(mask), mask_stride, ptr(o),
-                                        B, H, hd, T, S0, cache.capacity, stream))
-            # x = round(round(o Wo^T + bo) + x)   (transformer_decoder_layer.py:222-230)
-            self._linear(lib, stream, o, layer.self_attn.out_proj, M, D, D, residual=x, out=x)
-            self._layernorm(lib, stream, x, layer.final_layer_norm, M, D, out=h)
-            self._linear(lib, stream, h, layer.fc1, M, F, D, relu=True, out=u)
-            self._linear(lib, stream, u, layer.fc2, M, D, F, residual=x, out=x)
+                inner_states.append(None)
+            self._layernorm(lib, stream, x, self.layer_norm, M, D, h)
+            packed = False
+            features = h.view(B, T, D)
         cache.length = S0 + T
         if incremental_state is not None:
             incremental_state[self._state_key] = cache
-        if self.return_inner_states:
-            inner_states.append(x.view(B, T, D).transpose(0, 1).clone())
-        else:
-            inner_states.append(None)
-        self._layernorm(lib, stream, x, self.layer_norm, M, D, out=h)
-        return h.view(B, T, D), {"inner_states": inner_states}
+        return features, packed, (B, T), {"inner_states": inner_states}
+
+    def extract_features(self, prev_output_tokens, incremental_state=None,
+                         token_embeddings=None, self_attn_padding_mask=None):
+        """metaseq/models/transformer_decoder.py:348-396.  Returns features ``[B, T, D]`` (the
+        reference returns the same values as ``[T, B, D]``)."""
+        f, _, _, extra = self._forward_features(prev_output_tokens, incremental_state,
+                                                token_embeddings, self_attn_padding_mask, False)
+        return f, extra
+
+    def _project(self, features, packed, B, T):
+        lib = self._lib
+        D, V = self.cfg.decoder_embed_dim, self.cfg.vocab_size
+        y = torch.empty(B * T, V, dtype=torch.float16, device=features.device)
+        check(lib.msa_linear_f16(ptr(features), ptr(self._lm_head), None, None, ptr(y), B * T, V,
+                                 D, MSA_IN_PACKED if packed else 0, _capi.stream_ptr()))
+        return y.view(B, T, V)
 
     def output_layer(self, features, **kwargs):
         """Tied vocabulary projection without bias
-        (metaseq/models/transformer_decoder.py:398-428). features ``[B, T, D]``."""
-        lib = self._lib or _capi.load()
+        (metaseq/models/transformer_decoder.py:398-428). features ``[B, T, D]`` row-major."""
+        self.prepare_()
         B, T, D = features.shape
-        V = self.cfg.vocab_size
-        f = features.contiguous().view(B * T, D)
-        y = torch.empty(B * T, V, dtype=torch.float16, device=f.device)
-        check(lib.msa_linear_f16(ptr(f), ptr(self.embed_tokens.weight), None, None, ptr(y), B * T,
-                                 V, D, 0, None, 0, _capi.stream_ptr()))
-        return y.view(B, T, V)
+        return self._project(features.contiguous(), False, B, T)
 
     def forward(self, prev_output_tokens,
                 incremental_state: Optional[Dict[str, Any]] = None,
                 features_only: bool = False, src_lengths=None, token_embeddings=None,
                 self_attn_padding_mask=None):
         """metaseq/models/transformer_decoder.py:494-537."""
-        x, extra = self.extract_features(prev_output_tokens, incremental_state=incremental_state,
-                                         token_embeddings=token_embeddings,
-                                         self_attn_padding_mask=self_attn_padding_mask)
-        if not features_only:
-            x = self.output_layer(x)
-        return x, extra
+        f, packed, (B, T), extra = self._forward_features(
+            prev_output_tokens, incremental_state, token_embeddings, self_attn_padding_mask,
+            want_packed=not features_only)
+        if features_only:
+            return f, extra
+        return self._project(f, packed, B, T), extra
 
 
 # the name the reference's model code uses for this class

@@ -54,11 +54,11 @@ def test_loader_reports_version_and_fails_loudly_without_library(monkeypatch, tm
 def test_argument_validation_needs_no_gpu():
     """Entry points reject bad arguments before touching the device."""
     lib = _capi.load()
-    assert lib.msa_layernorm_f16(None, None, None, None, 1, 64, 1e-5, None) == -1
+    assert lib.msa_layernorm_f16(None, None, None, None, 1, 64, 1e-5, 0, None) == -1
     assert b"null pointer" in lib.msa_last_error()
     one = ctypes.c_void_p(16)
-    assert lib.msa_linear_f16(one, one, None, None, one, 4, 8, 40, 0, None, 0, None) == -1
+    assert lib.msa_linear_f16(one, one, None, None, one, 4, 16, 40, 0, None) == -1
     assert b"multiple of 32" in lib.msa_last_error()
-    assert lib.msa_attention_f16(one, one, one, None, 0, one, 1, 1, 64, 2, 9, 10, None) == -2
+    assert lib.msa_attention_f16(one, one, one, None, 0, one, 1, 1, 64, 2, 9, 10, 0, None) == -2
     with pytest.raises(ValueError):
         _capi.check(-2, lib)

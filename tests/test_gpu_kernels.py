@@ -57,6 +57,39 @@ def ok(rc, lib):
     assert rc == 0, lib.msa_last_error().decode()
 
 
+IN_PACKED, OUT_PACKED = 2, 4
+
+
+def pack_w(lib, w):
+    """row-major [N, K] fp16 device tensor -> tile-packed copy (through the C ABI)."""
+    out = torch.empty_like(w)
+    ok(lib.msa_pack_weight_f16(P(w), P(out), w.shape[0], w.shape[1], None), lib)
+    _KEEP.append(out)
+    return out
+
+
+def pack_w8(lib, q):
+    out = torch.empty_like(q)
+    ok(lib.msa_pack_weight_i8(P(q), P(out), q.shape[0], q.shape[1], None), lib)
+    _KEEP.append(out)
+    return out
+
+
+def pack_act(x):
+    """[M, K] -> packed activation layout (host-side restatement of the documented formula)."""
+    M, K = x.shape
+    MB = (M + 15) // 16
+    xp = torch.zeros(MB * 16, K, dtype=x.dtype)
+    xp[:M] = x
+    return xp.view(MB, 16, K // 32, 4, 8).permute(2, 0, 3, 1, 4).contiguous().view(-1)
+
+
+def unpack_act(xp, M, K):
+    MB = (M + 15) // 16
+    x = xp.view(K // 32, MB, 4, 16, 8).permute(1, 3, 0, 2, 4).contiguous().view(MB * 16, K)
+    return x[:M]
+
+
 def rnd(*shape, seed=0, std=1.0):
     g = torch.Generator().manual_seed(seed)
     return (torch.randn(*shape, generator=g) * std).half()
@@ -71,15 +104,22 @@ def test_layernorm(lib, rows, D):
     b = rnd(D, seed=3, std=0.1)
     want = O.layer_norm(x, g, b).half()
     y = torch.empty(rows, D, dtype=torch.float16, device=DEV)
-    ok(lib.msa_layernorm_f16(P(G(x)), P(G(g)), P(G(b)), P(y), rows, D, 1e-5, None),
+    ok(lib.msa_layernorm_f16(P(G(x)), P(G(g)), P(G(b)), P(y), rows, D, 1e-5, 0, None),
        lib)
     torch.cuda.synchronize()
     assert_fp16_close(y, want, what="layernorm")
+    if rows <= 64 and D % 32 == 0:
+        MB = (rows + 15) // 16
+        yp = torch.zeros(MB * 16 * D, dtype=torch.float16, device=DEV)
+        ok(lib.msa_layernorm_f16(P(G(x)), P(G(g)), P(G(b)), P(yp), rows, D, 1e-5, OUT_PACKED,
+                                 None), lib)
+        torch.cuda.synchronize()
+        assert torch.equal(unpack_act(yp.cpu(), rows, D), y.cpu())
 
 
 def test_layernorm_rejects_bad_dim(lib):
     x = torch.zeros(4, 12, dtype=torch.float16, device=DEV)
-    assert lib.msa_layernorm_f16(P(x), P(x), P(x), P(x), 4, 12, 1e-5, None) == -1
+    assert lib.msa_layernorm_f16(P(x), P(x), P(x), P(x), 4, 12, 1e-5, 0, None) == -1
     assert b"multiple of 8" in lib.msa_last_error()
 
 
@@ -122,74 +162,189 @@ def test_embed_flags_out_of_range_ids(lib):
     assert int(st) == 1
 
 
+def test_pack_roundtrip_and_layout(lib):
+    """pack/unpack are inverse, and the packed layout is the documented one."""
+    N, K = 48, 96
+    w = rnd(N, K, seed=1)
+    wp = pack_w(lib, G(w))
+    back = torch.empty_like(wp)
+    ok(lib.msa_unpack_weight_f16(P(wp), P(back), N, K, None), lib)
+    torch.cuda.synchronize()
+    assert torch.equal(back.cpu(), w)
+    want = w.view(N // 16, 16, K // 32, 4, 8).permute(0, 2, 3, 1, 4).contiguous()
+    assert torch.equal(wp.cpu().view(-1), want.view(-1))
+    q = torch.randint(-127, 128, (32, 128), dtype=torch.int8)
+    qp = pack_w8(lib, G(q))
+    qb = torch.empty_like(qp)
+    ok(lib.msa_unpack_weight_i8(P(qp), P(qb), 32, 128, None), lib)
+    torch.cuda.synchronize()
+    assert torch.equal(qb.cpu(), q)
+    # block (t, ks8): lane 16g+r holds [k = 64ks8+8g..+7 | k = 64ks8+32+8g..+7] of row 16t+r
+    want = q.view(2, 16, 2, 2, 4, 8).permute(0, 2, 4, 1, 3, 5).contiguous()
+    assert torch.equal(qp.cpu().view(-1), want.view(-1))
+    x = torch.zeros(4, 40, dtype=torch.float16, device=DEV)
+    assert lib.msa_pack_weight_f16(P(x), P(x), 16, 32, None) == -1      # aliased
+    assert lib.msa_pack_weight_f16(P(x), P(back), 24, 32, None) == -1   # N % 16
+
+
 LINEAR_SHAPES = [
     # M, N, K
     (1, 96, 64), (8, 768, 768), (32, 3072, 768), (32, 768, 3072), (33, 2048, 2048),
     (64, 4096, 4096), (17, 50272, 768), (65, 768, 768), (200, 2304, 768), (513, 4096, 1024),
-    (129, 1000, 96),
+    (129, 1008, 96),
 ]
+
+
+def _linear_want(x, W, b, res, relu):
+    want = O.linear(x.float(), W.float(), None if b is None else b.float(), r16)
+    if relu:
+        want = F.relu(want)
+    if res is not None:
+        want = r16(want + res.float())
+    return want
 
 
 @pytest.mark.parametrize("M,N,K", LINEAR_SHAPES)
 @pytest.mark.parametrize("epi", ["plain", "bias", "bias_relu", "bias_res"])
 def test_linear_f16(lib, M, N, K, epi):
+    """Row-major activations (tiled kernel) and, for M <= 64, packed activations (streaming
+    kernel, row-major and packed outputs) against the oracle's linear."""
     print("linear", M, N, K, epi, flush=True)
     x, W = rnd(M, K, seed=7), rnd(N, K, seed=8, std=0.05)
     b = rnd(N, seed=9, std=0.1) if epi != "plain" else None
     res = rnd(M, N, seed=10) if epi == "bias_res" else None
-    want = O.linear(x.float(), W.float(), None if b is None else b.float(), r16)
-    if epi == "bias_relu":
-        want = F.relu(want)
-    if res is not None:
-        want = r16(want + res.float())
-    y = torch.full((M, N), float("nan"), dtype=torch.float16, device=DEV)
-    dres = None if res is None else res.to(DEV)
-    ok(lib.msa_linear_f16(P(G(x)), P(G(W)), P(G(b)),
-                          P(dres), P(y), M, N, K, 1 if epi == "bias_relu" else 0, None, 0, None),
-       lib)
-    torch.cuda.synchronize()
+    relu = epi == "bias_relu"
+    want = _linear_want(x, W, b, res, relu).half()
     # with a second rounding point (bias / residual add) a 1-ulp difference of the intermediate
     # survives at the intermediate's magnitude even where the final value cancels to ~0
     atol = 2e-5 if epi == "plain" else float(want.abs().max()) * 2 ** -10
-    assert_fp16_close(y, want.half(), atol=atol, what="linear %s" % epi)
+    Wp = pack_w(lib, G(W))
+    flags = 1 if relu else 0
+    y = torch.full((M, N), float("nan"), dtype=torch.float16, device=DEV)
+    ok(lib.msa_linear_f16(P(G(x)), P(Wp), P(G(b)), P(G(res)), P(y), M, N, K, flags, None), lib)
+    torch.cuda.synchronize()
+    assert_fp16_close(y, want, atol=atol, what="linear %s (tiled)" % epi)
+    if M <= 64:
+        xp = G(pack_act(x))
+        y2 = torch.full((M, N), float("nan"), dtype=torch.float16, device=DEV)
+        ok(lib.msa_linear_f16(P(xp), P(Wp), P(G(b)), P(G(res)), P(y2), M, N, K,
+                              flags | IN_PACKED, None), lib)
+        torch.cuda.synchronize()
+        assert_fp16_close(y2, want, atol=atol, what="linear %s (stream)" % epi)
+        if N % 32 == 0:
+            MB = (M + 15) // 16
+            y3 = torch.zeros(MB * 16 * N, dtype=torch.float16, device=DEV)
+            ok(lib.msa_linear_f16(P(xp), P(Wp), P(G(b)), P(G(res)), P(y3), M, N, K,
+                                  flags | IN_PACKED | OUT_PACKED, None), lib)
+            torch.cuda.synchronize()
+            assert torch.equal(unpack_act(y3.cpu(), M, N), y2.cpu())
 
 
 def test_linear_in_place_residual(lib):
-    M, N, K = 32, 768, 3072
-    x, W, b, res = rnd(M, K, seed=1), rnd(N, K, seed=2, std=0.05), rnd(N, seed=3), rnd(M, N, seed=4)
-    want = r16(O.linear(x.float(), W.float(), b.float(), r16) + res.float())
-    y = res.to(DEV).clone()
-    ok(lib.msa_linear_f16(P(G(x)), P(G(W)), P(G(b)), P(y), P(y), M, N, K, 0, None,
-                          0, None), lib)
-    torch.cuda.synchronize()
-    assert_fp16_close(y, want.half(), atol=float(want.abs().max()) * 2 ** -10,
-                      what="in-place residual")
+    for M, flags in ((32, IN_PACKED), (200, 0)):
+        N, K = 768, 3072
+        x, W, b = rnd(M, K, seed=1), rnd(N, K, seed=2, std=0.05), rnd(N, seed=3)
+        res = rnd(M, N, seed=4)
+        want = _linear_want(x, W, b, res, False)
+        y = G(res).clone()
+        xin = G(pack_act(x)) if flags else G(x)
+        ok(lib.msa_linear_f16(P(xin), P(pack_w(lib, G(W))), P(G(b)), P(y), P(y), M, N, K, flags,
+                              None), lib)
+        torch.cuda.synchronize()
+        assert_fp16_close(y, want.half(), atol=float(want.abs().max()) * 2 ** -10,
+                          what="in-place residual")
 
 
 def test_linear_rejects_bad_shapes(lib):
-    x = torch.zeros(4, 40, dtype=torch.float16, device=DEV)
-    assert lib.msa_linear_f16(P(x), P(x), None, None, P(x), 4, 8, 40, 0, None, 0, None) == -1
-    assert lib.msa_linear_f16(None, P(x), None, None, P(x), 4, 8, 32, 0, None, 0, None) == -1
-    assert lib.msa_linear_f16(P(x), P(x), None, None, P(x), 4, 8, 32, 8, None, 0, None) == -1
+    x = torch.zeros(64, 64, dtype=torch.float16, device=DEV)
+    y = torch.zeros(64, 64, dtype=torch.float16, device=DEV)
+    assert lib.msa_linear_f16(P(x), P(x), None, None, P(y), 4, 16, 40, 0, None) == -1   # K % 32
+    assert lib.msa_linear_f16(P(x), P(x), None, None, P(y), 4, 8, 32, 0, None) == -1    # N % 16
+    assert lib.msa_linear_f16(None, P(x), None, None, P(y), 4, 16, 32, 0, None) == -1
+    assert lib.msa_linear_f16(P(x), P(x), None, None, P(y), 4, 16, 32, 64, None) == -1  # flags
+    assert lib.msa_linear_f16(P(x), P(x), None, None, P(y), 65, 16, 32, IN_PACKED, None) == -1
+    assert lib.msa_linear_partial_f16(P(x), P(x), P(y), 4, 16, 64, 1, 0, None) == -1    # not packed
+    assert lib.msa_linear_partial_f16(P(x), P(x), P(y), 4, 16, 64, 3, IN_PACKED, None) == -1
 
 
 @pytest.mark.parametrize("M,N,K", [(8, 768, 768), (64, 3072, 768), (32, 768, 3072),
-                                   (200, 2304, 768)])
+                                   (200, 2304, 768), (48, 4096, 4096)])
 def test_linear_w8a16(lib, M, N, K):
     print("w8a16", M, N, K, flush=True)
     x, W, b = rnd(M, K, seed=7), rnd(N, K, seed=8, std=0.02), rnd(N, seed=9, std=0.1)
     q, s = O.quantize_int8(W)
     Wd = O.dequantize_int8(q, s)
-    want = O.linear(x.float(), Wd.float(), b.float(), r16)
+    want = O.linear(x.float(), Wd.float(), b.float(), r16).half()
+    atol = float(want.abs().max()) * 2 ** -10
+    qp = pack_w8(lib, G(q))
     y = torch.empty(M, N, dtype=torch.float16, device=DEV)
-    ok(lib.msa_linear_w8a16(P(G(x)), P(G(q)), P(G(s)), P(G(b)), None, P(y), M,
-                            N, K, 0, None, 0, None), lib)
+    ok(lib.msa_linear_w8a16(P(G(x)), P(qp), P(G(s)), P(G(b)), None, P(y), M, N, K, 0, None), lib)
     torch.cuda.synchronize()
-    assert_fp16_close(y, want.half(), atol=float(want.abs().max()) * 2 ** -10, what="w8a16")
+    assert_fp16_close(y, want, atol=atol, what="w8a16 (tiled)")
+    if M <= 64:
+        y2 = torch.empty(M, N, dtype=torch.float16, device=DEV)
+        ok(lib.msa_linear_w8a16(P(G(pack_act(x))), P(qp), P(G(s)), P(G(b)), None, P(y2), M, N, K,
+                                IN_PACKED, None), lib)
+        torch.cuda.synchronize()
+        assert_fp16_close(y2, want, atol=atol, what="w8a16 (stream)")
+
+
+@pytest.mark.parametrize("M,N,K,S", [(32, 768, 768, 1), (32, 768, 3072, 4), (8, 4096, 4096, 4),
+                                     (33, 2048, 8192, 8), (64, 768, 3072, 3)])
+@pytest.mark.parametrize("w8", [False, True])
+def test_split_k_partials_and_fused_layernorm(lib, M, N, K, S, w8):
+    """msa_linear_partial_* followed by msa_residual_layernorm_f16 equals the oracle's
+    linear + bias, residual add and LayerNorm."""
+    print("splitk", M, N, K, S, w8, flush=True)
+    x, W, b = rnd(M, K, seed=7), rnd(N, K, seed=8, std=0.03), rnd(N, seed=9, std=0.1)
+    res, g, be = rnd(M, N, seed=10), (1 + rnd(N, seed=11, std=0.1).float()).half(), rnd(N, seed=12)
+    if w8:
+        q, sc = O.quantize_int8(W)
+        Wuse = O.dequantize_int8(q, sc)
+    else:
+        Wuse = W
+    xo = r16(O.linear(x.float(), Wuse.float(), b.float(), r16) + res.float())
+    want_h = O.layer_norm(xo, g, be).half()
+    part = torch.full((S, M, N), float("nan"), dtype=torch.float32, device=DEV)
+    xp = G(pack_act(x))
+    if w8:
+        ok(lib.msa_linear_partial_w8a16(P(xp), P(pack_w8(lib, G(q))), P(G(sc)), P(part), M, N, K,
+                                        S, IN_PACKED, None), lib)
+    else:
+        ok(lib.msa_linear_partial_f16(P(xp), P(pack_w(lib, G(W))), P(part), M, N, K, S, IN_PACKED,
+                                      None), lib)
+    xd = G(res).clone()
+    MB = (M + 15) // 16
+    hp = torch.zeros(MB * 16 * N, dtype=torch.float16, device=DEV)
+    ok(lib.msa_residual_layernorm_f16(P(part), S, P(G(b)), P(xd), P(G(g)), P(G(be)), P(hp), M, N,
+                                      1e-5, OUT_PACKED, None), lib)
+    torch.cuda.synchronize()
+    # the partials are exact fp32 sums of their K range
+    tot = part.sum(0).cpu()
+    assert (tot - x.float() @ Wuse.float().t()).abs().max() < 1e-3
+    atol = float(xo.abs().max()) * 2 ** -10
+    assert_fp16_close(xd, xo.half(), atol=atol, what="residual stream")
+    got_h = unpack_act(hp.cpu(), M, N)
+    # a 1-ulp difference in x moves the normalised value by about one ulp of x / sigma
+    assert_fp16_close(got_h, want_h, max_ulp=2, max_frac=2e-2, atol=4 * atol, what="fused LN")
+    # without LayerNorm outputs only the residual stream is updated
+    xd2 = G(res).clone()
+    ok(lib.msa_residual_layernorm_f16(P(part), S, P(G(b)), P(xd2), None, None, None, M, N, 1e-5, 0,
+                                      None), lib)
+    torch.cuda.synchronize()
+    assert torch.equal(xd2, xd)
+
+
+def test_default_splits_are_valid(lib):
+    for M, N, K in [(32, 4096, 4096), (32, 4096, 16384), (32, 12288, 4096), (1, 768, 768),
+                    (8, 2048, 8192), (64, 9216, 36864), (200, 4096, 4096)]:
+        S = lib.msa_linear_default_splits(M, N, K)
+        assert 1 <= S <= 8 and K // 64 >= S, (M, N, K, S)
+    assert lib.msa_linear_default_splits(32, 4096, 16384) > 1
 
 
 @pytest.mark.parametrize("B,T,H,hd,S0", [(3, 1, 2, 64, 5), (2, 7, 4, 128, 0), (32, 1, 12, 64, 40),
-                                         (2, 70, 2, 64, 0)])
+                                         (2, 70, 2, 64, 0), (64, 1, 4, 128, 3)])
 @pytest.mark.parametrize("w8", [False, True])
 def test_qkv_proj_scatter(lib, B, T, H, hd, S0, w8):
     print("qkv", B, T, H, hd, S0, w8, flush=True)
@@ -204,30 +359,33 @@ def test_qkv_proj_scatter(lib, B, T, H, hd, S0, w8):
     kvq = O.linear(x.float(), Wuse.float(), b.float(), r16)
     k, v, q = kvq.split(D, dim=-1)
     q = r16(q * (hd ** -0.5))
-    Kc = torch.zeros(B, H, S_cap, hd, dtype=torch.float16, device=DEV)
-    Vc = torch.zeros_like(Kc)
-    qo = torch.empty(B * T, D, dtype=torch.float16, device=DEV)
-    if w8:
-        ok(lib.msa_qkv_proj_w8a16(P(G(x)), P(G(qw)), P(G(sc)), P(G(b)), P(qo),
-                                  P(Kc), P(Vc), B, T, H, hd, S0, S_cap, D, None, 0, None), lib)
-    else:
-        ok(lib.msa_qkv_proj_f16(P(G(x)), P(G(W)), P(G(b)), P(qo), P(Kc), P(Vc), B,
-                                T, H, hd, S0, S_cap, D, None, 0, None), lib)
-    torch.cuda.synchronize()
-    atol = float(kvq.abs().max()) * 2 ** -10
-    assert_fp16_close(qo, q.half(), atol=atol, what="q")
     want_k = k.view(B, T, H, hd).permute(0, 2, 1, 3)
     want_v = v.view(B, T, H, hd).permute(0, 2, 1, 3)
-    assert_fp16_close(Kc[:, :, S0:S0 + T], want_k.half(), atol=atol, what="K cache")
-    assert_fp16_close(Vc[:, :, S0:S0 + T], want_v.half(), atol=atol, what="V cache")
-    # nothing outside the appended slice was touched
-    assert float(Kc[:, :, :S0].abs().sum()) == 0 and float(Kc[:, :, S0 + T:].abs().sum()) == 0
+    atol = float(kvq.abs().max()) * 2 ** -10
+    modes = [0] + ([IN_PACKED] if B * T <= 64 else [])
+    for flags in modes:
+        Kc = torch.zeros(B, H, S_cap, hd, dtype=torch.float16, device=DEV)
+        Vc = torch.zeros_like(Kc)
+        qo = torch.empty(B * T, D, dtype=torch.float16, device=DEV)
+        xin = G(pack_act(x)) if flags else G(x)
+        if w8:
+            ok(lib.msa_qkv_proj_w8a16(P(xin), P(pack_w8(lib, G(qw))), P(G(sc)), P(G(b)), P(qo),
+                                      P(Kc), P(Vc), B, T, H, hd, S0, S_cap, D, flags, None), lib)
+        else:
+            ok(lib.msa_qkv_proj_f16(P(xin), P(pack_w(lib, G(W))), P(G(b)), P(qo), P(Kc), P(Vc), B,
+                                    T, H, hd, S0, S_cap, D, flags, None), lib)
+        torch.cuda.synchronize()
+        assert_fp16_close(qo, q.half(), atol=atol, what="q")
+        assert_fp16_close(Kc[:, :, S0:S0 + T], want_k.half(), atol=atol, what="K cache")
+        assert_fp16_close(Vc[:, :, S0:S0 + T], want_v.half(), atol=atol, what="V cache")
+        # nothing outside the appended slice was touched
+        assert float(Kc[:, :, :S0].abs().sum()) == 0 and float(Kc[:, :, S0 + T:].abs().sum()) == 0
 
 
 def test_qkv_proj_capacity_error(lib):
     x = torch.zeros(2, 128, dtype=torch.float16, device=DEV)
-    rc = lib.msa_qkv_proj_f16(P(x), P(x), P(x), P(x), P(x), P(x), 2, 1, 2, 64, 10, 10, 128, None,
-                              0, None)
+    rc = lib.msa_qkv_proj_f16(P(x), P(x), P(x), P(x), P(x), P(x), 2, 1, 2, 64, 10, 10, 128, 0,
+                              None)
     assert rc == -2 and b"capacity" in lib.msa_last_error()
 
 
@@ -264,8 +422,16 @@ def test_attention(lib, B, H, hd, T, S0, masked):
     dm = None if mask is None else mask.to(torch.uint8).to(DEV)
     ok(lib.msa_attention_f16(P(G(q)), P(G(Kc)), P(G(Vc)), P(dm),
                              0 if dm is None else dm.stride(0), P(out), B, H, hd, T, S0, S_cap,
-                             None), lib)
+                             0, None), lib)
     torch.cuda.synchronize()
+    if T == 1 and B <= 64:
+        MB = (B + 15) // 16
+        op = torch.zeros(MB * 16 * D, dtype=torch.float16, device=DEV)
+        ok(lib.msa_attention_f16(P(G(q)), P(G(Kc)), P(G(Vc)), P(dm),
+                                 0 if dm is None else dm.stride(0), P(op), B, H, hd, T, S0, S_cap,
+                                 OUT_PACKED, None), lib)
+        torch.cuda.synchronize()
+        assert torch.equal(unpack_act(op.cpu(), B, D), out.cpu())
     # scores and probabilities are intermediate fp16 roundings: a 1-ulp flip of one of them
     # moves the output by up to one ulp of the largest output
     assert_fp16_close(out, want.half(), max_frac=2e-2, atol=float(want.abs().max()) * 2 ** -10,
@@ -274,8 +440,8 @@ def test_attention(lib, B, H, hd, T, S0, masked):
 
 def test_attention_rejects(lib):
     x = torch.zeros(64, 96, dtype=torch.float16, device=DEV)
-    assert lib.msa_attention_f16(P(x), P(x), P(x), None, 0, P(x), 1, 1, 96, 1, 0, 4, None) == -1
-    assert lib.msa_attention_f16(P(x), P(x), P(x), None, 0, P(x), 1, 1, 64, 1, 4, 4, None) == -2
+    assert lib.msa_attention_f16(P(x), P(x), P(x), None, 0, P(x), 1, 1, 96, 1, 0, 4, 0, None) == -1
+    assert lib.msa_attention_f16(P(x), P(x), P(x), None, 0, P(x), 1, 1, 64, 1, 4, 4, 0, None) == -2
 
 
 def _select(lib, logits, temperature=1.0, banned=(), stop=(), finished=None, force=0, eos=2):
