@@ -43,39 +43,43 @@ __global__ void attention_kernel(const half_t* __restrict__ q, const half_t* __r
   for (int i = 0; i < 8; ++i) qf[i] = (float)qv[i];
 
   // ---- scores ----
+  constexpr int U = 8;  // key rows in flight per lane group
   const int kstride = nw * RPW;
   float lmax = -INFINITY;
-  int key = wave * RPW + rsel;
-  for (; key + 3 * kstride < n_keys; key += 4 * kstride) {
-    half8_t kv[4];
-#pragma unroll
-    for (int u = 0; u < 4; ++u)
-      kv[u] = *reinterpret_cast<const half8_t*>(kbase + (int64_t)(key + u * kstride) * HD);
-#pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      float d = 0.f;
-#pragma unroll
-      for (int i = 0; i < 8; ++i) d = fmaf(qf[i], (float)kv[u][i], d);
-#pragma unroll
-      for (int o = LPR / 2; o > 0; o >>= 1) d += __shfl_xor(d, o, MSA_WAVE);
-      const int kk = key + u * kstride;
-      float s = round_h(d);
-      if (mrow && mrow[kk]) s = -INFINITY;
-      if (sub == 0) sc[kk] = s;
-      lmax = fmaxf(lmax, s);
-    }
-  }
-  for (; key < n_keys; key += kstride) {
-    const half8_t kv = *reinterpret_cast<const half8_t*>(kbase + (int64_t)key * HD);
+  auto score = [&](const half8_t& kv, int kk) {
     float d = 0.f;
 #pragma unroll
     for (int i = 0; i < 8; ++i) d = fmaf(qf[i], (float)kv[i], d);
 #pragma unroll
     for (int o = LPR / 2; o > 0; o >>= 1) d += __shfl_xor(d, o, MSA_WAVE);
     float s = round_h(d);
-    if (mrow && mrow[key]) s = -INFINITY;
-    if (sub == 0) sc[key] = s;
+    if (mrow && mrow[kk]) s = -INFINITY;
+    if (sub == 0) sc[kk] = s;
     lmax = fmaxf(lmax, s);
+  };
+  int key = wave * RPW + rsel;
+  for (; key + (U - 1) * kstride < n_keys; key += U * kstride) {
+    half8_t kv[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+      kv[u] = __builtin_nontemporal_load(
+          reinterpret_cast<const half8_t*>(kbase + (int64_t)(key + u * kstride) * HD));
+#pragma unroll
+    for (int u = 0; u < U; ++u) score(kv[u], key + u * kstride);
+  }
+  for (; key < n_keys; key += kstride)
+    score(__builtin_nontemporal_load(reinterpret_cast<const half8_t*>(kbase + (int64_t)key * HD)),
+          key);
+
+  // the first V rows are requested before the softmax so that HBM stays busy through it
+  half8_t vpre[U];
+  const int vkey0 = wave * RPW + rsel;
+  const bool have_pre = vkey0 + (U - 1) * kstride < n_keys;
+  if (have_pre) {
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+      vpre[u] = __builtin_nontemporal_load(
+          reinterpret_cast<const half8_t*>(vbase + (int64_t)(vkey0 + u * kstride) * HD));
   }
   const float m = block_max(lmax, red);  // barriers inside also publish sc[]
 
@@ -94,22 +98,32 @@ __global__ void attention_kernel(const half_t* __restrict__ q, const half_t* __r
   float acc[8];
 #pragma unroll
   for (int i = 0; i < 8; ++i) acc[i] = 0.f;
-  key = wave * RPW + rsel;
-  for (; key + 3 * kstride < n_keys; key += 4 * kstride) {
-    half8_t vv[4];
-    float p[4];
+  key = vkey0;
+  if (have_pre) {
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      vv[u] = *reinterpret_cast<const half8_t*>(vbase + (int64_t)(key + u * kstride) * HD);
-      p[u] = sc[key + u * kstride];
+    for (int u = 0; u < U; ++u) {
+      const float p = sc[key + u * kstride];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) acc[i] = fmaf(p, (float)vpre[u][i], acc[i]);
     }
+    key += U * kstride;
+  }
+  for (; key + (U - 1) * kstride < n_keys; key += U * kstride) {
+    half8_t vv[U];
 #pragma unroll
-    for (int u = 0; u < 4; ++u)
+    for (int u = 0; u < U; ++u)
+      vv[u] = __builtin_nontemporal_load(
+          reinterpret_cast<const half8_t*>(vbase + (int64_t)(key + u * kstride) * HD));
 #pragma unroll
-      for (int i = 0; i < 8; ++i) acc[i] = fmaf(p[u], (float)vv[u][i], acc[i]);
+    for (int u = 0; u < U; ++u) {
+      const float p = sc[key + u * kstride];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) acc[i] = fmaf(p, (float)vv[u][i], acc[i]);
+    }
   }
   for (; key < n_keys; key += kstride) {
-    const half8_t vv = *reinterpret_cast<const half8_t*>(vbase + (int64_t)key * HD);
+    const half8_t vv =
+        __builtin_nontemporal_load(reinterpret_cast<const half8_t*>(vbase + (int64_t)key * HD));
     const float p = sc[key];
 #pragma unroll
     for (int i = 0; i < 8; ++i) acc[i] = fmaf(p, (float)vv[i], acc[i]);

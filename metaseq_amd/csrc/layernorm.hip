@@ -7,8 +7,8 @@
 
 namespace {
 
-constexpr int LN_THREADS = 256;
-constexpr int LN_MAX_CHUNKS = 8;  // 8 halves per chunk per thread -> D <= 256*8*8 = 16384
+constexpr int LN_THREADS = 512;
+constexpr int LN_MAX_CHUNKS = 4;  // 8 halves per chunk per thread -> D <= 512*8*4 = 16384
 
 __global__ __launch_bounds__(LN_THREADS) void layernorm_f16_kernel(
     const half_t* x, const float* __restrict__ part, int S,
@@ -30,6 +30,7 @@ __global__ __launch_bounds__(LN_THREADS) void layernorm_f16_kernel(
         const float* p = part + (int64_t)row * D + (idx << 3);
         float4_t a0 = *reinterpret_cast<const float4_t*>(p);
         float4_t a1 = *reinterpret_cast<const float4_t*>(p + 4);
+#pragma unroll 4
         for (int i = 1; i < S; ++i) {
           const float* q = p + (int64_t)i * M * D;
           a0 += *reinterpret_cast<const float4_t*>(q);

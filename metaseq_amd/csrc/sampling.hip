@@ -14,24 +14,48 @@ struct RowStats {
   float lse;  // log(sum(exp(z - max)))   (so log_softmax(z) = z - max - lse)
 };
 
+// visits every element of a logits row as z = logit (/ temperature), 8 halves per load where the
+// row is 16-byte aligned
+template <typename F>
+__device__ __forceinline__ void for_each_z(const half_t* __restrict__ row, int V, float temp,
+                                           bool scale, F f) {
+  if ((reinterpret_cast<uintptr_t>(row) & 15) == 0) {
+    const int nv = V >> 3;
+    for (int c = threadIdx.x; c < nv; c += blockDim.x) {
+      const half8_t v = *reinterpret_cast<const half8_t*>(row + (c << 3));
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        float z = (float)v[i];
+        if (scale) z = z / temp;
+        f((c << 3) + i, z);
+      }
+    }
+    for (int i = (nv << 3) + threadIdx.x; i < V; i += blockDim.x) {
+      float z = (float)row[i];
+      if (scale) z = z / temp;
+      f(i, z);
+    }
+  } else {
+    for (int i = threadIdx.x; i < V; i += blockDim.x) {
+      float z = (float)row[i];
+      if (scale) z = z / temp;
+      f(i, z);
+    }
+  }
+}
+
 __device__ __forceinline__ RowStats row_logsumexp(const half_t* __restrict__ row, int V,
                                                   float temp, bool scale, float* red) {
   float mx = -INFINITY;
   bool nan = false;
-  for (int i = threadIdx.x; i < V; i += blockDim.x) {
-    float z = (float)row[i];
-    if (scale) z = z / temp;
+  for_each_z(row, V, temp, scale, [&](int, float z) {
     nan |= (z != z);
     mx = fmaxf(mx, z);
-  }
+  });
   mx = block_max(mx, red);
   const float any_nan = block_max(nan ? 1.f : 0.f, red);
   float s = 0.f;
-  for (int i = threadIdx.x; i < V; i += blockDim.x) {
-    float z = (float)row[i];
-    if (scale) z = z / temp;
-    s += expf(z - mx);
-  }
+  for_each_z(row, V, temp, scale, [&](int, float z) { s += expf(z - mx); });
   s = block_sum(s, red);
   RowStats r;
   r.max = mx;
@@ -44,58 +68,115 @@ struct IdList {
   int32_t id[16];
 };
 
+// (max, sum of exp(z - max)) pairs merge associatively: one pass over the row suffices
+__device__ __forceinline__ void lse_merge(float& m, float& s, float om, float os) {
+  if (om > m) {
+    s = s * expf(m - om) + os;
+    m = om;
+  } else if (om > -INFINITY) {
+    s += os * expf(om - m);
+  }
+}
+
 __global__ __launch_bounds__(SM_THREADS) void greedy_select_kernel(
     const half_t* __restrict__ logits, int64_t ld, int V, float temperature, bool scale,
     IdList banned, IdList stop, uint8_t* __restrict__ finished, int force_eos_all, int eos,
     int64_t* __restrict__ tok, int64_t tok_stride, float* __restrict__ score,
     int64_t score_stride) {
-  __shared__ float red[16];
-  __shared__ float wbest[16];
+  __shared__ float wm[16], ws[16], wbest[16], wnan[16];
   __shared__ int widx[16];
   const int b = blockIdx.x;
   const half_t* row = logits + (int64_t)b * ld;
-  const RowStats st = row_logsumexp(row, V, temperature, scale, red);
-  const bool dead = st.lse != st.lse;  // a NaN anywhere turns every log-prob into -inf
   const bool only_eos = force_eos_all || (finished && finished[b]);
 
-  float best = -INFINITY;
+  // single pass: running log-sum-exp over ALL ids, and the best eligible id (log-softmax is
+  // monotone in z, so the arg-max of the masked log-probs is the arg-max of the masked z)
+  float m = -INFINITY, s = 0.f, best = -INFINITY;
   int bidx = 0x7fffffff;
-  for (int i = threadIdx.x; i < V; i += blockDim.x) {
-    float z = (float)row[i];
-    if (scale) z = z / temperature;
-    float lp = dead ? -INFINITY : (z - st.max) - st.lse;
-    for (int j = 0; j < banned.n; ++j)
-      if (banned.id[j] == i) lp = -INFINITY;
-    if (only_eos && i != eos) lp = -INFINITY;
-    if (lp > best || (lp == best && i < bidx)) {
-      best = lp;
+  bool nan = false;
+  auto visit = [&](int i, float z) {  // arg-max bookkeeping of one id
+    nan |= (z != z);
+    bool ok = !(only_eos && i != eos);
+    for (int j = 0; j < banned.n; ++j) ok &= (banned.id[j] != i);
+    const float cand = ok ? z : -INFINITY;
+    if (cand > best || (cand == best && i < bidx)) {
+      best = cand;
       bidx = i;
     }
+  };
+  if ((reinterpret_cast<uintptr_t>(row) & 15) == 0) {
+    const int nv = V >> 3;
+    for (int c = threadIdx.x; c < nv; c += blockDim.x) {
+      const half8_t v = *reinterpret_cast<const half8_t*>(row + (c << 3));
+      float z[8], cm = -INFINITY;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        z[i] = (float)v[i];
+        if (scale) z[i] = z[i] / temperature;
+        cm = fmaxf(cm, z[i]);
+        visit((c << 3) + i, z[i]);
+      }
+      if (cm > m) {  // rescale once per 8 ids
+        s *= __expf(m - cm);
+        m = cm;
+      }
+      if (m > -INFINITY) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) s += __expf(z[i] - m);
+      }
+    }
+    for (int i = (nv << 3) + threadIdx.x; i < V; i += blockDim.x) {
+      float z = (float)row[i];
+      if (scale) z = z / temperature;
+      visit(i, z);
+      lse_merge(m, s, z, 1.f);
+    }
+  } else {
+    for (int i = threadIdx.x; i < V; i += blockDim.x) {
+      float z = (float)row[i];
+      if (scale) z = z / temperature;
+      visit(i, z);
+      lse_merge(m, s, z, 1.f);
+    }
   }
-  // wave then block arg-max; ties resolve to the lowest index
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) {
+    lse_merge(m, s, __shfl_xor(m, o, MSA_WAVE), __shfl_xor(s, o, MSA_WAVE));
     const float ob = __shfl_xor(best, o, MSA_WAVE);
     const int oi = __shfl_xor(bidx, o, MSA_WAVE);
     if (ob > best || (ob == best && oi < bidx)) {
       best = ob;
       bidx = oi;
     }
+    nan |= (bool)__shfl_xor((int)nan, o, MSA_WAVE);
   }
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   if (lane == 0) {
+    wm[wave] = m;
+    ws[wave] = s;
     wbest[wave] = best;
     widx[wave] = bidx;
+    wnan[wave] = nan ? 1.f : 0.f;
   }
   __syncthreads();
   if (threadIdx.x == 0) {
-    for (int w = 1; w < (int)(blockDim.x >> 6); ++w)
+    for (int w = 1; w < (int)(blockDim.x >> 6); ++w) {
+      lse_merge(m, s, wm[w], ws[w]);
       if (wbest[w] > best || (wbest[w] == best && widx[w] < bidx)) {
         best = wbest[w];
         bidx = widx[w];
       }
+      nan |= wnan[w] > 0.f;
+    }
+    // lprob = (z - max) - log(sum(exp(z - max))); a NaN anywhere, or no eligible finite id,
+    // leaves every eligible log-prob at -inf and the lowest index wins
+    float lp = (best - m) - logf(s);
+    if (nan || !(best > -INFINITY)) {
+      lp = -INFINITY;
+      bidx = 0;
+    }
     tok[b * tok_stride] = bidx;
-    score[b * score_stride] = best;
+    score[b * score_stride] = lp;
     if (finished) {
       bool f = bidx == eos;
       for (int j = 0; j < stop.n; ++j) f |= (stop.id[j] == bidx);
