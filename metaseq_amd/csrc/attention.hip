@@ -1,6 +1,7 @@
-// Causal attention over the contiguous per-layer KV cache [B, H, S_cap, hd].
+// Decode attention (one new query per row) over the contiguous per-layer KV cache
+// [B, H, S_cap, hd]; queries with T > 1 go to the MFMA kernel in attention_prefill.hip.
 //
-// One workgroup per (batch row, head, query).  The workgroup streams the K rows of its head
+// One workgroup per (batch row, head).  The workgroup streams the K rows of its head
 // once (16-byte loads, hd/8 lanes per key row, so each wave instruction reads whole 128- or
 // 256-byte rows), forms the fp16-rounded scores in LDS, normalises them with an fp32 softmax
 // whose probabilities are rounded to fp16 exactly like the reference's cast-back, then streams
@@ -173,6 +174,13 @@ extern "C" int msa_attention_f16(const void* q, const void* Kcache, const void* 
               "msa_attention_f16: packed output needs T == 1 and B <= 64 (T=%d B=%d)", T, B);
   const int out_mb = (flags & MSA_OUT_PACKED) ? (B + 15) / 16 : 0;
   const int64_t BH = (int64_t)B * H;
+  if (T > 1) {
+    MSA_REQUIRE(BH <= 0x7fffffff, MSA_ERR_INVALID_ARG, "msa_attention_f16: B*H too large");
+    msa_launch_prefill_attention(q, Kcache, Vcache, key_pad_mask, mask_stride, out, B, H, hd, T,
+                                 S0, S_cap, (hipStream_t)stream);
+    MSA_CHECK_LAUNCH("msa_attention_f16");
+    return MSA_OK;
+  }
   // few (b,h) pairs: spend more waves on each so the chip still fills
   const int threads = (T == 1 && BH < 512) ? 1024 : 256;
   const size_t lds = (size_t)(S0 + T) * sizeof(float);

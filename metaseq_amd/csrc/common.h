@@ -18,6 +18,12 @@ typedef float float16_t __attribute__((ext_vector_type(16)));
 
 void msa_set_error(const char* fmt, ...);
 
+// MFMA flash-style causal attention for T > 1 new queries (attention_prefill.hip)
+int msa_launch_prefill_attention(const void* q, const void* Kc, const void* Vc,
+                                 const uint8_t* key_pad_mask, int64_t mask_stride, void* out,
+                                 int B, int H, int hd, int T, int S0, int S_cap,
+                                 hipStream_t stream);
+
 #define MSA_REQUIRE(cond, code, ...) \
   do {                               \
     if (!(cond)) {                   \
