@@ -26,6 +26,11 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK = 8.0e12  # MI355X HBM3E, bytes/s
+MFMA_PEAK = 2.5e15  # dense fp16 MFMA, flop/s
+# HBM bytes per decode-attention launch over its algorithmic bytes, from rocprofv3 FETCH_SIZE +
+# WRITE_SIZE scaled by a 1 GiB copy (profiles/decode_attention_opt6.7b_bs32_pmc_traffic.txt):
+# 540.1 MB measured for 540.0 MB algorithmic.
+ATTN_TRAFFIC_RATIO = 540.1 / 540.0
 
 CONFIGS = {
     # name: (size, batch, prompt, generate)
@@ -45,6 +50,12 @@ def step_bytes(cfg, B, S, int8=False):
     if int8:
         weights += L * 9 * D * 2
     return weights + V * D * 2 + 2 * L * B * S * D * 2 + 2 * L * B * D * 2
+
+
+def prefill_flops(cfg, B, T):
+    """2*(12*D^2*L + V*D)*B*T for the GEMMs + 4*L*B*T^2*D for attention counted un-causal."""
+    L, D, V = cfg.decoder_layers, cfg.decoder_embed_dim, cfg.vocab_size
+    return 2.0 * (12 * D * D * L + V * D) * B * T + 4.0 * L * B * T * T * D
 
 
 def attn_bytes(cfg, B, S):
@@ -111,6 +122,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--config", default="6.7b", choices=sorted(CONFIGS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--pmc-calibration", action="store_true",
+                    help="also run a plain 1 GiB device copy, the known-size kernel that "
+                         "rocprofv3 FETCH_SIZE / WRITE_SIZE readings are scaled by")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU; --gpus %d is not supported (nothing in the "
@@ -135,6 +149,15 @@ def main():
     cfg = opt_config(size, max_target_positions=max(2048, max_len))
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+
+    if args.pmc_calibration:
+        a = torch.ones(1 << 29, dtype=torch.float16, device=dev)
+        bcopy = torch.empty_like(a)
+        for _ in range(3):
+            bcopy.copy_(a)
+        torch.cuda.synchronize()
+        del a, bcopy
+        torch.cuda.empty_cache()
 
     t0 = time.time()
     sd = random_state_dict(cfg, seed=1234, dtype=torch.float16, device=dev)
@@ -216,7 +239,9 @@ def main():
     achieved = ab / attn_s / 1e9
 
     result = {
-        "metric": "decode tokens/sec + % HBM roofline, OPT-6.7B-shape fp16 bs32, 1xMI355X",
+        "metric": ("decode tokens/sec + % HBM roofline, OPT-6.7B-shape fp16 bs32, 1xMI355X"
+                   if args.config == "6.7b" else
+                   "decode tokens/sec + %% HBM roofline, OPT-%s shape bs%d, 1xMI355X" % (size, B)),
         "value": B / t_step,
         "unit": "tokens/s",
         "n_gpus": 1,
@@ -237,11 +262,14 @@ def main():
         "step_bytes_mean": bytes_mean,
         "gpu_ms_per_step": gpu_s / K * 1e3,
         "prefill_s": prefill_s,
+        "prefill_tflops": prefill_flops(cfg, B, n0) / prefill_s / 1e12,
+        "prefill_mfma_frac": prefill_flops(cfg, B, n0) / prefill_s / MFMA_PEAK,
         "setup_s": t1 - t0,
         "roofline": {
             "kernel": "attention_kernel<%d> (decode, T=1)" % hd,
             "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK / 1e9, "unit": "GB/s",
-            "frac": achieved * 1e9 / HBM_PEAK, "traffic": None,
+            "frac": achieved * 1e9 / HBM_PEAK,
+            "traffic": ab * ATTN_TRAFFIC_RATIO if args.config == "6.7b" else None,
             "bytes_per_launch": ab, "avg_launch_us": attn_s * 1e6, "context": S_probe,
         },
     }

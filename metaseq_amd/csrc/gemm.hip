@@ -90,18 +90,25 @@ __device__ __forceinline__ void epilogue4(const Epilogue& e, int64_t m, int n, f
 
 __device__ __forceinline__ half8_t zero8() { return half8_t{0, 0, 0, 0, 0, 0, 0, 0}; }
 
-// 8 int8 (two dwords) times an fp16 per-row scale -> 8 fp16, each round(q * scale)
+// 8 int8 (two dwords) times an fp16 per-row scale -> 8 fp16, each round(q * scale).
+// Bytes are biased to unsigned (q + 128), dropped into the mantissa of fp16 1024.0 (0x6400 | u
+// is exactly 1024 + u), and 1152 is subtracted: q exactly, in packed fp16 arithmetic.  The
+// packed multiply then rounds the exact product q * scale once, as the fp32 route would.
 __device__ __forceinline__ half8_t dequant8(uint32_t lo, uint32_t hi, half_t scale) {
+  const half2_t bias = {(half_t)1152.0f, (half_t)1152.0f};
+  const half2_t sc = {scale, scale};
   half8_t r;
-  const uint32_t w[2] = {lo, hi};
-  const float s = (float)scale;
+  const uint32_t w[2] = {lo ^ 0x80808080u, hi ^ 0x80808080u};
 #pragma unroll
   for (int j = 0; j < 2; ++j) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int q = (int)(int8_t)((w[j] >> (8 * i)) & 0xff);
-      r[j * 4 + i] = (half_t)((float)q * s);
-    }
+    const uint32_t p0 = __builtin_amdgcn_perm(0x64646464u, w[j], 0x04010400u);  // bytes 0, 1
+    const uint32_t p1 = __builtin_amdgcn_perm(0x64646464u, w[j], 0x04030402u);  // bytes 2, 3
+    const half2_t h0 = (__builtin_bit_cast(half2_t, p0) - bias) * sc;
+    const half2_t h1 = (__builtin_bit_cast(half2_t, p1) - bias) * sc;
+    r[4 * j + 0] = h0[0];
+    r[4 * j + 1] = h0[1];
+    r[4 * j + 2] = h1[0];
+    r[4 * j + 3] = h1[1];
   }
   return r;
 }

@@ -433,9 +433,10 @@ def test_attention(lib, B, H, hd, T, S0, masked):
                                  OUT_PACKED, None), lib)
         torch.cuda.synchronize()
         assert torch.equal(unpack_act(op.cpu(), B, D), out.cpu())
-    # scores and probabilities are intermediate fp16 roundings: a 1-ulp flip of one of them
-    # moves the output by up to one ulp of the largest output
-    assert_fp16_close(out, want.half(), max_frac=2e-2, atol=float(want.abs().max()) * 2 ** -10,
+    # scores and probabilities are intermediate fp16 roundings.  A 1-ulp flip of a score of
+    # magnitude up to 16 (these inputs reach |s| ~ 15) scales its probability by e^(2^-7), so a
+    # few outputs may move by 2^-7 of the largest output; everything else is within 1 ulp.
+    assert_fp16_close(out, want.half(), max_frac=2e-2, atol=float(want.abs().max()) * 2 ** -7,
                       what="attention")
 
 
