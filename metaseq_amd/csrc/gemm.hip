@@ -158,14 +158,12 @@ __global__ __launch_bounds__(256) void pack_i8_kernel(const int8_t* __restrict__
 constexpr int ST_KG = 8;  // waves per workgroup = interleaved K lanes
 constexpr int ST_NT = 4;  // weight tiles sharing one activation fragment
 
-template <int MB, bool W8, int MODE>
-__global__ __launch_bounds__(ST_KG * 64) void linear_stream_kernel(
+template <int MB, bool W8, int MODE, int KG = ST_KG, int NT = ST_NT, int U = (MB <= 2 ? 4 : 2)>
+__global__ __launch_bounds__(KG * 64) void linear_stream_kernel(
     const half_t* __restrict__ xp, const void* __restrict__ Wp, const half_t* __restrict__ scales,
     float* __restrict__ part, int M, int N, int K, int tiles_per_wg, int ks_per_split,
     Epilogue epi) {
-  constexpr int KG = ST_KG, NT = ST_NT;
-  // K steps (32 wide) buffered per stage; an int8 block covers two steps
-  constexpr int U = MB <= 2 ? 4 : 2;
+  // U = K steps (32 wide) buffered per stage; an int8 block covers two steps
   constexpr int UA = W8 ? U / 2 : U;  // weight loads per stage and tile
   __shared__ float4_t red[KG][NT * MB][64];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -433,6 +431,7 @@ __global__ __launch_bounds__(TL_THREADS) void linear_tiled_kernel(
 }
 
 // ---- host side ------------------------------------------------------------------------------
+int g_tune = 0;  // kernel-shape experiments, see msa_internal_set_tune
 int g_num_cus = 0;
 int num_cus() {
   if (g_num_cus == 0) {
@@ -456,6 +455,28 @@ void launch_stream_mb(const void* xp, const void* W, const void* scales, float* 
   const int gx = (ntiles + tiles_per_wg - 1) / tiles_per_wg;
   int ks_per_split = (nks + S - 1) / S;
   if (W8) ks_per_split = (ks_per_split + 1) & ~1;  // int8 blocks cover two steps
+  if (g_tune != 0 && MB == 2 && !W8 && MODE == MODE_PLAIN) {
+    const int cfg = g_tune & 15, mult = (g_tune >> 4) ? (g_tune >> 4) : 1;
+    G = num_cus() * mult / S;
+    tiles_per_wg = (ntiles + G - 1) / G;
+    const int gx2 = (ntiles + tiles_per_wg - 1) / tiles_per_wg;
+#define MSA_TUNE(KG_, NT_, U_)                                                                  \
+  hipLaunchKernelGGL((linear_stream_kernel<2, false, MODE_PLAIN, KG_, NT_, U_>), dim3(gx2, S),  \
+                     dim3(KG_ * 64), 0, s, (const half_t*)xp, W, (const half_t*)scales, part, M, \
+                     N, K, tiles_per_wg, ks_per_split, epi)
+    switch (cfg) {
+      case 1: MSA_TUNE(4, 4, 4); break;
+      case 2: MSA_TUNE(8, 2, 8); break;
+      case 3: MSA_TUNE(16, 4, 2); break;
+      case 4: MSA_TUNE(8, 4, 2); break;
+      case 5: MSA_TUNE(4, 4, 8); break;
+      case 6: MSA_TUNE(8, 3, 4); break;
+      case 7: MSA_TUNE(4, 2, 8); break;
+      default: MSA_TUNE(8, 4, 4); break;
+    }
+#undef MSA_TUNE
+    return;
+  }
   hipLaunchKernelGGL((linear_stream_kernel<MB, W8, MODE>), dim3(gx, S), dim3(ST_KG * 64), 0, s,
                      (const half_t*)xp, W, (const half_t*)scales, part, M, N, K, tiles_per_wg,
                      ks_per_split, epi);
@@ -591,6 +612,9 @@ int pack_entry(const char* name, const void* src, void* dst, int N, int K, bool 
 }
 
 }  // namespace
+
+// Selects an experimental stream-kernel shape (tuning only; 0 = the shipped configuration).
+extern "C" void msa_internal_set_tune(int v) { g_tune = v; }
 
 extern "C" int msa_pack_weight_f16(const void* src, void* dst, int N, int K, void* stream) {
   return pack_entry("msa_pack_weight_f16", src, dst, N, K, false, false, stream);
