@@ -122,6 +122,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--config", default="6.7b", choices=sorted(CONFIGS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--graph", action="store_true",
+                    help="replay the captured decode-step hipGraph instead of launching every "
+                         "kernel from Python (measured slower on this ROCm: 5.81 vs 5.66 ms/step)")
     ap.add_argument("--pmc-calibration", action="store_true",
                     help="also run a plain 1 GiB device copy, the known-size kernel that "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE readings are scaled by")
@@ -186,7 +189,15 @@ def main():
     torch.cuda.synchronize()
     prefill_s = time.time() - t1
 
+    st = None
+    if args.graph and B <= 64:
+        st = gen.static_state(decoder, decoder.get_cache(inc), tokens, scores, finished,
+                              step_logits)
+
     def one_step(step, step_logits):
+        if st is not None:  # selection + forward + length advance as one graph replay
+            gen._graph_step(lib, st, step, max_len - 1, max_len)
+            return st["logits"]
         gen._select(lib, step_logits, step, max_len - 1, max_len, finished, tokens, scores)
         out = decoder(tokens[:, :step + 1], incremental_state=inc)[0]
         return out.view(B, -1)
@@ -225,7 +236,7 @@ def main():
         for i in range(cfg.decoder_layers):
             _capi.check(lib.msa_attention_f16(q.data_ptr(), cache.k(i).data_ptr(),
                                               cache.v(i).data_ptr(), None, 0, o.data_ptr(), B, H,
-                                              hd, 1, S_probe - 1, cache.capacity, 0, stream))
+                                              hd, 1, S_probe - 1, cache.capacity, 0, None, stream))
     attn_all_layers()
     torch.cuda.synchronize()
     a0, a1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -261,6 +272,7 @@ def main():
         "hbm_frac_step": bytes_mean / t_step / HBM_PEAK,
         "step_bytes_mean": bytes_mean,
         "gpu_ms_per_step": gpu_s / K * 1e3,
+        "graph_replay": st is not None,
         "prefill_s": prefill_s,
         "prefill_tflops": prefill_flops(cfg, B, n0) / prefill_s / 1e12,
         "prefill_mfma_frac": prefill_flops(cfg, B, n0) / prefill_s / MFMA_PEAK,

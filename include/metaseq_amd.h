@@ -60,6 +60,18 @@ int msa_unpack_weight_f16(const void* src, void* dst, int N, int K, void* stream
 int msa_pack_weight_i8(const int8_t* src, int8_t* dst, int N, int K, void* stream);
 int msa_unpack_weight_i8(const int8_t* src, int8_t* dst, int N, int K, void* stream);
 
+/* ---- device-resident sequence length (for hipGraph replay of a decode step) -------------------
+ * A captured graph must not bake the growing history length into launch arguments.  The four
+ * entry points that depend on it take an optional `len_dev` (int32 on the device, NULL = use the
+ * host arguments) holding the number of positions already in the KV cache:
+ *   msa_embed_f16 (T_out == 1): embeds column *len_dev of tokens (n = *len_dev + 1, capped by n);
+ *   msa_qkv_proj_* (T == 1):    appends at position *len_dev (skipped if that is >= S_cap);
+ *   msa_attention_f16 (T == 1): attends positions 0 .. *len_dev;
+ *   msa_greedy_select_f16:      writes tok[b*tok_stride + *len_dev], score likewise.
+ * msa_advance_len adds `delta` to *len_dev on the stream (a one-thread kernel).
+ * No reference counterpart (the reference re-launches every op from Python each step). */
+int msa_advance_len(int32_t* len_dev, int delta, void* stream);
+
 /* Pre-LN LayerNorm forward: y[r,:] = round(gamma * (x[r,:] - mean) * rsqrt(var + eps) + beta),
  * mean / biased variance in fp32.  D % 8 == 0, D <= 16384.  flags: MSA_OUT_PACKED.
  * Replaces metaseq/modules/layer_norm.py:28-33 -> apex cuApplyLayerNorm
@@ -92,7 +104,8 @@ int msa_residual_layernorm_f16(const float* part, int S, const void* bias, void*
  * (metaseq/modules/megatron/mpu/layers.py:220-250). */
 int msa_embed_f16(const int64_t* tokens, int64_t tok_stride, int B, int n, int T_out,
                   const void* E, int V, const void* P, int n_pos_rows, int pad_idx, int D,
-                  void* x, int64_t* positions_out, int32_t* status_dev, void* stream);
+                  void* x, int64_t* positions_out, int32_t* status_dev, const int32_t* len_dev,
+                  void* stream);
 
 /* y[M,N] = epilogue(x[M,K] . W[N,K]^T) with W tile-packed:
  *   t = round(acc); if bias: t = round(t + bias[n]); if RELU: t = max(t,0);
@@ -136,10 +149,11 @@ int msa_linear_default_splits(int64_t M, int N, int K);
  * (q scaling) and :449-479 (cache growth by torch.cat, here an in-place append). */
 int msa_qkv_proj_f16(const void* x, const void* Wqkv, const void* bqkv, void* q_out,
                      void* Kcache, void* Vcache, int B, int T, int H, int hd, int S0, int S_cap,
-                     int K, unsigned flags, void* stream);
+                     int K, unsigned flags, const int32_t* len_dev, void* stream);
 int msa_qkv_proj_w8a16(const void* x, const int8_t* Wq, const void* scales, const void* bqkv,
                        void* q_out, void* Kcache, void* Vcache, int B, int T, int H, int hd,
-                       int S0, int S_cap, int K, unsigned flags, void* stream);
+                       int S0, int S_cap, int K, unsigned flags, const int32_t* len_dev,
+                       void* stream);
 
 /* Causal attention of T new queries (already scaled, q[B*T, H*hd]) over the cache, whose
  * positions 0 .. S0+T-1 are valid: query t sees keys 0 .. S0+t.
@@ -152,7 +166,8 @@ int msa_qkv_proj_w8a16(const void* x, const int8_t* Wq, const void* scales, cons
  * padding masks), :533-534 (fp32 softmax, cast back), :543-552 (bmm p v, transpose). */
 int msa_attention_f16(const void* q, const void* Kcache, const void* Vcache,
                       const uint8_t* key_pad_mask, int64_t mask_stride, void* out, int B, int H,
-                      int hd, int T, int S0, int S_cap, unsigned flags, void* stream);
+                      int hd, int T, int S0, int S_cap, unsigned flags, const int32_t* len_dev,
+                      void* stream);
 
 /* One step of greedy selection over fp16 logits[B, V] (row stride ld_logits), with the
  * generator's bookkeeping fused in:
@@ -172,7 +187,7 @@ int msa_greedy_select_f16(const void* logits, int64_t ld_logits, int B, int V, f
                           const int32_t* banned_host, int n_banned, const int32_t* stop_host,
                           int n_stop, uint8_t* finished, int force_eos_all, int eos_idx,
                           int64_t* tok, int64_t tok_stride, float* score, int64_t score_stride,
-                          void* stream);
+                          const int32_t* len_dev, void* stream);
 
 /* Log-probabilities of given target ids under fp16 logits rows:
  *   out[r] = logits[r, target[r]]/temperature - logsumexp_fp32(logits[r,:]/temperature).

@@ -27,21 +27,22 @@ SIGNATURES = {
     "msa_layernorm_f16": [_P, _P, _P, _P, c_int64, c_int, c_float, c_uint, _P],
     "msa_residual_layernorm_f16": [_P, c_int, _P, _P, _P, _P, _P, c_int64, c_int, c_float, c_uint,
                                    _P],
+    "msa_advance_len": [_P, c_int, _P],
     "msa_embed_f16": [_P, c_int64, c_int, c_int, c_int, _P, c_int, _P, c_int, c_int, c_int, _P, _P,
-                      _P, _P],
+                      _P, _P, _P],
     "msa_linear_f16": [_P, _P, _P, _P, _P, c_int64, c_int, c_int, c_uint, _P],
     "msa_linear_w8a16": [_P, _P, _P, _P, _P, _P, c_int64, c_int, c_int, c_uint, _P],
     "msa_linear_partial_f16": [_P, _P, _P, c_int64, c_int, c_int, c_int, c_uint, _P],
     "msa_linear_partial_w8a16": [_P, _P, _P, _P, c_int64, c_int, c_int, c_int, c_uint, _P],
     "msa_linear_default_splits": [c_int64, c_int, c_int],
     "msa_qkv_proj_f16": [_P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
-                         c_uint, _P],
+                         c_uint, _P, _P],
     "msa_qkv_proj_w8a16": [_P, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int,
-                           c_int, c_uint, _P],
+                           c_int, c_uint, _P, _P],
     "msa_attention_f16": [_P, _P, _P, _P, c_int64, _P, c_int, c_int, c_int, c_int, c_int, c_int,
-                          c_uint, _P],
+                          c_uint, _P, _P],
     "msa_greedy_select_f16": [_P, c_int64, c_int, c_int, c_float, _P, c_int, _P, c_int, _P, c_int,
-                              c_int, _P, c_int64, _P, c_int64, _P],
+                              c_int, _P, c_int64, _P, c_int64, _P, _P],
     "msa_target_logprob_f16": [_P, c_int64, c_int64, c_int, c_float, _P, _P, _P],
 }
 OTHER_SYMBOLS = ["msa_last_error", "msa_version"]

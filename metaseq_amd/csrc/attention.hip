@@ -18,7 +18,7 @@ __global__ void attention_kernel(const half_t* __restrict__ q, const half_t* __r
                                  const half_t* __restrict__ Vc,
                                  const uint8_t* __restrict__ key_pad_mask, int64_t mask_stride,
                                  half_t* __restrict__ out, int H, int T, int S0, int S_cap,
-                                 int out_mb) {
+                                 int out_mb, const int32_t* __restrict__ len_dev) {
   constexpr int LPR = HD / 8;    // lanes per key row (16 bytes each)
   constexpr int RPW = 64 / LPR;  // key rows per wave instruction
   extern __shared__ float smem[];
@@ -30,6 +30,7 @@ __global__ void attention_kernel(const half_t* __restrict__ q, const half_t* __r
   const int b = bh / H, h = bh - b * H;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
   const int sub = lane % LPR, rsel = lane / LPR;
+  if (len_dev) S0 = min(*len_dev, S_cap - 1);  // cache length kept on the device (graph replay)
   const int n_keys = S0 + t + 1;
   const int D = H * HD;
 
@@ -154,7 +155,7 @@ __global__ void attention_kernel(const half_t* __restrict__ q, const half_t* __r
 extern "C" int msa_attention_f16(const void* q, const void* Kcache, const void* Vcache,
                                  const uint8_t* key_pad_mask, int64_t mask_stride, void* out, int B,
                                  int H, int hd, int T, int S0, int S_cap, unsigned flags,
-                                 void* stream) {
+                                 const int32_t* len_dev, void* stream) {
   MSA_REQUIRE(q && Kcache && Vcache && out, MSA_ERR_INVALID_ARG, "msa_attention_f16: null pointer");
   MSA_REQUIRE(B > 0 && H > 0 && T > 0 && S0 >= 0, MSA_ERR_INVALID_ARG,
               "msa_attention_f16: bad shape B=%d H=%d T=%d S0=%d", B, H, T, S0);
@@ -173,6 +174,10 @@ extern "C" int msa_attention_f16(const void* q, const void* Kcache, const void* 
   MSA_REQUIRE(!(flags & MSA_OUT_PACKED) || (T == 1 && B <= 64), MSA_ERR_INVALID_ARG,
               "msa_attention_f16: packed output needs T == 1 and B <= 64 (T=%d B=%d)", T, B);
   const int out_mb = (flags & MSA_OUT_PACKED) ? (B + 15) / 16 : 0;
+  MSA_REQUIRE(!len_dev || T == 1, MSA_ERR_INVALID_ARG,
+              "msa_attention_f16: a device-side length needs T == 1");
+  MSA_REQUIRE(!len_dev || S_cap <= 8192, MSA_ERR_CAPACITY,
+              "msa_attention_f16: S_cap %d exceeds the 8192 the score buffer holds", S_cap);
   const int64_t BH = (int64_t)B * H;
   if (T > 1) {
     MSA_REQUIRE(BH <= 0x7fffffff, MSA_ERR_INVALID_ARG, "msa_attention_f16: B*H too large");
@@ -183,17 +188,17 @@ extern "C" int msa_attention_f16(const void* q, const void* Kcache, const void* 
   }
   // few (b,h) pairs: spend more waves on each so the chip still fills
   const int threads = (T == 1 && BH < 512) ? 1024 : 256;
-  const size_t lds = (size_t)(S0 + T) * sizeof(float);
+  const size_t lds = (size_t)(len_dev ? S_cap : S0 + T) * sizeof(float);
   const dim3 grid((unsigned)BH, (unsigned)T);
   hipStream_t s = (hipStream_t)stream;
   if (hd == 64)
     hipLaunchKernelGGL(attention_kernel<64>, grid, dim3(threads), lds, s, (const half_t*)q,
                        (const half_t*)Kcache, (const half_t*)Vcache, key_pad_mask, mask_stride,
-                       (half_t*)out, H, T, S0, S_cap, out_mb);
+                       (half_t*)out, H, T, S0, S_cap, out_mb, len_dev);
   else
     hipLaunchKernelGGL(attention_kernel<128>, grid, dim3(threads), lds, s, (const half_t*)q,
                        (const half_t*)Kcache, (const half_t*)Vcache, key_pad_mask, mask_stride,
-                       (half_t*)out, H, T, S0, S_cap, out_mb);
+                       (half_t*)out, H, T, S0, S_cap, out_mb, len_dev);
   MSA_CHECK_LAUNCH("msa_attention_f16");
   return MSA_OK;
 }

@@ -43,10 +43,11 @@ __device__ __forceinline__ void clamp_ids(int64_t& tok, int& pos, int V, int n_p
 __global__ __launch_bounds__(EMB_THREADS) void embed_last_kernel(
     const int64_t* __restrict__ tokens, int64_t tok_stride, int n, const half_t* __restrict__ E,
     int V, const half_t* __restrict__ P, int n_pos_rows, int pad, int D, half_t* __restrict__ x,
-    int64_t* __restrict__ positions_out, int32_t* status) {
+    int64_t* __restrict__ positions_out, int32_t* status, const int32_t* __restrict__ len_dev) {
   __shared__ float red[16];
   const int b = blockIdx.x;
   const int64_t* row = tokens + b * tok_stride;
+  if (len_dev) n = min(*len_dev + 1, n);  // history length kept on the device (graph replay)
   int64_t tok = row[n - 1];
   int pos = pad;
   const int cnt = count_nonpad(row, n, pad, red);
@@ -96,7 +97,7 @@ __global__ __launch_bounds__(EMB_THREADS) void embed_rows_kernel(
 extern "C" int msa_embed_f16(const int64_t* tokens, int64_t tok_stride, int B, int n, int T_out,
                              const void* E, int V, const void* P, int n_pos_rows, int pad_idx,
                              int D, void* x, int64_t* positions_out, int32_t* status_dev,
-                             void* stream) {
+                             const int32_t* len_dev, void* stream) {
   MSA_REQUIRE(tokens && E && P && x, MSA_ERR_INVALID_ARG, "msa_embed_f16: null pointer");
   MSA_REQUIRE(B > 0 && n > 0 && T_out > 0 && T_out <= n && tok_stride >= n, MSA_ERR_INVALID_ARG,
               "msa_embed_f16: bad shape B=%d n=%d T_out=%d stride=%lld", B, n, T_out,
@@ -104,11 +105,13 @@ extern "C" int msa_embed_f16(const int64_t* tokens, int64_t tok_stride, int B, i
   MSA_REQUIRE(D > 0 && D % 8 == 0 && V > 0 && n_pos_rows > pad_idx && pad_idx >= 0,
               MSA_ERR_INVALID_ARG, "msa_embed_f16: bad sizes D=%d V=%d n_pos_rows=%d pad=%d", D, V,
               n_pos_rows, pad_idx);
+  MSA_REQUIRE(!len_dev || T_out == 1, MSA_ERR_INVALID_ARG,
+              "msa_embed_f16: a device-side length needs T_out == 1");
   hipStream_t s = (hipStream_t)stream;
   if (T_out == 1) {
     hipLaunchKernelGGL(embed_last_kernel, dim3(B), dim3(EMB_THREADS), 0, s, tokens, tok_stride, n,
                        (const half_t*)E, V, (const half_t*)P, n_pos_rows, pad_idx, D, (half_t*)x,
-                       positions_out, status_dev);
+                       positions_out, status_dev, len_dev);
   } else {
     MSA_REQUIRE(positions_out, MSA_ERR_INVALID_ARG,
                 "msa_embed_f16: positions_out is required when T_out > 1");
@@ -119,5 +122,16 @@ extern "C" int msa_embed_f16(const int64_t* tokens, int64_t tok_stride, int B, i
                        n_pos_rows, D, (half_t*)x, positions_out, status_dev);
   }
   MSA_CHECK_LAUNCH("msa_embed_f16");
+  return MSA_OK;
+}
+
+namespace {
+__global__ void advance_len_kernel(int32_t* len_dev, int delta) { *len_dev += delta; }
+}  // namespace
+
+extern "C" int msa_advance_len(int32_t* len_dev, int delta, void* stream) {
+  MSA_REQUIRE(len_dev, MSA_ERR_INVALID_ARG, "msa_advance_len: null pointer");
+  hipLaunchKernelGGL(advance_len_kernel, dim3(1), dim3(1), 0, (hipStream_t)stream, len_dev, delta);
+  MSA_CHECK_LAUNCH("msa_advance_len");
   return MSA_OK;
 }

@@ -37,6 +37,7 @@ struct Epilogue {
   half_t* Kc;
   half_t* Vc;
   int T, H, hd, S0, S_cap;
+  const int32_t* len_dev;  // if set (T == 1): the append position is read from the device
   float qscale;
 };
 
@@ -81,9 +82,12 @@ __device__ __forceinline__ void epilogue4(const Epilogue& e, int64_t m, int n, f
       for (int i = 0; i < 4; ++i) o[i] = (half_t)t[i];
       const int h = c / e.hd, d = c - h * e.hd;
       const int64_t b = m / e.T, tt = m - b * e.T;
-      half_t* dst = (part == 0 ? e.Kc : e.Vc) +
-                    ((b * e.H + h) * (int64_t)e.S_cap + e.S0 + tt) * e.hd + d;
-      *reinterpret_cast<half4_t*>(dst) = o;
+      const int s0 = e.len_dev ? *e.len_dev : e.S0;
+      if (s0 + tt < e.S_cap) {
+        half_t* dst = (part == 0 ? e.Kc : e.Vc) +
+                      ((b * e.H + h) * (int64_t)e.S_cap + s0 + tt) * e.hd + d;
+        *reinterpret_cast<half4_t*>(dst) = o;
+      }
     }
   }
 }
@@ -431,7 +435,6 @@ __global__ __launch_bounds__(TL_THREADS) void linear_tiled_kernel(
 }
 
 // ---- host side ------------------------------------------------------------------------------
-int g_tune = 0;  // kernel-shape experiments, see msa_internal_set_tune
 int g_num_cus = 0;
 int num_cus() {
   if (g_num_cus == 0) {
@@ -451,32 +454,10 @@ void launch_stream_mb(const void* xp, const void* W, const void* scales, float* 
   const int ntiles = N / 16, nks = K / 32;
   int G = num_cus() / S;
   if (G < 1) G = 1;
-  int tiles_per_wg = (ntiles + G - 1) / G;
+  const int tiles_per_wg = (ntiles + G - 1) / G;
   const int gx = (ntiles + tiles_per_wg - 1) / tiles_per_wg;
   int ks_per_split = (nks + S - 1) / S;
   if (W8) ks_per_split = (ks_per_split + 1) & ~1;  // int8 blocks cover two steps
-  if (g_tune != 0 && MB == 2 && !W8 && MODE == MODE_PLAIN) {
-    const int cfg = g_tune & 15, mult = (g_tune >> 4) ? (g_tune >> 4) : 1;
-    G = num_cus() * mult / S;
-    tiles_per_wg = (ntiles + G - 1) / G;
-    const int gx2 = (ntiles + tiles_per_wg - 1) / tiles_per_wg;
-#define MSA_TUNE(KG_, NT_, U_)                                                                  \
-  hipLaunchKernelGGL((linear_stream_kernel<2, false, MODE_PLAIN, KG_, NT_, U_>), dim3(gx2, S),  \
-                     dim3(KG_ * 64), 0, s, (const half_t*)xp, W, (const half_t*)scales, part, M, \
-                     N, K, tiles_per_wg, ks_per_split, epi)
-    switch (cfg) {
-      case 1: MSA_TUNE(4, 4, 4); break;
-      case 2: MSA_TUNE(8, 2, 8); break;
-      case 3: MSA_TUNE(16, 4, 2); break;
-      case 4: MSA_TUNE(8, 4, 2); break;
-      case 5: MSA_TUNE(4, 4, 8); break;
-      case 6: MSA_TUNE(8, 3, 4); break;
-      case 7: MSA_TUNE(4, 2, 8); break;
-      default: MSA_TUNE(8, 4, 4); break;
-    }
-#undef MSA_TUNE
-    return;
-  }
   hipLaunchKernelGGL((linear_stream_kernel<MB, W8, MODE>), dim3(gx, S), dim3(ST_KG * 64), 0, s,
                      (const half_t*)xp, W, (const half_t*)scales, part, M, N, K, tiles_per_wg,
                      ks_per_split, epi);
@@ -563,7 +544,9 @@ int partial_entry(const char* name, const void* x, const void* W, const void* sc
 template <bool W8>
 int qkv_entry(const char* name, const void* x, const void* W, const void* scales, const void* bqkv,
               void* q_out, void* Kc, void* Vc, int B, int T, int H, int hd, int S0, int S_cap,
-              int K, unsigned flags, void* stream) {
+              int K, unsigned flags, const int32_t* len_dev, void* stream) {
+  MSA_REQUIRE(!len_dev || T == 1, MSA_ERR_INVALID_ARG, "%s: a device-side length needs T == 1",
+              name);
   MSA_REQUIRE(q_out && Kc && Vc, MSA_ERR_INVALID_ARG, "%s: null pointer", name);
   MSA_REQUIRE(B > 0 && T > 0 && H > 0 && hd > 0 && hd % 8 == 0 && S0 >= 0, MSA_ERR_INVALID_ARG,
               "%s: bad shape B=%d T=%d H=%d hd=%d S0=%d", name, B, T, H, hd, S0);
@@ -584,6 +567,7 @@ int qkv_entry(const char* name, const void* x, const void* W, const void* scales
   e.H = H;
   e.hd = hd;
   e.S0 = S0;
+  e.len_dev = len_dev;
   e.S_cap = S_cap;
   e.qscale = (float)pow((double)hd, -0.5);  // the reference's head_dim ** -0.5, cast to fp32
   if (flags & MSA_IN_PACKED)
@@ -612,9 +596,6 @@ int pack_entry(const char* name, const void* src, void* dst, int N, int K, bool 
 }
 
 }  // namespace
-
-// Selects an experimental stream-kernel shape (tuning only; 0 = the shipped configuration).
-extern "C" void msa_internal_set_tune(int v) { g_tune = v; }
 
 extern "C" int msa_pack_weight_f16(const void* src, void* dst, int N, int K, void* stream) {
   return pack_entry("msa_pack_weight_f16", src, dst, N, K, false, false, stream);
@@ -667,15 +648,16 @@ extern "C" int msa_linear_partial_w8a16(const void* x, const int8_t* Wq, const v
 
 extern "C" int msa_qkv_proj_f16(const void* x, const void* Wqkv, const void* bqkv, void* q_out,
                                 void* Kcache, void* Vcache, int B, int T, int H, int hd, int S0,
-                                int S_cap, int K, unsigned flags, void* stream) {
+                                int S_cap, int K, unsigned flags, const int32_t* len_dev,
+                                void* stream) {
   return qkv_entry<false>("msa_qkv_proj_f16", x, Wqkv, nullptr, bqkv, q_out, Kcache, Vcache, B, T,
-                          H, hd, S0, S_cap, K, flags, stream);
+                          H, hd, S0, S_cap, K, flags, len_dev, stream);
 }
 
 extern "C" int msa_qkv_proj_w8a16(const void* x, const int8_t* Wq, const void* scales,
                                   const void* bqkv, void* q_out, void* Kcache, void* Vcache, int B,
                                   int T, int H, int hd, int S0, int S_cap, int K, unsigned flags,
-                                  void* stream) {
+                                  const int32_t* len_dev, void* stream) {
   return qkv_entry<true>("msa_qkv_proj_w8a16", x, Wq, scales, bqkv, q_out, Kcache, Vcache, B, T, H,
-                         hd, S0, S_cap, K, flags, stream);
+                         hd, S0, S_cap, K, flags, len_dev, stream);
 }

@@ -18,8 +18,19 @@ __global__ __launch_bounds__(LN_THREADS) void layernorm_f16_kernel(
   const int row = blockIdx.x;
   const int nchunk = D >> 3;  // 16-byte chunks in the row
 
-  half8_t v[LN_MAX_CHUNKS];
+  half8_t v[LN_MAX_CHUNKS], gv[LN_MAX_CHUNKS], bv[LN_MAX_CHUNKS];
   float s = 0.f;
+  // gamma / beta are requested first so that their latency hides behind the reductions
+  if (gamma) {
+#pragma unroll
+    for (int c = 0; c < LN_MAX_CHUNKS; ++c) {
+      const int idx = threadIdx.x + c * LN_THREADS;
+      if (idx < nchunk) {
+        gv[c] = *reinterpret_cast<const half8_t*>(gamma + (idx << 3));
+        bv[c] = *reinterpret_cast<const half8_t*>(beta + (idx << 3));
+      }
+    }
+  }
 #pragma unroll
   for (int c = 0; c < LN_MAX_CHUNKS; ++c) {
     const int idx = threadIdx.x + c * LN_THREADS;
@@ -72,12 +83,10 @@ __global__ __launch_bounds__(LN_THREADS) void layernorm_f16_kernel(
   for (int c = 0; c < LN_MAX_CHUNKS; ++c) {
     const int idx = threadIdx.x + c * LN_THREADS;
     if (idx < nchunk) {
-      const half8_t g = *reinterpret_cast<const half8_t*>(gamma + (idx << 3));
-      const half8_t b = *reinterpret_cast<const half8_t*>(beta + (idx << 3));
       half8_t o;
 #pragma unroll
       for (int i = 0; i < 8; ++i)
-        o[i] = (half_t)(((float)v[c][i] - mean) * rstd * (float)g[i] + (float)b[i]);
+        o[i] = (half_t)(((float)v[c][i] - mean) * rstd * (float)gv[c][i] + (float)bv[c][i]);
       half_t* dst = out_mb > 0 ? y + packed_act_offset(row, idx << 3, out_mb)
                                : y + (int64_t)row * D + (idx << 3);
       *reinterpret_cast<half8_t*>(dst) = o;

@@ -82,7 +82,7 @@ __global__ __launch_bounds__(SM_THREADS) void greedy_select_kernel(
     const half_t* __restrict__ logits, int64_t ld, int V, float temperature, bool scale,
     IdList banned, IdList stop, uint8_t* __restrict__ finished, int force_eos_all, int eos,
     int64_t* __restrict__ tok, int64_t tok_stride, float* __restrict__ score,
-    int64_t score_stride) {
+    int64_t score_stride, const int32_t* __restrict__ len_dev) {
   __shared__ float wm[16], ws[16], wbest[16], wnan[16];
   __shared__ int widx[16];
   const int b = blockIdx.x;
@@ -175,8 +175,9 @@ __global__ __launch_bounds__(SM_THREADS) void greedy_select_kernel(
       lp = -INFINITY;
       bidx = 0;
     }
-    tok[b * tok_stride] = bidx;
-    score[b * score_stride] = lp;
+    const int col = len_dev ? *len_dev : 0;  // column offset kept on the device (graph replay)
+    tok[b * tok_stride + col] = bidx;
+    score[b * score_stride + col] = lp;
     if (finished) {
       bool f = bidx == eos;
       for (int j = 0; j < stop.n; ++j) f |= (stop.id[j] == bidx);
@@ -208,7 +209,7 @@ extern "C" int msa_greedy_select_f16(const void* logits, int64_t ld_logits, int 
                                      const int32_t* stop_host, int n_stop, uint8_t* finished,
                                      int force_eos_all, int eos_idx, int64_t* tok,
                                      int64_t tok_stride, float* score, int64_t score_stride,
-                                     void* stream) {
+                                     const int32_t* len_dev, void* stream) {
   MSA_REQUIRE(logits && tok && score, MSA_ERR_INVALID_ARG, "msa_greedy_select_f16: null pointer");
   MSA_REQUIRE(B > 0 && V > 0 && ld_logits >= V, MSA_ERR_INVALID_ARG,
               "msa_greedy_select_f16: bad shape B=%d V=%d ld=%lld", B, V, (long long)ld_logits);
@@ -227,7 +228,8 @@ extern "C" int msa_greedy_select_f16(const void* logits, int64_t ld_logits, int 
   for (int i = 0; i < n_stop; ++i) stop.id[i] = stop_host[i];
   hipLaunchKernelGGL(greedy_select_kernel, dim3(B), dim3(SM_THREADS), 0, (hipStream_t)stream,
                      (const half_t*)logits, ld_logits, V, temperature, scale, banned, stop,
-                     finished, force_eos_all, eos_idx, tok, tok_stride, score, score_stride);
+                     finished, force_eos_all, eos_idx, tok, tok_stride, score, score_stride,
+                     len_dev);
   MSA_CHECK_LAUNCH("msa_greedy_select_f16");
   return MSA_OK;
 }

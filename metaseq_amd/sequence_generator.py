@@ -27,8 +27,11 @@ class SequenceGenerator(nn.Module):
                  topp: float = -1, profile=False, omega_bound: float = 0.3,
                  lambda_decay: float = -1, alpha_presence: float = 0.0,
                  alpha_frequency: float = 0.0, alpha_presence_src: float = 0.0,
-                 alpha_frequency_src: float = 0.0, alpha_src_penalty_end_idx: int = -1):
+                 alpha_frequency_src: float = 0.0, alpha_src_penalty_end_idx: int = -1,
+                 use_graph: bool = False):
         super().__init__()
+        # replay each decode step (selection + forward) as one captured hipGraph where possible
+        self.use_graph = use_graph
         self.model = models[0] if isinstance(models, (list, tuple)) else models
         self.tgt_dict = tgt_dict
         self.pad = tgt_dict.pad()
@@ -70,21 +73,60 @@ class SequenceGenerator(nn.Module):
         return self._generate(sample, **kwargs)
 
     # ------------------------------------------------------------------
-    def _select(self, lib, logits2d, step, min_len, max_len, finished, tokens, scores):
+    def _select(self, lib, logits2d, step, min_len, max_len, finished, tokens, scores,
+                len_dev=None):
         """Fused log-softmax + masks + arg-max + bookkeeping for one step
-        (metaseq/sequence_generator.py:272-308)."""
+        (metaseq/sequence_generator.py:272-308).  With ``len_dev`` the output column is read
+        from the device (``step`` then only selects the masks)."""
         banned = [self.pad]
         if step < min_len:
             banned += [self.eos] + self.stop
         B, V = logits2d.shape
         arr = (ctypes.c_int32 * len(banned))(*banned)
         stop = (ctypes.c_int32 * max(1, len(self.stop)))(*self.stop)
-        tok = tokens[:, step]
-        sc = scores[:, step]
+        col = 0 if len_dev is not None else step
+        tok = tokens[:, col]
+        sc = scores[:, col]
         check(lib.msa_greedy_select_f16(
             ptr(logits2d), logits2d.stride(0), B, V, float(self.temperature), arr, len(banned),
             stop, len(self.stop), ptr(finished), int(step >= max_len - 1), self.eos,
-            ptr(tok), tokens.stride(0), ptr(sc), scores.stride(0), _capi.stream_ptr()))
+            ptr(tok), tokens.stride(0), ptr(sc), scores.stride(0), ptr(len_dev),
+            _capi.stream_ptr()))
+
+    @staticmethod
+    def static_state(decoder, cache, tokens, scores, finished, step_logits):
+        """State of graph-replayed decoding: fixed-address buffers plus the device-side length
+        (= positions already in ``cache``; the next token goes to that column of ``tokens``)."""
+        return {"graphs": {}, "decoder": decoder, "cache": cache, "tokens": tokens,
+                "scores": scores, "finished": finished,
+                "logits": step_logits.contiguous().clone(),
+                "len_dev": torch.tensor([cache.length], dtype=torch.int32,
+                                        device=tokens.device)}
+
+    def _graph_body(self, lib, st, step, min_len, max_len):
+        """One decode step with nothing step-dependent in its launch arguments: select the token
+        for column *len_dev from the static logits, run the forward over the history including
+        it, advance the device-side length."""
+        self._select(lib, st["logits"], step, min_len, max_len, st["finished"], st["tokens"],
+                     st["scores"], st["len_dev"])
+        st["decoder"].decode_step_static(st["tokens"], st["cache"], st["len_dev"], st["logits"])
+        check(lib.msa_advance_len(ptr(st["len_dev"]), 1, _capi.stream_ptr()))
+
+    def _graph_step(self, lib, st, step, min_len, max_len):
+        """Runs the step through a captured graph; the first step of each masking regime
+        (before / after min_len) runs eagerly as the warm-up and is then captured."""
+        key = step < min_len
+        g = st["graphs"].get(key)
+        if g is None:
+            self._graph_body(lib, st, step, min_len, max_len)  # eager: a real step
+            torch.cuda.current_stream().synchronize()
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g):
+                self._graph_body(lib, st, step, min_len, max_len)  # recorded, not executed
+            st["graphs"][key] = g
+        else:
+            g.replay()
+        st["cache"].length += 1
 
     def _generate(self, sample: Dict[str, Dict[str, torch.Tensor]], prefix_tokens=None,
                   bos_token=None):
@@ -153,7 +195,18 @@ class SequenceGenerator(nn.Module):
             del logits, flat
 
             finished = torch.zeros(BB, dtype=torch.uint8, device=dev)
+            cache = decoder.get_cache(incremental_states) if hasattr(decoder, "get_cache") else None
+            st = None
+            if (self.use_graph and all_lprobs is None and cache is not None and BB <= 64
+                    and not cache.has_pads):
+                st = self.static_state(decoder, cache, tokens, scores, finished, step_logits)
             for step in range(start_step, max_len):
+                if st is not None and step < max_len - 1:
+                    self._graph_step(lib, st, step, min_len, max_len)
+                    if step >= min_len and bool(finished.all()):
+                        break
+                    step_logits = st["logits"]
+                    continue
                 if all_lprobs is not None:
                     all_lprobs[:, step] = self._masked_lprobs(step_logits, step, min_len, max_len,
                                                               finished)

@@ -243,14 +243,113 @@ class TransformerDecoder(nn.Module):
             check(lib.msa_linear_partial_f16(ptr(x), ptr(lin.weight), ptr(part), M, N, K, S,
                                              MSA_IN_PACKED, stream))
 
-    def _qkv(self, lib, stream, h, qkv, q, kc, vc, B, T, H, hd, S0, cap, D, flags):
+    def _qkv(self, lib, stream, h, qkv, q, kc, vc, B, T, H, hd, S0, cap, D, flags, len_dev=None):
         if qkv.qweight is not None:
             check(lib.msa_qkv_proj_w8a16(ptr(h), ptr(qkv.qweight), ptr(qkv.scales), ptr(qkv.bias),
                                          ptr(q), ptr(kc), ptr(vc), B, T, H, hd, S0, cap, D, flags,
-                                         stream))
+                                         ptr(len_dev), stream))
         else:
             check(lib.msa_qkv_proj_f16(ptr(h), ptr(qkv.weight), ptr(qkv.bias), ptr(q), ptr(kc),
-                                       ptr(vc), B, T, H, hd, S0, cap, D, flags, stream))
+                                       ptr(vc), B, T, H, hd, S0, cap, D, flags, ptr(len_dev),
+                                       stream))
+
+    def _step_buffers(self, cache, B):
+        """Work buffers of a decode step (<= 64 rows), allocated once per KV cache so that their
+        addresses stay fixed (a captured graph replays against them)."""
+        bufs = getattr(cache, "step_bufs", None)
+        if bufs is None:
+            cfg, dev = self.cfg, cache.device
+            D, F = cfg.decoder_embed_dim, cfg.decoder_ffn_embed_dim
+            MP = ((B + 15) // 16) * 16
+            lib = self._lib
+            S_o = lib.msa_linear_default_splits(B, D, D)
+            S_f = lib.msa_linear_default_splits(B, D, F)
+            f16 = dict(dtype=torch.float16, device=dev)
+            bufs = {
+                "x": torch.empty(B, D, **f16), "q": torch.empty(B, D, **f16),
+                "h": torch.empty(MP * D, **f16), "o": torch.empty(MP * D, **f16),
+                "u": torch.empty(MP * F, **f16), "feat": torch.empty(B, D, **f16),
+                "part": torch.empty(max(S_o, S_f) * B * D, dtype=torch.float32, device=dev),
+                "positions": torch.empty(B, 1, dtype=torch.long, device=dev),
+                "S_o": S_o, "S_f": S_f,
+            }
+            cache.step_bufs = bufs
+        return bufs
+
+    def _decode_core(self, lib, stream, tokens, n, B, cache, mask, bufs, len_dev, S0,
+                     want_packed):
+        """One decode step for at most 64 rows: packed activations, weight-streaming kernels,
+        split-K tails fused into the LayerNorm that follows.  With ``len_dev`` (int32 device
+        tensor holding the cache length) nothing in the launch arguments depends on the step,
+        so the sequence can be captured once and replayed."""
+        cfg = self.cfg
+        D, H, hd = cfg.decoder_embed_dim, cfg.decoder_attention_heads, cfg.head_dim
+        F, L, M = cfg.decoder_ffn_embed_dim, cfg.decoder_layers, B
+        x, q, h, o, u, part = (bufs[k] for k in ("x", "q", "h", "o", "u", "part"))
+        S_o, S_f = bufs["S_o"], bufs["S_f"]
+        IN, OUT = MSA_IN_PACKED, MSA_OUT_PACKED
+        mask_stride = mask.stride(0) if mask is not None else 0
+        ld = ptr(len_dev)
+        check(lib.msa_embed_f16(ptr(tokens), tokens.stride(0), B, n, 1,
+                                ptr(self.embed_tokens.weight), cfg.vocab_size,
+                                ptr(self.embed_positions.weight),
+                                self.embed_positions.weight.shape[0], self.padding_idx, D,
+                                ptr(x), ptr(bufs["positions"]), None, ld, stream))
+        self._layernorm(lib, stream, x, self.layers[0].self_attn_layer_norm, M, D, h, OUT)
+        x_last = None
+        feat = h
+        for i, layer in enumerate(self.layers):
+            kc, vc = cache.k(i), cache.v(i)
+            self._qkv(lib, stream, h, layer.self_attn.qkv_proj, q, kc, vc, B, 1, H, hd, S0,
+                      cache.capacity, D, IN, len_dev)
+            check(lib.msa_attention_f16(ptr(q), ptr(kc), ptr(vc), ptr(mask), mask_stride, ptr(o),
+                                        B, H, hd, 1, S0, cache.capacity, OUT, ld, stream))
+            op = layer.self_attn.out_proj
+            self._linear_partial(lib, stream, o, op, part, M, D, D, S_o)
+            ln = layer.final_layer_norm
+            check(lib.msa_residual_layernorm_f16(ptr(part), S_o, ptr(op.bias), ptr(x),
+                                                 ptr(ln.weight), ptr(ln.bias), ptr(h), M, D, 1e-5,
+                                                 OUT, stream))
+            self._linear(lib, stream, h, layer.fc1, M, F, D, relu=True, out=u, flags=IN | OUT)
+            self._linear_partial(lib, stream, u, layer.fc2, part, M, D, F, S_f)
+            last = i + 1 == L
+            ln = self.layer_norm if last else self.layers[i + 1].self_attn_layer_norm
+            b2 = layer.fc2.bias
+            if last and self.return_inner_states:
+                check(lib.msa_residual_layernorm_f16(ptr(part), S_f, ptr(b2), ptr(x), None, None,
+                                                     None, M, D, 1e-5, 0, stream))
+                x_last = x.view(B, 1, D).transpose(0, 1).clone()
+                feat = h if want_packed else torch.empty(M, D, dtype=torch.float16,
+                                                         device=x.device)
+                self._layernorm(lib, stream, x, ln, M, D, feat, OUT if want_packed else 0)
+            elif last and not want_packed:
+                feat = torch.empty(M, D, dtype=torch.float16, device=x.device)
+                check(lib.msa_residual_layernorm_f16(ptr(part), S_f, ptr(b2), ptr(x),
+                                                     ptr(ln.weight), ptr(ln.bias), ptr(feat), M,
+                                                     D, 1e-5, 0, stream))
+            else:
+                check(lib.msa_residual_layernorm_f16(ptr(part), S_f, ptr(b2), ptr(x),
+                                                     ptr(ln.weight), ptr(ln.bias), ptr(h), M, D,
+                                                     1e-5, OUT, stream))
+        return feat, x_last
+
+    def decode_step_static(self, tokens, cache, len_dev, logits_out):
+        """Graph-capturable decode step: embeds column ``*len_dev`` of the full ``tokens``
+        buffer, appends to ``cache`` at that position, attends ``*len_dev + 1`` positions and
+        writes ``logits_out[B, V]``.  No allocation, no sync, no step-dependent launch argument.
+        The caller advances ``len_dev`` (msa_advance_len) and ``cache.length``."""
+        lib = self.prepare_()
+        stream = _capi.stream_ptr()
+        B = tokens.shape[0]
+        if B > 64 or cache.has_pads:
+            raise ValueError("static decode steps need at most 64 rows and no padding")
+        bufs = self._step_buffers(cache, B)
+        feat, _ = self._decode_core(lib, stream, tokens, tokens.shape[1], B, cache, None, bufs,
+                                    len_dev, 0, True)
+        D, V = self.cfg.decoder_embed_dim, self.cfg.vocab_size
+        check(lib.msa_linear_f16(ptr(feat), ptr(self._lm_head), None, None, ptr(logits_out), B, V,
+                                 D, MSA_IN_PACKED, stream))
+        return logits_out
 
     def _layernorm(self, lib, stream, x, ln, rows, D, out, flags=0):
         check(lib.msa_layernorm_f16(ptr(x), ptr(ln.weight), ptr(ln.bias), ptr(out), rows, D, 1e-5,
@@ -323,96 +422,54 @@ class TransformerDecoder(nn.Module):
             cache.grow(min(max(self.max_positions(), S0 + 1), int(cache.capacity * 1.5) + 64))
 
         M = B * T
+        if T == 1 and M <= 64:
+            bufs = self._step_buffers(cache, B)
+            feat, x_last = self._decode_core(lib, stream, tokens, n, B, cache, mask, bufs, None,
+                                             S0, want_packed)
+            inner_states = [{"tok": None, "pos": bufs["positions"], "emb": None}, x_last]
+            packed = want_packed
+            features = feat if packed else feat.view(B, T, D)
+            cache.length = S0 + T
+            if incremental_state is not None:
+                incremental_state[self._state_key] = cache
+            return features, packed, (B, T), {"inner_states": inner_states}
         x = torch.empty(M, D, dtype=torch.float16, device=dev)
         positions = torch.empty(B, T, dtype=torch.long, device=dev)
         check(lib.msa_embed_f16(ptr(tokens), tokens.stride(0), B, n, T,
                                 ptr(self.embed_tokens.weight), cfg.vocab_size,
                                 ptr(self.embed_positions.weight),
                                 self.embed_positions.weight.shape[0], self.padding_idx, D,
-                                ptr(x), ptr(positions), None, stream))
+                                ptr(x), ptr(positions), None, None, stream))
         inner_states = [{"tok": None, "pos": positions, "emb": None}]
         if self.return_inner_states:
             inner_states[0]["emb"] = x.view(B, T, D).transpose(0, 1).clone()
         mask_stride = mask.stride(0) if mask is not None else 0
         q = torch.empty(M, D, dtype=torch.float16, device=dev)
-
-        if T == 1 and M <= 64:
-            # ---- decode step: packed activations, weight-streaming kernels, split-K tails
-            # fused into the LayerNorm that follows ----
-            MP = ((M + 15) // 16) * 16
-            h = torch.empty(MP * D, dtype=torch.float16, device=dev)
-            o = torch.empty(MP * D, dtype=torch.float16, device=dev)
-            u = torch.empty(MP * F, dtype=torch.float16, device=dev)
-            S_o = lib.msa_linear_default_splits(M, D, D)
-            S_f = lib.msa_linear_default_splits(M, D, F)
-            part = torch.empty(max(S_o, S_f) * M * D, dtype=torch.float32, device=dev)
-            IN, OUT = MSA_IN_PACKED, MSA_OUT_PACKED
-            self._layernorm(lib, stream, x, self.layers[0].self_attn_layer_norm, M, D, h, OUT)
-            for i, layer in enumerate(self.layers):
-                kc, vc = cache.k(i), cache.v(i)
-                self._qkv(lib, stream, h, layer.self_attn.qkv_proj, q, kc, vc, B, 1, H, hd, S0,
-                          cache.capacity, D, IN)
-                check(lib.msa_attention_f16(ptr(q), ptr(kc), ptr(vc), ptr(mask), mask_stride,
-                                            ptr(o), B, H, hd, 1, S0, cache.capacity, OUT, stream))
-                op = layer.self_attn.out_proj
-                self._linear_partial(lib, stream, o, op, part, M, D, D, S_o)
-                ln = layer.final_layer_norm
-                check(lib.msa_residual_layernorm_f16(ptr(part), S_o, ptr(op.bias), ptr(x),
-                                                     ptr(ln.weight), ptr(ln.bias), ptr(h), M, D,
-                                                     1e-5, OUT, stream))
-                self._linear(lib, stream, h, layer.fc1, M, F, D, relu=True, out=u,
-                             flags=IN | OUT)
-                self._linear_partial(lib, stream, u, layer.fc2, part, M, D, F, S_f)
-                last = i + 1 == L
-                ln = self.layer_norm if last else self.layers[i + 1].self_attn_layer_norm
-                if last and self.return_inner_states:
-                    check(lib.msa_residual_layernorm_f16(ptr(part), S_f, ptr(layer.fc2.bias),
-                                                         ptr(x), None, None, None, M, D, 1e-5, 0,
-                                                         stream))
-                    inner_states.append(x.view(B, T, D).transpose(0, 1).clone())
-                    out_flags = OUT if want_packed else 0
-                    feat = h if want_packed else torch.empty(M, D, dtype=torch.float16,
-                                                             device=dev)
-                    self._layernorm(lib, stream, x, ln, M, D, feat, out_flags)
-                elif last and not want_packed:
-                    feat = torch.empty(M, D, dtype=torch.float16, device=dev)
-                    check(lib.msa_residual_layernorm_f16(ptr(part), S_f, ptr(layer.fc2.bias),
-                                                         ptr(x), ptr(ln.weight), ptr(ln.bias),
-                                                         ptr(feat), M, D, 1e-5, 0, stream))
-                else:
-                    feat = h
-                    check(lib.msa_residual_layernorm_f16(ptr(part), S_f, ptr(layer.fc2.bias),
-                                                         ptr(x), ptr(ln.weight), ptr(ln.bias),
-                                                         ptr(h), M, D, 1e-5, OUT, stream))
-            if not self.return_inner_states:
-                inner_states.append(None)
-            packed = want_packed
-            features = feat if packed else feat.view(B, T, D)
+        # ---- prefill (or a decode batch above 64 rows): row-major activations, tiled MFMA
+        # kernels ----
+        h = torch.empty_like(x)
+        o = torch.empty_like(x)
+        u = torch.empty(M, F, dtype=torch.float16, device=dev)
+        for i, layer in enumerate(self.layers):
+            self._layernorm(lib, stream, x, layer.self_attn_layer_norm, M, D, h)
+            kc, vc = cache.k(i), cache.v(i)
+            self._qkv(lib, stream, h, layer.self_attn.qkv_proj, q, kc, vc, B, T, H, hd, S0,
+                      cache.capacity, D, 0)
+            check(lib.msa_attention_f16(ptr(q), ptr(kc), ptr(vc), ptr(mask), mask_stride,
+                                        ptr(o), B, H, hd, T, S0, cache.capacity, 0, None,
+                                        stream))
+            # x = round(round(o Wo^T + bo) + x)   (transformer_decoder_layer.py:222-230)
+            self._linear(lib, stream, o, layer.self_attn.out_proj, M, D, D, residual=x, out=x)
+            self._layernorm(lib, stream, x, layer.final_layer_norm, M, D, h)
+            self._linear(lib, stream, h, layer.fc1, M, F, D, relu=True, out=u)
+            self._linear(lib, stream, u, layer.fc2, M, D, F, residual=x, out=x)
+        if self.return_inner_states:
+            inner_states.append(x.view(B, T, D).transpose(0, 1).clone())
         else:
-            # ---- prefill (or a decode batch above 64 rows): row-major activations, tiled MFMA
-            # kernels ----
-            h = torch.empty_like(x)
-            o = torch.empty_like(x)
-            u = torch.empty(M, F, dtype=torch.float16, device=dev)
-            for i, layer in enumerate(self.layers):
-                self._layernorm(lib, stream, x, layer.self_attn_layer_norm, M, D, h)
-                kc, vc = cache.k(i), cache.v(i)
-                self._qkv(lib, stream, h, layer.self_attn.qkv_proj, q, kc, vc, B, T, H, hd, S0,
-                          cache.capacity, D, 0)
-                check(lib.msa_attention_f16(ptr(q), ptr(kc), ptr(vc), ptr(mask), mask_stride,
-                                            ptr(o), B, H, hd, T, S0, cache.capacity, 0, stream))
-                # x = round(round(o Wo^T + bo) + x)   (transformer_decoder_layer.py:222-230)
-                self._linear(lib, stream, o, layer.self_attn.out_proj, M, D, D, residual=x, out=x)
-                self._layernorm(lib, stream, x, layer.final_layer_norm, M, D, h)
-                self._linear(lib, stream, h, layer.fc1, M, F, D, relu=True, out=u)
-                self._linear(lib, stream, u, layer.fc2, M, D, F, residual=x, out=x)
-            if self.return_inner_states:
-                inner_states.append(x.view(B, T, D).transpose(0, 1).clone())
-            else:
-                inner_states.append(None)
-            self._layernorm(lib, stream, x, self.layer_norm, M, D, h)
-            packed = False
-            features = h.view(B, T, D)
+            inner_states.append(None)
+        self._layernorm(lib, stream, x, self.layer_norm, M, D, h)
+        packed = False
+        features = h.view(B, T, D)
         cache.length = S0 + T
         if incremental_state is not None:
             incremental_state[self._state_key] = cache

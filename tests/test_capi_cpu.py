@@ -59,6 +59,6 @@ def test_argument_validation_needs_no_gpu():
     one = ctypes.c_void_p(16)
     assert lib.msa_linear_f16(one, one, None, None, one, 4, 16, 40, 0, None) == -1
     assert b"multiple of 32" in lib.msa_last_error()
-    assert lib.msa_attention_f16(one, one, one, None, 0, one, 1, 1, 64, 2, 9, 10, 0, None) == -2
+    assert lib.msa_attention_f16(one, one, one, None, 0, one, 1, 1, 64, 2, 9, 10, 0, None, None) == -2
     with pytest.raises(ValueError):
         _capi.check(-2, lib)

@@ -35,9 +35,9 @@ def build(cfg, seed=1234, int8=False):
     return model, sd
 
 
-def run_generate(model, cfg, src, max_len_b, min_len):
+def run_generate(model, cfg, src, max_len_b, min_len, **kw):
     gen = SequenceGenerator([model], Dictionary(cfg.vocab_size), beam_size=1,
-                            max_len_b=max_len_b, min_len=min_len)
+                            max_len_b=max_len_b, min_len=min_len, **kw)
     return gen.generate([model], {"net_input": {"src_tokens": src.to(DEV)}})
 
 
@@ -192,3 +192,19 @@ def test_state_dict_uses_reference_names():
     keys = set(model.state_dict().keys())
     assert keys == set(sd.keys())
     assert tuple(model.state_dict()["decoder.layers.0.self_attn.qkv_proj.weight"].shape) == (384, 128)
+
+
+@pytest.mark.parametrize("min_len", [1, 12, 40])
+def test_graph_replay_matches_eager_generation(min_len):
+    """A captured decode step replayed many times (with the generator's own eager work and
+    synchronisations in between) produces the tokens and scores of the eager loop, across the
+    min_len boundary, stop tokens and early exit."""
+    cfg = opt_config("125m", max_target_positions=128)
+    model, _ = build(cfg, seed=11)
+    src = random_prompts(cfg, 5, 9, seed=3)
+    kw = dict(stop=[50118]) if min_len == 12 else {}
+    eager = run_generate(model, cfg, src, 41, min_len, **kw)
+    for _ in range(2):  # a second generation re-captures against a new cache
+        graph = run_generate(model, cfg, src, 41, min_len, use_graph=True, **kw)
+        assert torch.equal(graph["tokens"], eager["tokens"])
+        assert torch.equal(graph["scores"], eager["scores"])

@@ -143,7 +143,7 @@ def test_embed_positions_and_sum(lib, T_out):
     po = torch.empty(B, T_out, dtype=torch.long, device=DEV)
     st = torch.zeros(1, dtype=torch.int32, device=DEV)
     ok(lib.msa_embed_f16(P(td), td.stride(0), B, n, T_out, P(G(E)), V, P(G(Ptab)),
-                         Ptab.shape[0], pad, D, P(x), P(po), P(st), None), lib)
+                         Ptab.shape[0], pad, D, P(x), P(po), P(st), None, None), lib)
     torch.cuda.synchronize()
     assert torch.equal(po.cpu(), want_pos)
     assert torch.equal(x.cpu().float().view(B, T_out, D), want)
@@ -157,9 +157,51 @@ def test_embed_flags_out_of_range_ids(lib):
     x = torch.empty(1, D, dtype=torch.float16, device=DEV)
     st = torch.zeros(1, dtype=torch.int32, device=DEV)
     ok(lib.msa_embed_f16(P(toks), 3, 1, 3, 1, P(G(E)), V, P(G(Ptab)), 6, 1, D, P(x),
-                         None, P(st), None), lib)
+                         None, P(st), None, None), lib)
     torch.cuda.synchronize()
     assert int(st) == 1
+
+
+def test_device_side_length_matches_host_arguments(lib):
+    """embed / qkv append / attention / select with the history length read from device memory
+    give the results of the host-argument form, and msa_advance_len increments it."""
+    B, H, hd, V, S_cap = 4, 2, 64, 64, 24
+    D = H * hd
+    E, Ptab = rnd(V, D, seed=4), rnd(40, D, seed=5)
+    toks = torch.randint(4, V, (B, 20), generator=torch.Generator().manual_seed(1))
+    td = G(toks)
+    W, bq = rnd(3 * D, D, seed=2, std=0.05), rnd(3 * D, seed=3, std=0.1)
+    Wp = pack_w(lib, G(W))
+    Kc0, Vc0 = G(rnd(B, H, S_cap, hd, seed=6)), G(rnd(B, H, S_cap, hd, seed=7))
+    ln = torch.tensor([11], dtype=torch.int32, device=DEV)
+    outs = []
+    for len_dev, n, S0 in ((None, 12, 11), (ln, 20, 0)):
+        Kc, Vc = Kc0.clone(), Vc0.clone()
+        x = torch.empty(B, D, dtype=torch.float16, device=DEV)
+        ok(lib.msa_embed_f16(P(td), 20, B, n, 1, P(G(E)), V, P(G(Ptab)), 40, 1, D, P(x), None,
+                             None, P(len_dev), None), lib)
+        q = torch.empty(B, D, dtype=torch.float16, device=DEV)
+        xp = G(pack_act(x.cpu()))
+        ok(lib.msa_qkv_proj_f16(P(xp), P(Wp), P(G(bq)), P(q), P(Kc), P(Vc), B, 1, H, hd, S0, S_cap,
+                                D, IN_PACKED, P(len_dev), None), lib)
+        o = torch.empty(B, D, dtype=torch.float16, device=DEV)
+        ok(lib.msa_attention_f16(P(q), P(Kc), P(Vc), None, 0, P(o), B, H, hd, 1, S0, S_cap, 0,
+                                 P(len_dev), None), lib)
+        tok = torch.zeros(B, 20, dtype=torch.long, device=DEV)
+        sc = torch.zeros(B, 20, dtype=torch.float32, device=DEV)
+        ba = (ctypes.c_int32 * 1)(1)
+        col = 0 if len_dev is not None else 11
+        ok(lib.msa_greedy_select_f16(P(o), D, B, D, 1.0, ba, 1, ba, 0, None, 0, 2, P(tok[:, col]),
+                                     20, P(sc[:, col]), 20, P(len_dev), None), lib)
+        torch.cuda.synchronize()
+        outs.append((x.clone(), q.clone(), Kc.clone(), Vc.clone(), o.clone(), tok.clone(),
+                     sc.clone()))
+    for a, b in zip(*outs):
+        assert torch.equal(a, b)
+    assert int(outs[0][5][:, 11].abs().sum()) > 0
+    ok(lib.msa_advance_len(P(ln), 1, None), lib)
+    torch.cuda.synchronize()
+    assert int(ln) == 12
 
 
 def test_pack_roundtrip_and_layout(lib):
@@ -370,10 +412,10 @@ def test_qkv_proj_scatter(lib, B, T, H, hd, S0, w8):
         xin = G(pack_act(x)) if flags else G(x)
         if w8:
             ok(lib.msa_qkv_proj_w8a16(P(xin), P(pack_w8(lib, G(qw))), P(G(sc)), P(G(b)), P(qo),
-                                      P(Kc), P(Vc), B, T, H, hd, S0, S_cap, D, flags, None), lib)
+                                      P(Kc), P(Vc), B, T, H, hd, S0, S_cap, D, flags, None, None), lib)
         else:
             ok(lib.msa_qkv_proj_f16(P(xin), P(pack_w(lib, G(W))), P(G(b)), P(qo), P(Kc), P(Vc), B,
-                                    T, H, hd, S0, S_cap, D, flags, None), lib)
+                                    T, H, hd, S0, S_cap, D, flags, None, None), lib)
         torch.cuda.synchronize()
         assert_fp16_close(qo, q.half(), atol=atol, what="q")
         assert_fp16_close(Kc[:, :, S0:S0 + T], want_k.half(), atol=atol, what="K cache")
@@ -385,7 +427,7 @@ def test_qkv_proj_scatter(lib, B, T, H, hd, S0, w8):
 def test_qkv_proj_capacity_error(lib):
     x = torch.zeros(2, 128, dtype=torch.float16, device=DEV)
     rc = lib.msa_qkv_proj_f16(P(x), P(x), P(x), P(x), P(x), P(x), 2, 1, 2, 64, 10, 10, 128, 0,
-                              None)
+                              None, None)
     assert rc == -2 and b"capacity" in lib.msa_last_error()
 
 
@@ -423,14 +465,14 @@ def test_attention(lib, B, H, hd, T, S0, masked):
     dm = None if mask is None else mask.to(torch.uint8).to(DEV)
     ok(lib.msa_attention_f16(P(G(q)), P(G(Kc)), P(G(Vc)), P(dm),
                              0 if dm is None else dm.stride(0), P(out), B, H, hd, T, S0, S_cap,
-                             0, None), lib)
+                             0, None, None), lib)
     torch.cuda.synchronize()
     if T == 1 and B <= 64:
         MB = (B + 15) // 16
         op = torch.zeros(MB * 16 * D, dtype=torch.float16, device=DEV)
         ok(lib.msa_attention_f16(P(G(q)), P(G(Kc)), P(G(Vc)), P(dm),
                                  0 if dm is None else dm.stride(0), P(op), B, H, hd, T, S0, S_cap,
-                                 OUT_PACKED, None), lib)
+                                 OUT_PACKED, None, None), lib)
         torch.cuda.synchronize()
         assert torch.equal(unpack_act(op.cpu(), B, D), out.cpu())
     # scores and probabilities are intermediate fp16 roundings.  A 1-ulp flip of a score of
@@ -442,8 +484,8 @@ def test_attention(lib, B, H, hd, T, S0, masked):
 
 def test_attention_rejects(lib):
     x = torch.zeros(64, 96, dtype=torch.float16, device=DEV)
-    assert lib.msa_attention_f16(P(x), P(x), P(x), None, 0, P(x), 1, 1, 96, 1, 0, 4, 0, None) == -1
-    assert lib.msa_attention_f16(P(x), P(x), P(x), None, 0, P(x), 1, 1, 64, 1, 4, 4, 0, None) == -2
+    assert lib.msa_attention_f16(P(x), P(x), P(x), None, 0, P(x), 1, 1, 96, 1, 0, 4, 0, None, None) == -1
+    assert lib.msa_attention_f16(P(x), P(x), P(x), None, 0, P(x), 1, 1, 64, 1, 4, 4, 0, None, None) == -2
 
 
 def _select(lib, logits, temperature=1.0, banned=(), stop=(), finished=None, force=0, eos=2):
@@ -454,7 +496,7 @@ def _select(lib, logits, temperature=1.0, banned=(), stop=(), finished=None, for
     sa = (ctypes.c_int32 * max(1, len(stop)))(*stop)
     ok(lib.msa_greedy_select_f16(P(logits), logits.stride(0), B, V, temperature, ba, len(banned),
                                  sa, len(stop), P(finished), force, eos, P(tok[:, 1]), 3,
-                                 P(sc[:, 1]), 3, None), lib)
+                                 P(sc[:, 1]), 3, None, None), lib)
     torch.cuda.synchronize()
     assert float(tok[:, 0].abs().sum()) == 0 and float(tok[:, 2].abs().sum()) == 0
     return tok[:, 1].cpu(), sc[:, 1].cpu()
