@@ -18,6 +18,7 @@
 // Both share one epilogue that reproduces the reference's fp16 rounding points, and a QKV mode
 // that scatters K/V into the per-layer cache and scales Q.
 #include <math.h>
+#include <stdlib.h>
 
 #include "common.h"
 
@@ -434,6 +435,163 @@ __global__ __launch_bounds__(TL_THREADS) void linear_tiled_kernel(
     }
 }
 
+// ---- large tiled kernel -------------------------------------------------------------------
+// 256 x 256 x 64 per workgroup of 8 waves on v_mfma_f32_16x16x32_f16; every wave owns 32 output
+// features (two weight tiles) for all 256 activation rows.  Weight fragments come straight from
+// the packed layout in global memory into registers (one KB per wave instruction, no LDS round
+// trip, no two waves read the same weights); only the row-major activations are staged through
+// LDS, double buffered, one barrier per 64-wide K stage.  The stage is software pipelined by
+// hand: activations are fetched two stages ahead and parked in LDS one stage ahead, weights
+// are fetched one stage ahead, LDS fragment reads run TB_PD fragments ahead of the MFMAs, and
+// sched_group_barrier pins that order.  The main loop is branch free: rows and tiles past the
+// edge read clamped addresses and are dropped in the epilogue.  Needs K % 128 == 0.
+constexpr int TB_BM = 256, TB_BN = 256, TB_BK = 64, TB_LD = TB_BK + 8, TB_THREADS = 512;
+constexpr int TB_MF = TB_BM / 16;       // activation fragments per wave and 32-wide step
+constexpr int TB_NT = TB_BN / 8 / 16;   // weight tiles per wave
+constexpr int TB_PD = 4;                // LDS fragment reads in flight
+constexpr int TB_LDS_BYTES = 2 * TB_BM * TB_LD * (int)sizeof(half_t);
+
+template <bool W8>
+struct BigW {  // the weight fragments of one 64-wide stage; int8: the raw 16 bytes per tile
+  half8_t f[W8 ? 1 : 2][TB_NT];
+};
+
+template <bool W8, int MODE>
+__global__ __launch_bounds__(TB_THREADS) void linear_tiled_big_kernel(
+    const half_t* __restrict__ x, const void* __restrict__ Wp, const half_t* __restrict__ scales,
+    int64_t M, int N, int K, Epilogue epi) {
+  extern __shared__ __attribute__((aligned(16))) half_t lx_big[];  // [2][TB_BM * TB_LD]
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int lr = lane & 15, lg = lane >> 4;
+  const int64_t m0 = (int64_t)blockIdx.y * TB_BM;
+  const int n0 = blockIdx.x * TB_BN + wave * (TB_NT * 16);
+  const int nkt = K / TB_BK;
+  const int ntiles = N / 16;
+
+  // activation staging: piece c = row c/8, 16-byte chunk c%8 (8 lanes cover one 128-byte line)
+  const half_t* xsrc[4];
+  int xdst[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int c = tid + TB_THREADS * i;
+    const int row = c >> 3, ch = c & 7;
+    const int64_t m = min(m0 + row, M - 1);
+    xsrc[i] = x + m * K + ch * 8;
+    xdst[i] = row * TB_LD + ch * 8;
+  }
+  const char* wsrc[TB_NT];
+  half_t wscale[TB_NT];
+#pragma unroll
+  for (int j = 0; j < TB_NT; ++j) {
+    const int t = min(n0 / 16 + j, ntiles - 1);
+    // a tile's K sweep is K * 16 elements: K * 32 bytes in fp16, K * 16 bytes in int8
+    wsrc[j] = (const char*)Wp + (int64_t)t * K * (W8 ? 16 : 32) + lane * 16;
+    wscale[j] = W8 ? scales[t * 16 + lr] : (half_t)0.f;
+  }
+
+  auto gload_x = [&](half8_t(&xr)[4], int kt) {
+    kt = min(kt, nkt - 1);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) xr[i] = *reinterpret_cast<const half8_t*>(xsrc[i] + kt * TB_BK);
+  };
+  auto gload_w = [&](BigW<W8>& w, int kt) {
+    kt = min(kt, nkt - 1);
+#pragma unroll
+    for (int j = 0; j < TB_NT; ++j) {
+      if (W8) {
+        w.f[0][j] = *reinterpret_cast<const half8_t*>(wsrc[j] + (int64_t)kt * 1024);
+      } else {
+        w.f[0][j] = *reinterpret_cast<const half8_t*>(wsrc[j] + (int64_t)kt * 2048);
+        w.f[W8 ? 0 : 1][j] = *reinterpret_cast<const half8_t*>(wsrc[j] + (int64_t)kt * 2048 + 1024);
+      }
+    }
+  };
+  auto lstore = [&](const half8_t(&xr)[4], int buf) {
+    half_t* l = lx_big + buf * (TB_BM * TB_LD);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) *reinterpret_cast<half8_t*>(l + xdst[i]) = xr[i];
+  };
+
+  float4_t acc[TB_MF][TB_NT];
+#pragma unroll
+  for (int a = 0; a < TB_MF; ++a)
+#pragma unroll
+    for (int b = 0; b < TB_NT; ++b) acc[a][b] = float4_t{0.f, 0.f, 0.f, 0.f};
+
+  auto compute = [&](const BigW<W8>& w, int buf) {
+    const half_t* l = lx_big + buf * (TB_BM * TB_LD) + lr * TB_LD + lg * 8;
+    constexpr int F = 2 * TB_MF;  // fragment f = 32-wide step f / TB_MF, row block f % TB_MF
+    half8_t a[2][TB_NT];
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+      for (int j = 0; j < TB_NT; ++j) {
+        if (W8) {
+          const uint4 q = __builtin_bit_cast(uint4, w.f[0][j]);
+          a[ks][j] = ks == 0 ? dequant8(q.x, q.y, wscale[j]) : dequant8(q.z, q.w, wscale[j]);
+        } else {
+          a[ks][j] = w.f[W8 ? 0 : ks][j];
+        }
+      }
+    half8_t bx[TB_PD];
+#pragma unroll
+    for (int p = 0; p < TB_PD; ++p)
+      bx[p] = *reinterpret_cast<const half8_t*>(l + (p % TB_MF) * 16 * TB_LD + (p / TB_MF) * 32);
+    __builtin_amdgcn_sched_group_barrier(0x200, 4, 0);                         // LDS stores
+    __builtin_amdgcn_sched_group_barrier(0x020, 4 + (W8 ? 1 : 2) * TB_NT, 0);  // global loads
+    __builtin_amdgcn_sched_group_barrier(0x100, TB_PD, 0);                     // leading LDS reads
+#pragma unroll
+    for (int f = 0; f < F; ++f) {
+      const int ks = f / TB_MF, mf = f % TB_MF;
+      const half8_t cur = bx[f % TB_PD];
+#pragma unroll
+      for (int j = 0; j < TB_NT; ++j)
+        acc[mf][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[ks][j], cur, acc[mf][j], 0, 0, 0);
+      __builtin_amdgcn_sched_group_barrier(0x008, TB_NT, 0);
+      if (f + TB_PD < F) {
+        const int g = f + TB_PD;
+        bx[f % TB_PD] =
+            *reinterpret_cast<const half8_t*>(l + (g % TB_MF) * 16 * TB_LD + (g / TB_MF) * 32);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      }
+    }
+  };
+
+  half8_t xr[4];
+  BigW<W8> w0, w1;
+  gload_x(xr, 0);
+  gload_w(w0, 0);
+  lstore(xr, 0);
+  gload_x(xr, 1);
+  __syncthreads();
+  for (int kt = 0; kt < nkt; kt += 2) {
+    lstore(xr, 1);  // stage kt + 1, fetched during stage kt - 1
+    gload_x(xr, kt + 2);
+    gload_w(w1, kt + 1);
+    compute(w0, 0);
+    __syncthreads();
+    lstore(xr, 0);
+    gload_x(xr, kt + 3);
+    gload_w(w0, kt + 2);
+    compute(w1, 1);
+    __syncthreads();
+  }
+
+  // D of the 16x16 MFMA: lane holds activation row (lane & 15) and the 4 consecutive features
+  // 4 * (lane >> 4) .. + 3 of the weight tile
+#pragma unroll
+  for (int mf = 0; mf < TB_MF; ++mf) {
+    const int64_t m = m0 + mf * 16 + lr;
+    if (m >= M) continue;
+#pragma unroll
+    for (int j = 0; j < TB_NT; ++j) {
+      const int n = n0 + j * 16;
+      if (n >= N) continue;
+      epilogue4<MODE>(epi, m, n + lg * 4, acc[mf][j]);
+    }
+  }
+}
+
 // ---- host side ------------------------------------------------------------------------------
 int g_num_cus = 0;
 int num_cus() {
@@ -477,6 +635,22 @@ void launch_stream(const void* xp, const void* W, const void* scales, float* par
 template <bool W8, int MODE>
 void launch_tiled(const void* x, const void* W, const void* scales, int64_t M, int N, int K,
                   const Epilogue& epi, hipStream_t s) {
+  // the 256 x 256 kernel once it fills the chip; the 128 x 128 one for the shapes in between
+  const int64_t big_tiles = ((M + TB_BM - 1) / TB_BM) * ((N + TB_BN - 1) / TB_BN);
+  if (K % (2 * TB_BK) == 0 && big_tiles >= num_cus() && !getenv("MSA_NO_BIG")) {
+    static bool attr_set = false;  // one flag per instantiation
+    if (!attr_set) {
+      if (hipFuncSetAttribute((const void*)linear_tiled_big_kernel<W8, MODE>,
+                              hipFuncAttributeMaxDynamicSharedMemorySize,
+                              TB_LDS_BYTES) != hipSuccess)
+        return;  // the launch check below reports the error
+      attr_set = true;
+    }
+    const dim3 grid((N + TB_BN - 1) / TB_BN, (unsigned)((M + TB_BM - 1) / TB_BM));
+    hipLaunchKernelGGL((linear_tiled_big_kernel<W8, MODE>), grid, dim3(TB_THREADS), TB_LDS_BYTES,
+                       s, (const half_t*)x, W, (const half_t*)scales, M, N, K, epi);
+    return;
+  }
   const dim3 grid((N + TL_BN - 1) / TL_BN, (unsigned)((M + TL_BM - 1) / TL_BM));
   hipLaunchKernelGGL((linear_tiled_kernel<W8, MODE>), grid, dim3(TL_THREADS), 0, s,
                      (const half_t*)x, W, (const half_t*)scales, M, N, K, epi);

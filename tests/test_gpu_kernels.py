@@ -234,6 +234,8 @@ LINEAR_SHAPES = [
     (1, 96, 64), (8, 768, 768), (32, 3072, 768), (32, 768, 3072), (33, 2048, 2048),
     (64, 4096, 4096), (17, 50272, 768), (65, 768, 768), (200, 2304, 768), (513, 4096, 1024),
     (129, 1008, 96),
+    # enough 256 x 256 tiles to take the large tiled kernel, with ragged M and N edges
+    (1000, 16400, 128), (4099, 4096, 256),
 ]
 
 
@@ -310,7 +312,8 @@ def test_linear_rejects_bad_shapes(lib):
 
 
 @pytest.mark.parametrize("M,N,K", [(8, 768, 768), (64, 3072, 768), (32, 768, 3072),
-                                   (200, 2304, 768), (48, 4096, 4096)])
+                                   (200, 2304, 768), (48, 4096, 4096),
+                                   (1000, 16400, 128)])   # the last: large tiled kernel
 def test_linear_w8a16(lib, M, N, K):
     print("w8a16", M, N, K, flush=True)
     x, W, b = rnd(M, K, seed=7), rnd(N, K, seed=8, std=0.02), rnd(N, seed=9, std=0.1)
@@ -422,6 +425,40 @@ def test_qkv_proj_scatter(lib, B, T, H, hd, S0, w8):
         assert_fp16_close(Vc[:, :, S0:S0 + T], want_v.half(), atol=atol, what="V cache")
         # nothing outside the appended slice was touched
         assert float(Kc[:, :, :S0].abs().sum()) == 0 and float(Kc[:, :, S0 + T:].abs().sum()) == 0
+
+
+@pytest.mark.parametrize("w8", [False, True])
+def test_qkv_proj_scatter_large_tiled_kernel(lib, w8):
+    """A prefill-sized QKV projection (enough 256 x 256 tiles for the large tiled kernel): the
+    scatter into the cache and the q scaling, with an input width independent of H * hd."""
+    B, T, H, hd, S0, K = 2, 1100, 20, 128, 3, 256
+    D, S_cap = H * hd, S0 + T + 2
+    x, W, b = rnd(B * T, K, seed=1), rnd(3 * D, K, seed=2, std=0.05), rnd(3 * D, seed=3, std=0.1)
+    if w8:
+        qw, sc = O.quantize_int8(W)
+        Wuse = O.dequantize_int8(qw, sc)
+    else:
+        Wuse = W
+    kvq = O.linear(x.float(), Wuse.float(), b.float(), r16)
+    k, v, q = kvq.split(D, dim=-1)
+    q = r16(q * (hd ** -0.5))
+    atol = float(kvq.abs().max()) * 2 ** -10
+    Kc = torch.zeros(B, H, S_cap, hd, dtype=torch.float16, device=DEV)
+    Vc = torch.zeros_like(Kc)
+    qo = torch.empty(B * T, D, dtype=torch.float16, device=DEV)
+    if w8:
+        ok(lib.msa_qkv_proj_w8a16(P(G(x)), P(pack_w8(lib, G(qw))), P(G(sc)), P(G(b)), P(qo), P(Kc),
+                                  P(Vc), B, T, H, hd, S0, S_cap, K, 0, None, None), lib)
+    else:
+        ok(lib.msa_qkv_proj_f16(P(G(x)), P(pack_w(lib, G(W))), P(G(b)), P(qo), P(Kc), P(Vc), B, T,
+                                H, hd, S0, S_cap, K, 0, None, None), lib)
+    torch.cuda.synchronize()
+    assert_fp16_close(qo, q.half(), atol=atol, what="q")
+    assert_fp16_close(Kc[:, :, S0:S0 + T], k.view(B, T, H, hd).permute(0, 2, 1, 3).half(),
+                      atol=atol, what="K cache")
+    assert_fp16_close(Vc[:, :, S0:S0 + T], v.view(B, T, H, hd).permute(0, 2, 1, 3).half(),
+                      atol=atol, what="V cache")
+    assert float(Kc[:, :, :S0].abs().sum()) == 0 and float(Kc[:, :, S0 + T:].abs().sum()) == 0
 
 
 def test_qkv_proj_capacity_error(lib):
