@@ -180,14 +180,19 @@ def main():
     scores = torch.zeros(B, max_len, dtype=torch.float32, device=dev)
     finished = torch.zeros(B, dtype=torch.uint8, device=dev)
     tokens[:, :n0] = src
-    inc = {}
-    torch.cuda.synchronize()
-    t1 = time.time()
-    logits = model(tokens[:, :n0], incremental_state=inc)[0]
-    step_logits = logits[:, -1, :].contiguous()
-    del logits
-    torch.cuda.synchronize()
-    prefill_s = time.time() - t1
+    # the first prefill also packs the weights and grows the allocator's pools (reported as
+    # prefill_cold_s); the timed one is the second, as a serving process would see it
+    prefill_times = []
+    for _ in range(2):
+        inc = {}
+        torch.cuda.synchronize()
+        t1 = time.time()
+        logits = model(tokens[:, :n0], incremental_state=inc)[0]
+        step_logits = logits[:, -1, :].contiguous()
+        del logits
+        torch.cuda.synchronize()
+        prefill_times.append(time.time() - t1)
+    prefill_cold_s, prefill_s = prefill_times
 
     st = None
     if args.graph and B <= 64:
@@ -274,6 +279,7 @@ def main():
         "gpu_ms_per_step": gpu_s / K * 1e3,
         "graph_replay": st is not None,
         "prefill_s": prefill_s,
+        "prefill_cold_s": prefill_cold_s,
         "prefill_tflops": prefill_flops(cfg, B, n0) / prefill_s / 1e12,
         "prefill_mfma_frac": prefill_flops(cfg, B, n0) / prefill_s / MFMA_PEAK,
         "setup_s": t1 - t0,

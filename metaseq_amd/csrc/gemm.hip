@@ -188,6 +188,10 @@ __global__ __launch_bounds__(KG * 64) void linear_stream_kernel(
     half8_t b[U][MB];
   };
   Stage s0, s1;
+  // Loads are unconditional so that the hardware counters can keep two stages in flight (a
+  // load inside a branch makes the compiler wait for every outstanding load before the MFMAs).
+  // Steps and tiles past the end read a clamped, valid address: a surplus tile is dropped in
+  // finish(), a surplus step gets its activation fragment zeroed in mma().
   auto load = [&](Stage& s, int idx) {
     const int grp = idx / nstages, st = idx - grp * nstages;
     const int t0 = tile_begin + grp * NT;
@@ -196,29 +200,21 @@ __global__ __launch_bounds__(KG * 64) void linear_stream_kernel(
       // first 32-wide step covered by this load (wave-uniform)
       const int ks = W8 ? ks_begin + 2 * (wave + KG * (st * UA + u))
                         : ks_begin + wave + KG * (st * U + u);
-      const bool kv = idx < total && ks < ks_end;
 #pragma unroll
       for (int j = 0; j < NT; ++j) {
-        if (kv && t0 + j < tile_end) {
-          const int64_t blk = W8 ? (int64_t)(t0 + j) * (nks >> 1) + (ks >> 1)
-                                 : (int64_t)(t0 + j) * nks + ks;
-          s.a[u][j] = __builtin_nontemporal_load(
-              reinterpret_cast<const half8_t*>((const half_t*)Wp + blk * 512 + lane * 8));
-        } else {
-          s.a[u][j] = zero8();
-        }
+        const int t = min(t0 + j, tile_end - 1);
+        const int ksc = min(ks, ks_end - (W8 ? 2 : 1));
+        const int64_t blk = W8 ? (int64_t)t * (nks >> 1) + (ksc >> 1) : (int64_t)t * nks + ksc;
+        s.a[u][j] = __builtin_nontemporal_load(
+            reinterpret_cast<const half8_t*>((const half_t*)Wp + blk * 512 + lane * 8));
       }
 #pragma unroll
       for (int h = 0; h < (W8 ? 2 : 1); ++h) {
+        const int kk = min(ks + h, ks_end - 1);
 #pragma unroll
-        for (int mb = 0; mb < MB; ++mb) {
-          const int kk = ks + h;
-          if (kv && kk < ks_end)
-            s.b[W8 ? 2 * u + h : u][mb] = *reinterpret_cast<const half8_t*>(
-                xp + (((int64_t)kk * MB + mb) * 64 + lane) * 8);
-          else
-            s.b[W8 ? 2 * u + h : u][mb] = zero8();
-        }
+        for (int mb = 0; mb < MB; ++mb)
+          s.b[W8 ? 2 * u + h : u][mb] =
+              *reinterpret_cast<const half8_t*>(xp + (((int64_t)kk * MB + mb) * 64 + lane) * 8);
       }
     }
   };
@@ -230,13 +226,23 @@ __global__ __launch_bounds__(KG * 64) void linear_stream_kernel(
       for (int mb = 0; mb < MB; ++mb) acc[j][mb] = float4_t{0.f, 0.f, 0.f, 0.f};
   };
   auto mma = [&](Stage& s, int idx) {
+    const int grp = idx / nstages, st = idx - grp * nstages;
     half_t sc[NT];
     if (W8) {
-      const int grp = idx / nstages;
       const int t0 = tile_begin + grp * NT;
 #pragma unroll
       for (int j = 0; j < NT; ++j)
-        sc[j] = (t0 + j < tile_end) ? scales[(t0 + j) * 16 + (lane & 15)] : (half_t)0;
+        sc[j] = scales[min(t0 + j, tile_end - 1) * 16 + (lane & 15)];
+    }
+    // zero the activation fragments of steps past the end of this K range
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int ks = W8 ? ks_begin + 2 * (wave + KG * (st * UA + u / 2)) + (u & 1)
+                        : ks_begin + wave + KG * (st * U + u);
+      if (ks >= ks_end) {
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) s.b[u][mb] = zero8();
+      }
     }
 #pragma unroll
     for (int u = 0; u < UA; ++u)
@@ -290,15 +296,24 @@ __global__ __launch_bounds__(KG * 64) void linear_stream_kernel(
   };
   clear();
   load(s0, 0);
-  for (int idx = 0; idx < total; idx += 2) {
+  int idx = 0;
+  for (; idx + 2 < total; idx += 2) {  // steady state: every load is of a real stage
     load(s1, idx + 1);
     mma(s0, idx);
     if ((idx + 1) % nstages == 0) finish(idx);
     load(s0, idx + 2);
-    if (idx + 1 < total) {
-      mma(s1, idx + 1);
-      if ((idx + 2) % nstages == 0) finish(idx + 1);
-    }
+    mma(s1, idx + 1);
+    if ((idx + 2) % nstages == 0) finish(idx + 1);
+  }
+  if (idx + 1 < total) {  // two stages left
+    load(s1, idx + 1);
+    mma(s0, idx);
+    if ((idx + 1) % nstages == 0) finish(idx);
+    mma(s1, idx + 1);
+    finish(idx + 1);
+  } else {  // one stage left
+    mma(s0, idx);
+    finish(idx);
   }
 }
 
