@@ -2,6 +2,7 @@
 TransformerDecoder.forward / SequenceGenerator on one gfx950 GPU)."""
 from .config import OPTConfig, opt_config
 from .dictionary import Dictionary
+from .hub_utils import GeneratorInterface
 from .kv_cache import KVCache
 from .sequence_generator import SequenceGenerator
 from .synthetic import random_prompts, random_state_dict
@@ -9,7 +10,7 @@ from .transformer_decoder import ModelParallelTransformerDecoder, TransformerDec
 from .transformer_lm import TransformerLanguageModel
 
 __all__ = [
-    "OPTConfig", "opt_config", "Dictionary", "KVCache", "SequenceGenerator", "random_prompts",
+    "OPTConfig", "opt_config", "Dictionary", "GeneratorInterface", "KVCache", "SequenceGenerator", "random_prompts",
     "random_state_dict", "TransformerDecoder", "ModelParallelTransformerDecoder",
     "TransformerLanguageModel",
 ]

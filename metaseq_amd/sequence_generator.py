@@ -1,14 +1,17 @@
-"""Greedy generation loop with the constructor, call signature and return value of the
-reference's ``SequenceGenerator`` (metaseq/sequence_generator.py:26-534).
+"""Generation loop with the constructor, call signature and return value of the reference's
+``SequenceGenerator`` (metaseq/sequence_generator.py:26-534).
 
-The reference makes ~6 full-vocabulary fp32 passes and two device-to-host syncs per step; here
-one kernel per step does log-sum-exp, masking, arg-max, token/score write-back and the
-finished-row update on the device, and the host only syncs once end-of-sequence becomes
-possible (step >= min_len).
+Greedy decoding is the fast path: the reference makes ~6 full-vocabulary fp32 passes and two
+device-to-host syncs per step; here one kernel per step does log-sum-exp, masking, arg-max,
+token/score write-back and the finished-row update on the device, and the host only syncs
+once end-of-sequence becomes possible (step >= min_len).
 
-Implemented: beam_size replicas, min_len / max_len_b, stop tokens, temperature, prompt
-scoring, ``need_logprobs``.  Not implemented (raise): top-p / factual-nucleus sampling and
-repetition penalties.
+Nucleus (top-p) sampling, factual-nucleus decay and the repetition penalties take the general
+path: the step's masked fp32 log-probabilities are materialised with device tensor ops in
+the reference's order (:271-308) and the draw is ``torch.multinomial`` on the device, as in
+the reference (:431).  Factual-nucleus state is kept per row (the reference's indexing only
+works at beam_size 1, where the two agree), and prompt-token counts of a replica row come from
+its own prompt (the reference indexes past the prompt batch when beam_size > 1).
 """
 import ctypes
 from typing import Dict, List, Optional
@@ -49,14 +52,20 @@ class SequenceGenerator(nn.Module):
         self.sampling_topp = max(0, topp)
         self.temperature = temperature
         assert temperature >= 0, "--temperature must be >=0"
-        if not (self.temperature == 0.0 or self.sampling_topp == 0.0):
-            raise NotImplementedError("top-p sampling is not implemented; use topp <= 0 (greedy)")
-        if lambda_decay > 0:
-            raise NotImplementedError("factual-nucleus sampling is not implemented")
-        if max(alpha_presence, alpha_frequency, alpha_presence_src, alpha_frequency_src) > 0:
-            raise NotImplementedError("repetition penalties are not implemented")
         if len(self.stop) > 14:
             raise ValueError("at most 14 stop tokens are supported")
+        # factual nucleus (:107-116) and repetition penalties (:118-123)
+        self.lambda_decay = lambda_decay
+        self.omega_bound = float(omega_bound)
+        self.full_stop_list = [tgt_dict.index(w) for w in [".", "?", "!"]]
+        self.alpha_presence = alpha_presence
+        self.alpha_frequency = alpha_frequency
+        self.alpha_presence_src = alpha_presence_src
+        self.alpha_frequency_src = alpha_frequency_src
+        self.alpha_src_penalty_end_idx = alpha_src_penalty_end_idx
+        self.sampling = not (self.temperature == 0.0 or self.sampling_topp == 0.0)
+        self.penalties = max(alpha_presence, alpha_frequency) > 0
+        self.penalties_src = max(alpha_presence_src, alpha_frequency_src) > 0
         self.model.eval()
         self.profile = profile
 
@@ -196,11 +205,24 @@ class SequenceGenerator(nn.Module):
 
             finished = torch.zeros(BB, dtype=torch.uint8, device=dev)
             cache = decoder.get_cache(incremental_states) if hasattr(decoder, "get_cache") else None
+            general = self.sampling or self.penalties or self.penalties_src
+            gs = self._general_state(src_tokens, BB, V, dev) if general else None
             st = None
             if (self.use_graph and all_lprobs is None and cache is not None and BB <= 64
-                    and not cache.has_pads):
+                    and not cache.has_pads and not general):
                 st = self.static_state(decoder, cache, tokens, scores, finished, step_logits)
             for step in range(start_step, max_len):
+                if general:
+                    lprobs = self._masked_lprobs(step_logits, step, min_len, max_len, finished,
+                                                 gs)
+                    if all_lprobs is not None:
+                        all_lprobs[:, step] = lprobs
+                    self._choose(lprobs, step, gs, finished, tokens, scores)
+                    if bool(finished.all()) or step + 1 >= max_len:
+                        break
+                    out = decoder(tokens[:, :step + 1], incremental_state=incremental_states)[0]
+                    step_logits = out.view(BB, V)
+                    continue
                 if st is not None and step < max_len - 1:
                     self._graph_step(lib, st, step, min_len, max_len)
                     if step >= min_len and bool(finished.all()):
@@ -241,7 +263,9 @@ class SequenceGenerator(nn.Module):
             x = x / self.temperature
         return x
 
-    def _masked_lprobs(self, step_logits, step, min_len, max_len, finished):
+    def _masked_lprobs(self, step_logits, step, min_len, max_len, finished, gs=None):
+        """fp32 log-probabilities of one step with the reference's masks in the reference's
+        order (:272-293): min-length block, NaN, pad, forced eos, penalties, finished rows."""
         import math
         lprobs = self.model.get_normalized_probs(self._tempered(step_logits), log_probs=True)
         if step < min_len:
@@ -253,7 +277,88 @@ class SequenceGenerator(nn.Module):
         if step >= max_len - 1:
             lprobs[:, :self.eos] = -math.inf
             lprobs[:, self.eos + 1:] = -math.inf
+        if gs is not None:
+            lprobs = self._apply_repetition_penalties(lprobs, gs["count_tokens"],
+                                                      gs["count_tokens_src"])
         fin = finished.bool()
         lprobs[fin, :self.eos] = -math.inf
         lprobs[fin, self.eos + 1:] = -math.inf
         return lprobs
+
+    # ---- general path: nucleus sampling, factual-nucleus decay, repetition penalties ----
+    def _general_state(self, src_tokens, BB, V, dev):
+        """Per-call buffers of the general path (:372-395)."""
+        gs = {"count_tokens": None, "count_tokens_src": None}
+        if self.penalties:
+            gs["count_tokens"] = torch.zeros(BB, V, dtype=torch.long, device=dev)
+        if self.penalties_src:
+            src = src_tokens
+            if self.alpha_src_penalty_end_idx > 0 and not src_tokens.shape[0] > 1:
+                src = src[:, :self.alpha_src_penalty_end_idx]
+            src = src.repeat_interleave(self.beam_size, 0)
+            counts = torch.zeros(BB, V, dtype=torch.long, device=dev)
+            counts.scatter_add_(1, src.clamp(0, V - 1), torch.ones_like(src))
+            gs["count_tokens_src"] = counts
+        gs["init_p"] = torch.full((BB, 1), float(self.sampling_topp), device=dev)
+        gs["topp"] = gs["init_p"].clone()
+        gs["toks_since_reset"] = torch.zeros(BB, 1, device=dev)
+        gs["full_stop"] = torch.tensor(self.full_stop_list, device=dev)
+        gs["rows"] = torch.arange(BB, device=dev)
+        return gs
+
+    def _apply_repetition_penalties(self, lprobs, count_tokens, count_tokens_src):
+        """mu[j] - c[j] * alpha_frequency - [c[j] > 0] * alpha_presence (:478-523)."""
+        if self.penalties:
+            lprobs = (lprobs - count_tokens * self.alpha_frequency
+                      - count_tokens.gt(0) * self.alpha_presence)
+        if self.penalties_src:
+            lprobs = (lprobs - count_tokens_src * self.alpha_frequency_src
+                      - count_tokens_src.gt(0) * self.alpha_presence_src)
+        return lprobs
+
+    def _sample_topp(self, lprobs, gs):
+        """Draw among the smallest set of tokens whose probability mass reaches p (:399-441)."""
+        if not self.sampling:
+            return tuple(lprobs.max(dim=-1))
+        probs = torch.softmax(lprobs, dim=-1)
+        sprobs, sinds = probs.sort(dim=-1, descending=True)
+        p = self.sampling_topp if self.lambda_decay <= 0 else gs["topp"]
+        mask = (sprobs.cumsum(dim=-1) - sprobs) >= p
+        trunc = sprobs.masked_fill(mask, 0)
+        trunc.div_(trunc.sum(dim=-1, keepdim=True))
+        # A row with every token masked (min_len == max_len at the last step) has NaN
+        # probabilities: the reference's multinomial raises there, and on the device that check
+        # is an assertion that takes the GPU context down.  Such a row gets what the greedy
+        # branch's max() gives it: token 0 with score -inf.
+        dead = ~torch.isfinite(lprobs).any(dim=-1)
+        trunc = torch.nan_to_num(trunc, nan=0.0, posinf=0.0, neginf=0.0)
+        trunc[:, 0] += dead.to(trunc.dtype)
+        choices = torch.multinomial(trunc, 1)[:, 0]
+        tok_ids = sinds[gs["rows"], choices].masked_fill(dead, 0)
+        scores = sprobs[gs["rows"], choices].log().masked_fill(dead, float("-inf"))
+        if self.lambda_decay > 0:
+            self._update_sampling_topp(tok_ids, gs)
+        return scores, tok_ids
+
+    def _update_sampling_topp(self, tok_ids, gs):
+        """Factual-nucleus decay, vectorised over rows (:443-476): p restarts at its initial
+        value after ".", "?" or "!" and decays by lambda_decay per further token, never below
+        omega_bound."""
+        hit = (tok_ids.unsqueeze(1) == gs["full_stop"].unsqueeze(0)).any(dim=1, keepdim=True)
+        tsr = torch.where(hit, torch.zeros_like(gs["toks_since_reset"]),
+                          gs["toks_since_reset"] + 1)
+        gs["toks_since_reset"] = tsr
+        decay = (tsr - 1).clamp_(min=0)
+        gs["topp"] = torch.clamp(gs["init_p"] * self.lambda_decay ** decay, min=self.omega_bound)
+
+    def _choose(self, lprobs, step, gs, finished, tokens, scores):
+        """Selection and bookkeeping of one general-path step (:295-308)."""
+        next_scores, next_toks = self._sample_topp(lprobs, gs)
+        if gs["count_tokens"] is not None:
+            gs["count_tokens"][gs["rows"], next_toks] += 1
+        tokens[:, step] = next_toks
+        scores[:, step] = next_scores
+        done = next_toks == self.eos
+        for t in self.stop:
+            done |= next_toks == t
+        finished |= done.to(finished.dtype)

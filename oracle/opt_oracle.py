@@ -31,9 +31,15 @@ How each function is pinned (tests/test_oracle_*.py):
   position offset, pad mask      object with the same weights mapped in (the
                                  relation the reference's own
                                  gpu_tests/test_hf_compatibility.py:128-155 asserts).
-* ``greedy_generate``          - scripted-logit fake decoders with hand-derived
-                                 expected token/score tables (the idea of the
+* ``generate`` /               - scripted-logit fake decoders with hand-derived
+  ``greedy_generate``            expected token/score tables (the idea of the
                                  reference's tests/utils.py:420-465).
+* ``sample_topp``,             - hand-derived closed forms (mass-before-token rule,
+  ``update_sampling_topp``,      renormalisation, score of the untruncated probability,
+  ``apply_repetition_penalties`` decay / reset / bound sequence, penalty arithmetic) and
+                                 empirical draw frequencies; the reference holds no test of
+                                 these functions (tests/test_sequence_generator.py predates
+                                 them).
 * ``quantize_int8``            - parity unpinned by the reference (its int8
                                  quantiser lives in FasterTransformer and no
                                  reference test touches it); pinned by the closed
@@ -259,48 +265,123 @@ class OracleDecoder:
     __call__ = forward
 
 
-def greedy_generate(decoder, src_tokens: torch.Tensor, max_len_b: int, min_len: int = 1,
-                    pad: int = 1, eos: int = 2, stop: Optional[List[int]] = None,
-                    temperature: float = 1.0, max_positions: Optional[int] = None,
-                    return_step_logits: bool = False):
-    """SequenceGenerator._generate at beam 1 with greedy selection
-    (metaseq/sequence_generator.py:142-344; buffers :368-371; greedy :413-415).
+def sample_topp(lprobs: torch.Tensor, topp, generator=None):
+    """Nucleus choice of SequenceGenerator._sample_topp (metaseq/sequence_generator.py:399-441)
+    for ``topp`` a float or a [rows, 1] tensor.  Returns (scores, token ids, the truncated
+    renormalised distribution in sorted order, the sort indices)."""
+    probs = torch.softmax(lprobs, dim=-1)  # :416
+    sprobs, sinds = probs.sort(dim=-1, descending=True)
+    if torch.is_tensor(topp):
+        topp = topp.to(sprobs.device).expand(sprobs.size())
+    mask = (sprobs.cumsum(dim=-1) - sprobs) >= topp  # :420-427
+    trunc = sprobs.clone()
+    trunc[mask] = 0
+    trunc = trunc / trunc.sum(dim=-1, keepdim=True)  # :430
+    choices = torch.multinomial(trunc, 1, generator=generator)[:, 0]  # :431
+    rows = torch.arange(lprobs.size(0), device=lprobs.device)
+    return sprobs[rows, choices].log(), sinds[rows, choices], trunc, sinds  # :433-434
+
+
+def update_sampling_topp(tok_ids, toks_since_reset, init_p, full_stop_list, lambda_decay,
+                         omega_bound):
+    """Factual-nucleus decay of p, one value per row
+    (metaseq/sequence_generator.py:443-476, the 1-D-tokens branch :465-476).  Updates
+    ``toks_since_reset`` in place and returns the new p per row."""
+    new_p = init_p.clone()
+    for i, t in enumerate(tok_ids.tolist()):
+        if t in full_stop_list:
+            toks_since_reset[i] = 0
+        else:
+            toks_since_reset[i] += 1
+        decay = max(0, int(toks_since_reset[i]) - 1)
+        new_p[i] = max(omega_bound, float(init_p[i]) * lambda_decay ** decay)
+    return new_p
+
+
+def apply_repetition_penalties(lprobs, count_tokens, count_tokens_src, alpha_presence=0.0,
+                               alpha_frequency=0.0, alpha_presence_src=0.0,
+                               alpha_frequency_src=0.0):
+    """mu[j] - c[j] * alpha_frequency - [c[j] > 0] * alpha_presence, for the generated-token
+    counts and the prompt-token counts (metaseq/sequence_generator.py:478-523)."""
+    if alpha_frequency > 0 or alpha_presence > 0:
+        lprobs = lprobs - count_tokens * alpha_frequency - count_tokens.gt(0) * alpha_presence
+    if alpha_frequency_src > 0 or alpha_presence_src > 0:
+        lprobs = (lprobs - count_tokens_src * alpha_frequency_src
+                  - count_tokens_src.gt(0) * alpha_presence_src)
+    return lprobs
+
+
+def generate(decoder, src_tokens: torch.Tensor, max_len_b: int, min_len: int = 1,
+             pad: int = 1, eos: int = 2, stop: Optional[List[int]] = None,
+             temperature: float = 1.0, max_positions: Optional[int] = None,
+             return_step_logits: bool = False, beam_size: int = 1, topp: float = -1,
+             lambda_decay: float = -1, omega_bound: float = 0.3, full_stop_list=(3, 3, 3),
+             alpha_presence: float = 0.0, alpha_frequency: float = 0.0,
+             alpha_presence_src: float = 0.0, alpha_frequency_src: float = 0.0,
+             alpha_src_penalty_end_idx: int = -1, need_logprobs: bool = False,
+             generator=None):
+    """SequenceGenerator._generate (metaseq/sequence_generator.py:142-344; buffers :345-397;
+    selection :399-441; factual nucleus :443-476; penalties :478-534).
 
     ``decoder(tokens, incremental_state=dict)`` must return ``(logits[B, T, V], extra)``.
-    Returns {"tokens": [B, 1, max_len], "scores": [B, 1, max_len]} and, on request, the
-    list of logits tensors seen by the loop (prefill logits first).
+    ``full_stop_list`` holds the ids the dictionary gives ".", "?" and "!" (:116; the unk id for
+    a dictionary of BPE ids).  Factual-nucleus state is kept per row, which is what the
+    reference does at beam_size 1 (its indexing fails for more).
+    Returns {"tokens": [B, beam, max_len], "scores": [B, beam, max_len]} (+ "distributions"
+    with ``need_logprobs``) and, on request, the logits tensors seen by the loop.
     """
     stop = stop or []
+    topp = 0.0 if topp is None else max(0, topp)  # :96-98
+    greedy = temperature == 0.0 or topp == 0.0  # :412
     incremental_state: Dict = {}
     device = src_tokens.device
     src_lengths = (src_tokens.ne(eos) & src_tokens.ne(pad)).long().sum(dim=1)  # :164-166
     bsz = src_tokens.shape[0]
+    BB = bsz * beam_size
     if max_positions is None:
         max_positions = decoder.max_positions()
     max_len = int(min(max_positions, max_len_b or 1e99))  # :182
     min_len = min(max_len, min_len or 0)
     assert min_len <= max_len
-    scores = torch.zeros(bsz, max_len, device=device).float()  # :368-371
-    tokens = torch.full((bsz, max_len), pad, dtype=torch.long, device=device)
+    scores = torch.zeros(BB, max_len, device=device).float()  # :368-371
+    tokens = torch.full((BB, max_len), pad, dtype=torch.long, device=device)
     start_step = src_tokens.shape[1]
-    tokens[:, :start_step] = src_tokens
+    tokens[:, :start_step] = src_tokens.repeat_interleave(beam_size, 0)  # :225
+    V = None
     step_logits = []
     logits = decoder(tokens[:, :start_step], incremental_state=incremental_state)[0]
+    V = logits.shape[-1]
+    count_tokens = count_tokens_src = None  # :372-390
+    if alpha_presence > 0 or alpha_frequency > 0:
+        count_tokens = torch.zeros(BB, V, device=device, dtype=torch.long)
+    if alpha_presence_src > 0 or alpha_frequency_src > 0:
+        src = src_tokens
+        if alpha_src_penalty_end_idx > 0 and not bsz > 1:
+            src = src[:, :alpha_src_penalty_end_idx]
+        count_tokens_src = torch.zeros(BB, V, device=device, dtype=torch.long)
+        for i in range(BB):  # the reference fills rows 0..BB-1 from src rows 0..BB-1 (:385-390)
+            count_tokens_src[i] = torch.bincount(src[i], minlength=V)[:V]
+    init_p = torch.full((BB,), float(topp))
+    topp_rows = init_p.clone()
+    toks_since_reset = torch.zeros(BB)
+    all_lprobs = torch.zeros(BB, max_len, V, device=device) if need_logprobs else None
     if return_step_logits:
         step_logits.append(logits.clone())
     preds = logits.float()
     if temperature > 0 and temperature != 1.0:
         preds = preds / temperature
     lprobs = F.log_softmax(preds, dim=-1, dtype=torch.float32)  # :240
+    if all_lprobs is not None:
+        all_lprobs[:, 1:start_step] = lprobs[:, :-1]  # :247-250
     prompt_tokens = tokens[:, 1:start_step].unsqueeze(-1)
     scores[:, 1:start_step] = torch.gather(lprobs, -1, prompt_tokens).squeeze(-1)  # :255-258
     cut = []
     for i in range(bsz):  # :262-267
         prompt_len = int(src_lengths[i])
-        scores[i, prompt_len + 1:] = 0.0
-        cut.append(lprobs[i:i + 1, prompt_len])
+        scores[i * beam_size:(i + 1) * beam_size, prompt_len + 1:] = 0.0
+        cut.append(lprobs[i * beam_size:(i + 1) * beam_size, prompt_len])
     lprobs = torch.cat(cut, dim=0)
-    eos_mask = torch.zeros(bsz, dtype=torch.bool, device=device)
+    eos_mask = torch.zeros(BB, dtype=torch.bool, device=device)
     for step in range(start_step, max_len):  # :271
         if step < min_len:
             lprobs[:, eos] = -math.inf
@@ -311,11 +392,25 @@ def greedy_generate(decoder, src_tokens: torch.Tensor, max_len_b: int, min_len: 
         if step >= max_len - 1:  # :282-284
             lprobs[:, :eos] = -math.inf
             lprobs[:, eos + 1:] = -math.inf
+        lprobs = apply_repetition_penalties(lprobs, count_tokens, count_tokens_src,
+                                            alpha_presence, alpha_frequency, alpha_presence_src,
+                                            alpha_frequency_src)  # :287-289
         lprobs[eos_mask, :eos] = -math.inf  # :292-293
         lprobs[eos_mask, eos + 1:] = -math.inf
-        next_scores, next_toks = lprobs.max(dim=-1)  # :413-415
+        if greedy:
+            next_scores, next_toks = lprobs.max(dim=-1)  # :413-415
+        else:
+            p = topp if lambda_decay <= 0 else topp_rows.unsqueeze(1)
+            next_scores, next_toks, _, _ = sample_topp(lprobs, p, generator)
+            if lambda_decay > 0:
+                topp_rows = update_sampling_topp(next_toks, toks_since_reset, init_p,
+                                                 list(full_stop_list), lambda_decay, omega_bound)
+        if count_tokens is not None:  # :525-534
+            count_tokens[torch.arange(BB, device=device), next_toks] += 1
         tokens[:, step] = next_toks
         scores[:, step] = next_scores
+        if all_lprobs is not None:
+            all_lprobs[:, step] = lprobs
         eos_mask |= next_toks == eos
         for t in stop:
             eos_mask |= next_toks == t
@@ -328,7 +423,22 @@ def greedy_generate(decoder, src_tokens: torch.Tensor, max_len_b: int, min_len: 
         if temperature > 0 and temperature != 1.0:
             preds = preds / temperature
         lprobs = F.log_softmax(preds, dim=-1, dtype=torch.float32)[:, -1, :]
-    out = {"tokens": tokens.view(bsz, 1, -1), "scores": scores.view(bsz, 1, -1)}
+    beamscores = scores.view(bsz, beam_size, -1).cumsum(dim=-1)[:, :, -1]  # :326-333
+    indices = beamscores.sort(dim=-1, descending=True).indices
+    order = (indices + beam_size * torch.arange(bsz, device=device).unsqueeze(1)).view(-1)
+    out = {"tokens": tokens[order].view(bsz, beam_size, -1),
+           "scores": scores[order].view(bsz, beam_size, -1)}
+    if all_lprobs is not None:
+        out["distributions"] = all_lprobs[order].view(bsz, beam_size, -1, V)
     if return_step_logits:
         out["step_logits"] = step_logits
     return out
+
+
+def greedy_generate(decoder, src_tokens: torch.Tensor, max_len_b: int, min_len: int = 1,
+                    pad: int = 1, eos: int = 2, stop: Optional[List[int]] = None,
+                    temperature: float = 1.0, max_positions: Optional[int] = None,
+                    return_step_logits: bool = False):
+    """``generate`` at beam 1 with greedy selection (metaseq/sequence_generator.py:413-415)."""
+    return generate(decoder, src_tokens, max_len_b, min_len, pad, eos, stop, temperature,
+                    max_positions, return_step_logits)

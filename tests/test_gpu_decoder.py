@@ -179,8 +179,6 @@ def test_errors_are_loud():
     model(torch.tensor([[2, 5, 6]], device=DEV), incremental_state=inc)
     with pytest.raises(AssertionError):
         model.decoder(torch.tensor([[2, 5, 6, 7, 8]], device=DEV), incremental_state=inc)
-    with pytest.raises(NotImplementedError):
-        SequenceGenerator([model], Dictionary(64), topp=0.9)
     with pytest.raises(IndexError):
         SequenceGenerator([model], Dictionary(64), max_len_b=8).generate(
             [model], {"net_input": {"src_tokens": torch.tensor([[5, 6, 7]], device=DEV)}})
