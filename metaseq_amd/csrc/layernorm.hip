@@ -10,6 +10,10 @@ namespace {
 constexpr int LN_THREADS = 512;
 constexpr int LN_MAX_CHUNKS = 4;  // 8 halves per chunk per thread -> D <= 512*8*4 = 16384
 
+// ST > 0: the number of split-K slices is the compile-time constant ST, so that all slice loads
+// of a chunk are issued back to back (a run-time trip count makes them one round trip each);
+// ST == 0: any S.
+template <int ST>
 __global__ __launch_bounds__(LN_THREADS) void layernorm_f16_kernel(
     const half_t* x, const float* __restrict__ part, int S,
     const half_t* __restrict__ bias, half_t* x_out, const half_t* __restrict__ gamma,
@@ -37,18 +41,34 @@ __global__ __launch_bounds__(LN_THREADS) void layernorm_f16_kernel(
     if (idx < nchunk) {
       if (part) {
         // x_out = round(round(round(sum_s part) + bias) + x): the fp16 rounding points of
-        // "linear, + bias, + residual" in the reference layer
+        // "linear, + bias, + residual" in the reference layer; slices are summed in order
         const float* p = part + (int64_t)row * D + (idx << 3);
-        float4_t a0 = *reinterpret_cast<const float4_t*>(p);
-        float4_t a1 = *reinterpret_cast<const float4_t*>(p + 4);
-#pragma unroll 4
-        for (int i = 1; i < S; ++i) {
-          const float* q = p + (int64_t)i * M * D;
-          a0 += *reinterpret_cast<const float4_t*>(q);
-          a1 += *reinterpret_cast<const float4_t*>(q + 4);
-        }
+        const int64_t slice = (int64_t)M * D;
         const half8_t b = *reinterpret_cast<const half8_t*>(bias + (idx << 3));
         const half8_t r = *reinterpret_cast<const half8_t*>(x + (int64_t)row * D + (idx << 3));
+        float4_t a0, a1;
+        if (ST > 0) {
+          float4_t t0[ST > 0 ? ST : 1], t1[ST > 0 ? ST : 1];
+#pragma unroll
+          for (int i = 0; i < ST; ++i) {
+            t0[i] = *reinterpret_cast<const float4_t*>(p + i * slice);
+            t1[i] = *reinterpret_cast<const float4_t*>(p + i * slice + 4);
+          }
+          a0 = t0[0];
+          a1 = t1[0];
+#pragma unroll
+          for (int i = 1; i < ST; ++i) {
+            a0 += t0[i];
+            a1 += t1[i];
+          }
+        } else {
+          a0 = *reinterpret_cast<const float4_t*>(p);
+          a1 = *reinterpret_cast<const float4_t*>(p + 4);
+          for (int i = 1; i < S; ++i) {
+            a0 += *reinterpret_cast<const float4_t*>(p + i * slice);
+            a1 += *reinterpret_cast<const float4_t*>(p + i * slice + 4);
+          }
+        }
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
           float t = round_h(i < 4 ? a0[i] : a1[i - 4]);
@@ -117,7 +137,7 @@ extern "C" int msa_layernorm_f16(const void* x, const void* gamma, const void* b
   if (rc) return rc;
   if (rows == 0) return MSA_OK;
   const int out_mb = (flags & MSA_OUT_PACKED) ? (int)((rows + 15) / 16) : 0;
-  hipLaunchKernelGGL(layernorm_f16_kernel, dim3((unsigned)rows), dim3(LN_THREADS), 0,
+  hipLaunchKernelGGL(layernorm_f16_kernel<0>, dim3((unsigned)rows), dim3(LN_THREADS), 0,
                      (hipStream_t)stream, (const half_t*)x, (const float*)nullptr, 0,
                      (const half_t*)nullptr, (half_t*)nullptr, (const half_t*)gamma,
                      (const half_t*)beta, (half_t*)y, (int)rows, D, eps, out_mb);
@@ -138,10 +158,15 @@ extern "C" int msa_residual_layernorm_f16(const float* part, int S, const void* 
   if (rc) return rc;
   if (rows == 0) return MSA_OK;
   const int out_mb = (flags & MSA_OUT_PACKED) ? (int)((rows + 15) / 16) : 0;
-  hipLaunchKernelGGL(layernorm_f16_kernel, dim3((unsigned)rows), dim3(LN_THREADS), 0,
-                     (hipStream_t)stream, (const half_t*)x, part, S, (const half_t*)bias,
-                     (half_t*)x, (const half_t*)gamma, (const half_t*)beta, (half_t*)y, (int)rows,
-                     D, eps, out_mb);
+  auto kernel = S == 1   ? layernorm_f16_kernel<1>
+                : S == 2 ? layernorm_f16_kernel<2>
+                : S == 4 ? layernorm_f16_kernel<4>
+                : S == 8 ? layernorm_f16_kernel<8>
+                         : layernorm_f16_kernel<0>;
+  hipLaunchKernelGGL(kernel, dim3((unsigned)rows), dim3(LN_THREADS), 0, (hipStream_t)stream,
+                     (const half_t*)x, part, S, (const half_t*)bias, (half_t*)x,
+                     (const half_t*)gamma, (const half_t*)beta, (half_t*)y, (int)rows, D, eps,
+                     out_mb);
   MSA_CHECK_LAUNCH("msa_residual_layernorm_f16");
   return MSA_OK;
 }
