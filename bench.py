@@ -118,7 +118,9 @@ def cpu_baseline(size, B, S, seed=1234):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=128)
+    ap.add_argument("--steps", type=int, default=None,
+                    help="timed decode steps (default: the workload's generation length minus "
+                         "the warm-up steps, so warm-up + timed = the configured decode length)")
     ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--config", default="6.7b", choices=sorted(CONFIGS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -145,7 +147,8 @@ def main():
 
     size, B, P, G = CONFIGS[args.config]
     int8 = args.config.endswith("int8")
-    K, W = args.steps, args.warmup
+    W = args.warmup
+    K = args.steps if args.steps is not None else max(1, G - W)
     total_gen = max(G, K + W + 1)
     n0 = P + 1
     max_len = n0 + total_gen + 1

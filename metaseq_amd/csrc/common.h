@@ -52,16 +52,36 @@ __host__ __device__ __forceinline__ int64_t packed_act_offset(int m, int k, int 
 // round-to-nearest-even fp32 -> fp16 -> fp32 (a "materialise in fp16" point)
 __device__ __forceinline__ float round_h(float v) { return (float)(half_t)v; }
 
+// Cross-lane step of the wave reductions on the data-parallel-primitive path of the vector ALU
+// (no LDS round trip).  Lanes of a row that ROW_MASK leaves out receive `old`.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float dpp_move(float old, float v) {
+  return __builtin_bit_cast(
+      float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, old), __builtin_bit_cast(int, v),
+                                         CTRL, ROW_MASK, 0xf, false));
+}
+
+// Reductions over the 64 lanes of a wave; every lane gets the result.  Order: pairs, quads,
+// rows of 16 (two rotations), then the row totals are chained into lane 63 and broadcast.
+// All 64 lanes must be active.
 __device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, MSA_WAVE);
-  return v;
+  v += dpp_move<0xB1, 0xf>(0.f, v);   // quad_perm [1,0,3,2]
+  v += dpp_move<0x4E, 0xf>(0.f, v);   // quad_perm [2,3,0,1]
+  v += dpp_move<0x124, 0xf>(0.f, v);  // row_ror:4
+  v += dpp_move<0x128, 0xf>(0.f, v);  // row_ror:8
+  v += dpp_move<0x142, 0xa>(0.f, v);  // row_bcast15 into rows 1 and 3
+  v += dpp_move<0x143, 0xc>(0.f, v);  // row_bcast31 into rows 2 and 3
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
 }
 
 __device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, MSA_WAVE));
-  return v;
+  v = fmaxf(v, dpp_move<0xB1, 0xf>(-INFINITY, v));
+  v = fmaxf(v, dpp_move<0x4E, 0xf>(-INFINITY, v));
+  v = fmaxf(v, dpp_move<0x124, 0xf>(-INFINITY, v));
+  v = fmaxf(v, dpp_move<0x128, 0xf>(-INFINITY, v));
+  v = fmaxf(v, dpp_move<0x142, 0xa>(-INFINITY, v));
+  v = fmaxf(v, dpp_move<0x143, 0xc>(-INFINITY, v));
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
 }
 
 // Block-wide reductions for blocks of up to 16 waves; `red` is >= 16 floats of LDS.
@@ -72,8 +92,13 @@ __device__ __forceinline__ float block_sum(float v, float* red) {
   __syncthreads();
   if (lane == 0) red[wave] = v;
   __syncthreads();
+  // all 16 slots are read at once (slots past nw hold stale values and are not added)
   float t = 0.f;
-  for (int i = 0; i < nw; ++i) t += red[i];
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    const float r = red[i];
+    t += i < nw ? r : 0.f;
+  }
   return t;
 }
 
@@ -84,6 +109,10 @@ __device__ __forceinline__ float block_max(float v, float* red) {
   if (lane == 0) red[wave] = v;
   __syncthreads();
   float t = red[0];
-  for (int i = 1; i < nw; ++i) t = fmaxf(t, red[i]);
+#pragma unroll
+  for (int i = 1; i < 16; ++i) {
+    const float r = red[i];
+    t = fmaxf(t, i < nw ? r : t);
+  }
   return t;
 }

@@ -106,23 +106,32 @@ __global__ __launch_bounds__(SM_THREADS) void greedy_select_kernel(
   };
   if ((reinterpret_cast<uintptr_t>(row) & 15) == 0) {
     const int nv = V >> 3;
-    for (int c = threadIdx.x; c < nv; c += blockDim.x) {
-      const half8_t v = *reinterpret_cast<const half8_t*>(row + (c << 3));
-      float z[8], cm = -INFINITY;
+    constexpr int UNR = 4;  // chunks requested together: one memory round trip per UNR chunks
+    for (int c0 = threadIdx.x; c0 < nv; c0 += blockDim.x * UNR) {
+      half8_t vv[UNR];
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        z[i] = (float)v[i];
-        if (scale) z[i] = z[i] / temperature;
-        cm = fmaxf(cm, z[i]);
-        visit((c << 3) + i, z[i]);
-      }
-      if (cm > m) {  // rescale once per 8 ids
-        s *= __expf(m - cm);
-        m = cm;
-      }
-      if (m > -INFINITY) {
+      for (int u = 0; u < UNR; ++u)
+        vv[u] = *reinterpret_cast<const half8_t*>(row + (min(c0 + u * (int)blockDim.x, nv - 1) << 3));
 #pragma unroll
-        for (int i = 0; i < 8; ++i) s += __expf(z[i] - m);
+      for (int u = 0; u < UNR; ++u) {
+        const int c = c0 + u * blockDim.x;
+        if (c >= nv) break;
+        float z[8], cm = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          z[i] = (float)vv[u][i];
+          if (scale) z[i] = z[i] / temperature;
+          cm = fmaxf(cm, z[i]);
+          visit((c << 3) + i, z[i]);
+        }
+        if (cm > m) {  // rescale once per 8 ids
+          s *= __expf(m - cm);
+          m = cm;
+        }
+        if (m > -INFINITY) {
+#pragma unroll
+          for (int i = 0; i < 8; ++i) s += __expf(z[i] - m);
+        }
       }
     }
     for (int i = (nv << 3) + threadIdx.x; i < V; i += blockDim.x) {
