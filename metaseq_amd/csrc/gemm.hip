@@ -18,7 +18,6 @@
 // Both share one epilogue that reproduces the reference's fp16 rounding points, and a QKV mode
 // that scatters K/V into the per-layer cache and scales Q.
 #include <math.h>
-#include <stdlib.h>
 
 #include "common.h"
 
@@ -163,11 +162,15 @@ __global__ __launch_bounds__(256) void pack_i8_kernel(const int8_t* __restrict__
 constexpr int ST_KG = 8;  // waves per workgroup = interleaved K lanes
 constexpr int ST_NT = 4;  // weight tiles sharing one activation fragment
 
-template <int MB, bool W8, int MODE, int KG = ST_KG, int NT = ST_NT, int U = (MB <= 2 ? 4 : 2)>
+// XR: the activations are row-major ([rows, K], fragments gathered 16 bytes per lane) instead
+// of packed; the kernel then handles rows m_off .. m_off + M - 1 of a taller matrix (the ragged
+// bottom of a prefill-sized product) and the epilogue sees the global row numbers.
+template <int MB, bool W8, int MODE, bool XR = false, int KG = ST_KG, int NT = ST_NT,
+          int U = (MB <= 2 ? 4 : 2)>
 __global__ __launch_bounds__(KG * 64) void linear_stream_kernel(
     const half_t* __restrict__ xp, const void* __restrict__ Wp, const half_t* __restrict__ scales,
     float* __restrict__ part, int M, int N, int K, int tiles_per_wg, int ks_per_split,
-    Epilogue epi) {
+    Epilogue epi, int64_t m_off) {
   // U = K steps (32 wide) buffered per stage; an int8 block covers two steps
   constexpr int UA = W8 ? U / 2 : U;  // weight loads per stage and tile
   __shared__ float4_t red[KG][NT * MB][64];
@@ -212,9 +215,16 @@ __global__ __launch_bounds__(KG * 64) void linear_stream_kernel(
       for (int h = 0; h < (W8 ? 2 : 1); ++h) {
         const int kk = min(ks + h, ks_end - 1);
 #pragma unroll
-        for (int mb = 0; mb < MB; ++mb)
-          s.b[W8 ? 2 * u + h : u][mb] =
-              *reinterpret_cast<const half8_t*>(xp + (((int64_t)kk * MB + mb) * 64 + lane) * 8);
+        for (int mb = 0; mb < MB; ++mb) {
+          if (XR) {
+            const int64_t m = m_off + min(mb * 16 + (lane & 15), M - 1);
+            s.b[W8 ? 2 * u + h : u][mb] = *reinterpret_cast<const half8_t*>(
+                xp + m * K + kk * 32 + (lane >> 4) * 8);
+          } else {
+            s.b[W8 ? 2 * u + h : u][mb] = *reinterpret_cast<const half8_t*>(
+                xp + (((int64_t)kk * MB + mb) * 64 + lane) * 8);
+          }
+        }
       }
     }
   };
@@ -288,7 +298,7 @@ __global__ __launch_bounds__(KG * 64) void linear_stream_kernel(
         if (part)
           *reinterpret_cast<float4_t*>(part + ((int64_t)blockIdx.y * M + m) * N + n) = sum;
         else
-          epilogue4<MODE>(epi, m, n, sum);
+          epilogue4<MODE>(epi, m_off + m, n, sum);
       }
     }
     __syncthreads();
@@ -621,9 +631,9 @@ int num_cus() {
   return g_num_cus;
 }
 
-template <int MB, bool W8, int MODE>
+template <int MB, bool W8, int MODE, bool XR = false>
 void launch_stream_mb(const void* xp, const void* W, const void* scales, float* part, int S, int M,
-                      int N, int K, const Epilogue& epi, hipStream_t s) {
+                      int N, int K, const Epilogue& epi, hipStream_t s, int64_t m_off = 0) {
   const int ntiles = N / 16, nks = K / 32;
   int G = num_cus() / S;
   if (G < 1) G = 1;
@@ -631,19 +641,27 @@ void launch_stream_mb(const void* xp, const void* W, const void* scales, float* 
   const int gx = (ntiles + tiles_per_wg - 1) / tiles_per_wg;
   int ks_per_split = (nks + S - 1) / S;
   if (W8) ks_per_split = (ks_per_split + 1) & ~1;  // int8 blocks cover two steps
-  hipLaunchKernelGGL((linear_stream_kernel<MB, W8, MODE>), dim3(gx, S), dim3(ST_KG * 64), 0, s,
-                     (const half_t*)xp, W, (const half_t*)scales, part, M, N, K, tiles_per_wg,
-                     ks_per_split, epi);
+  hipLaunchKernelGGL((linear_stream_kernel<MB, W8, MODE, XR>), dim3(gx, S), dim3(ST_KG * 64), 0,
+                     s, (const half_t*)xp, W, (const half_t*)scales, part, M, N, K, tiles_per_wg,
+                     ks_per_split, epi, m_off);
 }
 
-template <bool W8, int MODE>
+template <bool W8, int MODE, bool XR = false>
 void launch_stream(const void* xp, const void* W, const void* scales, float* part, int S, int M,
-                   int N, int K, const Epilogue& epi, hipStream_t s) {
+                   int N, int K, const Epilogue& epi, hipStream_t s, int64_t m_off = 0) {
   switch ((M + 15) / 16) {
-    case 1: launch_stream_mb<1, W8, MODE>(xp, W, scales, part, S, M, N, K, epi, s); break;
-    case 2: launch_stream_mb<2, W8, MODE>(xp, W, scales, part, S, M, N, K, epi, s); break;
-    case 3: launch_stream_mb<3, W8, MODE>(xp, W, scales, part, S, M, N, K, epi, s); break;
-    default: launch_stream_mb<4, W8, MODE>(xp, W, scales, part, S, M, N, K, epi, s); break;
+    case 1:
+      launch_stream_mb<1, W8, MODE, XR>(xp, W, scales, part, S, M, N, K, epi, s, m_off);
+      break;
+    case 2:
+      launch_stream_mb<2, W8, MODE, XR>(xp, W, scales, part, S, M, N, K, epi, s, m_off);
+      break;
+    case 3:
+      launch_stream_mb<3, W8, MODE, XR>(xp, W, scales, part, S, M, N, K, epi, s, m_off);
+      break;
+    default:
+      launch_stream_mb<4, W8, MODE, XR>(xp, W, scales, part, S, M, N, K, epi, s, m_off);
+      break;
   }
 }
 
@@ -652,7 +670,7 @@ void launch_tiled(const void* x, const void* W, const void* scales, int64_t M, i
                   const Epilogue& epi, hipStream_t s) {
   // the 256 x 256 kernel once it fills the chip; the 128 x 128 one for the shapes in between
   const int64_t big_tiles = ((M + TB_BM - 1) / TB_BM) * ((N + TB_BN - 1) / TB_BN);
-  if (K % (2 * TB_BK) == 0 && big_tiles >= num_cus() && !getenv("MSA_NO_BIG")) {
+  if (K % (2 * TB_BK) == 0 && big_tiles >= num_cus()) {
     static bool attr_set = false;  // one flag per instantiation
     if (!attr_set) {
       if (hipFuncSetAttribute((const void*)linear_tiled_big_kernel<W8, MODE>,
@@ -661,9 +679,18 @@ void launch_tiled(const void* x, const void* W, const void* scales, int64_t M, i
         return;  // the launch check below reports the error
       attr_set = true;
     }
-    const dim3 grid((N + TB_BN - 1) / TB_BN, (unsigned)((M + TB_BM - 1) / TB_BM));
+    // A ragged bottom block would cost a full extra round of workgroups for a few rows (a
+    // prompt of 2^k tokens plus the leading end-of-sentence token always has one): up to 128
+    // leftover rows go through the weight-streaming kernel instead, 64 rows at a time.
+    int64_t M_main = M;
+    const int64_t rem = M % TB_BM;
+    if (rem > 0 && rem <= 128 && M > rem) M_main = M - rem;
+    const dim3 grid((N + TB_BN - 1) / TB_BN, (unsigned)((M_main + TB_BM - 1) / TB_BM));
     hipLaunchKernelGGL((linear_tiled_big_kernel<W8, MODE>), grid, dim3(TB_THREADS), TB_LDS_BYTES,
-                       s, (const half_t*)x, W, (const half_t*)scales, M, N, K, epi);
+                       s, (const half_t*)x, W, (const half_t*)scales, M_main, N, K, epi);
+    for (int64_t m0 = M_main; m0 < M; m0 += 64)
+      launch_stream<W8, MODE, true>(x, W, scales, nullptr, 1, (int)min((int64_t)64, M - m0), N, K,
+                                    epi, s, m0);
     return;
   }
   const dim3 grid((N + TL_BN - 1) / TL_BN, (unsigned)((M + TL_BM - 1) / TL_BM));

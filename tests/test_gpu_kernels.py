@@ -234,8 +234,9 @@ LINEAR_SHAPES = [
     (1, 96, 64), (8, 768, 768), (32, 3072, 768), (32, 768, 3072), (33, 2048, 2048),
     (64, 4096, 4096), (17, 50272, 768), (65, 768, 768), (200, 2304, 768), (513, 4096, 1024),
     (129, 1008, 96),
-    # enough 256 x 256 tiles to take the large tiled kernel, with ragged M and N edges
-    (1000, 16400, 128), (4099, 4096, 256),
+    # enough 256 x 256 tiles to take the large tiled kernel, with ragged M and N edges; a bottom
+    # block of at most 128 rows goes through the streaming kernel on row-major activations
+    (1000, 16400, 128), (4099, 4096, 256), (1124, 16400, 128),
 ]
 
 
@@ -313,7 +314,7 @@ def test_linear_rejects_bad_shapes(lib):
 
 @pytest.mark.parametrize("M,N,K", [(8, 768, 768), (64, 3072, 768), (32, 768, 3072),
                                    (200, 2304, 768), (48, 4096, 4096),
-                                   (1000, 16400, 128)])   # the last: large tiled kernel
+                                   (1000, 16400, 128), (1124, 16400, 128)])   # large tiled kernel
 def test_linear_w8a16(lib, M, N, K):
     print("w8a16", M, N, K, flush=True)
     x, W, b = rnd(M, K, seed=7), rnd(N, K, seed=8, std=0.02), rnd(N, seed=9, std=0.1)
@@ -431,7 +432,7 @@ def test_qkv_proj_scatter(lib, B, T, H, hd, S0, w8):
 def test_qkv_proj_scatter_large_tiled_kernel(lib, w8):
     """A prefill-sized QKV projection (enough 256 x 256 tiles for the large tiled kernel): the
     scatter into the cache and the q scaling, with an input width independent of H * hd."""
-    B, T, H, hd, S0, K = 2, 1100, 20, 128, 3, 256
+    B, T, H, hd, S0, K = 2, 1057, 20, 128, 3, 256   # 2114 rows = 8 * 256 + 66
     D, S_cap = H * hd, S0 + T + 2
     x, W, b = rnd(B * T, K, seed=1), rnd(3 * D, K, seed=2, std=0.05), rnd(3 * D, seed=3, std=0.1)
     if w8:
