@@ -13,8 +13,11 @@ constexpr int LN_MAX_CHUNKS = 4;  // 8 halves per chunk per thread -> D <= 512*8
 // ST > 0: the number of split-K slices is the compile-time constant ST, so that all slice loads
 // of a chunk are issued back to back (a run-time trip count makes them one round trip each);
 // ST == 0: any S.
-template <int ST>
-__global__ __launch_bounds__(LN_THREADS) void layernorm_f16_kernel(
+// THREADS: workgroup size; a row of D elements needs D / 8 <= THREADS * LN_MAX_CHUNKS.  Decode
+// (a few rows) uses wide workgroups to shorten the dependent chain, prefill (thousands of
+// rows) narrow ones so that several rows share a compute unit.
+template <int ST, int THREADS = LN_THREADS>
+__global__ __launch_bounds__(THREADS) void layernorm_f16_kernel(
     const half_t* x, const float* __restrict__ part, int S,
     const half_t* __restrict__ bias, half_t* x_out, const half_t* __restrict__ gamma,
     const half_t* __restrict__ beta, half_t* __restrict__ y, int M, int D, float eps, int out_mb) {
@@ -28,7 +31,7 @@ __global__ __launch_bounds__(LN_THREADS) void layernorm_f16_kernel(
   if (gamma) {
 #pragma unroll
     for (int c = 0; c < LN_MAX_CHUNKS; ++c) {
-      const int idx = threadIdx.x + c * LN_THREADS;
+      const int idx = threadIdx.x + c * THREADS;
       if (idx < nchunk) {
         gv[c] = *reinterpret_cast<const half8_t*>(gamma + (idx << 3));
         bv[c] = *reinterpret_cast<const half8_t*>(beta + (idx << 3));
@@ -37,7 +40,7 @@ __global__ __launch_bounds__(LN_THREADS) void layernorm_f16_kernel(
   }
 #pragma unroll
   for (int c = 0; c < LN_MAX_CHUNKS; ++c) {
-    const int idx = threadIdx.x + c * LN_THREADS;
+    const int idx = threadIdx.x + c * THREADS;
     if (idx < nchunk) {
       if (part) {
         // x_out = round(round(round(sum_s part) + bias) + x): the fp16 rounding points of
@@ -88,7 +91,7 @@ __global__ __launch_bounds__(LN_THREADS) void layernorm_f16_kernel(
   float q = 0.f;
 #pragma unroll
   for (int c = 0; c < LN_MAX_CHUNKS; ++c) {
-    const int idx = threadIdx.x + c * LN_THREADS;
+    const int idx = threadIdx.x + c * THREADS;
     if (idx < nchunk) {
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
@@ -101,7 +104,7 @@ __global__ __launch_bounds__(LN_THREADS) void layernorm_f16_kernel(
   const float rstd = rsqrtf(var + eps);
 #pragma unroll
   for (int c = 0; c < LN_MAX_CHUNKS; ++c) {
-    const int idx = threadIdx.x + c * LN_THREADS;
+    const int idx = threadIdx.x + c * THREADS;
     if (idx < nchunk) {
       half8_t o;
 #pragma unroll
@@ -137,10 +140,17 @@ extern "C" int msa_layernorm_f16(const void* x, const void* gamma, const void* b
   if (rc) return rc;
   if (rows == 0) return MSA_OK;
   const int out_mb = (flags & MSA_OUT_PACKED) ? (int)((rows + 15) / 16) : 0;
-  hipLaunchKernelGGL(layernorm_f16_kernel<0>, dim3((unsigned)rows), dim3(LN_THREADS), 0,
-                     (hipStream_t)stream, (const half_t*)x, (const float*)nullptr, 0,
-                     (const half_t*)nullptr, (half_t*)nullptr, (const half_t*)gamma,
-                     (const half_t*)beta, (half_t*)y, (int)rows, D, eps, out_mb);
+  // many rows: the narrowest workgroup that covers the row
+  const int threads = rows <= 64 || D > 256 * 8 * LN_MAX_CHUNKS ? LN_THREADS
+                      : D > 128 * 8 * LN_MAX_CHUNKS             ? 256
+                                                                : 128;
+  auto kernel = threads == LN_THREADS ? layernorm_f16_kernel<0, LN_THREADS>
+                : threads == 256      ? layernorm_f16_kernel<0, 256>
+                                      : layernorm_f16_kernel<0, 128>;
+  hipLaunchKernelGGL(kernel, dim3((unsigned)rows), dim3(threads), 0, (hipStream_t)stream,
+                     (const half_t*)x, (const float*)nullptr, 0, (const half_t*)nullptr,
+                     (half_t*)nullptr, (const half_t*)gamma, (const half_t*)beta, (half_t*)y,
+                     (int)rows, D, eps, out_mb);
   MSA_CHECK_LAUNCH("msa_layernorm_f16");
   return MSA_OK;
 }
