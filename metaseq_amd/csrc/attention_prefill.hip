@@ -35,7 +35,8 @@ __global__ __launch_bounds__(PF_THREADS) void prefill_attention_kernel(
   __shared__ __attribute__((aligned(16))) half_t lk[PF_BN * KLD];
   __shared__ __attribute__((aligned(16))) uint32_t lv[(PF_BN / 2) * VLD];
 
-  const int bh = blockIdx.x, qt = blockIdx.y;
+  // query tiles are issued last-first: the tiles with the most keys start earliest
+  const int bh = blockIdx.x, qt = gridDim.y - 1 - blockIdx.y;
   const int b = bh / H, h = bh - b * H;
   const int D = H * HD;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -147,7 +148,7 @@ __global__ __launch_bounds__(PF_THREADS) void prefill_attention_kernel(
     __syncthreads();  // previous tile fully consumed
     store_k();
     __syncthreads();
-    if (tile + 1 < ntiles) load_k(tile + 1);
+    if (tile + 1 < ntiles) load_k(tile + 1);  // the branch also pins the loads ahead of the MFMAs
     scores(tile);
     float tm = -INFINITY;
 #pragma unroll
@@ -161,7 +162,7 @@ __global__ __launch_bounds__(PF_THREADS) void prefill_attention_kernel(
 #pragma unroll
       for (int ib = 0; ib < 2; ++ib)
 #pragma unroll
-        for (int v = 0; v < 16; ++v) ts += __expf(s[ib][v] - mn);
+        for (int v = 0; v < 16; ++v) ts += __expf(s[ib][v] - mn);  // -inf - finite = -inf -> 0
       ts += __shfl_xor(ts, 32, MSA_WAVE);
       l = l * __expf(m - mn) + ts;
       m = mn;
