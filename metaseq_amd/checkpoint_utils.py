@@ -1,0 +1,135 @@
+"""State-dict level ingest of the reference's checkpoints: gluing the tensor-parallel parts of
+a `reshard-model_part-{r}.pt` set into the single-part state dict this decoder loads, the
+inverse split, and key normalisation.
+
+Gluing rules (metaseq/distributed/stitch_fsdp_ckpt.py:203-214, 246-339):
+* `qkv_proj` weight and bias: every part holds its own heads as local thirds K_r | V_r | Q_r;
+  the glued tensor is cat(K_r) | cat(V_r) | cat(Q_r).  (The reference's singleton form splits
+  these into k_proj / v_proj / q_proj; this decoder keeps the fused K | V | Q rows.)
+* column-parallel `fc1` (weight and bias) and the token embedding: concatenated along dim 0;
+* row-parallel `fc2` / `out_proj` weights: concatenated along dim 1, their biases replicated;
+* LayerNorms, positional table, everything else: replicated (taken from part 0 after checking
+  that the parts agree).
+
+Only tensors are read from files: `torch.load(..., weights_only=True)` executes nothing from the
+pickle, so a file whose "cfg" entry holds arbitrary Python objects is refused by the loader;
+re-save such a file as {"model": state_dict} with the reference's own tools first.
+"""
+import re
+from collections import OrderedDict
+from typing import Dict, List
+
+import torch
+
+_DROP = ("decoder.output_projection.weight",)
+
+
+def _agree(parts, key):
+    ref = parts[0][key]
+    for p in parts[1:]:
+        if p[key].shape != ref.shape or not torch.equal(p[key], ref):
+            raise ValueError("replicated parameter %s differs between model parts" % key)
+    return ref.clone()
+
+
+def glue_model_parts(parts: List[Dict[str, torch.Tensor]]) -> "OrderedDict[str, torch.Tensor]":
+    """Tensor-parallel parts (rank order) -> one state dict with fused K | V | Q rows."""
+    if not parts:
+        raise ValueError("no model parts")
+    keys = list(parts[0].keys())
+    for p in parts[1:]:
+        if list(p.keys()) != keys:
+            raise ValueError("model parts hold different parameter names")
+    out = OrderedDict()
+    for key in keys:
+        ts = [p[key] for p in parts]
+        if "qkv" in key:
+            thirds = [t.split(t.shape[0] // 3, dim=0) for t in ts]
+            out[key] = torch.cat([torch.cat([th[j] for th in thirds], dim=0) for j in range(3)],
+                                 dim=0)
+        elif "layer_norm" in key:
+            out[key] = _agree(parts, key)
+        elif "fc1" in key or re.search(r"\.(k|v|q)_proj\.", key):
+            out[key] = torch.cat(ts, dim=0)
+        elif "fc2" in key or "out_proj" in key:
+            out[key] = _agree(parts, key) if key.endswith("bias") else torch.cat(ts, dim=1)
+        elif "embed_tokens.weight" in key:
+            out[key] = torch.cat(ts, dim=0)
+        elif "_float_tensor" in key or "version" in key:
+            out[key] = ts[0].clone()
+        else:
+            out[key] = _agree(parts, key)
+    return out
+
+
+def split_model_parts(state: Dict[str, torch.Tensor], n: int) -> List["OrderedDict[str, torch.Tensor]"]:
+    """Inverse of glue_model_parts: the parts `n` tensor-parallel ranks would hold."""
+    parts = [OrderedDict() for _ in range(n)]
+    for key, t in state.items():
+        if "qkv" in key:
+            thirds = [th.chunk(n, dim=0) for th in t.split(t.shape[0] // 3, dim=0)]
+            for r in range(n):
+                parts[r][key] = torch.cat([thirds[j][r] for j in range(3)], dim=0).clone()
+        elif "layer_norm" in key:
+            for r in range(n):
+                parts[r][key] = t.clone()
+        elif "fc1" in key or "embed_tokens.weight" in key or re.search(r"\.(k|v|q)_proj\.", key):
+            for r, c in enumerate(t.chunk(n, dim=0)):
+                parts[r][key] = c.clone()
+        elif ("fc2" in key or "out_proj" in key) and key.endswith("weight"):
+            for r, c in enumerate(t.chunk(n, dim=1)):
+                parts[r][key] = c.clone()
+        else:
+            for r in range(n):
+                parts[r][key] = t.clone()
+    return parts
+
+
+def normalize_state_dict(state: Dict[str, torch.Tensor]) -> "OrderedDict[str, torch.Tensor]":
+    """Drops what the decoder re-creates itself (the tied `decoder.output_projection.weight`:
+    metaseq/checkpoint_utils.py:599-602, scripts/convert_to_singleton.py:160-166; sinusoidal
+    `_float_tensor` buffers) and fuses a
+    singleton checkpoint's k_proj / v_proj / q_proj back into `qkv_proj` rows K | V | Q."""
+    out = OrderedDict()
+    for key, t in state.items():
+        if key in _DROP or key.endswith("_float_tensor"):
+            continue
+        m = re.match(r"(.*\.self_attn\.)k_proj\.(weight|bias)$", key)
+        if m:
+            pre, kind = m.groups()
+            out[pre + "qkv_proj." + kind] = torch.cat(
+                [state[pre + "%s_proj.%s" % (n, kind)] for n in "kvq"], dim=0)
+            continue
+        if re.match(r".*\.self_attn\.(v|q)_proj\.(weight|bias)$", key):
+            continue
+        out[key] = t
+    return out
+
+
+def load_model_state(paths: List[str]) -> "OrderedDict[str, torch.Tensor]":
+    """Reads the tensor-parallel parts of one checkpoint (paths in rank order, e.g.
+    reshard-model_part-0.pt, reshard-model_part-1.pt), glues and normalises them.  Each file is
+    either a bare state dict or {"model": state_dict, ...} (metaseq/checkpoint_utils.py:540-557)."""
+    parts = []
+    for path in paths:
+        obj = torch.load(path, map_location="cpu", weights_only=True)
+        if isinstance(obj, dict) and "model" in obj and isinstance(obj["model"], dict):
+            obj = obj["model"]
+        if not isinstance(obj, dict) or not all(torch.is_tensor(v) for v in obj.values()):
+            raise ValueError("%s does not hold a state dict of tensors" % path)
+        parts.append(obj)
+    return normalize_state_dict(glue_model_parts(parts) if len(parts) > 1 else parts[0])
+
+
+def find_model_parts(names: List[str]) -> List[str]:
+    """Sorts file names of one checkpoint by their `-model_part-{r}` number
+    (metaseq/distributed/stitch_fsdp_ckpt.py:342-352) and checks that no rank is missing."""
+    numbered = []
+    for n in names:
+        m = re.search(r"-model_part-(\d+)", n)
+        if m is not None:
+            numbered.append((int(m.group(1)), n))
+    numbered.sort()
+    if [r for r, _ in numbered] != list(range(len(numbered))):
+        raise ValueError("model parts are not numbered 0..%d" % (len(numbered) - 1))
+    return [n for _, n in numbered]

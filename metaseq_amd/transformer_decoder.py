@@ -144,6 +144,9 @@ class TransformerDecoder(nn.Module):
         if any(k.startswith("decoder.") for k in sd):
             sd = {k[len("decoder."):]: v for k, v in sd.items() if k.startswith("decoder.")}
         sd.pop("output_projection.weight", None)
+        # the format marker is optional, as in the reference's upgrade_state_dict_named
+        # (metaseq/models/transformer_decoder.py:539-567)
+        sd.setdefault("version", torch.tensor([3.0]))
         for _, lin in self._linears():  # back to plain row-major parameters before loading
             if lin.packed or lin.qweight is not None:
                 lin.weight.data = torch.empty(lin.shape, dtype=torch.float16,
