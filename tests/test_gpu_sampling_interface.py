@@ -216,3 +216,18 @@ def test_fully_masked_step_does_not_reach_multinomial_with_nan():
     assert out["tokens"][:, 0, 7].tolist() == [0, 0]
     assert bool(torch.isinf(out["scores"][:, 0, 7]).all())
     assert bool(torch.isfinite(out["scores"][:, 0, :7]).all())
+
+
+def test_batching_service_over_the_interface_returns_what_direct_calls_return():
+    from metaseq_amd.service import BatchingService
+    gi, model, cfg, sd = _interface()
+    prompts = [[5, 9, 33, 12, 7], [40, 41], [8, 8, 8]]
+    svc = BatchingService(gi, max_seq_len=48, timeout_ms=5)
+    rets = [svc.submit(p, max_tokens=5, min_tokens=4, temperature=1.0, top_p=-1.0, n=1)
+            for p in prompts]
+    assert svc.step() == 3          # one padded batch for the three prompts
+    direct = gi.generate(prompts, max_tokens=[5] * 3, min_tokens=[4] * 3)
+    # the service hands prompts over cheapest first; every caller still gets its own row
+    for p, r, want in zip(prompts, rets, direct):
+        uid, got = r.get_nowait()
+        assert got[0]["tokens"] == want[0]["tokens"], p
