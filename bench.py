@@ -127,6 +127,9 @@ def main():
     ap.add_argument("--graph", action="store_true",
                     help="replay the captured decode-step hipGraph instead of launching every "
                          "kernel from Python (measured slower on this ROCm: 5.81 vs 5.66 ms/step)")
+    ap.add_argument("--unfused-select", action="store_true",
+                    help="store the logits and run the stand-alone selection kernel instead of "
+                         "selecting inside the vocabulary projection (for comparison)")
     ap.add_argument("--pmc-calibration", action="store_true",
                     help="also run a plain 1 GiB device copy, the known-size kernel that "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE readings are scaled by")
@@ -202,11 +205,27 @@ def main():
         st = gen.static_state(decoder, decoder.get_cache(inc), tokens, scores, finished,
                               step_logits)
 
+    min_len = max_len - 1
+    fused = st is None and B <= 64 and not args.unfused_select
+    if fused:
+        # the generator's fast path: the token at n0 comes from the prefill logits, every later
+        # one is chosen inside the decode step's vocabulary projection
+        gen._select(lib, step_logits, n0, min_len, max_len, finished, tokens, scores)
+
     def one_step(step, step_logits):
         if st is not None:  # selection + forward + length advance as one graph replay
-            gen._graph_step(lib, st, step, max_len - 1, max_len)
+            gen._graph_step(lib, st, step, min_len, max_len)
             return st["logits"]
-        gen._select(lib, step_logits, step, max_len - 1, max_len, finished, tokens, scores)
+        if fused:  # forward over the history up to `step`, selection of the token at step + 1
+            nxt = step + 1
+            decoder.forward_select(
+                tokens[:, :nxt], inc, temperature=gen.temperature,
+                banned=gen._banned(nxt, min_len), stop=gen.stop, finished=finished,
+                force_eos=nxt >= max_len - 1, eos=gen.eos, tok_out=tokens[:, nxt],
+                tok_stride=tokens.stride(0), score_out=scores[:, nxt],
+                score_stride=scores.stride(0))
+            return None
+        gen._select(lib, step_logits, step, min_len, max_len, finished, tokens, scores)
         out = decoder(tokens[:, :step + 1], incremental_state=inc)[0]
         return out.view(B, -1)
 

@@ -111,7 +111,10 @@ int msa_embed_f16(const int64_t* tokens, int64_t tok_stride, int B, int n, int T
  *   t = round(acc); if bias: t = round(t + bias[n]); if RELU: t = max(t,0);
  *   if residual: t = round(t + residual[m,n]);  y[m,n] = t.
  * N % 16 == 0, K % 32 == 0.  With MSA_IN_PACKED (M <= 64) the HBM-bound weight-streaming kernel
- * runs; otherwise the LDS-tiled MFMA kernel (any M, row-major x).  residual is row-major and may
+ * runs; otherwise (any M, row-major x) an MFMA kernel tiled for the product's size: 256 x 256
+ * tiles with weights read straight from the packed layout once they fill the chip (K % 128 == 0;
+ * a ragged bottom block of at most 128 rows is streamed instead), 128 x 128 LDS tiles for the
+ * shapes in between.  All variants round at the same points.  residual is row-major and may
  * alias a row-major y.  flags: MSA_EPI_RELU | MSA_IN_PACKED | MSA_OUT_PACKED.
  * Replaces LinearWithGradAccumulationAndAsyncCommunication.forward
  * (metaseq/modules/megatron/mpu/layers.py:290-292) as used by out_proj
@@ -195,6 +198,24 @@ int msa_greedy_select_f16(const void* logits, int64_t ld_logits, int B, int V, f
  * (metaseq/sequence_generator.py:235-258). */
 int msa_target_logprob_f16(const void* logits, int64_t ld_logits, int64_t rows, int V,
                            float temperature, const int64_t* target, float* out, void* stream);
+
+/* Vocabulary projection fused with the greedy selection (M <= 64 rows, packed activations):
+ * the logits round(x . E^T) of msa_linear_f16 are reduced inside the projection's epilogue to one
+ * (running log-sum-exp, best eligible id) partial per row and workgroup, and a second small
+ * kernel merges the partials and finishes the step exactly as msa_greedy_select_f16 does (same
+ * masks, tie-break, outputs and `len_dev` meaning).  The logits are only stored if `logits`
+ * ([M, V] fp16, row-major) is not NULL.  `workspace` needs
+ * msa_lm_head_select_workspace_bytes(M) bytes of device memory (contents are scratch).
+ * Replaces metaseq/models/transformer_decoder.py:398-428 (output_layer) followed by
+ * metaseq/sequence_generator.py:272-308,319-323 (log-softmax, masks, max, bookkeeping). */
+int64_t msa_lm_head_select_workspace_bytes(int M);
+int msa_lm_head_greedy_select_f16(const void* x, const void* Ep, void* logits, void* workspace,
+                                  int M, int V, int K, float temperature,
+                                  const int32_t* banned_host, int n_banned,
+                                  const int32_t* stop_host, int n_stop, uint8_t* finished,
+                                  int force_eos_all, int eos_idx, int64_t* tok,
+                                  int64_t tok_stride, float* score, int64_t score_stride,
+                                  const int32_t* len_dev, void* stream);
 
 #ifdef __cplusplus
 }

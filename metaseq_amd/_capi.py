@@ -44,8 +44,10 @@ SIGNATURES = {
     "msa_greedy_select_f16": [_P, c_int64, c_int, c_int, c_float, _P, c_int, _P, c_int, _P, c_int,
                               c_int, _P, c_int64, _P, c_int64, _P, _P],
     "msa_target_logprob_f16": [_P, c_int64, c_int64, c_int, c_float, _P, _P, _P],
+    "msa_lm_head_greedy_select_f16": [_P, _P, _P, _P, c_int, c_int, c_int, c_float, _P, c_int, _P,
+                                      c_int, _P, c_int, c_int, _P, c_int64, _P, c_int64, _P, _P],
 }
-OTHER_SYMBOLS = ["msa_last_error", "msa_version"]
+OTHER_SYMBOLS = ["msa_last_error", "msa_version", "msa_lm_head_select_workspace_bytes"]
 
 _lib = None
 
@@ -68,6 +70,8 @@ def load():
     lib.msa_last_error.restype = c_char_p
     lib.msa_version.argtypes = []
     lib.msa_version.restype = c_int
+    lib.msa_lm_head_select_workspace_bytes.argtypes = [c_int]
+    lib.msa_lm_head_select_workspace_bytes.restype = c_int64
     _lib = lib
     return lib
 

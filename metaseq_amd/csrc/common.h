@@ -41,6 +41,26 @@ int msa_launch_prefill_attention(const void* q, const void* Kc, const void* Vc,
     }                                                                       \
   } while (0)
 
+// up to 16 token ids passed by value to a kernel (banned / stop lists of the generator)
+struct IdList {
+  int32_t n;
+  int32_t id[16];
+};
+
+// Partial result of the greedy selection over a slice of one logits row: running log-sum-exp
+// (max, sum of exp(z - max)) over every id, best eligible z with its id, NaN seen.
+struct SelectPartial {
+  float m, s, best;
+  int32_t bidx;
+  float nan;
+  float pad[3];
+};
+
+int msa_launch_select_combine(const SelectPartial* partials, int n_parts, int B,
+                              const IdList& stop, uint8_t* finished, int eos, int64_t* tok,
+                              int64_t tok_stride, float* score, int64_t score_stride,
+                              const int32_t* len_dev, hipStream_t stream);
+
 // Packed activation layout for M <= 64 rows (the B operand of v_mfma_f32_16x16x32_f16, stored
 // in lane order): element (m, k) of a [M, K] activation with MB = ceil(M/16) row blocks lives
 // at half offset ((k/32 * MB + m/16) * 64 + 16*((k%32)/8) + m%16) * 8 + k%8.
@@ -51,6 +71,16 @@ __host__ __device__ __forceinline__ int64_t packed_act_offset(int m, int k, int 
 
 // round-to-nearest-even fp32 -> fp16 -> fp32 (a "materialise in fp16" point)
 __device__ __forceinline__ float round_h(float v) { return (float)(half_t)v; }
+
+// (max, sum of exp(z - max)) pairs merge associatively: one pass over a row suffices
+__device__ __forceinline__ void lse_merge(float& m, float& s, float om, float os) {
+  if (om > m) {
+    s = s * expf(m - om) + os;
+    m = om;
+  } else if (om > -INFINITY) {
+    s += os * expf(om - m);
+  }
+}
 
 // Cross-lane step of the wave reductions on the data-parallel-primitive path of the vector ALU
 // (no LDS round trip).  Lanes of a row that ROW_MASK leaves out receive `old`.

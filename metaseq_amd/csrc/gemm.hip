@@ -23,7 +23,7 @@
 
 namespace {
 
-enum { MODE_PLAIN = 0, MODE_QKV = 1 };
+enum { MODE_PLAIN = 0, MODE_QKV = 1, MODE_SELECT = 2 };
 
 struct Epilogue {
   const half_t* bias;
@@ -39,7 +39,68 @@ struct Epilogue {
   int T, H, hd, S0, S_cap;
   const int32_t* len_dev;  // if set (T == 1): the append position is read from the device
   float qscale;
+  // MODE_SELECT: greedy selection over the output row instead of (or besides) storing it
+  SelectPartial* partials;  // [M][gridDim.x]
+  const uint8_t* finished;  // rows that may only emit eos
+  IdList banned;
+  float temperature;  // logits are divided by it when `scale`
+  int scale, force_eos_all, eos;
 };
+
+// running selection state of one thread for one activation row (see SelectPartial)
+struct SelectState {
+  float m = -INFINITY, s = 0.f, best = -INFINITY;
+  int bidx = 0x7fffffff;
+  bool nan = false;
+};
+
+// 4 consecutive vocabulary ids n..n+3 of row m: the logit is round(acc), as the stored tensor
+// would hold it; log-softmax is monotone, so the arg-max of the masked log-probs is the
+// arg-max of the masked logits (lowest id on ties).
+__device__ __forceinline__ void select_update4(SelectState& st, const Epilogue& e, int64_t m,
+                                               int n, float4_t acc) {
+  float z[4], cm = -INFINITY;
+  const bool only_eos = e.force_eos_all || (e.finished && e.finished[m]);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    z[i] = round_h(acc[i]);
+    if (e.scale) z[i] = z[i] / e.temperature;
+    st.nan |= (z[i] != z[i]);
+    cm = fmaxf(cm, z[i]);
+    const int id = n + i;
+    bool ok = !(only_eos && id != e.eos);
+    for (int j = 0; j < e.banned.n; ++j) ok &= (e.banned.id[j] != id);
+    const float cand = ok ? z[i] : -INFINITY;
+    if (cand > st.best || (cand == st.best && id < st.bidx)) {
+      st.best = cand;
+      st.bidx = id;
+    }
+  }
+  if (cm > st.m) {
+    st.s *= __expf(st.m - cm);
+    st.m = cm;
+  }
+  if (st.m > -INFINITY) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) st.s += __expf(z[i] - st.m);
+  }
+  if (e.y) {
+    half4_t o;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) o[i] = (half_t)acc[i];
+    *reinterpret_cast<half4_t*>(e.y + m * e.N + n) = o;
+  }
+}
+
+__device__ __forceinline__ void select_merge(SelectState& a, float om, float os, float ob, int oi,
+                                             bool onan) {
+  lse_merge(a.m, a.s, om, os);
+  if (ob > a.best || (ob == a.best && oi < a.bidx)) {
+    a.best = ob;
+    a.bidx = oi;
+  }
+  a.nan |= onan;
+}
 
 // 4 consecutive output columns n..n+3 of row m
 template <int MODE>
@@ -228,6 +289,9 @@ __global__ __launch_bounds__(KG * 64) void linear_stream_kernel(
       }
     }
   };
+  // MODE_SELECT: slot e = threadIdx.x + it * KG * 64 of finish() always maps to the same row
+  constexpr int SEL_IT = (NT * MB * 64 + KG * 64 - 1) / (KG * 64);
+  SelectState sel[MODE == MODE_SELECT ? SEL_IT : 1];
   float4_t acc[NT][MB];
   auto clear = [&]() {
 #pragma unroll
@@ -286,7 +350,10 @@ __global__ __launch_bounds__(KG * 64) void linear_stream_kernel(
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb) red[wave][j * MB + mb][lane] = acc[j][mb];
     __syncthreads();
-    for (int e = threadIdx.x; e < NT * MB * 64; e += KG * 64) {
+#pragma unroll
+    for (int it = 0; it < SEL_IT; ++it) {
+      const int e = threadIdx.x + it * KG * 64;
+      if (e >= NT * MB * 64) break;
       const int jm = e >> 6, l = e & 63;
       const int j = jm / MB, mb = jm - j * MB;
       float4_t sum = red[0][jm][l];
@@ -297,8 +364,10 @@ __global__ __launch_bounds__(KG * 64) void linear_stream_kernel(
       if (m < M && t0 + j < tile_end) {
         if (part)
           *reinterpret_cast<float4_t*>(part + ((int64_t)blockIdx.y * M + m) * N + n) = sum;
+        else if (MODE == MODE_SELECT)
+          select_update4(sel[it], epi, m, n, sum);
         else
-          epilogue4<MODE>(epi, m_off + m, n, sum);
+          epilogue4<MODE == MODE_SELECT ? MODE_PLAIN : MODE>(epi, m_off + m, n, sum);
       }
     }
     __syncthreads();
@@ -324,6 +393,43 @@ __global__ __launch_bounds__(KG * 64) void linear_stream_kernel(
   } else {  // one stage left
     mma(s0, idx);
     finish(idx);
+  }
+  if (MODE == MODE_SELECT) {
+    // The 16 threads that hold one row (4 lane groups x NT tile slots of one row block) merge
+    // their states: lanes through shuffles, tile slots through LDS; one partial per row and
+    // workgroup goes to memory for the combine kernel.
+    SelectPartial* sp = reinterpret_cast<SelectPartial*>(&red[0][0][0]);  // [NT * MB * 16]
+#pragma unroll
+    for (int it = 0; it < SEL_IT; ++it) {
+      const int e = threadIdx.x + it * KG * 64;
+      SelectState st = sel[it];
+#pragma unroll
+      for (int o = 16; o <= 32; o <<= 1)
+        select_merge(st, __shfl_xor(st.m, o, MSA_WAVE), __shfl_xor(st.s, o, MSA_WAVE),
+                     __shfl_xor(st.best, o, MSA_WAVE), __shfl_xor(st.bidx, o, MSA_WAVE),
+                     (bool)__shfl_xor((int)st.nan, o, MSA_WAVE));
+      if (e < NT * MB * 64 && (e & 63) < 16) {
+        SelectPartial p;
+        p.m = st.m, p.s = st.s, p.best = st.best, p.bidx = st.bidx, p.nan = st.nan ? 1.f : 0.f;
+        sp[(e >> 6) * 16 + (e & 15)] = p;  // [jm][row in block]
+      }
+    }
+    __syncthreads();
+    if (threadIdx.x < MB * 16) {
+      const int mb = threadIdx.x >> 4, r = threadIdx.x & 15;
+      SelectState st;
+      for (int j = 0; j < NT; ++j) {  // jm = j * MB + mb
+        const SelectPartial p = sp[(j * MB + mb) * 16 + r];
+        select_merge(st, p.m, p.s, p.best, p.bidx, p.nan > 0.f);
+      }
+      const int m = mb * 16 + r;
+      if (m < M) {
+        SelectPartial p;
+        p.m = st.m, p.s = st.s, p.best = st.best, p.bidx = st.bidx, p.nan = st.nan ? 1.f : 0.f;
+        p.pad[0] = p.pad[1] = p.pad[2] = 0.f;
+        epi.partials[(int64_t)m * gridDim.x + blockIdx.x] = p;
+      }
+    }
   }
 }
 
@@ -824,6 +930,56 @@ extern "C" int msa_pack_weight_i8(const int8_t* src, int8_t* dst, int N, int K, 
 }
 extern "C" int msa_unpack_weight_i8(const int8_t* src, int8_t* dst, int N, int K, void* stream) {
   return pack_entry("msa_unpack_weight_i8", src, dst, N, K, true, true, stream);
+}
+
+extern "C" int64_t msa_lm_head_select_workspace_bytes(int M) {
+  // one partial per row and workgroup; the streaming kernel never launches more workgroups
+  // than there are compute units
+  return (int64_t)(M > 0 ? M : 0) * num_cus() * (int64_t)sizeof(SelectPartial);
+}
+
+extern "C" int msa_lm_head_greedy_select_f16(
+    const void* x, const void* Ep, void* logits, void* workspace, int M, int V, int K,
+    float temperature, const int32_t* banned_host, int n_banned, const int32_t* stop_host,
+    int n_stop, uint8_t* finished, int force_eos_all, int eos_idx, int64_t* tok,
+    int64_t tok_stride, float* score, int64_t score_stride, const int32_t* len_dev,
+    void* stream) {
+  const char* name = "msa_lm_head_greedy_select_f16";
+  MSA_REQUIRE(x && Ep && workspace && tok && score, MSA_ERR_INVALID_ARG, "%s: null pointer", name);
+  MSA_REQUIRE(M >= 1 && M <= 64 && V > 0 && V % 16 == 0 && K > 0 && K % 32 == 0,
+              MSA_ERR_INVALID_ARG, "%s: bad shape M=%d V=%d K=%d (1 <= M <= 64, V %% 16, K %% 32)",
+              name, M, V, K);
+  MSA_REQUIRE(n_banned >= 0 && n_banned <= 16 && (n_banned == 0 || banned_host),
+              MSA_ERR_INVALID_ARG, "%s: n_banned=%d (0..16)", name, n_banned);
+  MSA_REQUIRE(n_stop >= 0 && n_stop <= 16 && (n_stop == 0 || stop_host), MSA_ERR_INVALID_ARG,
+              "%s: n_stop=%d (0..16)", name, n_stop);
+  MSA_REQUIRE(eos_idx >= 0 && eos_idx < V, MSA_ERR_INVALID_ARG,
+              "%s: eos_idx=%d outside the vocabulary", name, eos_idx);
+  MSA_REQUIRE(temperature >= 0.f, MSA_ERR_INVALID_ARG, "%s: temperature < 0", name);
+  Epilogue e{};
+  e.y = (half_t*)logits;
+  e.N = V;
+  e.partials = (SelectPartial*)workspace;
+  e.finished = finished;
+  e.banned.n = n_banned;
+  for (int i = 0; i < n_banned; ++i) e.banned.id[i] = banned_host[i];
+  e.temperature = temperature;
+  e.scale = temperature > 0.f && temperature != 1.0f;
+  e.force_eos_all = force_eos_all;
+  e.eos = eos_idx;
+  IdList stop{};
+  stop.n = n_stop;
+  for (int i = 0; i < n_stop; ++i) stop.id[i] = stop_host[i];
+  // same decomposition as launch_stream_mb at S = 1: the partial stride is its grid size
+  const int ntiles = V / 16;
+  const int tiles_per_wg = (ntiles + num_cus() - 1) / num_cus();
+  const int gx = (ntiles + tiles_per_wg - 1) / tiles_per_wg;
+  launch_stream<false, MODE_SELECT>(x, Ep, nullptr, nullptr, 1, M, V, K, e, (hipStream_t)stream);
+  MSA_CHECK_LAUNCH(name);
+  msa_launch_select_combine((const SelectPartial*)workspace, gx, M, stop, finished, eos_idx, tok,
+                            tok_stride, score, score_stride, len_dev, (hipStream_t)stream);
+  MSA_CHECK_LAUNCH(name);
+  return MSA_OK;
 }
 
 extern "C" int msa_linear_default_splits(int64_t M, int N, int K) {

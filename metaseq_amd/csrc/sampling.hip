@@ -63,21 +63,6 @@ __device__ __forceinline__ RowStats row_logsumexp(const half_t* __restrict__ row
   return r;
 }
 
-struct IdList {
-  int32_t n;
-  int32_t id[16];
-};
-
-// (max, sum of exp(z - max)) pairs merge associatively: one pass over the row suffices
-__device__ __forceinline__ void lse_merge(float& m, float& s, float om, float os) {
-  if (om > m) {
-    s = s * expf(m - om) + os;
-    m = om;
-  } else if (om > -INFINITY) {
-    s += os * expf(om - m);
-  }
-}
-
 __global__ __launch_bounds__(SM_THREADS) void greedy_select_kernel(
     const half_t* __restrict__ logits, int64_t ld, int V, float temperature, bool scale,
     IdList banned, IdList stop, uint8_t* __restrict__ finished, int force_eos_all, int eos,
@@ -211,7 +196,82 @@ __global__ __launch_bounds__(SM_THREADS) void target_logprob_kernel(
   }
 }
 
+// Merges the per-workgroup partials that the vocabulary projection's selection epilogue
+// wrote for one row and finishes the step exactly as greedy_select_kernel does.
+__global__ __launch_bounds__(256) void select_combine_kernel(
+    const SelectPartial* __restrict__ partials, int n_parts, IdList stop,
+    uint8_t* __restrict__ finished, int eos, int64_t* __restrict__ tok, int64_t tok_stride,
+    float* __restrict__ score, int64_t score_stride, const int32_t* __restrict__ len_dev) {
+  __shared__ float wm[4], ws[4], wbest[4], wnan[4];
+  __shared__ int widx[4];
+  const int b = blockIdx.x;
+  float m = -INFINITY, s = 0.f, best = -INFINITY;
+  int bidx = 0x7fffffff;
+  bool nan = false;
+  for (int i = threadIdx.x; i < n_parts; i += blockDim.x) {
+    const SelectPartial p = partials[(int64_t)b * n_parts + i];
+    lse_merge(m, s, p.m, p.s);
+    if (p.best > best || (p.best == best && p.bidx < bidx)) {
+      best = p.best;
+      bidx = p.bidx;
+    }
+    nan |= p.nan > 0.f;
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    lse_merge(m, s, __shfl_xor(m, o, MSA_WAVE), __shfl_xor(s, o, MSA_WAVE));
+    const float ob = __shfl_xor(best, o, MSA_WAVE);
+    const int oi = __shfl_xor(bidx, o, MSA_WAVE);
+    if (ob > best || (ob == best && oi < bidx)) {
+      best = ob;
+      bidx = oi;
+    }
+    nan |= (bool)__shfl_xor((int)nan, o, MSA_WAVE);
+  }
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  if (lane == 0) {
+    wm[wave] = m;
+    ws[wave] = s;
+    wbest[wave] = best;
+    widx[wave] = bidx;
+    wnan[wave] = nan ? 1.f : 0.f;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < 4; ++w) {
+      lse_merge(m, s, wm[w], ws[w]);
+      if (wbest[w] > best || (wbest[w] == best && widx[w] < bidx)) {
+        best = wbest[w];
+        bidx = widx[w];
+      }
+      nan |= wnan[w] > 0.f;
+    }
+    float lp = (best - m) - logf(s);
+    if (nan || !(best > -INFINITY)) {
+      lp = -INFINITY;
+      bidx = 0;
+    }
+    const int col = len_dev ? *len_dev : 0;
+    tok[b * tok_stride + col] = bidx;
+    score[b * score_stride + col] = lp;
+    if (finished) {
+      bool f = bidx == eos;
+      for (int j = 0; j < stop.n; ++j) f |= (stop.id[j] == bidx);
+      if (f) finished[b] = 1;
+    }
+  }
+}
+
 }  // namespace
+
+int msa_launch_select_combine(const SelectPartial* partials, int n_parts, int B,
+                              const IdList& stop, uint8_t* finished, int eos, int64_t* tok,
+                              int64_t tok_stride, float* score, int64_t score_stride,
+                              const int32_t* len_dev, hipStream_t stream) {
+  hipLaunchKernelGGL(select_combine_kernel, dim3(B), dim3(256), 0, stream, partials, n_parts,
+                     stop, finished, eos, tok, tok_stride, score, score_stride, len_dev);
+  return 0;
+}
 
 extern "C" int msa_greedy_select_f16(const void* logits, int64_t ld_logits, int B, int V,
                                      float temperature, const int32_t* banned_host, int n_banned,

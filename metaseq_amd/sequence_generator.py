@@ -82,14 +82,20 @@ class SequenceGenerator(nn.Module):
         return self._generate(sample, **kwargs)
 
     # ------------------------------------------------------------------
+    def _banned(self, step, min_len):
+        """Ids that cannot be chosen at ``step``: pad always, eos and the stop tokens before the
+        minimum length (metaseq/sequence_generator.py:272-279)."""
+        banned = [self.pad]
+        if step < min_len:
+            banned += [self.eos] + self.stop
+        return banned
+
     def _select(self, lib, logits2d, step, min_len, max_len, finished, tokens, scores,
                 len_dev=None):
         """Fused log-softmax + masks + arg-max + bookkeeping for one step
         (metaseq/sequence_generator.py:272-308).  With ``len_dev`` the output column is read
         from the device (``step`` then only selects the masks)."""
-        banned = [self.pad]
-        if step < min_len:
-            banned += [self.eos] + self.stop
+        banned = self._banned(step, min_len)
         B, V = logits2d.shape
         arr = (ctypes.c_int32 * len(banned))(*banned)
         stop = (ctypes.c_int32 * max(1, len(self.stop)))(*self.stop)
@@ -211,7 +217,27 @@ class SequenceGenerator(nn.Module):
             if (self.use_graph and all_lprobs is None and cache is not None and BB <= 64
                     and not cache.has_pads and not general):
                 st = self.static_state(decoder, cache, tokens, scores, finished, step_logits)
-            for step in range(start_step, max_len):
+            fused = (not general and all_lprobs is None and st is None and BB <= 64
+                     and hasattr(decoder, "forward_select"))
+            if fused:
+                # the first token comes from the prefill logits; every later one is chosen inside
+                # the decode step's vocabulary projection, so logits are never materialised
+                step = start_step
+                self._select(lib, step_logits, step, min_len, max_len, finished, tokens, scores)
+                while True:
+                    if (step >= min_len or step >= max_len - 1) and bool(finished.all()):
+                        break
+                    if step + 1 >= max_len:
+                        break
+                    nxt = step + 1
+                    decoder.forward_select(
+                        tokens[:, :nxt], incremental_states, temperature=self.temperature,
+                        banned=self._banned(nxt, min_len), stop=self.stop, finished=finished,
+                        force_eos=nxt >= max_len - 1, eos=self.eos, tok_out=tokens[:, nxt],
+                        tok_stride=tokens.stride(0), score_out=scores[:, nxt],
+                        score_stride=scores.stride(0))
+                    step = nxt
+            for step in range(start_step, max_len if not fused else start_step):
                 if general:
                     lprobs = self._masked_lprobs(step_logits, step, min_len, max_len, finished,
                                                  gs)

@@ -7,6 +7,7 @@ parameter names in ``state_dict()``.
 All arithmetic runs in libmetaseq_amd.so through the C ABI; torch only owns the device
 memory and the stream.  There is no eager fallback.
 """
+import ctypes
 import uuid
 from typing import Any, Dict, Optional
 
@@ -512,6 +513,35 @@ class TransformerDecoder(nn.Module):
         if features_only:
             return f, extra
         return self._project(f, packed, B, T), extra
+
+    def forward_select(self, prev_output_tokens, incremental_state, *, temperature, banned, stop,
+                       finished, force_eos, eos, tok_out, tok_stride, score_out, score_stride,
+                       logits_out=None):
+        """One decode step (at most 64 rows) whose vocabulary projection is fused with the greedy
+        selection of the next token (metaseq/models/transformer_decoder.py:494-537 followed by
+        metaseq/sequence_generator.py:272-308,319-323): the logits are reduced inside the
+        projection's epilogue and never stored unless ``logits_out`` ([B, V] fp16) is given.
+        ``tok_out`` / ``score_out`` are views of the first row's output element (column of the
+        token being chosen) with the given row strides; ``banned`` / ``stop`` are id lists,
+        ``finished`` the uint8 row flags the call updates."""
+        if not incremental_state:
+            raise AssertionError("forward_select is a decode step: prefill first")
+        f, packed, (B, T), _ = self._forward_features(prev_output_tokens, incremental_state, None,
+                                                      None, want_packed=True)
+        if not packed:
+            raise ValueError("forward_select needs at most 64 rows")
+        lib = self._lib
+        D, V = self.cfg.decoder_embed_dim, self.cfg.vocab_size
+        need = lib.msa_lm_head_select_workspace_bytes(B)
+        ws = getattr(self, "_select_ws", None)
+        if ws is None or ws.numel() < need or ws.device != f.device:
+            ws = self._select_ws = torch.empty(need, dtype=torch.uint8, device=f.device)
+        ba = (ctypes.c_int32 * max(1, len(banned)))(*banned)
+        sa = (ctypes.c_int32 * max(1, len(stop)))(*stop)
+        check(lib.msa_lm_head_greedy_select_f16(
+            ptr(f), ptr(self._lm_head), ptr(logits_out), ptr(ws), B, V, D, float(temperature), ba,
+            len(banned), sa, len(stop), ptr(finished), int(force_eos), int(eos), ptr(tok_out),
+            tok_stride, ptr(score_out), score_stride, None, _capi.stream_ptr()))
 
 
 # the name the reference's model code uses for this class

@@ -205,4 +205,6 @@ def test_graph_replay_matches_eager_generation(min_len):
     for _ in range(2):  # a second generation re-captures against a new cache
         graph = run_generate(model, cfg, src, 41, min_len, use_graph=True, **kw)
         assert torch.equal(graph["tokens"], eager["tokens"])
-        assert torch.equal(graph["scores"], eager["scores"])
+        # the eager loop selects inside the vocabulary projection, the captured step with the
+        # stand-alone selection kernel: same logits, another fp32 order in the log-sum-exp
+        assert torch.allclose(graph["scores"], eager["scores"], atol=2e-5, rtol=1e-6)

@@ -586,3 +586,83 @@ def test_target_logprob(lib):
     ok(lib.msa_target_logprob_f16(P(d), d.stride(0), R, V, 1.0, P(G(tgt)), P(out), None), lib)
     torch.cuda.synchronize()
     assert torch.allclose(out.cpu(), want, atol=2e-5)
+
+
+@pytest.mark.parametrize("M,V,K", [(1, 96, 64), (17, 2048, 256), (32, 50272, 768), (64, 4000, 128),
+                                   (48, 50272, 256)])
+def test_lm_head_fused_selection_matches_projection_then_select(lib, M, V, K):
+    """msa_lm_head_greedy_select_f16 against msa_linear_f16 followed by msa_greedy_select_f16
+    (itself checked against the reference's passes above): identical tokens and finished flags,
+    identical stored logits, scores equal up to the fp32 summation order of the log-sum-exp."""
+    print("lm-head select", M, V, K, flush=True)
+    x, E = rnd(M, K, seed=3, std=1.0), rnd(V, K, seed=4, std=0.3)
+    Ep = pack_w(lib, G(E))
+    xp = G(pack_act(x))
+    logits = torch.empty(M, V, dtype=torch.float16, device=DEV)
+    ok(lib.msa_linear_f16(P(xp), P(Ep), None, None, P(logits), M, V, K, IN_PACKED, None), lib)
+    ws = torch.empty(lib.msa_lm_head_select_workspace_bytes(M), dtype=torch.uint8, device=DEV)
+    top = logits.float().argmax(-1)
+    cases = [
+        dict(),                                                     # plain
+        dict(temperature=0.7, banned=(1, 2)),                       # min-length regime
+        dict(banned=tuple({1, int(top[0]), int(top[-1])}), stop=(int(logits[0].float().topk(2).indices[1]),)),
+        dict(banned=(1,), force=1),                                 # last step: only eos
+        dict(banned=(1,), finished=[i % 3 == 0 for i in range(M)]),
+    ]
+    for c in cases:
+        banned, stop = list(c.get("banned", ())), list(c.get("stop", ()))
+        temp, force = c.get("temperature", 1.0), c.get("force", 0)
+        ba = (ctypes.c_int32 * max(1, len(banned)))(*banned)
+        sa = (ctypes.c_int32 * max(1, len(stop)))(*stop)
+        outs = []
+        for fused in (False, True):
+            fin = None
+            if "finished" in c:
+                fin = torch.tensor(c["finished"], dtype=torch.uint8, device=DEV)
+            elif stop:
+                fin = torch.zeros(M, dtype=torch.uint8, device=DEV)
+            tok = torch.full((M, 3), -7, dtype=torch.long, device=DEV)
+            sc = torch.full((M, 3), 9.0, dtype=torch.float32, device=DEV)
+            lg = torch.zeros(M, V, dtype=torch.float16, device=DEV)
+            if fused:
+                ok(lib.msa_lm_head_greedy_select_f16(
+                    P(xp), P(Ep), P(lg), P(ws), M, V, K, temp, ba, len(banned), sa, len(stop),
+                    P(fin), force, 2, P(tok[:, 1]), 3, P(sc[:, 1]), 3, None, None), lib)
+            else:
+                ok(lib.msa_greedy_select_f16(P(logits), V, M, V, temp, ba, len(banned), sa,
+                                             len(stop), P(fin), force, 2, P(tok[:, 1]), 3,
+                                             P(sc[:, 1]), 3, None, None), lib)
+                lg = logits
+            torch.cuda.synchronize()
+            outs.append((tok.cpu(), sc.cpu(), None if fin is None else fin.cpu(), lg.cpu()))
+        (t0, s0, f0, l0), (t1, s1, f1, l1) = outs
+        assert torch.equal(t0, t1), c
+        assert torch.allclose(s0, s1, atol=2e-5, rtol=1e-6), (c, (s0 - s1).abs().max())
+        assert (f0 is None and f1 is None) or torch.equal(f0, f1), c
+        assert torch.equal(l0, l1), c
+    # logits are optional, the column may come from the device, and a NaN row yields (0, -inf)
+    ln = torch.tensor([2], dtype=torch.int32, device=DEV)
+    tok = torch.full((M, 3), -7, dtype=torch.long, device=DEV)
+    sc = torch.zeros(M, 3, dtype=torch.float32, device=DEV)
+    ba = (ctypes.c_int32 * 1)(1)
+    ok(lib.msa_lm_head_greedy_select_f16(P(xp), P(Ep), None, P(ws), M, V, K, 1.0, ba, 1, ba, 0,
+                                         None, 0, 2, P(tok), 3, P(sc), 3, P(ln), None), lib)
+    xn = x.clone()
+    xn[0, 0] = float("nan")
+    tok2 = torch.full((M, 1), -7, dtype=torch.long, device=DEV)
+    sc2 = torch.zeros(M, 1, dtype=torch.float32, device=DEV)
+    ok(lib.msa_lm_head_greedy_select_f16(P(G(pack_act(xn))), P(Ep), None, P(ws), M, V, K, 1.0, ba,
+                                         1, ba, 0, None, 0, 2, P(tok2), 1, P(sc2), 1, None, None),
+       lib)
+    torch.cuda.synchronize()
+    lg = logits.float().clone()
+    lg[:, 1] = float("-inf")
+    assert torch.equal(tok[:, 2].cpu(), lg.argmax(-1).cpu()) and int((tok[:, :2] != -7).sum()) == 0
+    assert int(tok2[0]) == 0 and float(sc2[0]) == float("-inf")
+    if M > 1:
+        assert torch.equal(tok2[1:, 0].cpu(), lg[1:].argmax(-1).cpu())
+    # argument checks
+    assert lib.msa_lm_head_greedy_select_f16(P(xp), P(Ep), None, None, M, V, K, 1.0, ba, 1, ba, 0,
+                                             None, 0, 2, P(tok), 3, P(sc), 3, None, None) == -1
+    assert lib.msa_lm_head_greedy_select_f16(P(xp), P(Ep), None, P(ws), 65, V, K, 1.0, ba, 1, ba,
+                                             0, None, 0, 2, P(tok), 3, P(sc), 3, None, None) == -1
