@@ -142,6 +142,7 @@ int msa_linear_partial_f16(const void* x, const void* Wp, float* part, int64_t M
 int msa_linear_partial_w8a16(const void* x, const int8_t* Wq, const void* scales, float* part,
                              int64_t M, int N, int K, int S, unsigned flags, void* stream);
 int msa_linear_default_splits(int64_t M, int N, int K);
+int msa_linear_default_splits_w8a16(int64_t M, int N, int K);
 
 /* Fused QKV projection: kvq = round(round(x . Wqkv^T) + bqkv) with rows of Wqkv ordered
  * K | V | Q; then for row m = b*T + t and head h:

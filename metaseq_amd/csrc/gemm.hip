@@ -221,20 +221,26 @@ __global__ __launch_bounds__(256) void pack_i8_kernel(const int8_t* __restrict__
 // its operand; A rows are output features n, B rows are activation rows m.  The accumulator
 // of lane l holds m = l&15 and n = 4*(l>>4) .. +3.
 constexpr int ST_KG = 8;  // waves per workgroup = interleaved K lanes
-constexpr int ST_NT = 4;  // weight tiles sharing one activation fragment
+constexpr int ST_NT = 4;  // weight tiles sharing one activation fragment (<= 32 rows)
+constexpr int ST_RN = 4;  // tiles reduced across the waves per pass through LDS
 
 // XR: the activations are row-major ([rows, K], fragments gathered 16 bytes per lane) instead
 // of packed; the kernel then handles rows m_off .. m_off + M - 1 of a taller matrix (the ragged
 // bottom of a prefill-sized product) and the epilogue sees the global row numbers.
-template <int MB, bool W8, int MODE, bool XR = false, int KG = ST_KG, int NT = ST_NT,
-          int U = (MB <= 2 ? 4 : 2)>
+// With more than 32 activation rows the activation fragments (re-read from L2 once per tile
+// group) outweigh the weights in cache-fill traffic, so the fp16 kernel lets twice as many
+// tiles share each fragment and buffers fewer K steps to stay inside the register file (the
+// int8 kernel, whose stage also holds the raw bytes of two K steps, would spill).
+template <int MB, bool W8, int MODE, bool XR = false, int KG = ST_KG,
+          int NT = (MB <= 2 || W8 ? ST_NT : 2 * ST_NT), int U = (MB <= 2 ? 4 : (NT > ST_NT ? 1 : 2))>
 __global__ __launch_bounds__(KG * 64) void linear_stream_kernel(
     const half_t* __restrict__ xp, const void* __restrict__ Wp, const half_t* __restrict__ scales,
     float* __restrict__ part, int M, int N, int K, int tiles_per_wg, int ks_per_split,
     Epilogue epi, int64_t m_off) {
   // U = K steps (32 wide) buffered per stage; an int8 block covers two steps
   constexpr int UA = W8 ? U / 2 : U;  // weight loads per stage and tile
-  __shared__ float4_t red[KG][NT * MB][64];
+  constexpr int RN = ST_RN;  // NT is a multiple of RN
+  __shared__ float4_t red[KG][RN * MB][64];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int ntiles = N >> 4;
   const int nks = K >> 5;  // 32-wide steps in a row
@@ -289,8 +295,9 @@ __global__ __launch_bounds__(KG * 64) void linear_stream_kernel(
       }
     }
   };
-  // MODE_SELECT: slot e = threadIdx.x + it * KG * 64 of finish() always maps to the same row
-  constexpr int SEL_IT = (NT * MB * 64 + KG * 64 - 1) / (KG * 64);
+  // slot e = threadIdx.x + it * KG * 64 of a reduction pass of finish(); it always maps to the
+  // same activation row, whatever the pass (MODE_SELECT keeps one running state per slot)
+  constexpr int SEL_IT = (RN * MB * 64 + KG * 64 - 1) / (KG * 64);
   SelectState sel[MODE == MODE_SELECT ? SEL_IT : 1];
   float4_t acc[NT][MB];
   auto clear = [&]() {
@@ -318,10 +325,12 @@ __global__ __launch_bounds__(KG * 64) void linear_stream_kernel(
         for (int mb = 0; mb < MB; ++mb) s.b[u][mb] = zero8();
       }
     }
+    const int tiles_left = tile_end - (tile_begin + grp * NT);  // real tiles in this group
 #pragma unroll
     for (int u = 0; u < UA; ++u)
 #pragma unroll
       for (int j = 0; j < NT; ++j) {
+        if (NT > ST_NT && j >= tiles_left) continue;  // wave-uniform: no MFMAs for surplus tiles
         if (!W8) {
 #pragma unroll
           for (int mb = 0; mb < MB; ++mb)
@@ -346,31 +355,35 @@ __global__ __launch_bounds__(KG * 64) void linear_stream_kernel(
     const int grp = idx / nstages;
     const int t0 = tile_begin + grp * NT;
 #pragma unroll
-    for (int j = 0; j < NT; ++j)
+    for (int p = 0; p < NT / RN; ++p) {  // RN tiles per pass through the LDS buffer
 #pragma unroll
-      for (int mb = 0; mb < MB; ++mb) red[wave][j * MB + mb][lane] = acc[j][mb];
-    __syncthreads();
+      for (int jj = 0; jj < RN; ++jj)
 #pragma unroll
-    for (int it = 0; it < SEL_IT; ++it) {
-      const int e = threadIdx.x + it * KG * 64;
-      if (e >= NT * MB * 64) break;
-      const int jm = e >> 6, l = e & 63;
-      const int j = jm / MB, mb = jm - j * MB;
-      float4_t sum = red[0][jm][l];
+        for (int mb = 0; mb < MB; ++mb) red[wave][jj * MB + mb][lane] = acc[p * RN + jj][mb];
+      __syncthreads();
 #pragma unroll
-      for (int w = 1; w < KG; ++w) sum += red[w][jm][l];
-      const int m = mb * 16 + (l & 15);
-      const int n = (t0 + j) * 16 + ((l >> 4) << 2);
-      if (m < M && t0 + j < tile_end) {
-        if (part)
-          *reinterpret_cast<float4_t*>(part + ((int64_t)blockIdx.y * M + m) * N + n) = sum;
-        else if (MODE == MODE_SELECT)
-          select_update4(sel[it], epi, m, n, sum);
-        else
-          epilogue4<MODE == MODE_SELECT ? MODE_PLAIN : MODE>(epi, m_off + m, n, sum);
+      for (int it = 0; it < SEL_IT; ++it) {
+        const int e = threadIdx.x + it * KG * 64;
+        if (e >= RN * MB * 64) break;
+        const int jm = e >> 6, l = e & 63;
+        const int jj = jm / MB, mb = jm - jj * MB;
+        const int j = p * RN + jj;
+        float4_t sum = red[0][jm][l];
+#pragma unroll
+        for (int w = 1; w < KG; ++w) sum += red[w][jm][l];
+        const int m = mb * 16 + (l & 15);
+        const int n = (t0 + j) * 16 + ((l >> 4) << 2);
+        if (m < M && t0 + j < tile_end) {
+          if (part)
+            *reinterpret_cast<float4_t*>(part + ((int64_t)blockIdx.y * M + m) * N + n) = sum;
+          else if (MODE == MODE_SELECT)
+            select_update4(sel[it], epi, m, n, sum);
+          else
+            epilogue4<MODE == MODE_SELECT ? MODE_PLAIN : MODE>(epi, m_off + m, n, sum);
+        }
       }
+      __syncthreads();
     }
-    __syncthreads();
     clear();
   };
   clear();
@@ -395,10 +408,10 @@ __global__ __launch_bounds__(KG * 64) void linear_stream_kernel(
     finish(idx);
   }
   if (MODE == MODE_SELECT) {
-    // The 16 threads that hold one row (4 lane groups x NT tile slots of one row block) merge
+    // The 16 threads that hold one row (4 lane groups x RN tile slots of one row block) merge
     // their states: lanes through shuffles, tile slots through LDS; one partial per row and
     // workgroup goes to memory for the combine kernel.
-    SelectPartial* sp = reinterpret_cast<SelectPartial*>(&red[0][0][0]);  // [NT * MB * 16]
+    SelectPartial* sp = reinterpret_cast<SelectPartial*>(&red[0][0][0]);  // [RN * MB * 16]
 #pragma unroll
     for (int it = 0; it < SEL_IT; ++it) {
       const int e = threadIdx.x + it * KG * 64;
@@ -408,7 +421,7 @@ __global__ __launch_bounds__(KG * 64) void linear_stream_kernel(
         select_merge(st, __shfl_xor(st.m, o, MSA_WAVE), __shfl_xor(st.s, o, MSA_WAVE),
                      __shfl_xor(st.best, o, MSA_WAVE), __shfl_xor(st.bidx, o, MSA_WAVE),
                      (bool)__shfl_xor((int)st.nan, o, MSA_WAVE));
-      if (e < NT * MB * 64 && (e & 63) < 16) {
+      if (e < RN * MB * 64 && (e & 63) < 16) {
         SelectPartial p;
         p.m = st.m, p.s = st.s, p.best = st.best, p.bidx = st.bidx, p.nan = st.nan ? 1.f : 0.f;
         sp[(e >> 6) * 16 + (e & 15)] = p;  // [jm][row in block]
@@ -418,7 +431,7 @@ __global__ __launch_bounds__(KG * 64) void linear_stream_kernel(
     if (threadIdx.x < MB * 16) {
       const int mb = threadIdx.x >> 4, r = threadIdx.x & 15;
       SelectState st;
-      for (int j = 0; j < NT; ++j) {  // jm = j * MB + mb
+      for (int j = 0; j < RN; ++j) {  // jm = j * MB + mb
         const SelectPartial p = sp[(j * MB + mb) * 16 + r];
         select_merge(st, p.m, p.s, p.best, p.bidx, p.nan > 0.f);
       }
@@ -982,13 +995,41 @@ extern "C" int msa_lm_head_greedy_select_f16(
   return MSA_OK;
 }
 
+namespace {
+// Split count that minimises what one workgroup moves through its L1: its weight tiles over
+// its K range, the activation fragments of that K range once per tile group, and its fp32
+// partial sums (written here, read back by the LayerNorm tail).  More splits mean more tiles
+// per workgroup over a shorter K range, i.e. fewer activation bytes per weight byte.
+int pick_splits(int64_t M, int N, int K, int wbytes) {
+  if (M < 1 || M > 64 || N % 16 || K % 64) return 1;
+  const int MB = (int)((M + 15) / 16), ntiles = N / 16, nks = K / 32;
+  const int NT = MB <= 2 || wbytes == 1 ? ST_NT : 2 * ST_NT;
+  const int U = MB <= 2 ? 4 : (NT > ST_NT ? 1 : 2);
+  int best = 1;
+  double best_cost = 0;
+  for (int S = 1; S <= 8; S *= 2) {
+    const int G = num_cus() / S;
+    if (G < 1 || nks / S < ST_KG * U) break;  // every wave needs a full stage of K steps
+    const int tpw = (ntiles + G - 1) / G;
+    const int groups = (tpw + NT - 1) / NT;
+    const double Ks = (double)K / S;
+    double cost = tpw * 16.0 * Ks * wbytes + groups * MB * 16.0 * Ks * 2 + 2.0 * tpw * 16 * M * 4;
+    cost *= 1.0 + 0.02 * S;  // ties go to fewer splits (fewer partial slices to sum)
+    if (S == 1 || cost < best_cost) {
+      best = S;
+      best_cost = cost;
+    }
+  }
+  return best;
+}
+}  // namespace
+
 extern "C" int msa_linear_default_splits(int64_t M, int N, int K) {
-  // split K only where one split leaves most compute units without a tile group
-  if (M > 64 || N % 16 || K % 64) return 1;
-  const int groups = (N / 16 + ST_NT - 1) / ST_NT;
-  int S = 1;
-  while (S < 8 && groups * S * 2 <= num_cus() && K / 32 / (S * 2) >= ST_KG * 2) S *= 2;
-  return S;
+  return pick_splits(M, N, K, 2);
+}
+
+extern "C" int msa_linear_default_splits_w8a16(int64_t M, int N, int K) {
+  return pick_splits(M, N, K, 1);
 }
 
 extern "C" int msa_linear_f16(const void* x, const void* Wp, const void* bias,

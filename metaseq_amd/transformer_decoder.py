@@ -266,8 +266,9 @@ class TransformerDecoder(nn.Module):
             D, F = cfg.decoder_embed_dim, cfg.decoder_ffn_embed_dim
             MP = ((B + 15) // 16) * 16
             lib = self._lib
-            S_o = lib.msa_linear_default_splits(B, D, D)
-            S_f = lib.msa_linear_default_splits(B, D, F)
+            int8 = self.layers[0].fc2.qweight is not None
+            splits = lib.msa_linear_default_splits_w8a16 if int8 else lib.msa_linear_default_splits
+            S_o, S_f = splits(B, D, D), splits(B, D, F)
             f16 = dict(dtype=torch.float16, device=dev)
             bufs = {
                 "x": torch.empty(B, D, **f16), "q": torch.empty(B, D, **f16),
