@@ -21,7 +21,11 @@ Followed reference semantics (paths relative to the metaseq tree):
   concatenated along the vocabulary (models/transformer_decoder.py:398-428).
 
 Pinned by tests/test_checkpoint_cpu.py: at mp = 1 it must reproduce OracleDecoder exactly,
-which is itself pinned against Hugging Face OPT.
+which is itself pinned against Hugging Face OPT.  For mp > 1 the split of the computation over
+ranks is a restatement of the cited reference code with no reference fixture behind it (the
+reference ships no multi-part checkpoint or test vector): parity unpinned beyond the facts that
+the per-rank pieces sum / concatenate to the mp = 1 result when the parts are cut from one
+model, and that every rule is the one metaseq/distributed/stitch_fsdp_ckpt.py:203-339 applies.
 """
 from typing import Dict, List
 
