@@ -239,7 +239,7 @@ __global__ __launch_bounds__(KG * 64) void linear_stream_kernel(
     Epilogue epi, int64_t m_off) {
   // U = K steps (32 wide) buffered per stage; an int8 block covers two steps
   constexpr int UA = W8 ? U / 2 : U;  // weight loads per stage and tile
-  constexpr int RN = ST_RN;  // NT is a multiple of RN
+  constexpr int RN = NT < ST_RN ? NT : ST_RN;  // NT is a multiple of RN
   __shared__ float4_t red[KG][RN * MB][64];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int ntiles = N >> 4;
@@ -760,6 +760,17 @@ void launch_stream_mb(const void* xp, const void* W, const void* scales, float* 
   const int gx = (ntiles + tiles_per_wg - 1) / tiles_per_wg;
   int ks_per_split = (nks + S - 1) / S;
   if (W8) ks_per_split = (ks_per_split + 1) & ~1;  // int8 blocks cover two steps
+  // Up to 32 packed rows: groups of 3 tiles instead of 4 when that needs no more groups (no
+  // more sweeps over the activations) and leaves fewer empty tile slots, e.g. 3 tiles per
+  // workgroup for qkv_proj at d_model 4096.
+  if (MB <= 2 && !XR && (tiles_per_wg + 2) / 3 == (tiles_per_wg + 3) / 4 &&
+      (tiles_per_wg + 2) / 3 * 3 < (tiles_per_wg + 3) / 4 * 4) {
+    hipLaunchKernelGGL((linear_stream_kernel<(MB <= 2 ? MB : 1), W8, MODE, false, ST_KG, 3>),
+                       dim3(gx, S), dim3(ST_KG * 64), 0, s, (const half_t*)xp, W,
+                       (const half_t*)scales, part, M, N, K, tiles_per_wg, ks_per_split, epi,
+                       m_off);
+    return;
+  }
   hipLaunchKernelGGL((linear_stream_kernel<MB, W8, MODE, XR>), dim3(gx, S), dim3(ST_KG * 64), 0,
                      s, (const half_t*)xp, W, (const half_t*)scales, part, M, N, K, tiles_per_wg,
                      ks_per_split, epi, m_off);
