@@ -115,6 +115,64 @@ def cpu_baseline(size, B, S, seed=1234):
     }
 
 
+def torch_eager_steps(cfg, sd, B, S_first, K, warmup, dev):
+    """The reference's per-token forward written with stock PyTorch operators in fp16 on the same
+    GPU (linear / layer_norm / bmm / softmax, key and value history grown with torch.cat as
+    metaseq/modules/multihead_attention.py:451-467 does), greedy selection included; K timed
+    steps whose first one attends S_first positions.  Context figure only: what the same
+    arithmetic costs when every operator is a library call."""
+    import torch
+    import torch.nn.functional as F
+
+    L, D, H, hd = (cfg.decoder_layers, cfg.decoder_embed_dim, cfg.decoder_attention_heads,
+                   cfg.head_dim)
+    w = lambda k: sd["decoder." + k]
+    g = torch.Generator(device=dev).manual_seed(99)
+    n_hist = S_first - 1 - warmup
+    hist = [[torch.randn(B * H, n_hist, hd, device=dev, dtype=torch.float16, generator=g)
+             for _ in range(2)] for _ in range(L)]
+    tok = torch.randint(4, cfg.vocab_size, (B,), device=dev, generator=g)
+
+    def step(tok, n):
+        pos = torch.full((B,), n + 2, device=dev, dtype=torch.long)  # pad index 1 + 1 + n
+        x = F.embedding(tok, w("embed_tokens.weight")) + F.embedding(pos, w("embed_positions.weight"))
+        for i in range(L):
+            p = "layers.%d." % i
+            h = F.layer_norm(x, (D,), w(p + "self_attn_layer_norm.weight"),
+                             w(p + "self_attn_layer_norm.bias"))
+            k, v, q = F.linear(h, w(p + "self_attn.qkv_proj.weight"),
+                               w(p + "self_attn.qkv_proj.bias")).split(D, dim=-1)
+            q = (q * hd ** -0.5).reshape(B * H, 1, hd)
+            hist[i][0] = torch.cat([hist[i][0], k.reshape(B * H, 1, hd)], dim=1)
+            hist[i][1] = torch.cat([hist[i][1], v.reshape(B * H, 1, hd)], dim=1)
+            pr = F.softmax(torch.bmm(q, hist[i][0].transpose(1, 2)), dim=-1,
+                           dtype=torch.float32).to(x.dtype)
+            o = torch.bmm(pr, hist[i][1]).reshape(B, D)
+            x = F.linear(o, w(p + "self_attn.out_proj.weight")) + w(p + "self_attn.out_proj.bias") + x
+            h = F.layer_norm(x, (D,), w(p + "final_layer_norm.weight"), w(p + "final_layer_norm.bias"))
+            u = F.relu(F.linear(h, w(p + "fc1.weight"), w(p + "fc1.bias")))
+            x = x + F.linear(u, w(p + "fc2.weight"), w(p + "fc2.bias"))
+        x = F.layer_norm(x, (D,), w("layer_norm.weight"), w("layer_norm.bias"))
+        lprobs = F.log_softmax(F.linear(x, w("embed_tokens.weight")).float(), dim=-1)
+        return lprobs.max(dim=-1)[1]
+
+    with torch.no_grad():
+        n = n_hist
+        for _ in range(warmup):
+            tok = step(tok, n)
+            n += 1
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(K):
+            tok = step(tok, n)
+            n += 1
+        torch.cuda.synchronize()
+        dt = (time.perf_counter() - t0) / K
+    return {"value": B / dt, "unit": "tokens/s", "ms_per_step": dt * 1e3,
+            "what": "stock PyTorch fp16 operators, same shapes, same GPU, %d steps attending "
+                    "%d..%d positions" % (K, S_first, S_first + K - 1)}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -133,6 +191,9 @@ def main():
     ap.add_argument("--pmc-calibration", action="store_true",
                     help="also run a plain 1 GiB device copy, the known-size kernel that "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE readings are scaled by")
+    ap.add_argument("--torch-eager", action="store_true",
+                    help="also time the same decode steps written with stock PyTorch fp16 "
+                         "operators on this GPU (reported as torch_eager_same_gpu)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU; --gpus %d is not supported (nothing in the "
@@ -313,6 +374,14 @@ def main():
             "bytes_per_launch": ab, "avg_launch_us": attn_s * 1e6, "context": S_probe,
         },
     }
+    if args.torch_eager and not int8:
+        del inc, cache
+        sd = model.state_dict()
+        del model, gen, decoder
+        torch.cuda.empty_cache()
+        result["torch_eager_same_gpu"] = torch_eager_steps(cfg, sd, B, S_first, K, W, dev)
+        del sd
+        model = gen = inc = cache = decoder = None
     if not args.no_cpu_baseline:
         del model, gen, inc, cache, decoder
         torch.cuda.empty_cache()
