@@ -446,6 +446,206 @@ __global__ __launch_bounds__(KG * 64) void linear_stream_kernel(
   }
 }
 
+// ---- shared-activation stream kernel (33 .. 64 rows) ------------------------------------------
+// With more than 32 activation rows a wave that loads its own activation fragments moves more
+// bytes of activations (from L2) than of weights (from HBM) through the L1, and the L1 fill rate
+// becomes the limit.  Here the 8 waves form KL K lanes x NG tile lanes: the NG waves of a K lane
+// work on different weight tiles over the same K steps and read their activation fragments from
+// LDS, which the whole workgroup fills once per stage (SK = KL * U consecutive K steps, one
+// contiguous piece of the packed activations).  Weights still go from HBM straight to registers.
+// A tile group is NG * NT tiles, dealt round robin to the tile lanes; one barrier per stage;
+// activations are fetched two stages ahead and parked in LDS one stage ahead, weights (and int8
+// scales) one stage ahead.  The K lanes are summed through LDS in fixed order.
+constexpr int SH_THREADS = 512;
+
+template <int MB, bool W8, int NG, int NT, int U>
+struct ShareCfg {
+  static constexpr int KL = 8 / NG, SK = KL * U, UA = W8 ? U / 2 : U;
+  static constexpr int XH = SK * MB * 512;  // halves of activations per stage
+  static constexpr int XP = SK * MB / 8;    // 16-byte pieces per thread and stage
+  static constexpr int LDS_BYTES = 2 * XH * 2 + (KL - 1) * NG * NT * MB * 1024;
+  static_assert(SK * MB % 8 == 0 && U % 2 == 0, "stage must split evenly over the threads");
+};
+
+template <int MB, bool W8, int MODE, int NG, int NT, int U>
+__global__ __launch_bounds__(SH_THREADS) void linear_share_kernel(
+    const half_t* __restrict__ xp, const void* __restrict__ Wp, const half_t* __restrict__ scales,
+    float* __restrict__ part, int M, int N, int K, int tiles_per_wg, int ks_per_split,
+    Epilogue epi) {
+  static_assert(MODE != MODE_SELECT, "selection runs in the plain stream kernel");
+  using C = ShareCfg<MB, W8, NG, NT, U>;
+  constexpr int KL = C::KL, SK = C::SK, UA = C::UA, XH = C::XH, XP = C::XP;
+  extern __shared__ __attribute__((aligned(16))) half_t lx_share[];  // [2][XH], then red
+  float4_t* red = reinterpret_cast<float4_t*>(lx_share + 2 * XH);    // [KL-1][NG][NT*MB][64]
+  const int lane = threadIdx.x & 63;
+  // the wave number as a scalar: everything derived from it stays out of the vector registers
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int tid = wave * 64 + lane;
+  const int kl = wave / NG, ng = wave - kl * NG;
+  const int ntiles = N >> 4, nks = K >> 5;
+  const int tile_begin = blockIdx.x * tiles_per_wg;
+  const int tile_end = min(ntiles, tile_begin + tiles_per_wg);
+  const int ks_begin = blockIdx.y * ks_per_split;
+  const int ks_end = min(nks, ks_begin + ks_per_split);
+  if (tile_begin >= tile_end || ks_begin >= ks_end) return;
+  const int ngroups = (tile_end - tile_begin + NG * NT - 1) / (NG * NT);
+  const int nstages = (ks_end - ks_begin + SK - 1) / SK;
+  const int total = ngroups * nstages;
+
+  // Every load is unconditional (clamped address): K steps past the end are zeroed on their way
+  // into LDS, tiles past the end are dropped in finish().
+  half8_t xr[XP];
+  auto gload_x = [&](int idx) {
+    const int kb = ks_begin + (idx % nstages) * SK;
+#pragma unroll
+    for (int i = 0; i < XP; ++i) {
+      const int p = tid + SH_THREADS * i, f = p >> 6;
+      const int kk = min(kb + f / MB, ks_end - 1);
+      xr[i] = *reinterpret_cast<const half8_t*>(
+          xp + (((int64_t)kk * MB + f % MB) * 64 + (p & 63)) * 8);
+    }
+  };
+  auto lstore = [&](int idx) {
+    const int kb = ks_begin + (idx % nstages) * SK;
+    half_t* l = lx_share + (idx & 1) * XH;
+#pragma unroll
+    for (int i = 0; i < XP; ++i) {
+      const int p = tid + SH_THREADS * i;
+      const bool live = kb + (p >> 6) / MB < ks_end;
+      *reinterpret_cast<half8_t*>(l + p * 8) = live ? xr[i] : zero8();
+    }
+  };
+  struct Wst {
+    half8_t a[UA][NT];  // fp16: one A fragment; int8: 16 raw bytes = two A fragments
+    uint32_t sc[NT];    // int8: the row's fp16 scale in the low half
+  };
+  auto gload_w = [&](Wst& w, int idx) {
+    const int grp = idx / nstages, st = idx - grp * nstages;
+#pragma unroll
+    for (int j = 0; j < NT; ++j) {
+      const int t = min(tile_begin + (grp * NT + j) * NG + ng, tile_end - 1);
+#pragma unroll
+      for (int u = 0; u < UA; ++u) {
+        const int ks = ks_begin + st * SK + kl * U + (W8 ? 2 * u : u);
+        const int ksc = min(ks, ks_end - (W8 ? 2 : 1));
+        const int64_t blk = W8 ? (int64_t)t * (nks >> 1) + (ksc >> 1) : (int64_t)t * nks + ksc;
+        w.a[u][j] = __builtin_nontemporal_load(
+            reinterpret_cast<const half8_t*>((const half_t*)Wp + blk * 512 + lane * 8));
+      }
+      w.sc[j] = W8 ? reinterpret_cast<const uint16_t*>(scales)[t * 16 + (lane & 15)] : 0u;
+    }
+  };
+
+  float4_t acc[NT][MB];
+  auto clear = [&]() {
+#pragma unroll
+    for (int j = 0; j < NT; ++j)
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb) acc[j][mb] = float4_t{0.f, 0.f, 0.f, 0.f};
+  };
+  auto compute = [&](const Wst& w, int idx) {
+    const half_t* l = lx_share + (idx & 1) * XH + kl * U * MB * 512 + lane * 8;
+    constexpr int F = U * MB;  // fragment f = K step f / MB, row block f % MB
+    constexpr int PD = 4;      // LDS fragment reads in flight
+    half8_t bx[PD];
+#pragma unroll
+    for (int p = 0; p < PD; ++p) bx[p] = *reinterpret_cast<const half8_t*>(l + p * 512);
+    // the A fragments of K step u
+    half8_t a[2][NT];
+    auto expand = [&](int u) {
+#pragma unroll
+      for (int j = 0; j < NT; ++j) {
+        if (W8) {
+          typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+          const u4 raw = __builtin_bit_cast(u4, w.a[u / 2][j]);
+          const half_t sc = __builtin_bit_cast(half2_t, w.sc[j])[0];
+          a[u & 1][j] = (u & 1) ? dequant8(raw[2], raw[3], sc) : dequant8(raw[0], raw[1], sc);
+        } else {
+          a[u & 1][j] = w.a[W8 ? 0 : u][j];
+        }
+      }
+    };
+    // the stage's LDS stores and global loads go out first, then LDS reads and MFMAs alternate
+    __builtin_amdgcn_sched_group_barrier(0x200, XP, 0);
+    __builtin_amdgcn_sched_group_barrier(0x020, XP, 0);  // activations first: needed first
+    __builtin_amdgcn_sched_group_barrier(0x020, UA * NT + (W8 ? NT : 0), 0);
+    __builtin_amdgcn_sched_group_barrier(0x100, PD, 0);
+#pragma unroll
+    for (int f = 0; f < F; ++f) {
+      const int u = f / MB, mb = f % MB;
+      if (mb == 0) expand(u);
+      const half8_t cur = bx[f % PD];
+#pragma unroll
+      for (int j = 0; j < NT; ++j)
+        acc[j][mb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[u & 1][j], cur, acc[j][mb], 0, 0, 0);
+      __builtin_amdgcn_sched_group_barrier(0x008, NT, 0);
+      if (f + PD < F) {
+        bx[f % PD] = *reinterpret_cast<const half8_t*>(l + (f + PD) * 512);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      }
+    }
+  };
+  auto finish = [&](int idx) {  // after the last stage of a tile group
+    const int grp = idx / nstages;
+    if (kl > 0) {
+#pragma unroll
+      for (int j = 0; j < NT; ++j)
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb)
+          red[((((kl - 1) * NG + ng) * NT + j) * MB + mb) * 64 + lane] = acc[j][mb];
+    }
+    __syncthreads();
+    if (kl == 0) {
+#pragma unroll
+      for (int j = 0; j < NT; ++j) {
+        const int t = tile_begin + (grp * NT + j) * NG + ng;
+        if (t >= tile_end) continue;
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) {
+          float4_t sum = acc[j][mb];
+#pragma unroll
+          for (int k = 1; k < KL; ++k) sum += red[((((k - 1) * NG + ng) * NT + j) * MB + mb) * 64 + lane];
+          const int m = mb * 16 + (lane & 15);
+          const int n = t * 16 + ((lane >> 4) << 2);
+          if (m >= M) continue;
+          if (part)
+            *reinterpret_cast<float4_t*>(part + ((int64_t)blockIdx.y * M + m) * N + n) = sum;
+          else
+            epilogue4<MODE>(epi, m, n, sum);
+        }
+      }
+    }
+    clear();
+  };
+
+  // PF weight stages in flight (a third int8 stage measured no faster than two)
+  constexpr int PF = 2;
+  Wst w[PF];
+  clear();
+  // same issue order as in the loop (activations of the next stage, then weights), so that the
+  // wait before the loop's first LDS store does not cover the weight loads
+  gload_x(0);
+  lstore(0);
+  gload_x(1);
+#pragma unroll
+  for (int st = 0; st < PF - 1; ++st) gload_w(w[st], st);
+  __syncthreads();
+  // Stages are taken PF at a time; surplus stages at the end work on clamped addresses into
+  // accumulators that are never stored.
+  for (int idx = 0; idx < total; idx += PF) {
+#pragma unroll
+    for (int st = 0; st < PF; ++st) {
+      const int i = idx + st;
+      lstore(i + 1);  // fetched during stage i - 1
+      gload_x(i + 2);
+      gload_w(w[(st + PF - 1) % PF], i + PF - 1);
+      compute(w[st], i);
+      if (i < total && (i + 1) % nstages == 0) finish(i);
+      __syncthreads();
+    }
+  }
+}
+
 // sums split-K partials part[s][m][n] in slice order and applies the epilogue
 template <int MODE>
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ part, int S,
@@ -776,9 +976,71 @@ void launch_stream_mb(const void* xp, const void* W, const void* scales, float* 
                      ks_per_split, epi, m_off);
 }
 
+constexpr int SH_GROUP = 12;  // tiles per pass of the shared-activation kernel (4 lanes x 3)
+
+// The shared-activation kernel sweeps K once per pass of SH_GROUP tiles: it is used when the
+// workgroup's tiles fill their passes to at least three quarters.
+bool share_fits(int N, int S) {
+  int G = num_cus() / S;
+  if (G < 1) G = 1;
+  const int tpw = (N / 16 + G - 1) / G;
+  if (tpw <= SH_GROUP) return true;  // one pass, with the tile count per wave chosen to fit
+  const int passes = (tpw + SH_GROUP - 1) / SH_GROUP;
+  return 4 * tpw >= 3 * passes * SH_GROUP;
+}
+
+template <int MB, bool W8, int MODE, int NG, int NT, int U>
+void launch_share_cfg(const void* xp, const void* W, const void* scales, float* part, int S, int M,
+                      int N, int K, int tiles_per_wg, int gx, int ks_per_split, const Epilogue& epi,
+                      hipStream_t s) {
+  using C = ShareCfg<MB, W8, NG, NT, U>;
+  static bool attr_set = false;  // one flag per instantiation
+  if (!attr_set) {
+    if (hipFuncSetAttribute((const void*)linear_share_kernel<MB, W8, MODE, NG, NT, U>,
+                            hipFuncAttributeMaxDynamicSharedMemorySize,
+                            C::LDS_BYTES) != hipSuccess)
+      return;  // the caller's launch check reports the error
+    attr_set = true;
+  }
+  hipLaunchKernelGGL((linear_share_kernel<MB, W8, MODE, NG, NT, U>), dim3(gx, S),
+                     dim3(SH_THREADS), C::LDS_BYTES, s, (const half_t*)xp, W,
+                     (const half_t*)scales, part, M, N, K, tiles_per_wg, ks_per_split, epi);
+}
+
+// 33 .. 64 packed rows, no selection: the shared-activation kernel
+template <int MB, bool W8, int MODE>
+void launch_share(const void* xp, const void* W, const void* scales, float* part, int S, int M,
+                  int N, int K, const Epilogue& epi, hipStream_t s) {
+  const int ntiles = N / 16, nks = K / 32;
+  int G = num_cus() / S;
+  if (G < 1) G = 1;
+  const int tiles_per_wg = (ntiles + G - 1) / G;
+  const int gx = (ntiles + tiles_per_wg - 1) / tiles_per_wg;
+  int ks_per_split = (nks + S - 1) / S;
+  if (W8) ks_per_split = (ks_per_split + 1) & ~1;  // int8 blocks cover two steps
+  // tiles per wave and pass: the fewest that take the workgroup's tiles in one pass, at most 3
+  if (tiles_per_wg <= 4)
+    launch_share_cfg<MB, W8, MODE, 4, 1, 8>(xp, W, scales, part, S, M, N, K, tiles_per_wg, gx,
+                                            ks_per_split, epi, s);
+  else if (tiles_per_wg <= 8)
+    launch_share_cfg<MB, W8, MODE, 4, 2, 4>(xp, W, scales, part, S, M, N, K, tiles_per_wg, gx,
+                                            ks_per_split, epi, s);
+  else
+    launch_share_cfg<MB, W8, MODE, 4, 3, 4>(xp, W, scales, part, S, M, N, K, tiles_per_wg, gx,
+                                            ks_per_split, epi, s);
+}
+
 template <bool W8, int MODE, bool XR = false>
 void launch_stream(const void* xp, const void* W, const void* scales, float* part, int S, int M,
                    int N, int K, const Epilogue& epi, hipStream_t s, int64_t m_off = 0) {
+  if (!XR && MODE != MODE_SELECT && M > 32 && share_fits(N, S)) {
+    constexpr int PM = MODE == MODE_SELECT ? MODE_PLAIN : MODE;
+    if (M > 48)
+      launch_share<4, W8, PM>(xp, W, scales, part, S, M, N, K, epi, s);
+    else
+      launch_share<3, W8, PM>(xp, W, scales, part, S, M, N, K, epi, s);
+    return;
+  }
   switch ((M + 15) / 16) {
     case 1:
       launch_stream_mb<1, W8, MODE, XR>(xp, W, scales, part, S, M, N, K, epi, s, m_off);
@@ -1014,13 +1276,14 @@ namespace {
 int pick_splits(int64_t M, int N, int K, int wbytes) {
   if (M < 1 || M > 64 || N % 16 || K % 64) return 1;
   const int MB = (int)((M + 15) / 16), ntiles = N / 16, nks = K / 32;
-  const int NT = MB <= 2 || wbytes == 1 ? ST_NT : 2 * ST_NT;
-  const int U = MB <= 2 ? 4 : (NT > ST_NT ? 1 : 2);
+  // tiles that share one sweep over the activations, and K steps per stage of the workgroup
+  const int NT = MB > 2 ? SH_GROUP : ST_NT;
+  const int stage = MB > 2 ? 16 : ST_KG * 4;
   int best = 1;
   double best_cost = 0;
   for (int S = 1; S <= 8; S *= 2) {
     const int G = num_cus() / S;
-    if (G < 1 || nks / S < ST_KG * U) break;  // every wave needs a full stage of K steps
+    if (G < 1 || nks / S < stage) break;  // every wave needs a full stage of K steps
     const int tpw = (ntiles + G - 1) / G;
     const int groups = (tpw + NT - 1) / NT;
     const double Ks = (double)K / S;

@@ -236,6 +236,9 @@ LINEAR_SHAPES = [
     (1, 96, 64), (8, 768, 768), (32, 3072, 768), (32, 768, 3072), (33, 2048, 2048),
     (64, 4096, 4096), (17, 50272, 768), (65, 768, 768), (200, 2304, 768), (513, 4096, 1024),
     (129, 1008, 96),
+    # 33 .. 64 rows: the shared-activation kernel with 1, 2 and 3 tiles per wave, a K range
+    # shorter than one stage, and two passes over the workgroup's tiles
+    (64, 1008, 96), (50, 24576, 256), (40, 73728, 128),
     # enough 256 x 256 tiles to take the large tiled kernel, with ragged M and N edges; a bottom
     # block of at most 128 rows goes through the streaming kernel on row-major activations
     (1000, 16400, 128), (4099, 4096, 256), (1124, 16400, 128),
@@ -315,7 +318,8 @@ def test_linear_rejects_bad_shapes(lib):
 
 
 @pytest.mark.parametrize("M,N,K", [(8, 768, 768), (64, 3072, 768), (32, 768, 3072),
-                                   (200, 2304, 768), (48, 4096, 4096),
+                                   (200, 2304, 768), (48, 4096, 4096), (64, 24576, 256),
+                                   (40, 73728, 128),
                                    (1000, 16400, 128), (1124, 16400, 128)])   # large tiled kernel
 def test_linear_w8a16(lib, M, N, K):
     print("w8a16", M, N, K, flush=True)
@@ -338,7 +342,8 @@ def test_linear_w8a16(lib, M, N, K):
 
 
 @pytest.mark.parametrize("M,N,K,S", [(32, 768, 768, 1), (32, 768, 3072, 4), (8, 4096, 4096, 4),
-                                     (33, 2048, 8192, 8), (64, 768, 3072, 3)])
+                                     (33, 2048, 8192, 8), (64, 768, 3072, 3),
+                                     (48, 4608, 2048, 4)])
 @pytest.mark.parametrize("w8", [False, True])
 def test_split_k_partials_and_fused_layernorm(lib, M, N, K, S, w8):
     """msa_linear_partial_* followed by msa_residual_layernorm_f16 equals the oracle's
@@ -592,8 +597,10 @@ def test_target_logprob(lib):
                                    (48, 50272, 256)])
 def test_lm_head_fused_selection_matches_projection_then_select(lib, M, V, K):
     """msa_lm_head_greedy_select_f16 against msa_linear_f16 followed by msa_greedy_select_f16
-    (itself checked against the reference's passes above): identical tokens and finished flags,
-    identical stored logits, scores equal up to the fp32 summation order of the log-sum-exp."""
+    (itself checked against the reference's passes above).  The stand-alone selection runs on
+    the logits the fused call stored: identical tokens and finished flags, scores equal up to the
+    fp32 summation order of the log-sum-exp.  The stored logits equal msa_linear_f16's up to the
+    fp32 summation order over K (above 32 rows the two run different kernels)."""
     print("lm-head select", M, V, K, flush=True)
     x, E = rnd(M, K, seed=3, std=1.0), rnd(V, K, seed=4, std=0.3)
     Ep = pack_w(lib, G(E))
@@ -615,7 +622,8 @@ def test_lm_head_fused_selection_matches_projection_then_select(lib, M, V, K):
         ba = (ctypes.c_int32 * max(1, len(banned)))(*banned)
         sa = (ctypes.c_int32 * max(1, len(stop)))(*stop)
         outs = []
-        for fused in (False, True):
+        fused_logits = None
+        for fused in (True, False):
             fin = None
             if "finished" in c:
                 fin = torch.tensor(c["finished"], dtype=torch.uint8, device=DEV)
@@ -628,18 +636,22 @@ def test_lm_head_fused_selection_matches_projection_then_select(lib, M, V, K):
                 ok(lib.msa_lm_head_greedy_select_f16(
                     P(xp), P(Ep), P(lg), P(ws), M, V, K, temp, ba, len(banned), sa, len(stop),
                     P(fin), force, 2, P(tok[:, 1]), 3, P(sc[:, 1]), 3, None, None), lib)
+                fused_logits = lg
             else:
-                ok(lib.msa_greedy_select_f16(P(logits), V, M, V, temp, ba, len(banned), sa,
+                ok(lib.msa_greedy_select_f16(P(fused_logits), V, M, V, temp, ba, len(banned), sa,
                                              len(stop), P(fin), force, 2, P(tok[:, 1]), 3,
                                              P(sc[:, 1]), 3, None, None), lib)
-                lg = logits
             torch.cuda.synchronize()
-            outs.append((tok.cpu(), sc.cpu(), None if fin is None else fin.cpu(), lg.cpu()))
-        (t0, s0, f0, l0), (t1, s1, f1, l1) = outs
+            outs.append((tok.cpu(), sc.cpu(), None if fin is None else fin.cpu()))
+        (t0, s0, f0), (t1, s1, f1) = outs
         assert torch.equal(t0, t1), c
         assert torch.allclose(s0, s1, atol=2e-5, rtol=1e-6), (c, (s0 - s1).abs().max())
         assert (f0 is None and f1 is None) or torch.equal(f0, f1), c
-        assert torch.equal(l0, l1), c
+        if M <= 32:
+            assert torch.equal(fused_logits, logits), c
+        else:
+            assert_fp16_close(fused_logits, logits.cpu(),
+                              atol=float(logits.float().abs().max()) * 2 ** -10, what="logits")
     # logits are optional, the column may come from the device, and a NaN row yields (0, -inf)
     ln = torch.tensor([2], dtype=torch.int32, device=DEV)
     tok = torch.full((M, 3), -7, dtype=torch.long, device=DEV)
