@@ -5,17 +5,22 @@
 // the order the 64 lanes read it, and the blocks of one 16-row tile follow each other along K.
 // A wave instruction therefore reads one whole KB and a tile's K sweep is one linear stream.
 //
-// Two kernels:
-//   * stream (M <= 64, the decode step): HBM-bound.  A workgroup of 8 waves owns a contiguous
-//     range of 16-row tiles (and, with split-K, one K range); it walks the tiles 4 at a time,
-//     the waves taking interleaved K steps.  Activations come in the matching packed fragment
-//     layout from L2 and every activation fragment is reused for 4 weight tiles.  Fragments
-//     are double buffered several steps deep and the prefetch runs across tile-group
+// Four kernels:
+//   * stream (M <= 32 packed rows, the decode step; also the fused vocabulary projection +
+//     selection up to 64 rows): HBM-bound.  A workgroup of 8 waves owns a contiguous range of
+//     16-row tiles (and, with split-K, one K range); it walks the tiles 3 or 4 at a time, the
+//     waves taking interleaved K steps.  Activations come in the matching packed fragment
+//     layout from L2 and every activation fragment is reused for the tiles of the group.
+//     Fragments are double buffered several steps deep and the prefetch runs across tile-group
 //     boundaries, so the memory pipe never drains while a finished group is reduced across
 //     the waves through LDS (fixed order: results are run-to-run deterministic).
-//   * tiled (any M, the prefill): 128 x 128 x 32 LDS double-buffered tiles, 4 waves of 64 x 64,
+//   * shared-activation stream (33 .. 64 packed rows): the same weight streaming, with the
+//     activation fragments staged once per workgroup in LDS and shared by four waves.
+//   * large tiled (prefill-sized M): 256 x 256 x 64 per workgroup, weights straight from the
+//     packed layout into registers, activations through LDS, v_mfma_f32_16x16x32_f16.
+//   * tiled (shapes in between): 128 x 128 x 32 LDS double-buffered tiles, 4 waves of 64 x 64,
 //     v_mfma_f32_32x32x16_f16.
-// Both share one epilogue that reproduces the reference's fp16 rounding points, and a QKV mode
+// All share one epilogue that reproduces the reference's fp16 rounding points, and a QKV mode
 // that scatters K/V into the per-layer cache and scales Q.
 #include <math.h>
 
