@@ -337,6 +337,19 @@ def main():
     ab = attn_bytes(cfg, B, S_probe)
     achieved = ab / attn_s / 1e9
 
+    # ---- what a plain streaming read reaches on this GPU (context for the fractions of the
+    # published peak): 4 GiB read once per launch by the library's probe kernel
+    probe = torch.empty(1 << 31, dtype=torch.float16, device=dev).zero_()
+    _capi.check(lib.msa_probe_stream_read(probe.data_ptr(), probe.numel() * 2, stream))
+    torch.cuda.synchronize()
+    a0.record()
+    for _ in range(5):
+        _capi.check(lib.msa_probe_stream_read(probe.data_ptr(), probe.numel() * 2, stream))
+    a1.record()
+    torch.cuda.synchronize()
+    stream_read = probe.numel() * 2 / (a0.elapsed_time(a1) / 1e3 / 5) / 1e9
+    del probe
+
     result = {
         "metric": ("decode tokens/sec + % HBM roofline, OPT-6.7B-shape fp16 bs32, 1xMI355X"
                    if args.config == "6.7b" else
@@ -372,6 +385,7 @@ def main():
             "frac": achieved * 1e9 / HBM_PEAK,
             "traffic": ab * ATTN_TRAFFIC_RATIO if args.config == "6.7b" else None,
             "bytes_per_launch": ab, "avg_launch_us": attn_s * 1e6, "context": S_probe,
+            "plain_stream_read_GBps": stream_read,
         },
     }
     if args.torch_eager and not int8:

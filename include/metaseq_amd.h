@@ -218,6 +218,12 @@ int msa_lm_head_greedy_select_f16(const void* x, const void* Ep, void* logits, v
                                   int64_t tok_stride, float* score, int64_t score_stride,
                                   const int32_t* len_dev, void* stream);
 
+/* Measurement aid with no counterpart in the reference: reads `bytes` bytes (a multiple of 16,
+ * 16-byte aligned) of device memory once with 16-byte streaming loads and discards them.  The
+ * benchmark times it to report the read rate this GPU actually sustains beside the published
+ * peak that the roofline fractions are quoted against. */
+int msa_probe_stream_read(const void* p, int64_t bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

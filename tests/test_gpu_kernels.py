@@ -678,3 +678,20 @@ def test_lm_head_fused_selection_matches_projection_then_select(lib, M, V, K):
                                              None, 0, 2, P(tok), 3, P(sc), 3, None, None) == -1
     assert lib.msa_lm_head_greedy_select_f16(P(xp), P(Ep), None, P(ws), 65, V, K, 1.0, ba, 1, ba,
                                              0, None, 0, 2, P(tok), 3, P(sc), 3, None, None) == -1
+
+
+def test_stream_read_probe_runs_and_validates(lib):
+    """The measurement aid reads a buffer once; bad sizes and addresses are rejected."""
+    buf = torch.zeros(1 << 29, dtype=torch.float16, device=DEV)  # 1 GiB
+    ok(lib.msa_probe_stream_read(P(buf), buf.numel() * 2, None), lib)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    ok(lib.msa_probe_stream_read(P(buf), buf.numel() * 2, None), lib)
+    e1.record()
+    torch.cuda.synchronize()
+    rate = buf.numel() * 2 / (e0.elapsed_time(e1) * 1e-3)
+    assert 1e12 < rate < 8.5e12, rate  # it really reads the buffer: bounded by the memory system
+    assert lib.msa_probe_stream_read(P(buf), 24, None) == -1
+    assert lib.msa_probe_stream_read(ctypes.c_void_p(buf.data_ptr() + 2), 32, None) == -1
+    assert lib.msa_probe_stream_read(None, 32, None) == -1
