@@ -48,7 +48,8 @@ int msa_version(void);
  *   fp16: block (t = n/16, ks = k/32) at half offset (t*K/32 + ks)*512; lane l = 16*((k%32)/8) +
  *         n%16 owns halves 8l..8l+7 = W[n][8*(k/8) .. +7].                N % 16 == 0, K % 32 == 0.
  *   int8: block (t, ks8 = k/64) at byte offset (t*K/64 + ks8)*1024; lane l = 16g + r owns 16 bytes:
- *         0..7 = W[16t+r][64ks8 + 8g ..+7], 8..15 = W[16t+r][64ks8 + 32 + 8g ..+7].   K % 64 == 0.
+ *         0..7 = W[16t+r][64ks8 + 8g ..+7], 8..15 = W[16t+r][64ks8 + 32 + 8g ..+7], each byte
+ *         stored biased (q + 128, unsigned).                                     K % 64 == 0.
  * The pack / unpack calls convert from / to row-major [N,K] (src != dst).
  * Activations of at most 64 rows may be PACKED the same way (the MFMA B operand in lane order):
  * with MB = ceil(M/16), element (m,k) sits at half offset

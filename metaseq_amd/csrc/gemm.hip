@@ -160,15 +160,16 @@ __device__ __forceinline__ void epilogue4(const Epilogue& e, int64_t m, int n, f
 
 __device__ __forceinline__ half8_t zero8() { return half8_t{0, 0, 0, 0, 0, 0, 0, 0}; }
 
-// 8 int8 (two dwords) times an fp16 per-row scale -> 8 fp16, each round(q * scale).
-// Bytes are biased to unsigned (q + 128), dropped into the mantissa of fp16 1024.0 (0x6400 | u
-// is exactly 1024 + u), and 1152 is subtracted: q exactly, in packed fp16 arithmetic.  The
-// packed multiply then rounds the exact product q * scale once, as the fp32 route would.
+// 8 packed int8 weights (two dwords) times an fp16 per-row scale -> 8 fp16, each round(q * scale).
+// The packed layout stores every byte biased to unsigned (u = q + 128, done once by the pack
+// kernel).  u is dropped into the mantissa of fp16 1024.0 (0x6400 | u is exactly 1024 + u) and
+// 1152 is subtracted: q exactly, in packed fp16 arithmetic.  The packed multiply then rounds
+// the exact product q * scale once, as the fp32 route would.
 __device__ __forceinline__ half8_t dequant8(uint32_t lo, uint32_t hi, half_t scale) {
   const half2_t bias = {(half_t)1152.0f, (half_t)1152.0f};
   const half2_t sc = {scale, scale};
   half8_t r;
-  const uint32_t w[2] = {lo ^ 0x80808080u, hi ^ 0x80808080u};
+  const uint32_t w[2] = {lo, hi};
 #pragma unroll
   for (int j = 0; j < 2; ++j) {
     const uint32_t p0 = __builtin_amdgcn_perm(0x64646464u, w[j], 0x04010400u);  // bytes 0, 1
@@ -188,7 +189,8 @@ __device__ __forceinline__ half8_t dequant8(uint32_t lo, uint32_t hi, half_t sca
 // lane l = 16*((k%32)/8) + n%16 owns halves l*8 .. l*8+7 = W[n][8*(k/8) .. +7].
 // int8: block (t, ks8 = k/64) at bytes ((t * K/64 + ks8) * 1024); lane l = 16*g + r owns 16 bytes:
 // bytes 0..7 = W[16t+r][64*ks8 + 8g .. +7] and bytes 8..15 = W[16t+r][64*ks8 + 32 + 8g .. +7],
-// i.e. the A fragments of the two 32-wide steps the block covers.
+// i.e. the A fragments of the two 32-wide steps the block covers; every byte is stored as
+// q + 128.
 __global__ __launch_bounds__(256) void pack_f16_kernel(const half_t* __restrict__ src,
                                                        half_t* __restrict__ dst, int N, int K,
                                                        bool unpack) {
@@ -215,10 +217,12 @@ __global__ __launch_bounds__(256) void pack_i8_kernel(const int8_t* __restrict__
   const int64_t blk = piece >> 7;
   const int ks8 = (int)(blk % nks8), t = (int)(blk / nks8);
   const int64_t rm = ((int64_t)t * 16 + (lane & 15)) * K + ks8 * 64 + half * 32 + (lane >> 4) * 8;
-  if (unpack)
-    *reinterpret_cast<uint2*>(dst + rm) = *reinterpret_cast<const uint2*>(src + piece * 8);
-  else
-    *reinterpret_cast<uint2*>(dst + piece * 8) = *reinterpret_cast<const uint2*>(src + rm);
+  // packed bytes are q + 128 (the sign bit flipped): the kernels expand them without a
+  // sign fix-up
+  uint2 v = *reinterpret_cast<const uint2*>(unpack ? src + piece * 8 : src + rm);
+  v.x ^= 0x80808080u;
+  v.y ^= 0x80808080u;
+  *reinterpret_cast<uint2*>(unpack ? dst + rm : dst + piece * 8) = v;
 }
 
 // ---- stream kernel (M <= 64) --------------------------------------------------------------

@@ -223,9 +223,11 @@ def test_pack_roundtrip_and_layout(lib):
     ok(lib.msa_unpack_weight_i8(P(qp), P(qb), 32, 128, None), lib)
     torch.cuda.synchronize()
     assert torch.equal(qb.cpu(), q)
-    # block (t, ks8): lane 16g+r holds [k = 64ks8+8g..+7 | k = 64ks8+32+8g..+7] of row 16t+r
+    # block (t, ks8): lane 16g+r holds [k = 64ks8+8g..+7 | k = 64ks8+32+8g..+7] of row 16t+r,
+    # every byte stored as q + 128 (i.e. with the sign bit flipped)
     want = q.view(2, 16, 2, 2, 4, 8).permute(0, 2, 4, 1, 3, 5).contiguous()
-    assert torch.equal(qp.cpu().view(-1), want.view(-1))
+    want = (want.view(-1).to(torch.int16) + 128).to(torch.uint8)
+    assert torch.equal(qp.cpu().view(-1).view(torch.uint8), want)
     x = torch.zeros(4, 40, dtype=torch.float16, device=DEV)
     assert lib.msa_pack_weight_f16(P(x), P(x), 16, 32, None) == -1      # aliased
     assert lib.msa_pack_weight_f16(P(x), P(back), 24, 32, None) == -1   # N % 16
