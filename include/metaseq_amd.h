@@ -137,7 +137,9 @@ int msa_linear_w8a16(const void* x, const int8_t* Wq, const void* scales, const 
 /* Split-K form for the decode step (1 <= M <= 64, MSA_IN_PACKED required): K is cut into S
  * ranges and part[s][m][n] (fp32, [S, M, N]) receives the exact fp32 partial sums of range s;
  * the consumer adds them in slice order (msa_residual_layernorm_f16).  Used where N alone gives
- * the chip too few weight tiles (out_proj, fc2).  msa_linear_default_splits suggests S. */
+ * the chip too few weight tiles (out_proj, fc2).  msa_linear_default_splits suggests S.  The
+ * ranges hold ceil(K/32 / S) 32-wide steps (rounded up to an even count for int8); an S that would
+ * leave the last range(s) empty is rejected. */
 int msa_linear_partial_f16(const void* x, const void* Wp, float* part, int64_t M, int N, int K,
                            int S, unsigned flags, void* stream);
 int msa_linear_partial_w8a16(const void* x, const int8_t* Wq, const void* scales, float* part,

@@ -1152,6 +1152,16 @@ int partial_entry(const char* name, const void* x, const void* W, const void* sc
               "%s: needs packed activations and 1 <= M <= 64 (M=%lld)", name, (long long)M);
   MSA_REQUIRE(S >= 1 && S <= K / (W8 ? 64 : 32), MSA_ERR_INVALID_ARG,
               "%s: S=%d outside 1..%d", name, S, K / (W8 ? 64 : 32));
+  {
+    // the ranges are ceil(steps / S) 32-wide steps each (an even count for int8): every one of
+    // the S slices must get at least one step, or it would stay unwritten
+    const int nks = K / 32;
+    int per = (nks + S - 1) / S;
+    if (W8) per = (per + 1) & ~1;
+    MSA_REQUIRE((int64_t)(S - 1) * per < nks, MSA_ERR_INVALID_ARG,
+                "%s: S=%d leaves a K range empty (K=%d is cut into ranges of %d elements)", name, S,
+                K, per * 32);
+  }
   Epilogue e{};
   launch_stream<W8, MODE_PLAIN>(x, W, scales, part, S, (int)M, N, K, e, (hipStream_t)stream);
   MSA_CHECK_LAUNCH(name);

@@ -62,3 +62,8 @@ def test_argument_validation_needs_no_gpu():
     assert lib.msa_attention_f16(one, one, one, None, 0, one, 1, 1, 64, 2, 9, 10, 0, None, None) == -2
     with pytest.raises(ValueError):
         _capi.check(-2, lib)
+    # split-K counts that would leave a slice of the partial sums unwritten are refused
+    assert lib.msa_linear_partial_f16(one, one, one, 58, 50272, 160, 4, 2, None) == -1
+    assert b"leaves a K range empty" in lib.msa_last_error()
+    assert lib.msa_linear_partial_w8a16(one, one, one, one, 52, 8000, 768, 8, 2, None) == -1
+    assert b"leaves a K range empty" in lib.msa_last_error()
