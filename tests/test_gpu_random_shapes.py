@@ -1,0 +1,131 @@
+"""Seeded random shapes through the C ABI: the decode GEMM paths (1 .. 64 packed rows, fp16 and
+int8 weights, with and without split-K) and both attention kernels (one query per row over a
+history; a block of queries, causal, optionally appended to a history, optionally with a key
+padding mask), each against the same arithmetic written with torch ops on the device.  The fixed
+shapes of test_gpu_kernels.py pin the layouts and rounding points; these cases sweep the launch
+geometry (tiles per workgroup, K ranges shorter than a stage, ragged tiles, cache capacities)."""
+import random
+
+import pytest
+import torch
+
+from tests.test_gpu_kernels import pack_act
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+def r16(t):
+    return t.half().float()
+
+
+@pytest.fixture(scope="module")
+def lib():
+    from metaseq_amd import _capi
+    return _capi.load()
+
+
+def test_decode_gemm_random_shapes(lib):
+    rng = random.Random(7)
+    ran = 0
+    for it in range(60):
+        M = rng.randint(1, 64)
+        N = 16 * rng.choice([1, 3, 7, 20, 63, 64, 100, 257, 500, 1000, 2304, 3142])
+        w8 = rng.random() < 0.5
+        K = (64 if w8 else 32) * rng.choice([1, 2, 3, 5, 8, 12, 17, 32, 48, 64])
+        S = rng.choice([1, 1, 2, 3, 4, 8])
+        print("gemm case", it, M, N, K, "int8" if w8 else "fp16", "S", S, flush=True)
+        g = torch.Generator().manual_seed(it)
+        x = (torch.randn(M, K, generator=g) * 0.5).half()
+        xp = pack_act(x).to(DEV)
+        if w8:
+            q = torch.randint(-127, 128, (N, K), generator=g, dtype=torch.int8)
+            sc = (torch.rand(N, generator=g) * 0.01 + 0.001).half()
+            Wd = (q.float() * sc.float()[:, None]).half()
+            qd, scd = q.to(DEV), sc.to(DEV)
+            Wp = torch.empty_like(qd)
+            assert lib.msa_pack_weight_i8(qd.data_ptr(), Wp.data_ptr(), N, K, None) == 0
+        else:
+            Wd = (torch.randn(N, K, generator=g) * 0.05).half()
+            wd = Wd.to(DEV)
+            Wp = torch.empty_like(wd)
+            assert lib.msa_pack_weight_f16(wd.data_ptr(), Wp.data_ptr(), N, K, None) == 0
+        ref = x.to(DEV).float() @ Wd.to(DEV).float().t()
+        if S == 1:
+            b = (torch.randn(N, generator=g) * 0.1).half().to(DEV)
+            y = torch.full((M, N), float("nan"), dtype=torch.float16, device=DEV)
+            if w8:
+                rc = lib.msa_linear_w8a16(xp.data_ptr(), Wp.data_ptr(), scd.data_ptr(),
+                                          b.data_ptr(), None, y.data_ptr(), M, N, K, 2, None)
+            else:
+                rc = lib.msa_linear_f16(xp.data_ptr(), Wp.data_ptr(), b.data_ptr(), None,
+                                        y.data_ptr(), M, N, K, 2, None)
+            assert rc == 0, lib.msa_last_error()
+            torch.cuda.synchronize()
+            got, want = y.float(), r16(r16(ref) + b.float())
+        else:
+            part = torch.full((S, M, N), float("nan"), dtype=torch.float32, device=DEV)
+            if w8:
+                rc = lib.msa_linear_partial_w8a16(xp.data_ptr(), Wp.data_ptr(), scd.data_ptr(),
+                                                  part.data_ptr(), M, N, K, S, 2, None)
+            else:
+                rc = lib.msa_linear_partial_f16(xp.data_ptr(), Wp.data_ptr(), part.data_ptr(), M,
+                                                N, K, S, 2, None)
+            if rc != 0:  # a split count the K range cannot be cut into: refused, nothing ran
+                assert b"outside" in lib.msa_last_error() or b"empty" in lib.msa_last_error()
+                continue
+            torch.cuda.synchronize()
+            got, want = part.sum(0), ref  # every slice written (no NaN left), sums exact in fp32
+        ran += 1
+        assert torch.isfinite(got).all(), (it, "unwritten or non-finite output")
+        err = float((got - want).abs().max())
+        assert err <= max(1e-3, float(want.abs().max()) * 2e-3), (it, err)
+    assert ran >= 40
+
+
+def test_attention_random_shapes(lib):
+    rng = random.Random(11)
+    for it in range(45):
+        hd, H, B = rng.choice([64, 128]), rng.choice([1, 2, 3, 5]), rng.choice([1, 2, 3, 7, 33])
+        T = rng.choice([1, 1, 1, 2, 17, 64, 65, 127, 128, 129, 200, 300])
+        S0 = (rng.choice([0, 0, 1, 5, 63, 64, 100, 511, 700]) if T > 1
+              else rng.choice([0, 1, 7, 63, 64, 255, 256, 1000, 2047]))
+        S = S0 + T
+        S_cap = S + rng.choice([0, 1, 9, 64])
+        masked = rng.random() < 0.4
+        print("attention case", it, "B", B, "H", H, "hd", hd, "T", T, "S0", S0, "cap", S_cap,
+              "mask", masked, flush=True)
+        g = torch.Generator(device=DEV).manual_seed(it)
+        D = H * hd
+        q = (torch.randn(B * T, D, device=DEV, generator=g) * 0.3).half()
+        Kc = torch.randn(B, H, S_cap, hd, device=DEV, generator=g).half()
+        Vc = torch.randn(B, H, S_cap, hd, device=DEV, generator=g).half()
+        # rows past the history hold NaN: none of them may reach the result
+        Kc[:, :, S:] = float("nan")
+        Vc[:, :, S:] = float("nan")
+        mask = None
+        if masked:
+            mask = torch.zeros(B, S, dtype=torch.bool, device=DEV)
+            for b in range(B):
+                for _ in range(rng.randint(0, 3)):
+                    mask[b, rng.randint(1, S - 1) if S > 1 else 0] = True
+            mask[:, 0] = False  # key 0 stays visible: no fully masked row
+        qq = q.float().view(B, T, H, hd).permute(0, 2, 1, 3)
+        s = r16(qq @ Kc[:, :, :S].float().transpose(-1, -2))
+        s = s + torch.full((T, S), float("-inf"), device=DEV).triu(S0 + 1)
+        if mask is not None:
+            s = s.masked_fill(mask[:, None, None, :], float("-inf"))
+        p = r16(torch.softmax(s, -1, dtype=torch.float32))
+        want = r16(p @ Vc[:, :, :S].float()).permute(0, 2, 1, 3).reshape(B * T, D)
+        out = torch.full((B * T, D), float("nan"), dtype=torch.float16, device=DEV)
+        dm = None if mask is None else mask.to(torch.uint8)
+        rc = lib.msa_attention_f16(q.data_ptr(), Kc.data_ptr(), Vc.data_ptr(),
+                                   None if dm is None else dm.data_ptr(),
+                                   0 if dm is None else dm.stride(0), out.data_ptr(), B, H, hd, T,
+                                   S0, S_cap, 0, None, None)
+        assert rc == 0, lib.msa_last_error()
+        torch.cuda.synchronize()
+        assert torch.isfinite(out.float()).all(), it
+        err = float((out.float() - want).abs().max())
+        # a 1-ulp flip of an fp16 score scales its probability by up to e^(2^-7)
+        assert err <= float(want.abs().max()) * 2 ** -6 + 1e-3, (it, err)
