@@ -42,6 +42,7 @@ struct Epilogue {
   half_t* Kc;
   half_t* Vc;
   int T, H, hd, S0, S_cap;
+  int hd_shift;  // log2(hd) if hd is a power of two, else -1
   const int32_t* len_dev;  // if set (T == 1): the append position is read from the device
   float qscale;
   // MODE_SELECT: greedy selection over the output row instead of (or besides) storing it
@@ -136,8 +137,10 @@ __device__ __forceinline__ void epilogue4(const Epilogue& e, int64_t m, int n, f
     else
       *reinterpret_cast<half4_t*>(e.y + m * e.N + n) = o;
   } else {
+    // index arithmetic in 32 bits, without 64-bit division: the row count is below 2^31, the
+    // thirds are found by comparison, and a power-of-two head size (the usual case) is a shift
     const int D = e.H * e.hd;
-    const int part = n / D, c = n - part * D;  // 0 = K, 1 = V, 2 = Q
+    const int part = (n >= D) + (n >= 2 * D), c = n - part * D;  // 0 = K, 1 = V, 2 = Q
     half4_t o;
     if (part == 2) {
 #pragma unroll
@@ -146,12 +149,13 @@ __device__ __forceinline__ void epilogue4(const Epilogue& e, int64_t m, int n, f
     } else {
 #pragma unroll
       for (int i = 0; i < 4; ++i) o[i] = (half_t)t[i];
-      const int h = c / e.hd, d = c - h * e.hd;
-      const int64_t b = m / e.T, tt = m - b * e.T;
+      const int h = e.hd_shift >= 0 ? c >> e.hd_shift : c / e.hd, d = c - h * e.hd;
+      const int mi = (int)m;
+      const int b = e.T == 1 ? mi : mi / e.T, tt = mi - b * e.T;
       const int s0 = e.len_dev ? *e.len_dev : e.S0;
       if (s0 + tt < e.S_cap) {
         half_t* dst = (part == 0 ? e.Kc : e.Vc) +
-                      ((b * e.H + h) * (int64_t)e.S_cap + s0 + tt) * e.hd + d;
+                      (((int64_t)b * e.H + h) * e.S_cap + s0 + tt) * e.hd + d;
         *reinterpret_cast<half4_t*>(dst) = o;
       }
     }
@@ -1193,6 +1197,7 @@ int qkv_entry(const char* name, const void* x, const void* W, const void* scales
   e.T = T;
   e.H = H;
   e.hd = hd;
+  e.hd_shift = (hd & (hd - 1)) == 0 ? __builtin_ctz((unsigned)hd) : -1;
   e.S0 = S0;
   e.len_dev = len_dev;
   e.S_cap = S_cap;
