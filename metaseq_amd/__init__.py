@@ -5,12 +5,12 @@ from .dictionary import Dictionary
 from .hub_utils import GeneratorInterface
 from .kv_cache import KVCache
 from .sequence_generator import SequenceGenerator
-from .synthetic import random_prompts, random_state_dict
+from .synthetic import iter_random_state_dict, random_prompts, random_state_dict
 from .transformer_decoder import ModelParallelTransformerDecoder, TransformerDecoder
 from .transformer_lm import TransformerLanguageModel
 
 __all__ = [
     "OPTConfig", "opt_config", "Dictionary", "GeneratorInterface", "KVCache", "SequenceGenerator", "random_prompts",
-    "random_state_dict", "TransformerDecoder", "ModelParallelTransformerDecoder",
+    "random_state_dict", "iter_random_state_dict", "TransformerDecoder", "ModelParallelTransformerDecoder",
     "TransformerLanguageModel",
 ]

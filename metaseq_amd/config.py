@@ -5,6 +5,10 @@ metaseq/modules/transformer_decoder_layer.py:44-98), and the OPT size table
 from dataclasses import dataclass, replace
 
 
+# head sizes the attention kernels are instantiated for (lanes per key row = head_dim / 8)
+SUPPORTED_HEAD_DIMS = (64, 128)
+
+
 @dataclass
 class OPTConfig:
     decoder_layers: int
@@ -38,13 +42,22 @@ class OPTConfig:
     def head_dim(self):
         return self.decoder_embed_dim // self.decoder_attention_heads
 
+    def require_supported_head_dim(self):
+        """Raised when a decoder is built, before any weight is allocated or packed."""
+        if self.head_dim not in SUPPORTED_HEAD_DIMS:
+            raise NotImplementedError(
+                "head_dim %d (decoder_embed_dim %d / %d heads) is not supported: the attention "
+                "kernels are built for head_dim %s" % (
+                    self.head_dim, self.decoder_embed_dim, self.decoder_attention_heads,
+                    " or ".join(str(h) for h in SUPPORTED_HEAD_DIMS)))
 
-# name -> (layers, embed dim, heads)
+
+# name -> (layers, embed dim, heads).  OPT-2.7B (32 layers, 2560 / 32 heads = head_dim 80) is
+# left out: no attention kernel is built for that head size.
 _OPT_SIZES = {
     "125m": (12, 768, 12),
     "350m": (24, 1024, 16),
     "1.3b": (24, 2048, 32),
-    "2.7b": (32, 2560, 32),
     "6.7b": (32, 4096, 32),
     "13b": (40, 5120, 40),
     "30b": (48, 7168, 56),

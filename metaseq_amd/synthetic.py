@@ -7,15 +7,17 @@ order from one generator: matrices, embeddings and biases ~ N(0, 0.02), LayerNor
 1 + N(0, 0.02), and the padding rows of both embedding tables are zero as in the reference
 (metaseq/modules/positional_embedding.py:46-47).
 """
-from typing import Dict
+from typing import Dict, Iterator, Tuple
 
 import torch
 
 from .config import OPTConfig
 
 
-def random_state_dict(cfg: OPTConfig, seed: int = 1234, dtype=torch.float16,
-                      device="cpu", std: float = 0.02) -> Dict[str, torch.Tensor]:
+def iter_random_state_dict(cfg: OPTConfig, seed: int = 1234, dtype=torch.float16,
+                           device="cpu", std: float = 0.02) -> Iterator[Tuple[str, torch.Tensor]]:
+    """Yields (name, tensor) one at a time, in the fixed drawing order, so that a model far
+    larger than the spare memory can be filled without ever holding a second copy of it."""
     device = torch.device(device)
     gen = torch.Generator(device=device)
     gen.manual_seed(seed)
@@ -26,31 +28,36 @@ def random_state_dict(cfg: OPTConfig, seed: int = 1234, dtype=torch.float16,
         return t.to(dtype)
 
     D, F, V = cfg.decoder_embed_dim, cfg.decoder_ffn_embed_dim, cfg.vocab_size
-    sd: Dict[str, torch.Tensor] = {}
-    sd["decoder.version"] = torch.tensor([3.0])
+    yield "decoder.version", torch.tensor([3.0])
     e = normal(V, D)
     e[cfg.padding_idx].zero_()
-    sd["decoder.embed_tokens.weight"] = e
+    yield "decoder.embed_tokens.weight", e
+    del e
     p = normal(cfg.max_target_positions + cfg.padding_idx + 1, D)
     p[cfg.padding_idx].zero_()
-    sd["decoder.embed_positions.weight"] = p
+    yield "decoder.embed_positions.weight", p
+    del p
     for i in range(cfg.decoder_layers):
         pre = f"decoder.layers.{i}."
-        sd[pre + "self_attn_layer_norm.weight"] = normal(D, mean=1.0)
-        sd[pre + "self_attn_layer_norm.bias"] = normal(D)
-        sd[pre + "self_attn.qkv_proj.weight"] = normal(3 * D, D)
-        sd[pre + "self_attn.qkv_proj.bias"] = normal(3 * D)
-        sd[pre + "self_attn.out_proj.weight"] = normal(D, D)
-        sd[pre + "self_attn.out_proj.bias"] = normal(D)
-        sd[pre + "final_layer_norm.weight"] = normal(D, mean=1.0)
-        sd[pre + "final_layer_norm.bias"] = normal(D)
-        sd[pre + "fc1.weight"] = normal(F, D)
-        sd[pre + "fc1.bias"] = normal(F)
-        sd[pre + "fc2.weight"] = normal(D, F)
-        sd[pre + "fc2.bias"] = normal(D)
-    sd["decoder.layer_norm.weight"] = normal(D, mean=1.0)
-    sd["decoder.layer_norm.bias"] = normal(D)
-    return sd
+        yield pre + "self_attn_layer_norm.weight", normal(D, mean=1.0)
+        yield pre + "self_attn_layer_norm.bias", normal(D)
+        yield pre + "self_attn.qkv_proj.weight", normal(3 * D, D)
+        yield pre + "self_attn.qkv_proj.bias", normal(3 * D)
+        yield pre + "self_attn.out_proj.weight", normal(D, D)
+        yield pre + "self_attn.out_proj.bias", normal(D)
+        yield pre + "final_layer_norm.weight", normal(D, mean=1.0)
+        yield pre + "final_layer_norm.bias", normal(D)
+        yield pre + "fc1.weight", normal(F, D)
+        yield pre + "fc1.bias", normal(F)
+        yield pre + "fc2.weight", normal(D, F)
+        yield pre + "fc2.bias", normal(D)
+    yield "decoder.layer_norm.weight", normal(D, mean=1.0)
+    yield "decoder.layer_norm.bias", normal(D)
+
+
+def random_state_dict(cfg: OPTConfig, seed: int = 1234, dtype=torch.float16,
+                      device="cpu", std: float = 0.02) -> Dict[str, torch.Tensor]:
+    return dict(iter_random_state_dict(cfg, seed, dtype, device, std))
 
 
 def random_prompts(cfg: OPTConfig, batch: int, prompt_len: int, seed: int = 4321,

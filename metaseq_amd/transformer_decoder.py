@@ -107,6 +107,7 @@ class TransformerDecoder(nn.Module):
     def __init__(self, cfg: OPTConfig, state_dict: Optional[Dict[str, torch.Tensor]] = None,
                  device="cuda"):
         super().__init__()
+        cfg.require_supported_head_dim()
         self.cfg = cfg
         self.args = cfg  # the reference exposes its namespace as .args
         D, F = cfg.decoder_embed_dim, cfg.decoder_ffn_embed_dim
@@ -155,6 +156,41 @@ class TransformerDecoder(nn.Module):
                 lin.packed, lin.qweight, lin.scales = False, None, None
         self._lm_head = None
         return super().load_state_dict(sd, strict=strict, **kw)
+
+    def load_tensors(self, named_tensors, quantize_int8=False):
+        """Streaming form of ``load_state_dict`` for checkpoints that leave no room for a second
+        copy: ``named_tensors`` yields (reference parameter name, tensor) pairs, each is copied
+        into place and may be freed by the producer right away.  With ``quantize_int8`` every
+        linear layer is quantised and packed as soon as its weight has arrived, so the fp16
+        matrices never all exist at once.  Every parameter must arrive exactly once."""
+        lib = self._lib = self._lib or _capi.load()
+        if quantize_int8:
+            self.cfg.quantize_int8 = True
+        own = dict(self.named_parameters())
+        linears = dict(self._linears())
+        for lin in linears.values():
+            if lin.packed or lin.qweight is not None:
+                raise RuntimeError("load_tensors needs a freshly constructed decoder")
+        self._lm_head = None
+        seen = set()
+        for name, t in named_tensors:
+            if name.startswith("decoder."):
+                name = name[len("decoder."):]
+            if name in ("version", "output_projection.weight"):
+                continue
+            if name not in own or name in seen:
+                raise KeyError("unexpected or repeated parameter %r" % name)
+            if tuple(own[name].shape) != tuple(t.shape):
+                raise ValueError("shape of %s: expected %s, got %s"
+                                 % (name, tuple(own[name].shape), tuple(t.shape)))
+            own[name].data.copy_(t)
+            seen.add(name)
+            if quantize_int8 and name.endswith(".weight") and name[:-len(".weight")] in linears:
+                linears[name[:-len(".weight")]].prepare_(lib, int8=True)
+        missing = sorted(set(own) - seen)
+        if missing:
+            raise KeyError("missing parameters: %s" % ", ".join(missing[:8]))
+        return self
 
     def state_dict(self, *args, **kwargs):
         """Reference-layout (row-major, fp16) state dict; quantised matrices come back as their

@@ -6,7 +6,10 @@ leg compare the HIP path against.  It is written from the reference's sources (c
 per function, paths relative to the metaseq tree) in plain PyTorch ops and runs on
 any torch device.
 
-Two arithmetic modes, selected by ``dtype``:
+Two arithmetic modes, selected by ``dtype`` (and, orthogonally, ``lean=True`` keeps weights
+and the key/value history stored in ``dtype`` and upcasts them where they are used, and walks
+the attention over batch rows in chunks: the same values at a fraction of the memory, for the
+30B / 66B shapes):
 
 * ``torch.float32`` - everything in fp32.
 * ``torch.float16`` - "rounding faithful": every tensor the reference materialises
@@ -119,6 +122,23 @@ def linear(x, w, b, r):
     return y
 
 
+class _Weights:
+    """name -> fp32 tensor; the stored tensor may be narrower (lean mode) and is then upcast on
+    access, which changes no value."""
+
+    def __init__(self, tensors):
+        self.t = tensors
+
+    def __getitem__(self, k):
+        return self.t[k].float()
+
+    def raw(self, k):
+        return self.t[k]
+
+    def __contains__(self, k):
+        return k in self.t
+
+
 class OracleDecoder:
     """Restates ModelParallelTransformerDecoder.forward at tensor-parallel size 1
     (metaseq/models/transformer_decoder.py:494-537) with the inference branch of
@@ -133,17 +153,29 @@ class OracleDecoder:
     """
 
     def __init__(self, cfg: OracleConfig, state_dict: Dict[str, torch.Tensor],
-                 dtype=torch.float32, device="cpu"):
+                 dtype=torch.float32, device="cpu", lean=False, native_matmul=False):
         self.cfg = cfg
         self.dtype = dtype
         self.device = torch.device(device)
-        # weights are held as fp32 copies of values already rounded to `dtype`
-        self.w = {
-            k: v.detach().to(self.device).to(dtype).float()
+        self.lean = lean
+        # native_matmul: matrix products are handed to torch in `dtype` itself (what the
+        # reference does on a GPU: the BLAS accumulates in fp32 and rounds once on output)
+        # instead of as fp32 products of `dtype` values that are rounded afterwards.  Same
+        # rounding points, another summation order: a second valid evaluation of the reference,
+        # used to measure how far two such evaluations drift apart.
+        self.native_matmul = native_matmul and dtype != torch.float32
+        # weights are values already rounded to `dtype`, held as fp32 copies - or, when lean, in
+        # `dtype` itself (no copy if the caller's tensor already is) and upcast at each use
+        self.w = _Weights({
+            k: (v.detach().to(self.device).to(dtype) if lean
+                else v.detach().to(self.device).to(dtype).float())
             for k, v in state_dict.items()
             if v.is_floating_point()
-        }
+        })
         self.layer_ids = [str(uuid.uuid4()) for _ in range(cfg.decoder_layers)]
+        # lean: rows of the batch whose attention is evaluated together (bounds the fp32
+        # score tensors to about 2 GB)
+        self.attn_chunk_bytes = 2 << 30
 
     # -- rounding point --------------------------------------------------
     def _r(self, t: torch.Tensor) -> torch.Tensor:
@@ -155,12 +187,21 @@ class OracleDecoder:
         # transformer_decoder.py:430-434 with learned_positional_embedding.py:25-28
         return min(
             self.cfg.max_target_positions,
-            self.w["decoder.embed_positions.weight"].shape[0] - self.cfg.padding_idx - 1,
+            self.w.raw("decoder.embed_positions.weight").shape[0] - self.cfg.padding_idx - 1,
         )
 
     # -- linear: matmul -> round -> (+ bias -> round) ----------------------
     def _linear(self, x, wname, bname=None):
-        return linear(x, self.w[wname], self.w[bname] if bname is not None else None, self._r)
+        b = self.w[bname] if bname is not None else None
+        if self.native_matmul:
+            y = (x.to(self.dtype) @ self.w.raw(wname).to(self.dtype).t()).float()
+            return self._r(y + b) if b is not None else y
+        return linear(x, self.w[wname], b, self._r)
+
+    def _bmm(self, a, b):
+        if self.native_matmul:
+            return torch.bmm(a.to(self.dtype), b.to(self.dtype)).float()
+        return self._r(torch.bmm(a, b))
 
     def attention_core(self, q, k, v, B, attn_mask=None, key_padding_mask=None):
         """multihead_attention.py:492-543 on q [B*H, T, hd] (already scaled) and
@@ -168,7 +209,7 @@ class OracleDecoder:
         back to the activation dtype, weighted sum of values."""
         BH, T, _ = q.shape
         H, S = BH // B, k.shape[1]
-        s = self._r(torch.bmm(q, k.transpose(1, 2)))  # :492
+        s = self._bmm(q, k.transpose(1, 2))  # :492
         if attn_mask is not None:
             s = s + attn_mask.unsqueeze(0)  # :516-518
         if key_padding_mask is not None:  # :520-531
@@ -177,7 +218,25 @@ class OracleDecoder:
                 key_padding_mask.unsqueeze(1).unsqueeze(2).to(torch.bool), float("-inf")
             ).view(BH, T, S)
         pr = self._r(F.softmax(s, dim=-1, dtype=torch.float32))  # :533-534
-        return self._r(torch.bmm(pr, v))  # :543
+        return self._bmm(pr, v)  # :543
+
+    def _attention_rows(self, q, k, v, B, attn_mask, key_padding_mask):
+        """attention_core over the whole batch, or (lean) over groups of batch rows: rows are
+        independent, so the values are the same."""
+        BH, T, _ = q.shape
+        H, S = BH // B, k.shape[1]
+        rows = B
+        if self.lean:
+            rows = max(1, min(B, int(self.attn_chunk_bytes // max(1, H * T * S * 4))))
+        if rows >= B:
+            return self.attention_core(q, k, v, B, attn_mask, key_padding_mask)
+        out = []
+        for b0 in range(0, B, rows):
+            b1 = min(B, b0 + rows)
+            kp = None if key_padding_mask is None else key_padding_mask[b0:b1]
+            out.append(self.attention_core(q[b0 * H:b1 * H], k[b0 * H:b1 * H],
+                                           v[b0 * H:b1 * H], b1 - b0, attn_mask, kp))
+        return torch.cat(out, dim=0)
 
     def _attention(self, i, x, incremental_state, attn_mask, key_padding_mask):
         """multihead_attention.py:278-556, inference branch. x is [T, B, D]."""
@@ -195,13 +254,16 @@ class OracleDecoder:
             key = self.layer_ids[i] + ".attn_state"
             saved = incremental_state.get(key, {})
             if "prev_key" in saved:  # :451-467
-                k = torch.cat([saved["prev_key"].view(B * H, -1, hd), k], dim=1)
-                v = torch.cat([saved["prev_value"].view(B * H, -1, hd), v], dim=1)
-            saved["prev_key"] = k.view(B, H, -1, hd)
-            saved["prev_value"] = v.view(B, H, -1, hd)
+                k = torch.cat([saved["prev_key"].view(B * H, -1, hd).float(), k], dim=1)
+                v = torch.cat([saved["prev_value"].view(B * H, -1, hd).float(), v], dim=1)
+            # the history holds values already rounded to `dtype`: storing it in `dtype` (lean)
+            # loses nothing
+            keep = (lambda t: t.to(self.dtype)) if self.lean else (lambda t: t)
+            saved["prev_key"] = keep(k.view(B, H, -1, hd))
+            saved["prev_value"] = keep(v.view(B, H, -1, hd))
             saved["prev_key_padding_mask"] = key_padding_mask
             incremental_state[key] = saved
-        o = self.attention_core(q, k, v, B, attn_mask, key_padding_mask)
+        o = self._attention_rows(q, k, v, B, attn_mask, key_padding_mask)
         o = o.transpose(0, 1).contiguous().view(T, B, D)  # :552
         return self._linear(o, p + "out_proj.weight", None), self.w[p + "out_proj.bias"]
 
@@ -229,11 +291,11 @@ class OracleDecoder:
         if self_attn_padding_mask is None and bool(tokens.eq(cfg.padding_idx).any()):
             self_attn_padding_mask = tokens.eq(cfg.padding_idx)  # :357-361
         positions = make_positions(tokens, cfg.padding_idx)
-        pos_emb = F.embedding(positions, self.w["decoder.embed_positions.weight"])
+        pos_emb = F.embedding(positions, self.w.raw("decoder.embed_positions.weight")).float()
         if incremental_state:  # non-empty dict == decode step (:324-327)
             tokens = tokens[:, -1:]
             pos_emb = pos_emb[:, -1:]
-        emb = F.embedding(tokens, self.w["decoder.embed_tokens.weight"])
+        emb = F.embedding(tokens, self.w.raw("decoder.embed_tokens.weight")).float()
         x = self._r(emb + pos_emb)  # embed_scale == 1.0 (:89, :329-335)
         x = x.transpose(0, 1).contiguous()  # [T, B, D] (:341)
         T = x.shape[0]
@@ -252,7 +314,7 @@ class OracleDecoder:
 
     def output_layer(self, features):
         """transformer_decoder.py:398-428: tied projection, no bias."""
-        return self._r(features @ self.w["decoder.embed_tokens.weight"].t())
+        return self._linear(features, "decoder.embed_tokens.weight")
 
     def forward(self, prev_output_tokens, incremental_state=None, features_only=False,
                 self_attn_padding_mask=None):

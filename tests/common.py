@@ -16,5 +16,5 @@ def oracle_cfg(cfg):
                         cfg.padding_idx, cfg.eos_idx)
 
 
-def make_oracle(cfg, sd, dtype=torch.float32, device="cpu"):
-    return OracleDecoder(oracle_cfg(cfg), sd, dtype=dtype, device=device)
+def make_oracle(cfg, sd, dtype=torch.float32, device="cpu", lean=False):
+    return OracleDecoder(oracle_cfg(cfg), sd, dtype=dtype, device=device, lean=lean)

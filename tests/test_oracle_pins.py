@@ -230,3 +230,25 @@ def test_quantize_int8_closed_form():
     assert (deq.float() - w.float()).abs().max() <= float(s.float().max()) * 0.51
     # the largest-magnitude entry of each row maps to +-127
     assert torch.equal(q.abs().amax(1), torch.full((6,), 127, dtype=torch.int8))
+
+
+def test_lean_mode_changes_no_value():
+    """lean=True (weights and history stored in fp16, attention walked over batch rows in
+    chunks) is a memory layout of the same arithmetic: logits and tokens equal the plain
+    oracle's bit for bit, with a padded row, prefill and incremental steps."""
+    from metaseq_amd import random_prompts, random_state_dict
+    from oracle.opt_oracle import greedy_generate
+    from tests.common import make_oracle, tiny_cfg
+    cfg = tiny_cfg(layers=3, dim=128, heads=2, vocab=128, max_pos=64)
+    sd = random_state_dict(cfg, seed=7, dtype=torch.float16)
+    plain = make_oracle(cfg, sd, torch.float16)
+    lean = make_oracle(cfg, sd, torch.float16, lean=True)
+    lean.attn_chunk_bytes = 2 * 12 * 12 * 4  # one batch row per chunk
+    toks = random_prompts(cfg, 3, 20, seed=5)
+    toks[1, 15:] = 1
+    a = greedy_generate(plain, toks[:, :12], max_len_b=30, min_len=29, return_step_logits=True)
+    b = greedy_generate(lean, toks[:, :12], max_len_b=30, min_len=29, return_step_logits=True)
+    assert torch.equal(a["tokens"], b["tokens"]) and torch.equal(a["scores"], b["scores"])
+    for x, y in zip(a["step_logits"], b["step_logits"]):
+        assert torch.equal(x, y)
+    assert torch.equal(plain(toks)[0], lean(toks)[0])
