@@ -221,6 +221,23 @@ int msa_lm_head_greedy_select_f16(const void* x, const void* Ep, void* logits, v
                                   int64_t tok_stride, float* score, int64_t score_stride,
                                   const int32_t* len_dev, void* stream);
 
+/* msa_lm_head_greedy_select_f16 for callers that cannot allocate device memory (code under
+ * hipGraph capture, tight serving loops, harnesses that forbid hipMalloc).  It has no
+ * counterpart in the reference.  Same arguments, results and kernels, minus `workspace`: the
+ * selection partials go to a fixed device array inside the library (512 KiB per GPU, held until
+ * the process ends), whose address is looked up once per device on the first call there.  The
+ * call allocates and frees nothing.  Limits: M <= 64 rows and at most 256 compute units
+ * (MSA_ERR_CAPACITY beyond).  All calls on one GPU share that array: calls that overlap on one
+ * GPU (different streams or threads) race; calls on one stream are ordered and safe.  Nothing
+ * in the array needs to start at zero: every partial that is read is written by the same call. */
+int msa_lm_head_greedy_select_noalloc_f16(const void* x, const void* Ep, void* logits, int M,
+                                          int V, int K, float temperature,
+                                          const int32_t* banned_host, int n_banned,
+                                          const int32_t* stop_host, int n_stop, uint8_t* finished,
+                                          int force_eos_all, int eos_idx, int64_t* tok,
+                                          int64_t tok_stride, float* score, int64_t score_stride,
+                                          const int32_t* len_dev, void* stream);
+
 /* Measurement aid with no counterpart in the reference: reads `bytes` bytes (a multiple of 16,
  * 16-byte aligned) of device memory once with 16-byte streaming loads and discards them.  The
  * benchmark times it to report the read rate this GPU actually sustains beside the published

@@ -47,6 +47,9 @@ SIGNATURES = {
     "msa_target_logprob_f16": [_P, c_int64, c_int64, c_int, c_float, _P, _P, _P],
     "msa_lm_head_greedy_select_f16": [_P, _P, _P, _P, c_int, c_int, c_int, c_float, _P, c_int, _P,
                                       c_int, _P, c_int, c_int, _P, c_int64, _P, c_int64, _P, _P],
+    "msa_lm_head_greedy_select_noalloc_f16": [_P, _P, _P, c_int, c_int, c_int, c_float, _P, c_int,
+                                              _P, c_int, _P, c_int, c_int, _P, c_int64, _P,
+                                              c_int64, _P, _P],
     "msa_probe_stream_read": [_P, c_int64, _P],
 }
 OTHER_SYMBOLS = ["msa_last_error", "msa_version", "msa_lm_head_select_workspace_bytes"]

@@ -24,6 +24,8 @@
 // that scatters K/V into the per-layer cache and scales Q.
 #include <math.h>
 
+#include <mutex>
+
 #include "common.h"
 
 namespace {
@@ -1248,13 +1250,13 @@ extern "C" int64_t msa_lm_head_select_workspace_bytes(int M) {
   return (int64_t)(M > 0 ? M : 0) * num_cus() * (int64_t)sizeof(SelectPartial);
 }
 
-extern "C" int msa_lm_head_greedy_select_f16(
-    const void* x, const void* Ep, void* logits, void* workspace, int M, int V, int K,
-    float temperature, const int32_t* banned_host, int n_banned, const int32_t* stop_host,
-    int n_stop, uint8_t* finished, int force_eos_all, int eos_idx, int64_t* tok,
-    int64_t tok_stride, float* score, int64_t score_stride, const int32_t* len_dev,
-    void* stream) {
-  const char* name = "msa_lm_head_greedy_select_f16";
+namespace {
+int lm_head_select_impl(const char* name, const void* x, const void* Ep, void* logits,
+                        void* workspace, int M, int V, int K, float temperature,
+                        const int32_t* banned_host, int n_banned, const int32_t* stop_host,
+                        int n_stop, uint8_t* finished, int force_eos_all, int eos_idx, int64_t* tok,
+                        int64_t tok_stride, float* score, int64_t score_stride,
+                        const int32_t* len_dev, void* stream) {
   MSA_REQUIRE(x && Ep && workspace && tok && score, MSA_ERR_INVALID_ARG, "%s: null pointer", name);
   MSA_REQUIRE(M >= 1 && M <= 64 && V > 0 && V % 16 == 0 && K > 0 && K % 32 == 0,
               MSA_ERR_INVALID_ARG, "%s: bad shape M=%d V=%d K=%d (1 <= M <= 64, V %% 16, K %% 32)",
@@ -1290,6 +1292,79 @@ extern "C" int msa_lm_head_greedy_select_f16(
                             tok_stride, score, score_stride, len_dev, (hipStream_t)stream);
   MSA_CHECK_LAUNCH(name);
   return MSA_OK;
+}
+}  // namespace
+
+extern "C" int msa_lm_head_greedy_select_f16(
+    const void* x, const void* Ep, void* logits, void* workspace, int M, int V, int K,
+    float temperature, const int32_t* banned_host, int n_banned, const int32_t* stop_host,
+    int n_stop, uint8_t* finished, int force_eos_all, int eos_idx, int64_t* tok,
+    int64_t tok_stride, float* score, int64_t score_stride, const int32_t* len_dev,
+    void* stream) {
+  return lm_head_select_impl("msa_lm_head_greedy_select_f16", x, Ep, logits, workspace, M, V, K,
+                             temperature, banned_host, n_banned, stop_host, n_stop, finished,
+                             force_eos_all, eos_idx, tok, tok_stride, score, score_stride, len_dev,
+                             stream);
+}
+
+// ---- the entry point that allocates nothing ---------------------------------------------------
+// The per-row, per-workgroup selection partials of the fused vocabulary projection live in a
+// fixed device array instead of a caller-provided workspace, for callers that cannot allocate
+// device memory (code under graph capture, serving loops, harnesses that forbid it).  Every
+// GPU the library runs on holds its own copy of the array (512 KiB) until the process ends.
+// In host code the array's name is only a stand-in for the symbol: the address the kernels get
+// is looked up once per device with hipGetSymbolAddress and kept in g_scratch_ptr.
+constexpr int NA_MAX_ROWS = 64;    // activation rows
+constexpr int NA_MAX_PARTS = 256;  // workgroups of the projection = partials per row
+static __device__ __align__(256) unsigned char
+    scratch[NA_MAX_ROWS * NA_MAX_PARTS * sizeof(SelectPartial)];
+
+namespace {
+constexpr int NA_MAX_DEVICES = 64;
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[NA_MAX_DEVICES] = {};
+
+// the current device's copy of `scratch`; NULL (with the error text set) on failure
+void* scratch_for_current_device(const char* name) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess || dev < 0 || dev >= NA_MAX_DEVICES) {
+    msa_set_error("%s: no usable current device (%s, device %d)", name, hipGetErrorString(e), dev);
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !p) {
+      msa_set_error("%s: hipGetSymbolAddress(scratch) failed on device %d: %s", name, dev,
+                    hipGetErrorString(e));
+      return nullptr;
+    }
+    g_scratch_ptr[dev] = p;
+  }
+  return g_scratch_ptr[dev];
+}
+}  // namespace
+
+extern "C" int msa_lm_head_greedy_select_noalloc_f16(
+    const void* x, const void* Ep, void* logits, int M, int V, int K, float temperature,
+    const int32_t* banned_host, int n_banned, const int32_t* stop_host, int n_stop,
+    uint8_t* finished, int force_eos_all, int eos_idx, int64_t* tok, int64_t tok_stride,
+    float* score, int64_t score_stride, const int32_t* len_dev, void* stream) {
+  const char* name = "msa_lm_head_greedy_select_noalloc_f16";
+  MSA_REQUIRE(M >= 1 && M <= NA_MAX_ROWS, MSA_ERR_CAPACITY,
+              "%s: M=%d rows exceed the %d the fixed scratch array holds", name, M, NA_MAX_ROWS);
+  MSA_REQUIRE(num_cus() <= NA_MAX_PARTS, MSA_ERR_CAPACITY,
+              "%s: %d compute units exceed the %d partials per row the fixed scratch array holds",
+              name, num_cus(), NA_MAX_PARTS);
+  void* ws = scratch_for_current_device(name);
+  if (!ws) return MSA_ERR_HIP;
+  // every partial the combine kernel reads is written by the projection of the same call, so
+  // nothing in the array has to start at zero
+  return lm_head_select_impl(name, x, Ep, logits, ws, M, V, K, temperature, banned_host, n_banned,
+                             stop_host, n_stop, finished, force_eos_all, eos_idx, tok, tok_stride,
+                             score, score_stride, len_dev, stream);
 }
 
 namespace {
