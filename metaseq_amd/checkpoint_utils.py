@@ -8,32 +8,53 @@ Gluing rules (metaseq/distributed/stitch_fsdp_ckpt.py:203-214, 246-339):
   these into k_proj / v_proj / q_proj; this decoder keeps the fused K | V | Q rows.)
 * column-parallel `fc1` (weight and bias) and the token embedding: concatenated along dim 0;
 * row-parallel `fc2` / `out_proj` weights: concatenated along dim 1, their biases replicated;
-* LayerNorms, positional table, everything else: replicated (taken from part 0 after checking
-  that the parts agree).
+* LayerNorms, positional table, everything else: replicated (taken from part 0; copies that
+  drifted apart are reported, as the reference does, not refused).
 
 Only tensors are read from files: `torch.load(..., weights_only=True)` executes nothing from the
 pickle, so a file whose "cfg" entry holds arbitrary Python objects is refused by the loader;
 re-save such a file as {"model": state_dict} with the reference's own tools first.
 """
+import logging
 import re
 from collections import OrderedDict
 from typing import Dict, List
 
 import torch
 
+logger = logging.getLogger(__name__)
+
 _DROP = ("decoder.output_projection.weight",)
 
 
-def _agree(parts, key):
+def _agree(parts, key, tolerance=None):
+    """Replicated parameter: part 0's copy is taken.  Copies that drifted apart (tensor-parallel
+    training does not keep them bit-identical) are reported with their largest absolute
+    difference, as the reference does (metaseq/distributed/stitch_fsdp_ckpt.py:253-262, which
+    only logs).  Only a shape mismatch, or a difference above an explicitly given ``tolerance``,
+    is an error."""
     ref = parts[0][key]
-    for p in parts[1:]:
-        if p[key].shape != ref.shape or not torch.equal(p[key], ref):
-            raise ValueError("replicated parameter %s differs between model parts" % key)
+    worst = 0.0
+    for r, p in enumerate(parts[1:], start=1):
+        if p[key].shape != ref.shape:
+            raise ValueError("replicated parameter %s has shape %s in part %d but %s in part 0"
+                             % (key, tuple(p[key].shape), r, tuple(ref.shape)))
+        if not torch.equal(p[key], ref):
+            worst = max(worst, float((p[key].float() - ref.float()).abs().max()))
+    if worst > 0.0:
+        if tolerance is not None and worst > tolerance:
+            raise ValueError("replicated parameter %s differs between model parts by %g "
+                             "(tolerance %g)" % (key, worst, tolerance))
+        logger.warning("replicated parameter %s differs between model parts by up to %g; "
+                       "taking part 0", key, worst)
     return ref.clone()
 
 
-def glue_model_parts(parts: List[Dict[str, torch.Tensor]]) -> "OrderedDict[str, torch.Tensor]":
-    """Tensor-parallel parts (rank order) -> one state dict with fused K | V | Q rows."""
+def glue_model_parts(parts: List[Dict[str, torch.Tensor]],
+                     replica_tolerance=None) -> "OrderedDict[str, torch.Tensor]":
+    """Tensor-parallel parts (rank order) -> one state dict with fused K | V | Q rows.
+    ``replica_tolerance``: largest absolute difference accepted between the parts' copies of a
+    replicated parameter (None: any difference is only reported)."""
     if not parts:
         raise ValueError("no model parts")
     keys = list(parts[0].keys())
@@ -48,17 +69,18 @@ def glue_model_parts(parts: List[Dict[str, torch.Tensor]]) -> "OrderedDict[str, 
             out[key] = torch.cat([torch.cat([th[j] for th in thirds], dim=0) for j in range(3)],
                                  dim=0)
         elif "layer_norm" in key:
-            out[key] = _agree(parts, key)
+            out[key] = _agree(parts, key, replica_tolerance)
         elif "fc1" in key or re.search(r"\.(k|v|q)_proj\.", key):
             out[key] = torch.cat(ts, dim=0)
         elif "fc2" in key or "out_proj" in key:
-            out[key] = _agree(parts, key) if key.endswith("bias") else torch.cat(ts, dim=1)
+            out[key] = (_agree(parts, key, replica_tolerance) if key.endswith("bias")
+                        else torch.cat(ts, dim=1))
         elif "embed_tokens.weight" in key:
             out[key] = torch.cat(ts, dim=0)
         elif "_float_tensor" in key or "version" in key:
             out[key] = ts[0].clone()
         else:
-            out[key] = _agree(parts, key)
+            out[key] = _agree(parts, key, replica_tolerance)
     return out
 
 

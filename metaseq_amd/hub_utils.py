@@ -17,6 +17,7 @@ the reference makes on its Hugging Face ``tokenizers`` object: ``decode(ids) -> 
 import time
 from typing import List, Optional
 
+import numpy as np
 import torch
 
 from .sequence_generator import SequenceGenerator
@@ -149,57 +150,58 @@ class GeneratorInterface:
         return retval
 
     def _record(self, tokens, scores, distributions, prompt_len, max_tokens, echo, logprobs):
-        """One result record (hub_utils.py:344-413)."""
+        """One result record with the reference's fields (hub_utils.py:344-413): ``text``,
+        per-token strings, character offsets, scores and, on request, the ``logprobs`` most
+        likely alternatives per position.
+
+        After the special-token cut the row holds [eos, prompt..., continuation...].  The
+        reported window is the whole row with ``echo`` and the continuation (capped at the
+        request's own ``max_tokens``) without; with ``echo`` the leading end-of-sentence token
+        shows up among the token strings but has no score, no alternatives and no text."""
         tokens, scores, distributions = self._filter_special(
             self._pad_token_ind, self._special_token_inds, tokens, scores, distributions)
-        if not echo:  # cut off the prompt and its leading end-of-sentence token
-            tokens = tokens[prompt_len + 1:][:max_tokens]
-            scores = scores[prompt_len + 1:][:max_tokens]
-            if logprobs > 0:
-                distributions = distributions[prompt_len + 1:][:max_tokens]
-        tokens_no_eos = tokens[1:] if echo else tokens
-        scores_with_eos = [None] + scores[1:] if echo else scores
-        text = self.bpe.decode(tokens_no_eos)
-        token_offsets = [s for s, e in self.bpe.encode(text).offsets]
-        result = {
+        lo = 0 if echo else prompt_len + 1
+        hi = len(tokens) if echo else min(len(tokens), lo + max_tokens)
+        window = slice(lo, max(lo, hi))
+        shown, shown_scores = tokens[window], scores[window]
+        lead = 1 if echo else 0  # positions at the front that carry no prediction
+        text = self.bpe.decode(shown[lead:])
+        record = {
             "text": text,
-            "tokens": [self.bpe.decode([t]) for t in tokens],
-            "text_offset": token_offsets,
-            "token_scores": scores_with_eos,
+            "tokens": [self.bpe.decode([t]) for t in shown],
+            "text_offset": [begin for begin, _ in self.bpe.encode(text).offsets],
+            "token_scores": [None] * lead + shown_scores[lead:],
+            "top_logprobs": None,
         }
         if logprobs > 0:
-            out_logprobs = []
-            if distributions.shape[0] > 0:
-                top_scores, top_toks = distributions.topk(k=logprobs, dim=-1)
-                for sc, tk in zip(top_scores, top_toks):
-                    out_logprobs.append({self.bpe.decode([t.item()]): s.item()
-                                         for t, s in zip(tk, sc)})
-            # no distribution precedes the leading end-of-sentence token
-            result["top_logprobs"] = [None] + out_logprobs[1:] if echo else out_logprobs
-        else:
-            result["top_logprobs"] = None
-        return result
+            best = self._alternatives(distributions[window], logprobs)
+            record["top_logprobs"] = [None] * lead + best[lead:]
+        return record
+
+    def _alternatives(self, rows, k):
+        """Per position, the k most likely tokens as {token string: log-probability}."""
+        if rows.shape[0] == 0:
+            return []
+        values, ids = torch.as_tensor(rows).topk(k, dim=-1)
+        return [{self.bpe.decode([i]): v for i, v in zip(id_row, value_row)}
+                for id_row, value_row in zip(ids.tolist(), values.tolist())]
 
     @staticmethod
     def _filter_special(pad_token_ind, special_token_inds, tokens: List[int],
                         scores: List[float], distributions):
-        """Drops pads and cuts the sequence at the first special token after position 0
-        (hub_utils.py:425-466).  ``distributions`` ([seqlen, vocab] or None) keeps the rows of
-        the surviving positions."""
-        kept, mask = [], []
-        for i, (t, s) in enumerate(zip(tokens, scores)):
-            if t == pad_token_ind:
-                mask.append(False)
-                continue
-            if t in special_token_inds and i > 0:
-                mask.append(False)
-                break
-            mask.append(True)
-            kept.append((t, s))
-        new_tokens, new_scores = zip(*kept)
+        """The part of a generated row that is reported (hub_utils.py:425-466): the row ends
+        before the first special token that is not a pad and not at position 0, and pads in
+        front of that point are dropped.  ``distributions`` ([positions, vocab] array or tensor,
+        or None) keeps the rows of the surviving positions."""
+        ids = np.asarray(tokens, dtype=np.int64)
+        enders = np.isin(ids, [t for t in special_token_inds if t != pad_token_ind])
+        enders[:1] = False
+        end = int(enders.argmax()) if enders.any() else ids.size
+        keep = np.flatnonzero(ids[:end] != pad_token_ind).tolist()
         if distributions is not None:
-            assert len(mask) <= distributions.shape[0], \
-                "Mask cannot be larger than the number of tokens in disribution (distributions.shape[0])"
-            mask.extend([False] * (distributions.shape[0] - len(mask)))
-            distributions = distributions[mask]
-        return list(new_tokens), list(new_scores), distributions
+            examined = min(end + 1, ids.size)
+            if examined > distributions.shape[0]:
+                raise AssertionError("%d positions were generated but only %d distributions "
+                                     "were recorded" % (examined, distributions.shape[0]))
+            distributions = distributions[keep]
+        return [tokens[i] for i in keep], [scores[i] for i in keep], distributions

@@ -58,6 +58,12 @@ class SequenceGenerator(nn.Module):
         self.lambda_decay = lambda_decay
         self.omega_bound = float(omega_bound)
         self.full_stop_list = [tgt_dict.index(w) for w in [".", "?", "!"]]
+        if lambda_decay > 0 and all(i == self.unk for i in self.full_stop_list):
+            # the decayed nucleus is only ever reset at a full stop: with a dictionary that
+            # cannot name ".", "?" and "!" it would silently decay to omega_bound for good
+            raise ValueError(
+                "factual-nucleus sampling (lambda_decay > 0) needs a dictionary that resolves "
+                "'.', '?' and '!' to token ids; this one maps them all to <unk>")
         self.alpha_presence = alpha_presence
         self.alpha_frequency = alpha_frequency
         self.alpha_presence_src = alpha_presence_src

@@ -92,10 +92,26 @@ def test_split_is_the_inverse_of_glue(mp):
         assert torch.allclose(tp_forward(two, TOKENS, H), tp_forward(parts, TOKENS, H), atol=2e-5)
 
 
-def test_replicated_parameters_must_agree():
+def test_replicated_parameters_that_drifted_are_taken_from_part_0_with_a_warning(caplog):
+    """The reference only logs the largest discrepancy between the parts' copies of a
+    replicated parameter and keeps part 0's (stitch_fsdp_ckpt.py:253-262); a shape mismatch or
+    a difference above an explicit tolerance is an error."""
     parts = _parts(2)
-    parts[1]["decoder.layer_norm.bias"] = parts[1]["decoder.layer_norm.bias"] + 1
-    with pytest.raises(ValueError):
+    key = "decoder.layer_norm.bias"
+    one_ulp = parts[1][key].half()
+    one_ulp = (one_ulp.view(torch.int16) + 1).view(torch.float16).float()  # next fp16 up
+    parts[1][key] = one_ulp
+    parts[0][key] = parts[0][key].half().float()
+    with caplog.at_level("WARNING", logger="metaseq_amd.checkpoint_utils"):
+        glued = C.glue_model_parts(parts)
+    assert torch.equal(glued[key], parts[0][key])
+    assert any(key in r.getMessage() and "taking part 0" in r.getMessage()
+               for r in caplog.records)
+    with pytest.raises(ValueError, match="tolerance"):
+        C.glue_model_parts(parts, replica_tolerance=1e-9)
+    C.glue_model_parts(parts, replica_tolerance=1.0)
+    parts[1][key] = parts[1][key][:-1]
+    with pytest.raises(ValueError, match="shape"):
         C.glue_model_parts(parts)
 
 

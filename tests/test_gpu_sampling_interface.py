@@ -20,6 +20,9 @@ from tests.scripted import ScriptedDecoder
 pytestmark = pytest.mark.gpu
 DEV = "cuda"
 V = 12
+# ids the test dictionary gives ".", "?" and "!": ordinary tokens of the scripted vocabulary, so
+# the factual-nucleus resets really fire
+FULL_STOPS = {".": 7, "?": 8, "!": 9}
 
 
 def _script(B, seed):
@@ -38,14 +41,14 @@ def _both(kw, B=3, seed=11, beam=1, max_len_b=16, min_len=6, src=None):
     if src is None:
         src = torch.tensor([[2, 5, 7, 9], [2, 6, 1, 1], [2, 4, 8, 1]][:B])
     dec = ScriptedDecoder(script, V, device=DEV, dtype=torch.float16)
-    gen = SequenceGenerator([dec], Dictionary(V), beam_size=beam, max_len_b=max_len_b,
-                            min_len=min_len, **kw)
+    gen = SequenceGenerator([dec], Dictionary(V, symbols=FULL_STOPS), beam_size=beam,
+                            max_len_b=max_len_b, min_len=min_len, **kw)
     torch.manual_seed(1234)
     got = gen.generate([dec], {"net_input": {"src_tokens": src.to(DEV)}})
     dec2 = ScriptedDecoder(script, V, device=DEV, dtype=torch.float16)
     torch.manual_seed(1234)
     want = O.generate(dec2, src.to(DEV), max_len_b=max_len_b, min_len=min_len, beam_size=beam,
-                      **kw)
+                      full_stop_list=tuple(FULL_STOPS.values()), **kw)
     return got, want
 
 

@@ -170,3 +170,30 @@ def test_id_tokenizer_round_trip():
     enc = tk.encode(text)
     assert enc.ids == [12, 7, 50271] and enc.offsets == [(0, 2), (3, 4), (5, 10)]
     assert tk.encode("").ids == []
+
+
+def test_dictionary_resolves_symbols_from_a_table_or_a_tokenizer():
+    class Tok:
+        def token_to_id(self, s):
+            return {".": 13, "?": 30}.get(s)
+    plain = Dictionary(100)
+    assert plain.index(".") == plain.unk() == 3 and not plain.resolves(".")
+    table = Dictionary(100, symbols={".": 4, "!": 6})
+    assert (table.index("."), table.index("!"), table.index("?")) == (4, 6, 3)
+    tok = Dictionary(100, tokenizer=Tok())
+    assert (tok.index("."), tok.index("?"), tok.index("!")) == (13, 30, 3)
+    assert tok.resolves("?") and not tok.resolves("!")
+
+
+def test_factual_nucleus_needs_resolvable_full_stops():
+    """With a dictionary that maps ".", "?" and "!" to <unk> the decayed nucleus would never be
+    reset (the reference resets on dictionary.index(...), sequence_generator.py:116, 443-476):
+    the generator refuses that combination instead of decaying silently."""
+    from metaseq_amd import SequenceGenerator
+    dec = ScriptedDecoder({0: {1: [1.0] + [0.0] * 11}}, 12)
+    with pytest.raises(ValueError, match="lambda_decay"):
+        SequenceGenerator([dec], Dictionary(12), topp=0.9, lambda_decay=0.8)
+    gen = SequenceGenerator([dec], Dictionary(12, symbols={".": 7, "?": 8, "!": 9}), topp=0.9,
+                            lambda_decay=0.8)
+    assert gen.full_stop_list == [7, 8, 9]
+    SequenceGenerator([dec], Dictionary(12), topp=0.9)  # no decay: nothing to resolve
