@@ -52,3 +52,13 @@ def test_more_than_one_gpu_is_refused_with_a_message():
                        capture_output=True, text=True, timeout=120)
     assert r.returncode == 2
     assert "one GPU" in r.stderr and r.stdout.strip() == ""
+
+
+def test_cpu_baseline_is_a_measured_run_of_the_cpu_runnable_case():
+    """The baseline leg runs the oracle's greedy generation on OPT-125m (batch 1, prompt 32, 32
+    generated tokens) and reports decode tokens/s over the timed generations."""
+    r = bench.cpu_baseline(warm=0, timed=1)
+    assert r["kind"] == "port" and r["timing"] == "measured" and r["unit"] == "tokens/s"
+    assert r["cores"] >= 1 and "OPT-125m" in r["sample"]
+    assert r["value"] == pytest.approx(32 / r["decode_s_mean"])
+    assert 0 < r["prefill_s_mean"] < r["decode_s_mean"]
