@@ -36,6 +36,11 @@ typedef enum {
 #define MSA_EPI_RELU 1u   /* y = max(y, 0) after the bias add                                  */
 #define MSA_IN_PACKED 2u  /* the input activation is in the packed layout (M <= 64, see below) */
 #define MSA_OUT_PACKED 4u /* write the output activation in the packed layout (M <= 64)        */
+#define MSA_EMBED_COL_FROM_LEN 8u /* msa_embed_f16: the new token sits in column len_dev[b]      */
+/* per-row bits of the optional `row_mode` array of the selection entry points */
+#define MSA_ROW_BAN_EARLY 1u /* eos_idx and the stop ids are not eligible for this row (the row
+                                has not reached its minimum length)                             */
+#define MSA_ROW_ONLY_EOS 2u  /* only eos_idx is eligible for this row (its last allowed step)   */
 
 const char* msa_last_error(void);
 int msa_version(void);
@@ -61,17 +66,32 @@ int msa_unpack_weight_f16(const void* src, void* dst, int N, int K, void* stream
 int msa_pack_weight_i8(const int8_t* src, int8_t* dst, int N, int K, void* stream);
 int msa_unpack_weight_i8(const int8_t* src, int8_t* dst, int N, int K, void* stream);
 
-/* ---- device-resident sequence length (for hipGraph replay of a decode step) -------------------
- * A captured graph must not bake the growing history length into launch arguments.  The four
- * entry points that depend on it take an optional `len_dev` (int32 on the device, NULL = use the
- * host arguments) holding the number of positions already in the KV cache:
- *   msa_embed_f16 (T_out == 1): embeds column *len_dev of tokens (n = *len_dev + 1, capped by n);
- *   msa_qkv_proj_* (T == 1):    appends at position *len_dev (skipped if that is >= S_cap);
- *   msa_attention_f16 (T == 1): attends positions 0 .. *len_dev;
- *   msa_greedy_select_f16:      writes tok[b*tok_stride + *len_dev], score likewise.
- * msa_advance_len adds `delta` to *len_dev on the stream (a one-thread kernel).
- * No reference counterpart (the reference re-launches every op from Python each step). */
-int msa_advance_len(int32_t* len_dev, int delta, void* stream);
+/* ---- device-resident per-row sequence lengths -------------------------------------------------
+ * The entry points of a decode step (T == 1) take an optional `len_dev`: int32 [B] on the device,
+ * len_dev[b] = number of positions of row b already in the KV cache (= the number of non-pad
+ * tokens of its history before the new one); NULL = use the host arguments, every row at S0.
+ * With it, rows of one batch may have different lengths (right-padded prompts, requests that
+ * joined a running batch at different times): each row appends at, and attends up to, its own
+ * length, and pads are never stored.  A NEGATIVE entry marks a row as inactive (an empty slot):
+ * nothing is appended or attended for it and its outputs are undefined.  A captured hipGraph
+ * bakes no length into its launch arguments and replays for every step.
+ *   msa_embed_f16 (T_out == 1): position = pad_idx + 1 + len_dev[b] (no scan of the history);
+ *                               the token is column n - 1 of the row, or column len_dev[b] with
+ *                               MSA_EMBED_COL_FROM_LEN (a full-history token buffer, no pads);
+ *                               step_len_out (optional int32 [B]) receives len_dev[b], or -1 if
+ *                               the row is inactive or its new token is a pad: passed on as the
+ *                               `len_dev` of the step's other kernels and as the gate of
+ *                               msa_advance_len, it keeps such a row out of the step, the way
+ *                               the reference masks a pad for good;
+ *   msa_qkv_proj_* (T == 1):    row b appends at position len_dev[b] (skipped if >= S_cap);
+ *   msa_attention_f16 (T == 1): row b attends positions 0 .. len_dev[b];
+ *   msa_greedy_select_f16 and the fused forms: the output column is len_dev[0] (graph replay of
+ *                               a batch whose rows all have the same length).
+ * msa_advance_len adds `delta` to those of the n entries of len_dev that are not negative and
+ * whose gate entry (optional int32 [n]) is not negative either, on the stream.
+ * No reference counterpart: the reference re-launches every op from Python each step and keeps
+ * pads inside its key/value history, masked (metaseq/modules/multihead_attention.py:485-531). */
+int msa_advance_len(int32_t* len_dev, const int32_t* gate, int n, int delta, void* stream);
 
 /* Pre-LN LayerNorm forward: y[r,:] = round(gamma * (x[r,:] - mean) * rsqrt(var + eps) + beta),
  * mean / biased variance in fp32.  D % 8 == 0, D <= 16384.  flags: MSA_OUT_PACKED.
@@ -98,7 +118,7 @@ int msa_residual_layernorm_f16(const float* part, int S, const void* bias, void*
  *   x[b*T_out + j, :] = round(E[tokens[b,t], :] + P[pos(b,t), :]),  t = n - T_out + j
  * tokens are int64 with row stride `tok_stride` elements.  positions_out (optional, int64
  * [B, T_out]) receives pos.  Ids outside [0,V) or positions >= n_pos_rows set *status_dev
- * (optional int32) to 1 and are clamped.
+ * (optional int32) to 1 and are clamped.  flags: MSA_EMBED_COL_FROM_LEN (with len_dev).
  * Replaces TransformerDecoder.forward_embedding (metaseq/models/transformer_decoder.py:263-346),
  * utils.make_positions (metaseq/utils.py:83-93), LearnedPositionalEmbedding.forward
  * (metaseq/modules/learned_positional_embedding.py:30-54) and VocabParallelEmbedding.forward
@@ -106,7 +126,7 @@ int msa_residual_layernorm_f16(const float* part, int S, const void* bias, void*
 int msa_embed_f16(const int64_t* tokens, int64_t tok_stride, int B, int n, int T_out,
                   const void* E, int V, const void* P, int n_pos_rows, int pad_idx, int D,
                   void* x, int64_t* positions_out, int32_t* status_dev, const int32_t* len_dev,
-                  void* stream);
+                  int32_t* step_len_out, unsigned flags, void* stream);
 
 /* y[M,N] = epilogue(x[M,K] . W[N,K]^T) with W tile-packed:
  *   t = round(acc); if bias: t = round(t + bias[n]); if RELU: t = max(t,0);
@@ -151,7 +171,7 @@ int msa_linear_default_splits_w8a16(int64_t M, int N, int K);
  * K | V | Q; then for row m = b*T + t and head h:
  *   Kcache[b,h,S0+t,:] = k,  Vcache[b,h,S0+t,:] = v,  q_out[m, h*hd:(h+1)*hd] = round(q * hd^-0.5).
  * Caches are [B, H, S_cap, hd] fp16, q_out row-major.  Same size rules as msa_linear_f16 with
- * N = 3*H*hd.  flags: MSA_IN_PACKED.
+ * N = 3*H*hd.  flags: MSA_IN_PACKED.  With len_dev (T == 1) row b appends at len_dev[b].
  * Replaces metaseq/modules/multihead_attention.py:316-319 (projection + split), :429
  * (q scaling) and :449-479 (cache growth by torch.cat, here an in-place append). */
 int msa_qkv_proj_f16(const void* x, const void* Wqkv, const void* bqkv, void* q_out,
@@ -168,7 +188,8 @@ int msa_qkv_proj_w8a16(const void* x, const int8_t* Wq, const void* scales, cons
  *   p = round(softmax_fp32(s));  out[b*T+t, h*hd:(h+1)*hd] = round(sum_key p * v).
  * key_pad_mask (optional) is uint8 [B, mask_stride].  hd in {64, 128}.  T == 1 is the
  * bandwidth-bound decode kernel; T > 1 the prefill kernel.  q is row-major; flags:
- * MSA_OUT_PACKED (T == 1, B <= 64).
+ * MSA_OUT_PACKED (T == 1, B <= 64).  With len_dev (T == 1) row b attends its own
+ * len_dev[b] + 1 positions and S0 only has to bound them.
  * Replaces metaseq/modules/multihead_attention.py:492 (bmm q k^T), :516-531 (causal and
  * padding masks), :533-534 (fp32 softmax, cast back), :543-552 (bmm p v, transpose). */
 int msa_attention_f16(const void* q, const void* Kcache, const void* Vcache,
@@ -183,18 +204,22 @@ int msa_attention_f16(const void* q, const void* Kcache, const void* Vcache,
  *   lprob of the row is -inf;
  *   ids in banned_host[0..n_banned) -> -inf (pad always, eos and stop ids while step < min_len);
  *   if force_eos_all != 0 (last step) or finished[b] != 0, only eos_idx stays eligible;
+ *   row_mode (optional uint8[B], device) adds the same two regimes per row, for batches whose
+ *   rows are at different points of their own requests: MSA_ROW_BAN_EARLY makes eos_idx and
+ *   the stop ids ineligible for row b, MSA_ROW_ONLY_EOS leaves only eos_idx eligible;
  *   tok[b*tok_stride] = lowest index attaining the max lprob; score[b*score_stride] = that max;
  *   finished[b] |= tok == eos_idx or tok in stop_host[0..n_stop).
- * banned_host / stop_host are HOST arrays of at most 16 ids, copied into the launch.
- * finished (uint8[B], device, in/out) is optional.
+ * banned_host / stop_host are HOST arrays of at most 16 (stop: 15 in the fused forms) ids,
+ * copied into the launch.  finished (uint8[B], device, in/out) is optional.
  * Replaces the per-step vocabulary passes of SequenceGenerator._generate
  * (metaseq/sequence_generator.py:272-308, :319-323), _sample_topp's greedy branch (:413-415)
  * and BaseDecoder.get_normalized_probs (metaseq/models/base_decoder.py:95-100). */
 int msa_greedy_select_f16(const void* logits, int64_t ld_logits, int B, int V, float temperature,
                           const int32_t* banned_host, int n_banned, const int32_t* stop_host,
-                          int n_stop, uint8_t* finished, int force_eos_all, int eos_idx,
-                          int64_t* tok, int64_t tok_stride, float* score, int64_t score_stride,
-                          const int32_t* len_dev, void* stream);
+                          int n_stop, uint8_t* finished, const uint8_t* row_mode,
+                          int force_eos_all, int eos_idx, int64_t* tok, int64_t tok_stride,
+                          float* score, int64_t score_stride, const int32_t* len_dev,
+                          void* stream);
 
 /* Log-probabilities of given target ids under fp16 logits rows:
  *   out[r] = logits[r, target[r]]/temperature - logsumexp_fp32(logits[r,:]/temperature).
@@ -217,9 +242,9 @@ int msa_lm_head_greedy_select_f16(const void* x, const void* Ep, void* logits, v
                                   int M, int V, int K, float temperature,
                                   const int32_t* banned_host, int n_banned,
                                   const int32_t* stop_host, int n_stop, uint8_t* finished,
-                                  int force_eos_all, int eos_idx, int64_t* tok,
-                                  int64_t tok_stride, float* score, int64_t score_stride,
-                                  const int32_t* len_dev, void* stream);
+                                  const uint8_t* row_mode, int force_eos_all, int eos_idx,
+                                  int64_t* tok, int64_t tok_stride, float* score,
+                                  int64_t score_stride, const int32_t* len_dev, void* stream);
 
 /* msa_lm_head_greedy_select_f16 for callers that cannot allocate device memory (code under
  * hipGraph capture, tight serving loops, harnesses that forbid hipMalloc).  It has no
@@ -234,9 +259,10 @@ int msa_lm_head_greedy_select_noalloc_f16(const void* x, const void* Ep, void* l
                                           int V, int K, float temperature,
                                           const int32_t* banned_host, int n_banned,
                                           const int32_t* stop_host, int n_stop, uint8_t* finished,
-                                          int force_eos_all, int eos_idx, int64_t* tok,
-                                          int64_t tok_stride, float* score, int64_t score_stride,
-                                          const int32_t* len_dev, void* stream);
+                                          const uint8_t* row_mode, int force_eos_all, int eos_idx,
+                                          int64_t* tok, int64_t tok_stride, float* score,
+                                          int64_t score_stride, const int32_t* len_dev,
+                                          void* stream);
 
 /* Measurement aid with no counterpart in the reference: reads `bytes` bytes (a multiple of 16,
  * 16-byte aligned) of device memory once with 16-byte streaming loads and discards them.  The

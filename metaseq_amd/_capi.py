@@ -15,6 +15,9 @@ LIB_PATH = os.path.join(_HERE, "csrc", "libmetaseq_amd.so")
 MSA_EPI_RELU = 1
 MSA_IN_PACKED = 2
 MSA_OUT_PACKED = 4
+MSA_EMBED_COL_FROM_LEN = 8
+MSA_ROW_BAN_EARLY = 1
+MSA_ROW_ONLY_EOS = 2
 
 _P = c_void_p
 
@@ -27,9 +30,9 @@ SIGNATURES = {
     "msa_layernorm_f16": [_P, _P, _P, _P, c_int64, c_int, c_float, c_uint, _P],
     "msa_residual_layernorm_f16": [_P, c_int, _P, _P, _P, _P, _P, c_int64, c_int, c_float, c_uint,
                                    _P],
-    "msa_advance_len": [_P, c_int, _P],
+    "msa_advance_len": [_P, _P, c_int, c_int, _P],
     "msa_embed_f16": [_P, c_int64, c_int, c_int, c_int, _P, c_int, _P, c_int, c_int, c_int, _P, _P,
-                      _P, _P, _P],
+                      _P, _P, _P, c_uint, _P],
     "msa_linear_f16": [_P, _P, _P, _P, _P, c_int64, c_int, c_int, c_uint, _P],
     "msa_linear_w8a16": [_P, _P, _P, _P, _P, _P, c_int64, c_int, c_int, c_uint, _P],
     "msa_linear_partial_f16": [_P, _P, _P, c_int64, c_int, c_int, c_int, c_uint, _P],
@@ -42,13 +45,14 @@ SIGNATURES = {
                            c_int, c_uint, _P, _P],
     "msa_attention_f16": [_P, _P, _P, _P, c_int64, _P, c_int, c_int, c_int, c_int, c_int, c_int,
                           c_uint, _P, _P],
-    "msa_greedy_select_f16": [_P, c_int64, c_int, c_int, c_float, _P, c_int, _P, c_int, _P, c_int,
-                              c_int, _P, c_int64, _P, c_int64, _P, _P],
+    "msa_greedy_select_f16": [_P, c_int64, c_int, c_int, c_float, _P, c_int, _P, c_int, _P, _P,
+                              c_int, c_int, _P, c_int64, _P, c_int64, _P, _P],
     "msa_target_logprob_f16": [_P, c_int64, c_int64, c_int, c_float, _P, _P, _P],
     "msa_lm_head_greedy_select_f16": [_P, _P, _P, _P, c_int, c_int, c_int, c_float, _P, c_int, _P,
-                                      c_int, _P, c_int, c_int, _P, c_int64, _P, c_int64, _P, _P],
+                                      c_int, _P, _P, c_int, c_int, _P, c_int64, _P, c_int64, _P,
+                                      _P],
     "msa_lm_head_greedy_select_noalloc_f16": [_P, _P, _P, c_int, c_int, c_int, c_float, _P, c_int,
-                                              _P, c_int, _P, c_int, c_int, _P, c_int64, _P,
+                                              _P, c_int, _P, _P, c_int, c_int, _P, c_int64, _P,
                                               c_int64, _P, _P],
     "msa_probe_stream_read": [_P, c_int64, _P],
 }

@@ -30,7 +30,11 @@ __global__ void attention_kernel(const half_t* __restrict__ q, const half_t* __r
   const int b = bh / H, h = bh - b * H;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
   const int sub = lane % LPR, rsel = lane / LPR;
-  if (len_dev) S0 = min(*len_dev, S_cap - 1);  // cache length kept on the device (graph replay)
+  if (len_dev) {  // per-row cache lengths kept on the device (ragged batches, graph replay)
+    S0 = len_dev[b];
+    if (S0 < 0) return;  // inactive row: nothing to attend, the output row keeps its contents
+    S0 = min(S0, S_cap - 1);
+  }
   const int n_keys = S0 + t + 1;
   const int D = H * HD;
 

@@ -39,19 +39,31 @@ __device__ __forceinline__ void clamp_ids(int64_t& tok, int& pos, int V, int n_p
   }
 }
 
-// decode step: one block per batch row, last token only
+// decode step: one block per batch row, last token only.  With len_dev (per-row number of
+// positions already in the KV cache = number of non-pad tokens before this one) the position
+// comes from there instead of a scan over the row's history.
 __global__ __launch_bounds__(EMB_THREADS) void embed_last_kernel(
     const int64_t* __restrict__ tokens, int64_t tok_stride, int n, const half_t* __restrict__ E,
     int V, const half_t* __restrict__ P, int n_pos_rows, int pad, int D, half_t* __restrict__ x,
-    int64_t* __restrict__ positions_out, int32_t* status, const int32_t* __restrict__ len_dev) {
+    int64_t* __restrict__ positions_out, int32_t* status, const int32_t* __restrict__ len_dev,
+    int32_t* __restrict__ step_len_out, bool col_from_len) {
   __shared__ float red[16];
   const int b = blockIdx.x;
   const int64_t* row = tokens + b * tok_stride;
-  if (len_dev) n = min(*len_dev + 1, n);  // history length kept on the device (graph replay)
-  int64_t tok = row[n - 1];
+  int64_t tok;
   int pos = pad;
-  const int cnt = count_nonpad(row, n, pad, red);
-  if (tok != pad) pos = pad + cnt;
+  if (len_dev) {
+    const int raw = len_dev[b];
+    const int len = max(raw, 0);  // an inactive row (negative) embeds as an empty one
+    tok = row[col_from_len ? min(len, n - 1) : n - 1];
+    if (tok != pad) pos = pad + 1 + len;
+    // a pad as the new token leaves the row out of this step, like an inactive row
+    if (step_len_out && threadIdx.x == 0) step_len_out[b] = (raw >= 0 && tok != pad) ? raw : -1;
+  } else {
+    tok = row[n - 1];
+    const int cnt = count_nonpad(row, n, pad, red);
+    if (tok != pad) pos = pad + cnt;
+  }
   clamp_ids(tok, pos, V, n_pos_rows, status);
   if (positions_out && threadIdx.x == 0) positions_out[b] = pos;
   gather_row(E, P, tok, pos, x + (int64_t)b * D, D);
@@ -97,7 +109,8 @@ __global__ __launch_bounds__(EMB_THREADS) void embed_rows_kernel(
 extern "C" int msa_embed_f16(const int64_t* tokens, int64_t tok_stride, int B, int n, int T_out,
                              const void* E, int V, const void* P, int n_pos_rows, int pad_idx,
                              int D, void* x, int64_t* positions_out, int32_t* status_dev,
-                             const int32_t* len_dev, void* stream) {
+                             const int32_t* len_dev, int32_t* step_len_out, unsigned flags,
+                             void* stream) {
   MSA_REQUIRE(tokens && E && P && x, MSA_ERR_INVALID_ARG, "msa_embed_f16: null pointer");
   MSA_REQUIRE(B > 0 && n > 0 && T_out > 0 && T_out <= n && tok_stride >= n, MSA_ERR_INVALID_ARG,
               "msa_embed_f16: bad shape B=%d n=%d T_out=%d stride=%lld", B, n, T_out,
@@ -106,12 +119,18 @@ extern "C" int msa_embed_f16(const int64_t* tokens, int64_t tok_stride, int B, i
               MSA_ERR_INVALID_ARG, "msa_embed_f16: bad sizes D=%d V=%d n_pos_rows=%d pad=%d", D, V,
               n_pos_rows, pad_idx);
   MSA_REQUIRE(!len_dev || T_out == 1, MSA_ERR_INVALID_ARG,
-              "msa_embed_f16: a device-side length needs T_out == 1");
+              "msa_embed_f16: device-side lengths need T_out == 1");
+  MSA_REQUIRE((flags & ~MSA_EMBED_COL_FROM_LEN) == 0 && (!flags || len_dev), MSA_ERR_INVALID_ARG,
+              "msa_embed_f16: unsupported flags 0x%x (MSA_EMBED_COL_FROM_LEN needs len_dev)",
+              flags);
+  MSA_REQUIRE(!step_len_out || len_dev, MSA_ERR_INVALID_ARG,
+              "msa_embed_f16: step_len_out needs len_dev");
   hipStream_t s = (hipStream_t)stream;
   if (T_out == 1) {
     hipLaunchKernelGGL(embed_last_kernel, dim3(B), dim3(EMB_THREADS), 0, s, tokens, tok_stride, n,
                        (const half_t*)E, V, (const half_t*)P, n_pos_rows, pad_idx, D, (half_t*)x,
-                       positions_out, status_dev, len_dev);
+                       positions_out, status_dev, len_dev, step_len_out,
+                       (flags & MSA_EMBED_COL_FROM_LEN) != 0);
   } else {
     MSA_REQUIRE(positions_out, MSA_ERR_INVALID_ARG,
                 "msa_embed_f16: positions_out is required when T_out > 1");
@@ -126,12 +145,20 @@ extern "C" int msa_embed_f16(const int64_t* tokens, int64_t tok_stride, int B, i
 }
 
 namespace {
-__global__ void advance_len_kernel(int32_t* len_dev, int delta) { *len_dev += delta; }
+__global__ __launch_bounds__(64) void advance_len_kernel(int32_t* len_dev,
+                                                         const int32_t* __restrict__ gate, int n,
+                                                         int delta) {
+  const int i = blockIdx.x * 64 + threadIdx.x;
+  // inactive rows (negative) and rows the gate leaves out of this step stay as they are
+  if (i < n && len_dev[i] >= 0 && (!gate || gate[i] >= 0)) len_dev[i] += delta;
+}
 }  // namespace
 
-extern "C" int msa_advance_len(int32_t* len_dev, int delta, void* stream) {
-  MSA_REQUIRE(len_dev, MSA_ERR_INVALID_ARG, "msa_advance_len: null pointer");
-  hipLaunchKernelGGL(advance_len_kernel, dim3(1), dim3(1), 0, (hipStream_t)stream, len_dev, delta);
+extern "C" int msa_advance_len(int32_t* len_dev, const int32_t* gate, int n, int delta,
+                               void* stream) {
+  MSA_REQUIRE(len_dev && n > 0, MSA_ERR_INVALID_ARG, "msa_advance_len: null pointer or n=%d", n);
+  hipLaunchKernelGGL(advance_len_kernel, dim3((n + 63) / 64), dim3(64), 0, (hipStream_t)stream,
+                     len_dev, gate, n, delta);
   MSA_CHECK_LAUNCH("msa_advance_len");
   return MSA_OK;
 }

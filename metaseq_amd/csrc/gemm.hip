@@ -45,12 +45,14 @@ struct Epilogue {
   half_t* Vc;
   int T, H, hd, S0, S_cap;
   int hd_shift;  // log2(hd) if hd is a power of two, else -1
-  const int32_t* len_dev;  // if set (T == 1): the append position is read from the device
+  const int32_t* len_dev;  // if set (T == 1): per-row append positions on the device (< 0: skip)
   float qscale;
   // MODE_SELECT: greedy selection over the output row instead of (or besides) storing it
   SelectPartial* partials;  // [M][gridDim.x]
   const uint8_t* finished;  // rows that may only emit eos
+  const uint8_t* row_mode;  // optional per-row MSA_ROW_* bits
   IdList banned;
+  IdList early;  // eos and the stop ids: not eligible for rows with MSA_ROW_BAN_EARLY
   float temperature;  // logits are divided by it when `scale`
   int scale, force_eos_all, eos;
 };
@@ -68,7 +70,10 @@ struct SelectState {
 __device__ __forceinline__ void select_update4(SelectState& st, const Epilogue& e, int64_t m,
                                                int n, float4_t acc) {
   float z[4], cm = -INFINITY;
-  const bool only_eos = e.force_eos_all || (e.finished && e.finished[m]);
+  const unsigned rm = e.row_mode ? e.row_mode[m] : 0u;
+  const bool only_eos =
+      e.force_eos_all || (e.finished && e.finished[m]) || (rm & MSA_ROW_ONLY_EOS);
+  const int n_early = (rm & MSA_ROW_BAN_EARLY) ? e.early.n : 0;
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     z[i] = round_h(acc[i]);
@@ -78,6 +83,7 @@ __device__ __forceinline__ void select_update4(SelectState& st, const Epilogue& 
     const int id = n + i;
     bool ok = !(only_eos && id != e.eos);
     for (int j = 0; j < e.banned.n; ++j) ok &= (e.banned.id[j] != id);
+    for (int j = 0; j < n_early; ++j) ok &= (e.early.id[j] != id);
     const float cand = ok ? z[i] : -INFINITY;
     if (cand > st.best || (cand == st.best && id < st.bidx)) {
       st.best = cand;
@@ -154,8 +160,8 @@ __device__ __forceinline__ void epilogue4(const Epilogue& e, int64_t m, int n, f
       const int h = e.hd_shift >= 0 ? c >> e.hd_shift : c / e.hd, d = c - h * e.hd;
       const int mi = (int)m;
       const int b = e.T == 1 ? mi : mi / e.T, tt = mi - b * e.T;
-      const int s0 = e.len_dev ? *e.len_dev : e.S0;
-      if (s0 + tt < e.S_cap) {
+      const int s0 = e.len_dev ? e.len_dev[b] : e.S0;  // per-row lengths: T == 1, b = row
+      if (s0 >= 0 && s0 + tt < e.S_cap) {
         half_t* dst = (part == 0 ? e.Kc : e.Vc) +
                       (((int64_t)b * e.H + h) * e.S_cap + s0 + tt) * e.hd + d;
         *reinterpret_cast<half4_t*>(dst) = o;
@@ -1254,17 +1260,17 @@ namespace {
 int lm_head_select_impl(const char* name, const void* x, const void* Ep, void* logits,
                         void* workspace, int M, int V, int K, float temperature,
                         const int32_t* banned_host, int n_banned, const int32_t* stop_host,
-                        int n_stop, uint8_t* finished, int force_eos_all, int eos_idx, int64_t* tok,
-                        int64_t tok_stride, float* score, int64_t score_stride,
-                        const int32_t* len_dev, void* stream) {
+                        int n_stop, uint8_t* finished, const uint8_t* row_mode, int force_eos_all,
+                        int eos_idx, int64_t* tok, int64_t tok_stride, float* score,
+                        int64_t score_stride, const int32_t* len_dev, void* stream) {
   MSA_REQUIRE(x && Ep && workspace && tok && score, MSA_ERR_INVALID_ARG, "%s: null pointer", name);
   MSA_REQUIRE(M >= 1 && M <= 64 && V > 0 && V % 16 == 0 && K > 0 && K % 32 == 0,
               MSA_ERR_INVALID_ARG, "%s: bad shape M=%d V=%d K=%d (1 <= M <= 64, V %% 16, K %% 32)",
               name, M, V, K);
   MSA_REQUIRE(n_banned >= 0 && n_banned <= 16 && (n_banned == 0 || banned_host),
               MSA_ERR_INVALID_ARG, "%s: n_banned=%d (0..16)", name, n_banned);
-  MSA_REQUIRE(n_stop >= 0 && n_stop <= 16 && (n_stop == 0 || stop_host), MSA_ERR_INVALID_ARG,
-              "%s: n_stop=%d (0..16)", name, n_stop);
+  MSA_REQUIRE(n_stop >= 0 && n_stop <= 15 && (n_stop == 0 || stop_host), MSA_ERR_INVALID_ARG,
+              "%s: n_stop=%d (0..15)", name, n_stop);
   MSA_REQUIRE(eos_idx >= 0 && eos_idx < V, MSA_ERR_INVALID_ARG,
               "%s: eos_idx=%d outside the vocabulary", name, eos_idx);
   MSA_REQUIRE(temperature >= 0.f, MSA_ERR_INVALID_ARG, "%s: temperature < 0", name);
@@ -1273,6 +1279,10 @@ int lm_head_select_impl(const char* name, const void* x, const void* Ep, void* l
   e.N = V;
   e.partials = (SelectPartial*)workspace;
   e.finished = finished;
+  e.row_mode = row_mode;
+  e.early.n = 1 + n_stop;
+  e.early.id[0] = eos_idx;
+  for (int i = 0; i < n_stop; ++i) e.early.id[1 + i] = stop_host[i];
   e.banned.n = n_banned;
   for (int i = 0; i < n_banned; ++i) e.banned.id[i] = banned_host[i];
   e.temperature = temperature;
@@ -1298,13 +1308,13 @@ int lm_head_select_impl(const char* name, const void* x, const void* Ep, void* l
 extern "C" int msa_lm_head_greedy_select_f16(
     const void* x, const void* Ep, void* logits, void* workspace, int M, int V, int K,
     float temperature, const int32_t* banned_host, int n_banned, const int32_t* stop_host,
-    int n_stop, uint8_t* finished, int force_eos_all, int eos_idx, int64_t* tok,
-    int64_t tok_stride, float* score, int64_t score_stride, const int32_t* len_dev,
+    int n_stop, uint8_t* finished, const uint8_t* row_mode, int force_eos_all, int eos_idx,
+    int64_t* tok, int64_t tok_stride, float* score, int64_t score_stride, const int32_t* len_dev,
     void* stream) {
   return lm_head_select_impl("msa_lm_head_greedy_select_f16", x, Ep, logits, workspace, M, V, K,
                              temperature, banned_host, n_banned, stop_host, n_stop, finished,
-                             force_eos_all, eos_idx, tok, tok_stride, score, score_stride, len_dev,
-                             stream);
+                             row_mode, force_eos_all, eos_idx, tok, tok_stride, score,
+                             score_stride, len_dev, stream);
 }
 
 // ---- the entry point that allocates nothing ---------------------------------------------------
@@ -1350,8 +1360,8 @@ void* scratch_for_current_device(const char* name) {
 extern "C" int msa_lm_head_greedy_select_noalloc_f16(
     const void* x, const void* Ep, void* logits, int M, int V, int K, float temperature,
     const int32_t* banned_host, int n_banned, const int32_t* stop_host, int n_stop,
-    uint8_t* finished, int force_eos_all, int eos_idx, int64_t* tok, int64_t tok_stride,
-    float* score, int64_t score_stride, const int32_t* len_dev, void* stream) {
+    uint8_t* finished, const uint8_t* row_mode, int force_eos_all, int eos_idx, int64_t* tok,
+    int64_t tok_stride, float* score, int64_t score_stride, const int32_t* len_dev, void* stream) {
   const char* name = "msa_lm_head_greedy_select_noalloc_f16";
   MSA_REQUIRE(M >= 1 && M <= NA_MAX_ROWS, MSA_ERR_CAPACITY,
               "%s: M=%d rows exceed the %d the fixed scratch array holds", name, M, NA_MAX_ROWS);
@@ -1363,8 +1373,8 @@ extern "C" int msa_lm_head_greedy_select_noalloc_f16(
   // every partial the combine kernel reads is written by the projection of the same call, so
   // nothing in the array has to start at zero
   return lm_head_select_impl(name, x, Ep, logits, ws, M, V, K, temperature, banned_host, n_banned,
-                             stop_host, n_stop, finished, force_eos_all, eos_idx, tok, tok_stride,
-                             score, score_stride, len_dev, stream);
+                             stop_host, n_stop, finished, row_mode, force_eos_all, eos_idx, tok,
+                             tok_stride, score, score_stride, len_dev, stream);
 }
 
 namespace {

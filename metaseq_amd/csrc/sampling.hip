@@ -65,14 +65,17 @@ __device__ __forceinline__ RowStats row_logsumexp(const half_t* __restrict__ row
 
 __global__ __launch_bounds__(SM_THREADS) void greedy_select_kernel(
     const half_t* __restrict__ logits, int64_t ld, int V, float temperature, bool scale,
-    IdList banned, IdList stop, uint8_t* __restrict__ finished, int force_eos_all, int eos,
+    IdList banned, IdList stop, uint8_t* __restrict__ finished,
+    const uint8_t* __restrict__ row_mode, int force_eos_all, int eos,
     int64_t* __restrict__ tok, int64_t tok_stride, float* __restrict__ score,
     int64_t score_stride, const int32_t* __restrict__ len_dev) {
   __shared__ float wm[16], ws[16], wbest[16], wnan[16];
   __shared__ int widx[16];
   const int b = blockIdx.x;
   const half_t* row = logits + (int64_t)b * ld;
-  const bool only_eos = force_eos_all || (finished && finished[b]);
+  const unsigned rm = row_mode ? row_mode[b] : 0u;
+  const bool only_eos = force_eos_all || (finished && finished[b]) || (rm & MSA_ROW_ONLY_EOS);
+  const bool ban_early = rm & MSA_ROW_BAN_EARLY;  // eos and the stop ids are not eligible
 
   // single pass: running log-sum-exp over ALL ids, and the best eligible id (log-softmax is
   // monotone in z, so the arg-max of the masked log-probs is the arg-max of the masked z)
@@ -81,8 +84,10 @@ __global__ __launch_bounds__(SM_THREADS) void greedy_select_kernel(
   bool nan = false;
   auto visit = [&](int i, float z) {  // arg-max bookkeeping of one id
     nan |= (z != z);
-    bool ok = !(only_eos && i != eos);
+    bool ok = !(only_eos && i != eos) && !(ban_early && i == eos);
     for (int j = 0; j < banned.n; ++j) ok &= (banned.id[j] != i);
+    if (ban_early)
+      for (int j = 0; j < stop.n; ++j) ok &= (stop.id[j] != i);
     const float cand = ok ? z : -INFINITY;
     if (cand > best || (cand == best && i < bidx)) {
       best = cand;
@@ -276,7 +281,8 @@ int msa_launch_select_combine(const SelectPartial* partials, int n_parts, int B,
 extern "C" int msa_greedy_select_f16(const void* logits, int64_t ld_logits, int B, int V,
                                      float temperature, const int32_t* banned_host, int n_banned,
                                      const int32_t* stop_host, int n_stop, uint8_t* finished,
-                                     int force_eos_all, int eos_idx, int64_t* tok,
+                                     const uint8_t* row_mode, int force_eos_all, int eos_idx,
+                                     int64_t* tok,
                                      int64_t tok_stride, float* score, int64_t score_stride,
                                      const int32_t* len_dev, void* stream) {
   MSA_REQUIRE(logits && tok && score, MSA_ERR_INVALID_ARG, "msa_greedy_select_f16: null pointer");
@@ -297,8 +303,8 @@ extern "C" int msa_greedy_select_f16(const void* logits, int64_t ld_logits, int 
   for (int i = 0; i < n_stop; ++i) stop.id[i] = stop_host[i];
   hipLaunchKernelGGL(greedy_select_kernel, dim3(B), dim3(SM_THREADS), 0, (hipStream_t)stream,
                      (const half_t*)logits, ld_logits, V, temperature, scale, banned, stop,
-                     finished, force_eos_all, eos_idx, tok, tok_stride, score, score_stride,
-                     len_dev);
+                     finished, row_mode, force_eos_all, eos_idx, tok, tok_stride, score,
+                     score_stride, len_dev);
   MSA_CHECK_LAUNCH("msa_greedy_select_f16");
   return MSA_OK;
 }

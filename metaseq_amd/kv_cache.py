@@ -3,7 +3,10 @@
 The reference grows its cache by ``torch.cat`` every step and every layer
 (metaseq/modules/multihead_attention.py:449-479), re-copying the whole history.  Here each
 layer owns one fp16 tensor ``[2, B, H, S_cap, hd]`` (K then V) that the QKV kernel appends to
-in place; ``length`` counts the valid positions.  The object lives inside the caller-owned
+in place; ``length`` counts the valid positions (columns of the token history).  A "ragged"
+cache (prefilled from right-padded prompts, or filled slot by slot) stores every row without
+pads and keeps the per-row lengths in ``lens`` (int32 [B] on the device, negative = empty
+slot).  The object lives inside the caller-owned
 ``incremental_state`` dict, as the reference's per-module buffers do
 (metaseq/incremental_decoding_utils.py:30-69), and is freed with it.
 """
@@ -17,6 +20,8 @@ class KVCache:
         self.length = 0
         self.device = device
         self.has_pads = False
+        self.ragged = False
+        self.lens = None  # int32 [B] device tensor when ragged
         self.layers = [
             torch.empty(2, batch, heads, self.capacity, head_dim, dtype=torch.float16,
                         device=device)

@@ -110,19 +110,20 @@ class SequenceGenerator(nn.Module):
         sc = scores[:, col]
         check(lib.msa_greedy_select_f16(
             ptr(logits2d), logits2d.stride(0), B, V, float(self.temperature), arr, len(banned),
-            stop, len(self.stop), ptr(finished), int(step >= max_len - 1), self.eos,
+            stop, len(self.stop), ptr(finished), None, int(step >= max_len - 1), self.eos,
             ptr(tok), tokens.stride(0), ptr(sc), scores.stride(0), ptr(len_dev),
             _capi.stream_ptr()))
 
     @staticmethod
     def static_state(decoder, cache, tokens, scores, finished, step_logits):
-        """State of graph-replayed decoding: fixed-address buffers plus the device-side length
-        (= positions already in ``cache``; the next token goes to that column of ``tokens``)."""
+        """State of graph-replayed decoding: fixed-address buffers plus the device-side per-row
+        lengths (= positions already in ``cache``; all rows equal here, and the next token goes
+        to that column of ``tokens``)."""
         return {"graphs": {}, "decoder": decoder, "cache": cache, "tokens": tokens,
                 "scores": scores, "finished": finished,
                 "logits": step_logits.contiguous().clone(),
-                "len_dev": torch.tensor([cache.length], dtype=torch.int32,
-                                        device=tokens.device)}
+                "len_dev": torch.full((tokens.shape[0],), cache.length, dtype=torch.int32,
+                                      device=tokens.device)}
 
     def _graph_body(self, lib, st, step, min_len, max_len):
         """One decode step with nothing step-dependent in its launch arguments: select the token
@@ -131,7 +132,8 @@ class SequenceGenerator(nn.Module):
         self._select(lib, st["logits"], step, min_len, max_len, st["finished"], st["tokens"],
                      st["scores"], st["len_dev"])
         st["decoder"].decode_step_static(st["tokens"], st["cache"], st["len_dev"], st["logits"])
-        check(lib.msa_advance_len(ptr(st["len_dev"]), 1, _capi.stream_ptr()))
+        check(lib.msa_advance_len(ptr(st["len_dev"]), None, st["len_dev"].numel(), 1,
+                                  _capi.stream_ptr()))
 
     def _graph_step(self, lib, st, step, min_len, max_len):
         """Runs the step through a captured graph; the first step of each masking regime

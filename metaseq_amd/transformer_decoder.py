@@ -15,7 +15,8 @@ import torch
 from torch import nn
 
 from . import _capi
-from ._capi import MSA_EPI_RELU, MSA_IN_PACKED, MSA_OUT_PACKED, check, ptr
+from ._capi import (MSA_EMBED_COL_FROM_LEN, MSA_EPI_RELU, MSA_IN_PACKED, MSA_OUT_PACKED, check,
+                    ptr)
 from .config import OPTConfig
 from .kv_cache import KVCache
 
@@ -312,17 +313,20 @@ class TransformerDecoder(nn.Module):
                 "u": torch.empty(MP * F, **f16), "feat": torch.empty(B, D, **f16),
                 "part": torch.empty(max(S_o, S_f) * B * D, dtype=torch.float32, device=dev),
                 "positions": torch.empty(B, 1, dtype=torch.long, device=dev),
+                "step_len": torch.empty(B, dtype=torch.int32, device=dev),
                 "S_o": S_o, "S_f": S_f,
             }
             cache.step_bufs = bufs
         return bufs
 
     def _decode_core(self, lib, stream, tokens, n, B, cache, mask, bufs, len_dev, S0,
-                     want_packed):
+                     want_packed, col_from_len=False):
         """One decode step for at most 64 rows: packed activations, weight-streaming kernels,
-        split-K tails fused into the LayerNorm that follows.  With ``len_dev`` (int32 device
-        tensor holding the cache length) nothing in the launch arguments depends on the step,
-        so the sequence can be captured once and replayed."""
+        split-K tails fused into the LayerNorm that follows.  With ``len_dev`` (int32 [B] device
+        tensor: positions of each row already in the cache, negative = inactive row) every row
+        appends at and attends up to its own length, and nothing in the launch arguments
+        depends on the step, so the sequence can be captured once and replayed.  The new tokens
+        are the last column of ``tokens`` (or column ``len_dev[b]`` with ``col_from_len``)."""
         cfg = self.cfg
         D, H, hd = cfg.decoder_embed_dim, cfg.decoder_attention_heads, cfg.head_dim
         F, L, M = cfg.decoder_ffn_embed_dim, cfg.decoder_layers, B
@@ -330,12 +334,18 @@ class TransformerDecoder(nn.Module):
         S_o, S_f = bufs["S_o"], bufs["S_f"]
         IN, OUT = MSA_IN_PACKED, MSA_OUT_PACKED
         mask_stride = mask.stride(0) if mask is not None else 0
-        ld = ptr(len_dev)
+        # a row whose new token is a pad sits this step out (step_len = -1), as does an
+        # inactive row; under graph replay there are no pads and the lengths are used as is
+        step_len = bufs["step_len"] if (len_dev is not None and not col_from_len) else None
         check(lib.msa_embed_f16(ptr(tokens), tokens.stride(0), B, n, 1,
                                 ptr(self.embed_tokens.weight), cfg.vocab_size,
                                 ptr(self.embed_positions.weight),
                                 self.embed_positions.weight.shape[0], self.padding_idx, D,
-                                ptr(x), ptr(bufs["positions"]), None, ld, stream))
+                                ptr(x), ptr(bufs["positions"]), None, ptr(len_dev), ptr(step_len),
+                                MSA_EMBED_COL_FROM_LEN if col_from_len else 0, stream))
+        if step_len is not None:
+            len_dev = step_len
+        ld = ptr(len_dev)
         self._layernorm(lib, stream, x, self.layers[0].self_attn_layer_norm, M, D, h, OUT)
         x_last = None
         feat = h
@@ -375,8 +385,8 @@ class TransformerDecoder(nn.Module):
         return feat, x_last
 
     def decode_step_static(self, tokens, cache, len_dev, logits_out):
-        """Graph-capturable decode step: embeds column ``*len_dev`` of the full ``tokens``
-        buffer, appends to ``cache`` at that position, attends ``*len_dev + 1`` positions and
+        """Graph-capturable decode step: embeds column ``len_dev[b]`` of the full ``tokens``
+        buffer, appends to ``cache`` at that position, attends ``len_dev[b] + 1`` positions and
         writes ``logits_out[B, V]``.  No allocation, no sync, no step-dependent launch argument.
         The caller advances ``len_dev`` (msa_advance_len) and ``cache.length``."""
         lib = self.prepare_()
@@ -386,7 +396,7 @@ class TransformerDecoder(nn.Module):
             raise ValueError("static decode steps need at most 64 rows and no padding")
         bufs = self._step_buffers(cache, B)
         feat, _ = self._decode_core(lib, stream, tokens, tokens.shape[1], B, cache, None, bufs,
-                                    len_dev, 0, True)
+                                    len_dev, 0, True, col_from_len=True)
         D, V = self.cfg.decoder_embed_dim, self.cfg.vocab_size
         check(lib.msa_linear_f16(ptr(feat), ptr(self._lm_head), None, None, ptr(logits_out), B, V,
                                  D, MSA_IN_PACKED, stream))
@@ -438,13 +448,27 @@ class TransformerDecoder(nn.Module):
 
         # key padding mask: the reference tests tokens.eq(pad).any() on every call (a
         # device-to-host sync, transformer_decoder.py:357-361); here only the prefill syncs.
-        mask = None
+        # Right-padded prompts (the only padding a serving batch has) make the cache "ragged":
+        # every row's keys and values are stored without its pads, per-row lengths live on the
+        # device, and decode steps neither mask nor stream pad positions.  Pads anywhere else
+        # keep the reference's layout (pads stored, masked at every step).
+        mask, ragged, lens = None, False, None
         if self_attn_padding_mask is not None:
+            if not prefill and cache.ragged:
+                raise AssertionError("a cache prefilled from right-padded prompts stores no "
+                                     "pads: decode steps take no padding mask")
             mask = self_attn_padding_mask
         elif prefill:
             m = tokens.eq(self.padding_idx)
-            if bool(m.any()):
+            counts = n - m.sum(dim=1)
+            trailing = m == (torch.arange(n, device=dev).unsqueeze(0) >= counts.unsqueeze(1))
+            any_pad, all_trailing = torch.stack([m.any(), trailing.all()]).tolist()
+            if any_pad:
                 mask = m
+                ragged = bool(all_trailing) and B <= 64
+                lens = counts.to(torch.int32)
+        elif cache.ragged:
+            lens = cache.lens
         elif cache.has_pads:
             mask = tokens.eq(self.padding_idx)
         if mask is not None:
@@ -459,14 +483,18 @@ class TransformerDecoder(nn.Module):
             cap = max(int(cap), n)
             cache = KVCache(L, B, H, hd, cap, dev)
             cache.has_pads = mask is not None
+            cache.ragged = ragged
+            cache.lens = lens if ragged else None
         elif S0 + 1 > cache.capacity:
             cache.grow(min(max(self.max_positions(), S0 + 1), int(cache.capacity * 1.5) + 64))
 
         M = B * T
         if T == 1 and M <= 64:
             bufs = self._step_buffers(cache, B)
-            feat, x_last = self._decode_core(lib, stream, tokens, n, B, cache, mask, bufs, None,
+            feat, x_last = self._decode_core(lib, stream, tokens, n, B, cache, mask, bufs, lens,
                                              S0, want_packed)
+            if lens is not None:
+                check(lib.msa_advance_len(ptr(lens), ptr(bufs["step_len"]), B, 1, stream))
             inner_states = [{"tok": None, "pos": bufs["positions"], "emb": None}, x_last]
             packed = want_packed
             features = feat if packed else feat.view(B, T, D)
@@ -480,7 +508,7 @@ class TransformerDecoder(nn.Module):
                                 ptr(self.embed_tokens.weight), cfg.vocab_size,
                                 ptr(self.embed_positions.weight),
                                 self.embed_positions.weight.shape[0], self.padding_idx, D,
-                                ptr(x), ptr(positions), None, None, stream))
+                                ptr(x), ptr(positions), None, None, None, 0, stream))
         inner_states = [{"tok": None, "pos": positions, "emb": None}]
         if self.return_inner_states:
             inner_states[0]["emb"] = x.view(B, T, D).transpose(0, 1).clone()
@@ -553,7 +581,7 @@ class TransformerDecoder(nn.Module):
 
     def forward_select(self, prev_output_tokens, incremental_state, *, temperature, banned, stop,
                        finished, force_eos, eos, tok_out, tok_stride, score_out, score_stride,
-                       logits_out=None):
+                       logits_out=None, row_mode=None):
         """One decode step (at most 64 rows) whose vocabulary projection is fused with the greedy
         selection of the next token (metaseq/models/transformer_decoder.py:494-537 followed by
         metaseq/sequence_generator.py:272-308,319-323): the logits are reduced inside the
@@ -577,8 +605,8 @@ class TransformerDecoder(nn.Module):
         sa = (ctypes.c_int32 * max(1, len(stop)))(*stop)
         check(lib.msa_lm_head_greedy_select_f16(
             ptr(f), ptr(self._lm_head), ptr(logits_out), ptr(ws), B, V, D, float(temperature), ba,
-            len(banned), sa, len(stop), ptr(finished), int(force_eos), int(eos), ptr(tok_out),
-            tok_stride, ptr(score_out), score_stride, None, _capi.stream_ptr()))
+            len(banned), sa, len(stop), ptr(finished), ptr(row_mode), int(force_eos), int(eos),
+            ptr(tok_out), tok_stride, ptr(score_out), score_stride, None, _capi.stream_ptr()))
 
 
 # the name the reference's model code uses for this class

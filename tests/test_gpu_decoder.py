@@ -9,7 +9,7 @@ import torch
 from metaseq_amd import (Dictionary, OPTConfig, SequenceGenerator, TransformerLanguageModel,
                          opt_config, random_prompts, random_state_dict)
 from oracle.opt_oracle import greedy_generate
-from tests.common import make_oracle, tiny_cfg
+from tests.common import assert_tokens_match_up_to_ties, make_oracle, tiny_cfg
 from tests.scripted import CASES, ScriptedDecoder
 
 pytestmark = pytest.mark.gpu
@@ -138,6 +138,51 @@ def test_batch4_padded_generation_matches_oracle():
     got = run_generate(model, cfg, src, max_len_b, max_len_b - 1)
     assert torch.equal(got["tokens"].cpu(), want["tokens"])
     assert torch.allclose(got["scores"].cpu(), want["scores"], atol=5e-2)
+
+
+def test_ragged_batch_keeps_per_row_lengths_and_matches_oracle():
+    """Right-padded prompts of different lengths (what a serving batch looks like): the cache
+    stores no pads, every row's length lives on the device and advances by one per step, and
+    greedy tokens are the oracle's (which keeps the pads and masks them,
+    metaseq/modules/multihead_attention.py:485-531) up to numerical ties.  Teacher-forced logits
+    of every decode step are within tolerance, and a left-padded batch still takes the masked
+    layout."""
+    cfg = opt_config("125m", max_target_positions=128)
+    model, sd = build(cfg, seed=31)
+    src = random_prompts(cfg, 6, 30, seed=13)
+    real = [31, 3, 17, 31, 9, 24]            # tokens per row, the leading eos included
+    for b, n in enumerate(real):
+        src[b, n:] = 1
+    oracle = make_oracle(cfg, sd, torch.float16)
+    n0, G = src.shape[1], 20
+    max_len_b = n0 + G + 1
+    want = greedy_generate(oracle, src, max_len_b=max_len_b, min_len=max_len_b - 1,
+                           return_step_logits=True)
+    got = run_generate(model, cfg, src, max_len_b, max_len_b - 1)
+    diverged = assert_tokens_match_up_to_ties(got["tokens"][:, 0], want["tokens"][:, 0],
+                                              want["step_logits"], n0,
+                                              prefill_index=[n - 1 for n in real])
+    assert len(diverged) <= 2
+    wt = want["tokens"][:, 0].to(DEV)
+    inc = {}
+    model.decoder.kv_cache_capacity = max_len_b
+    logits = model(wt[:, :n0], incremental_state=inc)[0]
+    cache = model.decoder.get_cache(inc)
+    assert cache.ragged and cache.lens.tolist() == real
+    valid = src.ne(1)
+    check_logits(logits.cpu()[valid], want["step_logits"][0][valid], "ragged prefill")
+    for i, t in enumerate(range(n0, n0 + G)):
+        step = model.decoder(wt[:, :t + 1], incremental_state=inc)[0]
+        check_logits(step, want["step_logits"][i + 1], "ragged step %d" % t)
+    assert cache.lens.tolist() == [n + G for n in real] and cache.length == n0 + G
+    model.decoder.kv_cache_capacity = None
+    # pads in front: not ragged, the masked layout of the reference
+    left = random_prompts(cfg, 2, 12, seed=5)
+    left[1, 1:4] = 1
+    inc2 = {}
+    model(left.to(DEV), incremental_state=inc2)
+    c2 = model.decoder.get_cache(inc2)
+    assert c2.has_pads and not c2.ragged
 
 
 @pytest.mark.parametrize("name", sorted(CASES))

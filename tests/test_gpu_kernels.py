@@ -145,7 +145,7 @@ def test_embed_positions_and_sum(lib, T_out):
     po = torch.empty(B, T_out, dtype=torch.long, device=DEV)
     st = torch.zeros(1, dtype=torch.int32, device=DEV)
     ok(lib.msa_embed_f16(P(td), td.stride(0), B, n, T_out, P(G(E)), V, P(G(Ptab)),
-                         Ptab.shape[0], pad, D, P(x), P(po), P(st), None, None), lib)
+                         Ptab.shape[0], pad, D, P(x), P(po), P(st), None, None, 0, None), lib)
     torch.cuda.synchronize()
     assert torch.equal(po.cpu(), want_pos)
     assert torch.equal(x.cpu().float().view(B, T_out, D), want)
@@ -159,14 +159,18 @@ def test_embed_flags_out_of_range_ids(lib):
     x = torch.empty(1, D, dtype=torch.float16, device=DEV)
     st = torch.zeros(1, dtype=torch.int32, device=DEV)
     ok(lib.msa_embed_f16(P(toks), 3, 1, 3, 1, P(G(E)), V, P(G(Ptab)), 6, 1, D, P(x),
-                         None, P(st), None, None), lib)
+                         None, P(st), None, None, 0, None), lib)
     torch.cuda.synchronize()
     assert int(st) == 1
 
 
+COL_FROM_LEN = 8
+
+
 def test_device_side_length_matches_host_arguments(lib):
     """embed / qkv append / attention / select with the history length read from device memory
-    give the results of the host-argument form, and msa_advance_len increments it."""
+    (one entry per row, all equal here) give the results of the host-argument form, and
+    msa_advance_len increments every entry."""
     B, H, hd, V, S_cap = 4, 2, 64, 64, 24
     D = H * hd
     E, Ptab = rnd(V, D, seed=4), rnd(40, D, seed=5)
@@ -175,13 +179,14 @@ def test_device_side_length_matches_host_arguments(lib):
     W, bq = rnd(3 * D, D, seed=2, std=0.05), rnd(3 * D, seed=3, std=0.1)
     Wp = pack_w(lib, G(W))
     Kc0, Vc0 = G(rnd(B, H, S_cap, hd, seed=6)), G(rnd(B, H, S_cap, hd, seed=7))
-    ln = torch.tensor([11], dtype=torch.int32, device=DEV)
+    ln = torch.full((B,), 11, dtype=torch.int32, device=DEV)
     outs = []
     for len_dev, n, S0 in ((None, 12, 11), (ln, 20, 0)):
         Kc, Vc = Kc0.clone(), Vc0.clone()
         x = torch.empty(B, D, dtype=torch.float16, device=DEV)
         ok(lib.msa_embed_f16(P(td), 20, B, n, 1, P(G(E)), V, P(G(Ptab)), 40, 1, D, P(x), None,
-                             None, P(len_dev), None), lib)
+                             None, P(len_dev), None, COL_FROM_LEN if len_dev is not None else 0,
+                             None), lib)
         q = torch.empty(B, D, dtype=torch.float16, device=DEV)
         xp = G(pack_act(x.cpu()))
         ok(lib.msa_qkv_proj_f16(P(xp), P(Wp), P(G(bq)), P(q), P(Kc), P(Vc), B, 1, H, hd, S0, S_cap,
@@ -193,17 +198,129 @@ def test_device_side_length_matches_host_arguments(lib):
         sc = torch.zeros(B, 20, dtype=torch.float32, device=DEV)
         ba = (ctypes.c_int32 * 1)(1)
         col = 0 if len_dev is not None else 11
-        ok(lib.msa_greedy_select_f16(P(o), D, B, D, 1.0, ba, 1, ba, 0, None, 0, 2, P(tok[:, col]),
-                                     20, P(sc[:, col]), 20, P(len_dev), None), lib)
+        ok(lib.msa_greedy_select_f16(P(o), D, B, D, 1.0, ba, 1, ba, 0, None, None, 0, 2,
+                                     P(tok[:, col]), 20, P(sc[:, col]), 20, P(len_dev), None), lib)
         torch.cuda.synchronize()
         outs.append((x.clone(), q.clone(), Kc.clone(), Vc.clone(), o.clone(), tok.clone(),
                      sc.clone()))
     for a, b in zip(*outs):
         assert torch.equal(a, b)
     assert int(outs[0][5][:, 11].abs().sum()) > 0
-    ok(lib.msa_advance_len(P(ln), 1, None), lib)
+    ok(lib.msa_advance_len(P(ln), None, B, 1, None), lib)
     torch.cuda.synchronize()
-    assert int(ln) == 12
+    assert ln.tolist() == [12] * B
+
+
+@pytest.mark.parametrize("hd,H", [(64, 3), (128, 2)])
+def test_per_row_lengths_append_and_attend_each_row_at_its_own_length(lib, hd, H):
+    """A decode step over rows of different lengths (and one inactive row, length -1): every row
+    gets the position embedding of its own length, appends its key and value at its own slot
+    and attends exactly its own history.  Checked against the oracle's attention arithmetic
+    row by row on that row's history; slots past a row's length hold NaN, so a key read beyond
+    the length would poison the result."""
+    print("per-row lengths", hd, H, flush=True)
+    V, S_cap, pad = 64, 40, 1
+    D = H * hd
+    lens = [0, 7, 19, -1, 38, 3, 5]
+    B = len(lens)
+    E, Ptab = rnd(V, D, seed=4), rnd(S_cap + 4, D, seed=5)
+    toks = torch.randint(4, V, (B, 1), generator=torch.Generator().manual_seed(1))
+    toks[6, 0] = pad  # a pad as the new token: the row sits the step out
+    W, bq = rnd(3 * D, D, seed=2, std=0.05), rnd(3 * D, seed=3, std=0.1)
+    Wp = pack_w(lib, G(W))
+    Kc, Vc = rnd(B, H, S_cap, hd, seed=6), rnd(B, H, S_cap, hd, seed=7)
+    for b, n in enumerate(lens):
+        Kc[b, :, max(n, 0):] = float("nan")
+        Vc[b, :, max(n, 0):] = float("nan")
+    Kd, Vd = G(Kc.clone()), G(Vc.clone())
+    ln = torch.tensor(lens, dtype=torch.int32, device=DEV)
+    x = torch.empty(B, D, dtype=torch.float16, device=DEV)
+    po = torch.empty(B, 1, dtype=torch.long, device=DEV)
+    sl = torch.full((B,), 99, dtype=torch.int32, device=DEV)
+    ok(lib.msa_embed_f16(P(G(toks)), 1, B, 1, 1, P(G(E)), V, P(G(Ptab)), Ptab.shape[0], pad, D,
+                         P(x), P(po), None, P(ln), P(sl), 0, None), lib)
+    q = torch.zeros(B, D, dtype=torch.float16, device=DEV)
+    ok(lib.msa_qkv_proj_f16(P(G(pack_act(x.cpu()))), P(Wp), P(G(bq)), P(q), P(Kd), P(Vd), B, 1, H,
+                            hd, 0, S_cap, D, IN_PACKED, P(sl), None), lib)
+    o = torch.full((B, D), 7.0, dtype=torch.float16, device=DEV)
+    ok(lib.msa_attention_f16(P(q), P(Kd), P(Vd), None, 0, P(o), B, H, hd, 1, max(lens), S_cap, 0,
+                             P(sl), None), lib)
+    ok(lib.msa_advance_len(P(ln), P(sl), B, 1, None), lib)
+    torch.cuda.synchronize()
+    assert sl.tolist() == [0, 7, 19, -1, 38, 3, -1]
+    assert ln.tolist() == [1, 8, 20, -1, 39, 4, 5]
+    lens[6] = -1  # from here on row 6 is checked like the inactive row
+    dec = O.OracleDecoder(O.OracleConfig(1, D, H, 4 * D, V, S_cap), {}, dtype=torch.float16)
+    for b, n in enumerate(lens):
+        if n < 0:  # inactive: nothing appended, output row untouched
+            assert torch.equal(o[b].cpu(), torch.full((D,), 7.0, dtype=torch.float16))
+            assert torch.equal(torch.isnan(Kd[b].cpu()), torch.isnan(Kc[b]))
+            continue
+        assert int(po[b]) == pad + 1 + n
+        xb = r16(E[toks[b, 0]].float() + Ptab[pad + 1 + n].float())
+        assert torch.equal(x[b].cpu().float(), xb)
+        kvq = O.linear(xb.unsqueeze(0), W.float(), bq.float(), r16)[0]
+        k, v, qq = kvq.split(D)
+        qq = r16(qq * hd ** -0.5)
+        assert_fp16_close(q[b], qq, atol=2e-3, max_frac=0.05, what="q")
+        # the new key / value sit at slot n; slots before keep the history, slots after NaN
+        kb, vb = Kd[b].cpu(), Vd[b].cpu()
+        assert_fp16_close(kb[:, n].reshape(-1), k, atol=2e-3, max_frac=0.05, what="appended k")
+        assert_fp16_close(vb[:, n].reshape(-1), v, atol=2e-3, max_frac=0.05, what="appended v")
+        assert torch.equal(kb[:, :n], Kc[b, :, :n]) and bool(torch.isnan(kb[:, n + 1:]).all())
+        want = dec.attention_core(q[b].cpu().float().view(H, 1, hd), kb[:, :n + 1].float(),
+                                  vb[:, :n + 1].float(), 1)
+        assert_fp16_close(o[b], want.reshape(-1), atol=2e-3, max_frac=0.05, what="attention row %d" % b)
+
+
+def test_selection_with_per_row_modes(lib):
+    """row_mode gives every row its own regime: MSA_ROW_BAN_EARLY removes eos and the stop ids,
+    MSA_ROW_ONLY_EOS leaves only eos.  Both selection entry points, against masked arg-max."""
+    M, V, K, eos = 12, 4000, 128, 2
+    x, E = rnd(M, K, seed=3, std=1.0), rnd(V, K, seed=4, std=0.3)
+    Ep = pack_w(lib, G(E))
+    xp = G(pack_act(x))
+    logits = torch.empty(M, V, dtype=torch.float16, device=DEV)
+    ok(lib.msa_linear_f16(P(xp), P(Ep), None, None, P(logits), M, V, K, IN_PACKED, None), lib)
+    # make eos or a stop id the plain arg-max of some rows, so the bans change the outcome
+    lg = logits.float().cpu()
+    stop = [int(lg[1].argmax()), int(lg[4].argmax())]
+    modes = torch.tensor([0, 1, 2, 0, 1, 3, 0, 1, 2, 0, 1, 0], dtype=torch.uint8)
+    want = []
+    for m in range(M):
+        z = lg[m].clone()
+        z[1] = float("-inf")  # pad is always banned
+        if modes[m] & 1:
+            z[[eos] + stop] = float("-inf")
+        if modes[m] & 2:
+            keep = z[eos].clone()
+            z[:] = float("-inf")
+            z[eos] = keep
+        want.append(int(z.argmax()) if bool(torch.isfinite(z).any()) else 0)
+    ba = (ctypes.c_int32 * 1)(1)
+    sa = (ctypes.c_int32 * 2)(*stop)
+    ws = torch.empty(lib.msa_lm_head_select_workspace_bytes(M), dtype=torch.uint8, device=DEV)
+    md = G(modes)
+    for fused in (True, False):
+        tok = torch.full((M,), -7, dtype=torch.long, device=DEV)
+        sc = torch.zeros(M, dtype=torch.float32, device=DEV)
+        fin = torch.zeros(M, dtype=torch.uint8, device=DEV)
+        if fused:
+            ok(lib.msa_lm_head_greedy_select_f16(P(xp), P(Ep), None, P(ws), M, V, K, 1.0, ba, 1, sa,
+                                                 2, P(fin), P(md), 0, eos, P(tok), 1, P(sc), 1,
+                                                 None, None), lib)
+        else:
+            ok(lib.msa_greedy_select_f16(P(logits), V, M, V, 1.0, ba, 1, sa, 2, P(fin), P(md), 0,
+                                         eos, P(tok), 1, P(sc), 1, None, None), lib)
+        torch.cuda.synchronize()
+        assert tok.tolist() == want, (fused, tok.tolist(), want)
+        assert fin.tolist() == [int(t == eos or t in stop) for t in want]
+        lp = torch.log_softmax(lg, -1)
+        for m in range(M):  # mode 3: eos banned and alone eligible -> (0, -inf)
+            if modes[m] == 3:
+                assert float(sc[m]) == float("-inf")
+            else:
+                assert abs(float(sc[m]) - float(lp[m, want[m]])) < 2e-5
 
 
 def test_pack_roundtrip_and_layout(lib):
@@ -542,7 +659,7 @@ def _select(lib, logits, temperature=1.0, banned=(), stop=(), finished=None, for
     ba = (ctypes.c_int32 * max(1, len(banned)))(*banned)
     sa = (ctypes.c_int32 * max(1, len(stop)))(*stop)
     ok(lib.msa_greedy_select_f16(P(logits), logits.stride(0), B, V, temperature, ba, len(banned),
-                                 sa, len(stop), P(finished), force, eos, P(tok[:, 1]), 3,
+                                 sa, len(stop), P(finished), None, force, eos, P(tok[:, 1]), 3,
                                  P(sc[:, 1]), 3, None, None), lib)
     torch.cuda.synchronize()
     assert float(tok[:, 0].abs().sum()) == 0 and float(tok[:, 2].abs().sum()) == 0
@@ -637,11 +754,11 @@ def test_lm_head_fused_selection_matches_projection_then_select(lib, M, V, K):
             if fused:
                 ok(lib.msa_lm_head_greedy_select_f16(
                     P(xp), P(Ep), P(lg), P(ws), M, V, K, temp, ba, len(banned), sa, len(stop),
-                    P(fin), force, 2, P(tok[:, 1]), 3, P(sc[:, 1]), 3, None, None), lib)
+                    P(fin), None, force, 2, P(tok[:, 1]), 3, P(sc[:, 1]), 3, None, None), lib)
                 fused_logits = lg
             else:
                 ok(lib.msa_greedy_select_f16(P(fused_logits), V, M, V, temp, ba, len(banned), sa,
-                                             len(stop), P(fin), force, 2, P(tok[:, 1]), 3,
+                                             len(stop), P(fin), None, force, 2, P(tok[:, 1]), 3,
                                              P(sc[:, 1]), 3, None, None), lib)
             torch.cuda.synchronize()
             outs.append((tok.cpu(), sc.cpu(), None if fin is None else fin.cpu()))
@@ -660,14 +777,14 @@ def test_lm_head_fused_selection_matches_projection_then_select(lib, M, V, K):
     sc = torch.zeros(M, 3, dtype=torch.float32, device=DEV)
     ba = (ctypes.c_int32 * 1)(1)
     ok(lib.msa_lm_head_greedy_select_f16(P(xp), P(Ep), None, P(ws), M, V, K, 1.0, ba, 1, ba, 0,
-                                         None, 0, 2, P(tok), 3, P(sc), 3, P(ln), None), lib)
+                                         None, None, 0, 2, P(tok), 3, P(sc), 3, P(ln), None), lib)
     xn = x.clone()
     xn[0, 0] = float("nan")
     tok2 = torch.full((M, 1), -7, dtype=torch.long, device=DEV)
     sc2 = torch.zeros(M, 1, dtype=torch.float32, device=DEV)
     ok(lib.msa_lm_head_greedy_select_f16(P(G(pack_act(xn))), P(Ep), None, P(ws), M, V, K, 1.0, ba,
-                                         1, ba, 0, None, 0, 2, P(tok2), 1, P(sc2), 1, None, None),
-       lib)
+                                         1, ba, 0, None, None, 0, 2, P(tok2), 1, P(sc2), 1, None,
+                                         None), lib)
     torch.cuda.synchronize()
     lg = logits.float().clone()
     lg[:, 1] = float("-inf")
@@ -677,9 +794,11 @@ def test_lm_head_fused_selection_matches_projection_then_select(lib, M, V, K):
         assert torch.equal(tok2[1:, 0].cpu(), lg[1:].argmax(-1).cpu())
     # argument checks
     assert lib.msa_lm_head_greedy_select_f16(P(xp), P(Ep), None, None, M, V, K, 1.0, ba, 1, ba, 0,
-                                             None, 0, 2, P(tok), 3, P(sc), 3, None, None) == -1
+                                             None, None, 0, 2, P(tok), 3, P(sc), 3, None,
+                                             None) == -1
     assert lib.msa_lm_head_greedy_select_f16(P(xp), P(Ep), None, P(ws), 65, V, K, 1.0, ba, 1, ba,
-                                             0, None, 0, 2, P(tok), 3, P(sc), 3, None, None) == -1
+                                             0, None, None, 0, 2, P(tok), 3, P(sc), 3, None,
+                                             None) == -1
 
 
 def test_stream_read_probe_runs_and_validates(lib):

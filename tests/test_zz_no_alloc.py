@@ -46,12 +46,12 @@ def _case(lib, M, V, K, seed, banned, stop, temperature, finished_rows):
             before = torch.cuda.memory_stats()["allocation.all.allocated"]
             rc = lib.msa_lm_head_greedy_select_noalloc_f16(
                 P(xp), P(Ep), P(lg), M, V, K, temperature, ba, len(banned), sa, len(stop), P(fin),
-                0, 2, P(tok[:, 1]), 3, P(sc[:, 1]), 3, None, None)
+                None, 0, 2, P(tok[:, 1]), 3, P(sc[:, 1]), 3, None, None)
             assert torch.cuda.memory_stats()["allocation.all.allocated"] == before
         else:
             rc = lib.msa_lm_head_greedy_select_f16(
                 P(xp), P(Ep), P(lg), P(ws), M, V, K, temperature, ba, len(banned), sa, len(stop),
-                P(fin), 0, 2, P(tok[:, 1]), 3, P(sc[:, 1]), 3, None, None)
+                P(fin), None, 0, 2, P(tok[:, 1]), 3, P(sc[:, 1]), 3, None, None)
         assert rc == 0, lib.msa_last_error().decode()
         torch.cuda.synchronize()
         outs.append((tok.cpu(), sc.cpu(), fin.cpu(), lg.cpu()))
@@ -88,5 +88,5 @@ def test_noalloc_entry_rejects_sizes_beyond_the_fixed_array():
     one = ctypes.c_void_p(256)
     ba = (ctypes.c_int32 * 1)(1)
     rc = lib.msa_lm_head_greedy_select_noalloc_f16(one, one, None, 65, 4000, 128, 1.0, ba, 1, ba,
-                                                   0, None, 0, 2, one, 1, one, 1, None, None)
+                                                   0, None, None, 0, 2, one, 1, one, 1, None, None)
     assert rc == -2 and b"exceed" in lib.msa_last_error()
