@@ -1,173 +1,437 @@
-"""Dynamic batching in front of ``GeneratorInterface``: the work queue, cost model and batching
-loop of the reference's hosted service (metaseq/service/queue.py, metaseq/service/workers.py,
-metaseq/cli/interactive_hosted.py:66-175), without its web layer.
+"""Serving loops in front of ``GeneratorInterface``, without a web layer.
 
-Requests are queued per generation-argument signature (requests that sample differently cannot
-share a batch), served smallest-cost first from the fullest queue, and grouped until the padded
-batch would exceed ``max_tokens`` or ``max_prompt + max_gen`` would exceed the model's sequence
-length; an unfilled batch runs after ``timeout`` milliseconds.  One thread drives the GPU
-(interactive_hosted.py:205); callers block on their own return queue.
+Two engines share one front (``submit`` from any thread, ``step`` / ``serve_forever`` on the one
+thread that drives the GPU, results delivered through a per-request queue):
+
+* ``BatchingService`` - run-to-completion batches, the policy of the reference's hosted service
+  (metaseq/cli/interactive_hosted.py:66-175 with metaseq/service/queue.py and workers.py):
+  requests wait in one backlog per sampling signature, the fullest backlog is served cheapest
+  request first, and a batch - a padded rectangle - closes when one more request would push
+  ``longest cost x rows`` over the token budget or ``longest prompt + longest continuation`` over
+  the sequence length, or when nothing arrives for ``timeout_ms``.
+* ``ContinuousBatcher`` - no reference counterpart: a fixed set of slots over one KV cache with
+  per-row lengths; a request is prefilled into a free slot whenever one exists and leaves it the
+  moment it ends, while the other rows keep decoding.  Greedy requests only; each row follows
+  its own ``min_tokens`` / ``max_tokens`` / end-of-sequence rules, and gets the record a
+  single-request ``GeneratorInterface.generate`` call would give it.
 """
+import heapq
+import itertools
 import math
 import queue
 import random
 import threading
-from dataclasses import dataclass, field
 from typing import Any, Dict, List, Optional
 
-# arguments that must agree within a batch (metaseq/service/workers.py:13-23)
-QUEUE_KEYS = ["temperature", "top_p", "n", "lambda_decay", "omega_bound", "alpha_presence",
-              "alpha_frequency", "alpha_presence_src", "alpha_frequency_src"]
-# arguments copied from the batch's requests into the generate() call
+# options that must agree within a run-to-completion batch (metaseq/service/workers.py:13-23)
+SIGNATURE_OPTIONS = ("temperature", "top_p", "n", "lambda_decay", "omega_bound", "alpha_presence",
+                     "alpha_frequency", "alpha_presence_src", "alpha_frequency_src")
+# options handed through to generate() from the requests of a batch
 # (interactive_hosted.py:125-142)
-SHARED_ARGS = ["temperature", "top_p", "n", "best_of", "echo", "logprobs", "stop", "omega_bound",
-               "lambda_decay", "alpha_presence", "alpha_frequency", "alpha_presence_src",
-               "alpha_frequency_src", "alpha_src_penalty_end_idx"]
+CALL_OPTIONS = ("temperature", "top_p", "n", "best_of", "echo", "logprobs", "stop", "omega_bound",
+                "lambda_decay", "alpha_presence", "alpha_frequency", "alpha_presence_src",
+                "alpha_frequency_src", "alpha_src_penalty_end_idx")
 MAX_SEQ_LEN = 2048        # metaseq/service/constants.py:8
 MAX_BATCH_TOKENS = 3072   # metaseq/service/constants.py:10
 
 
 def prompt_cost(n_tokens: int) -> int:
-    """Linear layers plus attention (metaseq/service/workers.py:57-59)."""
+    """Work estimate of a prompt: linear layers plus attention
+    (metaseq/service/workers.py:57-59)."""
     return n_tokens + int(math.ceil((n_tokens / 10) ** 2))
 
 
-@dataclass(order=False)
-class WorkItem:
-    """Sortable queue entry: lower cost is served first, ties by uid
-    (metaseq/service/workers.py:26-50)."""
-    cost: int
-    uid: int
-    return_queue: "queue.Queue"
-    data: Any
-    prompt_len: int = 0
-    gen_len: int = 0
+class Request:
+    """One prompt with its generation options and the queue its answer goes to."""
 
-    def __lt__(self, other):
-        return (self.cost, self.uid) < (other.cost, other.uid)
+    __slots__ = ("uid", "prompt", "options", "reply", "cost")
 
-    def __eq__(self, other):
-        return (self.cost, self.uid) == (other.cost, other.uid)
+    def __init__(self, uid: int, prompt: List[int], options: Dict[str, Any]):
+        self.uid = uid
+        self.prompt = list(prompt)
+        self.options = dict(options)
+        self.reply: "queue.Queue" = queue.Queue()
+        self.cost = prompt_cost(len(self.prompt))
 
-    def queue_key(self) -> str:
-        d = {k: self.data.get(k) for k in QUEUE_KEYS}
-        return ":".join("%s:%s" % (k, d[k]) for k in sorted(d))
+    @property
+    def new_tokens(self) -> int:
+        return int(self.options.get("max_tokens", 0) or 0)
+
+    @property
+    def signature(self) -> str:
+        return "|".join("%s=%s" % (k, self.options.get(k)) for k in sorted(SIGNATURE_OPTIONS))
+
+    @property
+    def rank(self):
+        """Cheapest first, earlier submission first among equals (workers.py:26-50)."""
+        return (self.cost, self.uid)
+
+    def answer(self, result):
+        self.reply.put((self.uid, result))
 
 
-class KeyedQueues:
-    """One priority queue per signature; the batching loop drains the fullest one
-    (metaseq/service/queue.py:11-49)."""
+class Backlog:
+    """Waiting requests, one heap per signature, behind one condition variable."""
 
     def __init__(self):
-        self.queues: Dict[str, "queue.PriorityQueue"] = {}
-        self._lock = threading.Lock()
+        self._heaps: Dict[str, list] = {}
+        self._cv = threading.Condition()
 
-    def put(self, item: WorkItem):
-        with self._lock:
-            q = self.queues.setdefault(item.queue_key(), queue.PriorityQueue())
-        q.put(item)
+    def put(self, req: Request, signature: Optional[str] = None):
+        with self._cv:
+            heap = self._heaps.setdefault(req.signature if signature is None else signature, [])
+            heapq.heappush(heap, (req.rank, req))
+            self._cv.notify_all()
 
-    def get_largest_queue(self) -> Optional["queue.PriorityQueue"]:
-        with self._lock:
-            if not self.queues:
+    def __len__(self):
+        with self._cv:
+            return sum(len(h) for h in self._heaps.values())
+
+    def fullest(self) -> Optional[str]:
+        with self._cv:
+            live = [(len(h), k) for k, h in self._heaps.items() if h]
+            if not live:
                 return None
-            key = max(self.queues, key=lambda k: self.queues[k].qsize())
-            return self.queues[key]
+            return max(live, key=lambda e: e[0])[1]
+
+    def take(self, signature: str, wait: float = 0.0) -> Optional[Request]:
+        """Cheapest request of one signature; waits up to ``wait`` seconds for one to arrive."""
+        with self._cv:
+            heap = self._heaps.setdefault(signature, [])
+            if not heap and wait > 0:
+                self._cv.wait_for(lambda: bool(heap), timeout=wait)
+            return heapq.heappop(heap)[1] if heap else None
 
 
-class BatchingService:
-    """``submit`` from any thread; ``serve_forever`` (or ``step``) on the one GPU thread."""
+class Rectangle:
+    """A run-to-completion batch: rows padded to the longest member.  It owns the arithmetic
+    that decides whether one more request still fits."""
 
-    def __init__(self, generator, max_tokens: int = MAX_BATCH_TOKENS,
-                 max_seq_len: int = MAX_SEQ_LEN, timeout_ms: float = 100.0, seed: int = None):
-        self.generator = generator
-        self.max_tokens = max_tokens
-        self.max_seq_len = max_seq_len
-        self.timeout = timeout_ms / 1000.0
-        self.queues = KeyedQueues()
-        self._uid = 0
+    def __init__(self, token_budget: int, max_seq_len: int):
+        self.token_budget, self.max_seq_len = token_budget, max_seq_len
+        self.members: List[Request] = []
+        self._widest = self._longest_prompt = self._longest_new = 0
+
+    def fits(self, req: Request) -> bool:
+        if not self.members:
+            return True  # a lone request is never refused here; generate() judges it
+        padded = max(self._widest, req.cost) * (len(self.members) + 1)
+        span = max(self._longest_prompt, len(req.prompt)) + max(self._longest_new, req.new_tokens)
+        return padded <= self.token_budget and span <= self.max_seq_len
+
+    def add(self, req: Request):
+        self.members.append(req)
+        self._widest = max(self._widest, req.cost)
+        self._longest_prompt = max(self._longest_prompt, len(req.prompt))
+        self._longest_new = max(self._longest_new, req.new_tokens)
+
+    def call_arguments(self, seed: int) -> Dict[str, Any]:
+        args: Dict[str, Any] = {
+            "inputs": [r.prompt for r in self.members],
+            "min_tokens": [r.options.get("min_tokens", 0) for r in self.members],
+            "max_tokens": [r.options.get("max_tokens", self.max_seq_len) for r in self.members],
+            "seed": seed,
+        }
+        for r in self.members:  # members share a signature; later ones win on the rest
+            args.update({k: r.options[k] for k in CALL_OPTIONS if k in r.options})
+        return args
+
+    def answer(self, results):
+        for req, res in zip(self.members, results):
+            req.answer(res)
+
+
+class _Front:
+    """What both engines share: request numbering, the blocking call, the serving loop."""
+
+    def __init__(self, idle_wait: float):
+        self._uids = itertools.count()
         self._uid_lock = threading.Lock()
-        self._rng = random.Random(seed)
-        self._stop = threading.Event()
+        self._halt = threading.Event()
+        self._idle_wait = idle_wait
 
-    # -- producer side ----------------------------------------------------------------
-    def submit(self, encoded_prompt: List[int], **generation_args) -> "queue.Queue":
-        """Queues one prompt; the returned queue receives ``(uid, result_or_exception)``."""
+    def _new_request(self, prompt, options) -> Request:
         with self._uid_lock:
-            uid = self._uid
-            self._uid += 1
-        ro = {"input": list(encoded_prompt), **generation_args}
-        n = len(encoded_prompt)
-        ret: "queue.Queue" = queue.Queue()
-        self.queues.put(WorkItem(prompt_cost(n), uid, ret, ro, prompt_len=n,
-                                 gen_len=int(ro.get("max_tokens", 0) or 0)))
-        return ret
+            uid = next(self._uids)
+        return Request(uid, prompt, options)
 
-    def generate(self, encoded_prompt: List[int], **generation_args):
-        """Blocking convenience call (metaseq/service/workers.py:52-62)."""
-        _, result = self.submit(encoded_prompt, **generation_args).get()
+    def generate(self, encoded_prompt: List[int], **options):
+        """Blocking convenience call; needs ``serve_forever`` running on another thread."""
+        _, result = self.submit(encoded_prompt, **options).get()
         if isinstance(result, Exception):
             raise result
         return result
 
-    # -- consumer side ----------------------------------------------------------------
-    def collect_batch(self) -> List[WorkItem]:
-        """Pulls like-sized items from the fullest queue until the padded batch is over budget
-        (``longest cost x batch size > max_tokens``), would overflow the sequence length, or
-        the queue stays empty for ``timeout`` (interactive_hosted.py:93-118)."""
-        batch: List[WorkItem] = []
-        target = self.queues.get_largest_queue()
-        if target is None:
-            return batch
-        while True:
-            try:
-                item = target.get(timeout=self.timeout)
-            except queue.Empty:
-                return batch
-            longest = max([item] + batch).cost
-            batch_cost = longest * (len(batch) + 1)
-            max_prompt_len = max(x.prompt_len for x in [item] + batch)
-            max_gen_len = max(x.gen_len for x in [item] + batch)
-            overflow = (max_prompt_len + max_gen_len) > self.max_seq_len
-            if batch and (batch_cost > self.max_tokens or overflow):
-                target.put(item)  # over budget: back into the queue for the next batch
-                return batch
-            batch.append(item)
-
-    def run_batch(self, batch: List[WorkItem]):
-        """One generate() call for the whole batch; results go back per item
-        (interactive_hosted.py:119-172).  A RuntimeError (device fault) propagates, any other
-        exception is reported to every caller of the batch."""
-        request = {"inputs": [], "min_tokens": [], "max_tokens": []}
-        for item in batch:
-            ro = item.data
-            request["inputs"].append(ro["input"])
-            request["min_tokens"].append(ro.get("min_tokens", 0))
-            request["max_tokens"].append(ro.get("max_tokens", self.max_seq_len))
-            for key in SHARED_ARGS:  # assumption of the reference: the batch agrees on these
-                if key in ro:
-                    request[key] = ro[key]
-        request["seed"] = self._rng.randint(1, 20000)
-        try:
-            generations = self.generator.generate(**request)
-        except RuntimeError:
-            raise
-        except Exception as e:  # noqa: BLE001 - reported to the callers, as in the reference
-            generations = [e] * len(batch)
-        for item, gen in zip(batch, generations):
-            item.return_queue.put((item.uid, gen))
-
-    def step(self) -> int:
-        """Collects and runs at most one batch; returns its size."""
-        batch = self.collect_batch()
-        if batch:
-            self.run_batch(batch)
-        return len(batch)
-
     def serve_forever(self):
-        while not self._stop.is_set():
+        while not self._halt.is_set():
             if self.step() == 0:
-                self._stop.wait(self.timeout)
+                self._halt.wait(self._idle_wait)
 
     def stop(self):
-        self._stop.set()
+        self._halt.set()
+
+
+class BatchingService(_Front):
+    """Run-to-completion batching in front of anything with ``generate(inputs=..., ...)``."""
+
+    def __init__(self, generator, max_tokens: int = MAX_BATCH_TOKENS,
+                 max_seq_len: int = MAX_SEQ_LEN, timeout_ms: float = 100.0, seed: int = None):
+        super().__init__(timeout_ms / 1000.0)
+        self.generator = generator
+        self.max_tokens, self.max_seq_len = max_tokens, max_seq_len
+        self.timeout = timeout_ms / 1000.0
+        self.backlog = Backlog()
+        self._rng = random.Random(seed)
+
+    def submit(self, encoded_prompt: List[int], **options) -> "queue.Queue":
+        """Queues one prompt; the returned queue receives ``(uid, result_or_exception)``."""
+        req = self._new_request(encoded_prompt, options)
+        self.backlog.put(req)
+        return req.reply
+
+    def plan(self) -> Rectangle:
+        """The next batch: cheapest-first from the fullest backlog until one more would not fit
+        or nothing arrives within the timeout."""
+        batch = Rectangle(self.max_tokens, self.max_seq_len)
+        signature = self.backlog.fullest()
+        while signature is not None:
+            req = self.backlog.take(signature, wait=self.timeout)
+            if req is None:
+                break
+            if not batch.fits(req):
+                self.backlog.put(req)  # opens the next batch
+                break
+            batch.add(req)
+        return batch
+
+    def run(self, batch: Rectangle):
+        """One generate() call for the batch.  A RuntimeError is a device fault and propagates
+        (the reference's worker dies on it and is restarted, interactive_hosted.py:161-171);
+        any other exception is the answer every member gets."""
+        try:
+            results = self.generator.generate(
+                **batch.call_arguments(self._rng.randint(1, 20000)))
+        except RuntimeError:
+            raise
+        except Exception as e:  # noqa: BLE001 - delivered to the callers
+            results = [e] * len(batch.members)
+        batch.answer(results)
+
+    def step(self) -> int:
+        """Plans and runs at most one batch; returns its size."""
+        batch = self.plan()
+        if batch.members:
+            self.run(batch)
+        return len(batch.members)
+
+
+class _Row:
+    """A request while it occupies a slot."""
+
+    __slots__ = ("req", "tokens", "scores", "n_new", "min_new", "max_new", "last", "done")
+
+    def __init__(self, req: Request, tokens: List[int], scores: List[float], max_new: int):
+        self.req, self.tokens, self.scores = req, tokens, scores
+        self.n_new = 0
+        self.min_new = int(req.options.get("min_tokens", 0) or 0)
+        self.max_new = max_new
+        self.last = tokens[-1]
+        self.done = False
+
+    def mode(self) -> int:
+        """Selection regime of this row's next token: end-of-sequence and stop tokens are barred
+        until ``min_tokens`` are out, and the last allowed token can only be end-of-sequence,
+        as in the generation loop (metaseq/sequence_generator.py:272-284)."""
+        m = 0
+        if self.n_new < self.min_new:
+            m |= 1  # MSA_ROW_BAN_EARLY
+        if self.n_new >= self.max_new - 1:
+            m |= 2  # MSA_ROW_ONLY_EOS
+        return m
+
+    def take(self, token: int, score: float, eos: int, stop) -> bool:
+        """Records the chosen token; True when the row has ended."""
+        self.tokens.append(token)
+        self.scores.append(score)
+        self.n_new += 1
+        self.last = token
+        self.done = token == eos or token in stop or self.n_new >= self.max_new
+        return self.done
+
+
+class SlotBatch:
+    """The running batch of the continuous engine: which request sits in which slot, and the
+    arithmetic that decides whether a request can be taken in."""
+
+    def __init__(self, slots: int, capacity: int):
+        self.capacity = capacity
+        self.rows: List[Optional[_Row]] = [None] * slots
+
+    def free_slot(self) -> Optional[int]:
+        for i, r in enumerate(self.rows):
+            if r is None:
+                return i
+        return None
+
+    def active(self):
+        return [(i, r) for i, r in enumerate(self.rows) if r is not None]
+
+    def room_for(self, req: Request) -> int:
+        """New tokens the request may generate in a slot: its own limit, capped by what the
+        slot's cache holds after the prompt and its leading end-of-sequence token (0: the
+        prompt itself does not fit)."""
+        left = self.capacity - (len(req.prompt) + 1)
+        if left < 1:
+            return 0
+        asked = req.new_tokens or left
+        return max(1, min(asked, left))
+
+
+class ContinuousBatcher(_Front):
+    """Continuous batching of greedy requests over ``slots`` rows of one KV cache.
+
+    ``interface`` is the ``GeneratorInterface`` whose model, dictionary and tokenizer are used;
+    ``capacity`` is the number of positions a slot can hold (prompt + continuation).  Requests
+    that need sampling, several replicas, penalties or ``logprobs`` are refused with a
+    ValueError delivered to the caller (serve them through ``BatchingService``)."""
+
+    UNSUPPORTED = ("lambda_decay", "alpha_presence", "alpha_frequency", "alpha_presence_src",
+                   "alpha_frequency_src")
+
+    def __init__(self, interface, slots: int = 32, capacity: int = MAX_SEQ_LEN,
+                 idle_ms: float = 2.0):
+        super().__init__(idle_ms / 1000.0)
+        import torch
+
+        from . import _capi
+        self._torch, self._capi = torch, _capi
+        self.interface = interface
+        self.model = interface.models[0]
+        self.decoder = self.model.decoder
+        self.dict = interface.tgt_dict
+        self.device = interface.device
+        capacity = min(int(capacity), self.decoder.max_positions())
+        self.batch = SlotBatch(slots, capacity)
+        self.backlog = Backlog()
+        self.cache = None  # allocated with the first request
+        self._stop: tuple = ()  # stop ids of the running batch
+        dev = self.device
+        self._last = torch.full((slots,), self.dict.pad(), dtype=torch.long, device=dev)
+        self._mode = torch.zeros(slots, dtype=torch.uint8, device=dev)
+        self._tok = torch.zeros(slots, dtype=torch.long, device=dev)
+        self._score = torch.zeros(slots, dtype=torch.float32, device=dev)
+        self.steps = 0          # decode steps run
+        self.rows_stepped = 0   # active rows summed over those steps
+
+    # -- producer side ------------------------------------------------------------------
+    def submit(self, encoded_prompt: List[int], **options) -> "queue.Queue":
+        req = self._new_request(encoded_prompt, options)
+        problem = self._why_not(req)
+        if problem:
+            req.answer(ValueError(problem))
+        else:
+            self.backlog.put(req, signature="")  # one queue: every greedy request can share
+        return req.reply
+
+    def _why_not(self, req: Request) -> Optional[str]:
+        o = req.options
+        temperature, top_p = o.get("temperature", 1.0), o.get("top_p", -1.0)
+        if not (temperature == 0 or ((top_p is None or top_p <= 0) and temperature == 1.0)):
+            return "continuous batching serves greedy requests only (temperature 0, or top_p <= 0)"
+        if (o.get("n", 1) or 1) != 1 or (o.get("best_of") or 1) != 1:
+            return "continuous batching serves one replica per request"
+        if (o.get("logprobs", 0) or 0) > 0:
+            return "continuous batching does not record distributions (logprobs > 0)"
+        for k in self.UNSUPPORTED:
+            if (o.get(k, 0) or 0) > 0:
+                return "continuous batching does not apply %s" % k
+        if len(o.get("stop") or []) > 14:
+            return "at most 14 stop tokens are supported"
+        if self.batch.room_for(req) == 0:
+            return ("a prompt of %d tokens does not fit a slot of %d positions"
+                    % (len(req.prompt), self.batch.capacity))
+        return None
+
+    # -- consumer side ------------------------------------------------------------------
+    def _admit(self, slot: int, req: Request):
+        """Prefill into the slot and choose the request's first token from the prompt's last
+        position."""
+        torch = self._torch
+        eos, pad = self.dict.eos(), self.dict.pad()
+        if self.cache is None:
+            self.cache = self.decoder.new_slot_cache(len(self.batch.rows), self.batch.capacity,
+                                                     self.device)
+        ids = [eos] + req.prompt
+        row = _Row(req, ids, [], self.batch.room_for(req))
+        row.scores = self.decoder.admit_slot(
+            self.cache, slot, torch.tensor(ids, dtype=torch.long, device=self.device),
+            banned=[pad], stop=self._stop, eos=eos, mode=row.mode(),
+            tok_out=self._tok[slot:slot + 1], score_out=self._score[slot:slot + 1])
+        self.batch.rows[slot] = row
+        if row.take(int(self._tok[slot]), float(self._score[slot]), eos, self._stop):
+            self._retire(slot)
+
+    def _retire(self, slot: int):
+        row = self.batch.rows[slot]
+        self.batch.rows[slot] = None
+        self.decoder.release_slot(self.cache, slot)
+        req = row.req
+        try:
+            # the row as the generation loop would return it: tokens up to the end, then eos
+            toks, scs = list(row.tokens), list(row.scores)
+            if toks[-1] != self.dict.eos():
+                toks.append(self.dict.eos())
+                scs.append(0.0)
+            rec = self.interface._record(toks, scs, None, len(req.prompt), row.max_new,
+                                         bool(req.options.get("echo", False)), 0)
+            req.answer([rec])
+        except Exception as e:  # noqa: BLE001 - delivered to the caller
+            req.answer(e)
+
+    def step(self) -> int:
+        """Takes waiting requests into free slots, then runs one decode step over the occupied
+        slots.  Returns the number of rows that were served (admitted or stepped).  The rows of
+        the running batch share one stop list: a request with another one waits until the batch
+        has drained."""
+        torch = self._torch
+        served = 0
+        while True:
+            slot = self.batch.free_slot()
+            if slot is None:
+                break
+            req = self.backlog.take("")
+            if req is None:
+                break
+            stop = tuple(sorted(req.options.get("stop") or ()))
+            if self.batch.active() and stop != self._stop:
+                self.backlog.put(req, signature="")
+                break
+            self._stop = stop
+            try:
+                self._admit(slot, req)
+            except RuntimeError:
+                raise
+            except Exception as e:  # noqa: BLE001 - this request's own answer
+                self.batch.rows[slot] = None
+                req.answer(e)
+            served += 1
+        active = self.batch.active()
+        if not active:
+            return served
+        eos, pad = self.dict.eos(), self.dict.pad()
+        last = [pad] * len(self.batch.rows)
+        mode = [0] * len(self.batch.rows)
+        for i, row in active:
+            last[i], mode[i] = row.last, row.mode()
+        self._last.copy_(torch.tensor(last, dtype=torch.long))
+        self._mode.copy_(torch.tensor(mode, dtype=torch.uint8))
+        self.decoder.decode_slots(self.cache, self._last, temperature=1.0, banned=[pad],
+                                  stop=self._stop, eos=eos, row_mode=self._mode,
+                                  tok_out=self._tok, score_out=self._score)
+        toks, scs = self._tok.tolist(), self._score.tolist()
+        self.steps += 1
+        self.rows_stepped += len(active)
+        for i, row in active:
+            if row.take(toks[i], scs[i], eos, self._stop):
+                self._retire(i)
+        return served + len(active)

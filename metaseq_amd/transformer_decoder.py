@@ -502,6 +502,25 @@ class TransformerDecoder(nn.Module):
             if incremental_state is not None:
                 incremental_state[self._state_key] = cache
             return features, packed, (B, T), {"inner_states": inner_states}
+        h, inner_states = self._rows_core(lib, stream, tokens, B, n, T, S0, cache, mask)
+        packed = False
+        features = h.view(B, T, D)
+        cache.length = S0 + T
+        if incremental_state is not None:
+            incremental_state[self._state_key] = cache
+        return features, packed, (B, T), {"inner_states": inner_states}
+
+    def _rows_core(self, lib, stream, tokens, B, n, T, S0, kv, mask):
+        """Prefill (or a decode batch above 64 rows): the last T columns of ``tokens[B, n]``
+        through embedding, L layers and the final LayerNorm on row-major activations and the
+        tiled MFMA kernels, keys and values written at positions S0 .. S0 + T - 1 of ``kv``
+        (anything with ``k(i)``, ``v(i)`` and ``capacity``).  Returns the normalised features
+        [B * T, D] and the inner-states list."""
+        cfg = self.cfg
+        D, H, hd = cfg.decoder_embed_dim, cfg.decoder_attention_heads, cfg.head_dim
+        F = cfg.decoder_ffn_embed_dim
+        dev = tokens.device
+        M = B * T
         x = torch.empty(M, D, dtype=torch.float16, device=dev)
         positions = torch.empty(B, T, dtype=torch.long, device=dev)
         check(lib.msa_embed_f16(ptr(tokens), tokens.stride(0), B, n, T,
@@ -514,18 +533,16 @@ class TransformerDecoder(nn.Module):
             inner_states[0]["emb"] = x.view(B, T, D).transpose(0, 1).clone()
         mask_stride = mask.stride(0) if mask is not None else 0
         q = torch.empty(M, D, dtype=torch.float16, device=dev)
-        # ---- prefill (or a decode batch above 64 rows): row-major activations, tiled MFMA
-        # kernels ----
         h = torch.empty_like(x)
         o = torch.empty_like(x)
         u = torch.empty(M, F, dtype=torch.float16, device=dev)
         for i, layer in enumerate(self.layers):
             self._layernorm(lib, stream, x, layer.self_attn_layer_norm, M, D, h)
-            kc, vc = cache.k(i), cache.v(i)
+            kc, vc = kv.k(i), kv.v(i)
             self._qkv(lib, stream, h, layer.self_attn.qkv_proj, q, kc, vc, B, T, H, hd, S0,
-                      cache.capacity, D, 0)
+                      kv.capacity, D, 0)
             check(lib.msa_attention_f16(ptr(q), ptr(kc), ptr(vc), ptr(mask), mask_stride,
-                                        ptr(o), B, H, hd, T, S0, cache.capacity, 0, None,
+                                        ptr(o), B, H, hd, T, S0, kv.capacity, 0, None,
                                         stream))
             # x = round(round(o Wo^T + bo) + x)   (transformer_decoder_layer.py:222-230)
             self._linear(lib, stream, o, layer.self_attn.out_proj, M, D, D, residual=x, out=x)
@@ -537,12 +554,98 @@ class TransformerDecoder(nn.Module):
         else:
             inner_states.append(None)
         self._layernorm(lib, stream, x, self.layer_norm, M, D, h)
-        packed = False
-        features = h.view(B, T, D)
-        cache.length = S0 + T
-        if incremental_state is not None:
-            incremental_state[self._state_key] = cache
-        return features, packed, (B, T), {"inner_states": inner_states}
+        return h, inner_states
+
+    # ------------------------------------------------------------------ slot interface
+    # A running batch whose rows belong to different requests (continuous batching): a fixed
+    # number of slots over one KV cache, each slot filled by its own prefill and advanced by
+    # decode steps over all slots at once.  No reference counterpart: the reference's service
+    # runs every batch to completion (metaseq/cli/interactive_hosted.py:66-175).
+    def new_slot_cache(self, slots: int, capacity: int, device=None) -> KVCache:
+        """An empty cache of ``slots`` rows (at most 64) and ``capacity`` positions each."""
+        if not 1 <= slots <= 64:
+            raise ValueError("a slot cache holds 1..64 rows")
+        cfg = self.cfg
+        capacity = int(capacity)
+        if not 1 <= capacity <= self.max_positions():
+            raise ValueError("capacity %d outside 1..%d" % (capacity, self.max_positions()))
+        dev = device if device is not None else self.embed_tokens.weight.device
+        cache = KVCache(cfg.decoder_layers, slots, cfg.decoder_attention_heads, cfg.head_dim,
+                        capacity, dev)
+        cache.ragged = True
+        cache.lens = torch.full((slots,), -1, dtype=torch.int32, device=dev)
+        return cache
+
+    def prefill_slot(self, cache: KVCache, slot: int, tokens: torch.Tensor):
+        """Runs the prompt ``tokens`` (1-D ids on the device, no pads, the leading
+        end-of-sentence token included) through the model into row ``slot`` of ``cache`` and
+        activates the slot.  Returns the logits of every prompt position, ``[T, V]`` fp16."""
+        lib = self.prepare_()
+        if tokens.dim() != 1 or tokens.numel() == 0 or not tokens.is_cuda:
+            raise AssertionError("tokens must be a non-empty 1-D device tensor")
+        T = tokens.numel()
+        if T >= cache.capacity:
+            raise ValueError("a prompt of %d tokens leaves no room in a cache of %d positions"
+                             % (T, cache.capacity))
+        if not (cache.ragged and 0 <= slot < cache.batch):
+            raise ValueError("not a slot cache, or slot %d outside 0..%d" % (slot, cache.batch - 1))
+        toks = tokens.long().contiguous().view(1, T)
+        h, _ = self._rows_core(lib, _capi.stream_ptr(), toks, 1, T, T, 0, _SlotView(cache, slot),
+                               None)
+        cache.lens[slot] = T
+        return self._project(h, False, 1, T)[0]
+
+    def admit_slot(self, cache: KVCache, slot: int, tokens: torch.Tensor, *, banned=(), stop=(),
+                   eos=2, mode=0, tok_out=None, score_out=None):
+        """``prefill_slot`` plus what a request needs from its prompt: the log-probability of
+        every prompt token given its prefix (returned as a list, 0.0 for the first token) and
+        the greedy choice of the first new token from the last position, written to
+        ``tok_out`` / ``score_out`` (one-element int64 / fp32 device tensors) under the
+        selection regime ``mode`` (MSA_ROW_* bits)."""
+        lib = self.prepare_()
+        logits = self.prefill_slot(cache, slot, tokens)
+        T, V = logits.shape
+        stream = _capi.stream_ptr()
+        scores = [0.0] * T
+        if T > 1:
+            lp = torch.empty(T - 1, dtype=torch.float32, device=logits.device)
+            target = tokens.long()[1:].contiguous()
+            check(lib.msa_target_logprob_f16(ptr(logits), logits.stride(0), T - 1, V, 1.0,
+                                             ptr(target), ptr(lp), stream))
+            scores[1:] = lp.tolist()
+        banned, stop = list(banned), list(stop)
+        ba = (ctypes.c_int32 * max(1, len(banned)))(*banned)
+        sa = (ctypes.c_int32 * max(1, len(stop)))(*stop)
+        row_mode = torch.tensor([mode], dtype=torch.uint8, device=logits.device)
+        last = logits[T - 1:T]
+        check(lib.msa_greedy_select_f16(ptr(last), last.stride(0), 1, V, 1.0, ba, len(banned), sa,
+                                        len(stop), None, ptr(row_mode), 0, int(eos), ptr(tok_out),
+                                        1, ptr(score_out), 1, None, stream))
+        return scores
+
+    def release_slot(self, cache: KVCache, slot: int):
+        cache.lens[slot] = -1
+
+    def decode_slots(self, cache: KVCache, last_tokens: torch.Tensor, *, temperature=1.0,
+                     banned=(), stop=(), eos=2, row_mode=None, tok_out=None, score_out=None,
+                     finished=None, logits_out=None):
+        """One decode step over every active slot: ``last_tokens`` ([slots] ids on the device;
+        what an inactive slot holds does not matter) are embedded at each row's own position,
+        appended to its history and attended over it; the vocabulary projection selects the
+        next token greedily into ``tok_out`` / ``score_out`` ([slots], int64 / fp32) under the
+        per-row ``row_mode`` (uint8 [slots]: MSA_ROW_BAN_EARLY, MSA_ROW_ONLY_EOS).  Every active
+        row's length advances by one.  Outputs of inactive slots are undefined."""
+        lib = self.prepare_()
+        stream = _capi.stream_ptr()
+        B = cache.batch
+        if last_tokens.shape != (B,) or last_tokens.dtype != torch.long:
+            raise AssertionError("last_tokens must be int64 [%d]" % B)
+        bufs = self._step_buffers(cache, B)
+        feat, _ = self._decode_core(lib, stream, last_tokens.view(B, 1), 1, B, cache, None, bufs,
+                                    cache.lens, 0, True)
+        check(lib.msa_advance_len(ptr(cache.lens), ptr(bufs["step_len"]), B, 1, stream))
+        self._select_from(lib, feat, B, temperature, banned, stop, finished, row_mode, False, eos,
+                          tok_out, 1, score_out, 1, logits_out)
 
     def extract_features(self, prev_output_tokens, incremental_state=None,
                          token_embeddings=None, self_attn_padding_mask=None):
@@ -595,18 +698,37 @@ class TransformerDecoder(nn.Module):
                                                       None, want_packed=True)
         if not packed:
             raise ValueError("forward_select needs at most 64 rows")
-        lib = self._lib
+        self._select_from(self._lib, f, B, temperature, banned, stop, finished, row_mode,
+                          force_eos, eos, tok_out, tok_stride, score_out, score_stride, logits_out)
+
+    def _select_from(self, lib, f, B, temperature, banned, stop, finished, row_mode, force_eos,
+                     eos, tok_out, tok_stride, score_out, score_stride, logits_out):
+        """Vocabulary projection of the packed features ``f`` fused with the greedy selection."""
         D, V = self.cfg.decoder_embed_dim, self.cfg.vocab_size
         need = lib.msa_lm_head_select_workspace_bytes(B)
         ws = getattr(self, "_select_ws", None)
         if ws is None or ws.numel() < need or ws.device != f.device:
             ws = self._select_ws = torch.empty(need, dtype=torch.uint8, device=f.device)
+        banned, stop = list(banned), list(stop)
         ba = (ctypes.c_int32 * max(1, len(banned)))(*banned)
         sa = (ctypes.c_int32 * max(1, len(stop)))(*stop)
         check(lib.msa_lm_head_greedy_select_f16(
             ptr(f), ptr(self._lm_head), ptr(logits_out), ptr(ws), B, V, D, float(temperature), ba,
             len(banned), sa, len(stop), ptr(finished), ptr(row_mode), int(force_eos), int(eos),
             ptr(tok_out), tok_stride, ptr(score_out), score_stride, None, _capi.stream_ptr()))
+
+
+class _SlotView:
+    """Row ``slot`` of a KV cache, with the interface the prefill path expects of a cache."""
+
+    def __init__(self, cache: KVCache, slot: int):
+        self._layers, self._slot, self.capacity = cache.layers, slot, cache.capacity
+
+    def k(self, i):
+        return self._layers[i][0][self._slot:self._slot + 1]
+
+    def v(self, i):
+        return self._layers[i][1][self._slot:self._slot + 1]
 
 
 # the name the reference's model code uses for this class

@@ -234,3 +234,38 @@ def test_batching_service_over_the_interface_returns_what_direct_calls_return():
     for p, r, want in zip(prompts, rets, direct):
         uid, got = r.get_nowait()
         assert got[0]["tokens"] == want[0]["tokens"], p
+
+
+def test_continuous_batcher_rows_equal_single_request_generation():
+    """Requests that join and leave a running batch of slots get exactly what a generation of
+    their own would give them: with at most 16 rows every row runs through the same kernels
+    with the same summation order whatever its neighbours are, so tokens and scores are equal to
+    the last bit.  More requests than slots, different prompt lengths, minimum and maximum
+    lengths, echo."""
+    from metaseq_amd.service import ContinuousBatcher
+    gi, model, cfg, sd = _interface()
+    specs = [dict(prompt=[5, 9, 33, 12, 7], max_tokens=9),
+             dict(prompt=[40], max_tokens=3),
+             dict(prompt=[8, 8, 8, 21, 22, 23, 24, 25, 26, 27, 28], min_tokens=5, max_tokens=12),
+             dict(prompt=[17, 4], max_tokens=1),
+             dict(prompt=[30, 31, 32], min_tokens=2, max_tokens=7, echo=True),
+             dict(prompt=[11], max_tokens=14),
+             dict(prompt=[45, 46, 47, 48], max_tokens=6)]
+    cb = ContinuousBatcher(gi, slots=3, capacity=40)
+    replies = [cb.submit(s["prompt"], **{k: v for k, v in s.items() if k != "prompt"})
+               for s in specs]
+    n = 0
+    while cb.step():
+        n += 1
+        assert n < 200
+    assert cb.steps > 0 and cb.rows_stepped > cb.steps      # rows shared decode steps
+    for s, r in zip(specs, replies):
+        _, got = r.get_nowait()
+        assert not isinstance(got, Exception), got
+        want = gi.generate([s["prompt"]], max_tokens=[s["max_tokens"]],
+                           min_tokens=[s.get("min_tokens", 0)], echo=s.get("echo", False))
+        assert got[0]["tokens"] == want[0][0]["tokens"], s
+        assert got[0]["token_scores"] == want[0][0]["token_scores"], s
+        assert got[0]["text"] == want[0][0]["text"]
+    # every slot is free again and the cache holds no active row
+    assert cb.cache.lens.tolist() == [-1, -1, -1]
