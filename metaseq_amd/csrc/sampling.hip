@@ -267,6 +267,242 @@ __global__ __launch_bounds__(256) void select_combine_kernel(
   }
 }
 
+
+// ---- nucleus (top-p) sampling --------------------------------------------------------------
+// One workgroup per row.  The nucleus boundary is found without sorting, by a radix descent over
+// the bit pattern of the probabilities (positive floats order like their bit patterns): four
+// passes over the row, each adding the mass of the ids that match the bits decided so far into
+// a 256-bucket histogram.  Masses are accumulated as 2^-48 fixed-point integers, so the sums
+// are exact and do not depend on the order of the additions (run-to-run deterministic although
+// the buckets are filled with LDS atomics).  Ties at the boundary are cut by id.  Nothing of the
+// row is kept between passes: a pass re-reads the fp16 logits (L2) and recomputes p.
+// The draw is an exponential race: arg-max of p / noise over the nucleus, noise ~ Exp(1) per id,
+// which picks id v with probability p[v] / mass(nucleus).
+constexpr int SP_THREADS = 1024;
+constexpr float SP_FIXED = 281474976710656.f;  // 2^48
+
+struct Penalties {
+  int64_t* counts;            // [B, V] generated-token counts (updated) or NULL
+  const int64_t* counts_src;  // [B, V] prompt-token counts or NULL
+  float presence, frequency, presence_src, frequency_src;
+};
+
+__device__ __forceinline__ void argbest(float& v, int& i, float ov, int oi) {
+  if (ov > v || (ov == v && oi < i)) {
+    v = ov;
+    i = oi;
+  }
+}
+
+__global__ __launch_bounds__(SP_THREADS) void sample_topp_kernel(
+    const half_t* __restrict__ logits, int64_t ld, int V, float temperature, bool scale,
+    IdList banned, IdList stop, uint8_t* __restrict__ finished,
+    const uint8_t* __restrict__ row_mode, int force_eos_all, int eos,
+    const float* __restrict__ topp_rows, float topp_all, const float* __restrict__ noise,
+    Penalties pen, int64_t* __restrict__ tok, int64_t tok_stride, float* __restrict__ score,
+    int64_t score_stride) {
+  __shared__ float red[16];
+  __shared__ float rbest[16], rprob[16];
+  __shared__ int ridx[16];
+  __shared__ unsigned long long hist[256];
+  __shared__ unsigned sh_bucket;
+  __shared__ unsigned long long sh_above;
+  const int b = blockIdx.x;
+  const half_t* row = logits + (int64_t)b * ld;
+  const unsigned rm = row_mode ? row_mode[b] : 0u;
+  const bool only_eos = force_eos_all || (finished && finished[b]) || (rm & MSA_ROW_ONLY_EOS);
+  const bool ban_early = rm & MSA_ROW_BAN_EARLY;
+  const float topp = topp_rows ? topp_rows[b] : topp_all;
+
+  // e(id) = z - penalties for an eligible id, -inf otherwise; nan_out collects NaN logits
+  auto eligible = [&](int id) {
+    bool ok = !(only_eos && id != eos) && !(ban_early && id == eos);
+    for (int t = 0; t < banned.n; ++t) ok &= (banned.id[t] != id);
+    if (ban_early)
+      for (int t = 0; t < stop.n; ++t) ok &= (stop.id[t] != id);
+    return ok;
+  };
+  auto e_of = [&](int id, bool& nan_out) {
+    float z = (float)row[id];
+    if (scale) z = z / temperature;
+    nan_out |= (z != z);
+    if (!eligible(id)) return -INFINITY;
+    if (pen.counts) {
+      const float cnt = (float)pen.counts[(int64_t)b * V + id];
+      z -= cnt * pen.frequency + (cnt > 0.f ? pen.presence : 0.f);
+    }
+    if (pen.counts_src) {
+      const float cnt = (float)pen.counts_src[(int64_t)b * V + id];
+      z -= cnt * pen.frequency_src + (cnt > 0.f ? pen.presence_src : 0.f);
+    }
+    return z;
+  };
+
+  // ---- softmax statistics: over the eligible ids (after penalties), and over every id of the
+  // raw z for the log-softmax that the greedy branch's score is taken from ----
+  bool nan = false;
+  float mx = -INFINITY, mx_all = -INFINITY;
+  for (int id = threadIdx.x; id < V; id += SP_THREADS) {
+    mx = fmaxf(mx, e_of(id, nan));
+    float z = (float)row[id];
+    if (scale) z = z / temperature;
+    mx_all = fmaxf(mx_all, z);
+  }
+  mx = block_max(mx, red);
+  mx_all = block_max(mx_all, red);
+  const bool dead = block_max(nan ? 1.f : 0.f, red) > 0.f || !(mx > -INFINITY);
+  float s = 0.f, s_all = 0.f;
+  if (!dead) {
+    bool unused = false;
+    for (int id = threadIdx.x; id < V; id += SP_THREADS) {
+      const float e = e_of(id, unused);
+      s += e > -INFINITY ? expf(e - mx) : 0.f;
+      float z = (float)row[id];
+      if (scale) z = z / temperature;
+      s_all += expf(z - mx_all);
+    }
+  }
+  s = block_sum(s, red);
+  s_all = block_sum(s_all, red);
+  const float inv = dead ? 0.f : 1.f / s;
+  auto p_of = [&](int id) {
+    bool unused = false;
+    const float e = e_of(id, unused);
+    return e > -INFINITY ? expf(e - mx) * inv : 0.f;
+  };
+
+  // ---- nucleus: ids in order of decreasing p (ties: increasing id) belong while the mass
+  // before them is < topp.  T = the smallest probability whose strictly-greater mass is below
+  // topp: everything above T is in, of the ids equal to T those below tie_limit.
+  const bool sampling = noise != nullptr && topp > 0.f && !dead;
+  unsigned tbits = 0;
+  int tie_limit = V;
+  if (sampling) {
+    const unsigned long long P =
+        topp >= 1.f ? ~0ull : (unsigned long long)((double)topp * (double)SP_FIXED);
+    unsigned prefix = 0;            // bits decided so far (the top 8 * level bits)
+    unsigned long long above = 0;   // mass of the ids whose decided bits are greater
+    for (int level = 0; level < 4; ++level) {
+      const int shift = 24 - 8 * level;
+      if (threadIdx.x < 256) hist[threadIdx.x] = 0;
+      __syncthreads();
+      for (int id = threadIdx.x; id < V; id += SP_THREADS) {
+        const float pv = p_of(id);
+        const unsigned u = __float_as_uint(pv);
+        if (pv > 0.f && (level == 0 || (u >> (shift + 8)) == prefix))
+          atomicAdd(&hist[(u >> shift) & 255u], (unsigned long long)(pv * SP_FIXED));
+      }
+      __syncthreads();
+      if (threadIdx.x == 0) {
+        // the lowest non-empty bucket that still has less than topp above it
+        unsigned long long cum = above, found_above = above;
+        unsigned found = 255;
+        bool any = false;
+        for (int d = 255; d >= 0; --d) {
+          if (hist[d] != 0 && cum < P) {
+            found = (unsigned)d;
+            found_above = cum;
+            any = true;
+          }
+          cum += hist[d];
+        }
+        sh_bucket = any ? found : 0u;
+        sh_above = any ? found_above : above;
+      }
+      __syncthreads();
+      prefix = (prefix << 8) | sh_bucket;
+      above = sh_above;
+      __syncthreads();
+    }
+    tbits = prefix;
+    const float T = __uint_as_float(tbits);
+    const unsigned long long Tfx = (unsigned long long)(T * SP_FIXED);
+    const unsigned long long tie_mass = hist[tbits & 255u];
+    const long long n_ties = Tfx ? (long long)(tie_mass / Tfx) : 0;
+    // the i-th tied id (from 0) has above + i * T before it
+    long long n_in = n_ties;
+    if (Tfx && P != ~0ull && above < P) n_in = min(n_ties, (long long)((P - above + Tfx - 1) / Tfx));
+    if (n_in < n_ties) {  // the smallest id bound below which exactly n_in tied ids lie
+      int lo = 0, hi = V;
+      while (lo < hi) {
+        const int mid = lo + ((hi - lo) >> 1);
+        float cnt = 0.f;
+        for (int id = threadIdx.x; id < mid; id += SP_THREADS)
+          cnt += __float_as_uint(p_of(id)) == tbits ? 1.f : 0.f;
+        if ((long long)block_sum(cnt, red) >= n_in)
+          hi = mid;
+        else
+          lo = mid + 1;
+      }
+      tie_limit = lo;
+    }
+  }
+
+  // ---- the draw: exponential race over the nucleus (the arg-max of p when not sampling)
+  float best = -1.f, bestp = 0.f;
+  int bidx = 0x7fffffff;
+  if (!dead) {
+    for (int id = threadIdx.x; id < V; id += SP_THREADS) {
+      const float pv = p_of(id);
+      if (!(pv > 0.f)) continue;
+      float key = pv;
+      if (sampling) {
+        const unsigned u = __float_as_uint(pv);
+        if (!(u > tbits || (u == tbits && id < tie_limit))) continue;
+        key = pv / noise[(int64_t)b * V + id];
+      }
+      if (key > best || (key == best && id < bidx)) {
+        best = key;
+        bidx = id;
+        bestp = pv;
+      }
+    }
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    const float ov = __shfl_xor(best, o, MSA_WAVE), op = __shfl_xor(bestp, o, MSA_WAVE);
+    const int oi = __shfl_xor(bidx, o, MSA_WAVE);
+    if (ov > best || (ov == best && oi < bidx)) {
+      best = ov;
+      bidx = oi;
+      bestp = op;
+    }
+  }
+  if ((threadIdx.x & 63) == 0) {
+    rbest[threadIdx.x >> 6] = best;
+    ridx[threadIdx.x >> 6] = bidx;
+    rprob[threadIdx.x >> 6] = bestp;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < SP_THREADS / 64; ++w)
+      if (rbest[w] > best || (rbest[w] == best && ridx[w] < bidx)) {
+        best = rbest[w];
+        bidx = ridx[w];
+        bestp = rprob[w];
+      }
+    // sampling: the log of the probability among the eligible ids (the reference takes it from
+    // softmax(lprobs)); greedy: the penalised log-softmax value itself (lprobs.max())
+    float lp = logf(bestp);
+    if (!sampling && !dead && bidx != 0x7fffffff) {
+      bool unused = false;
+      lp = (e_of(bidx, unused) - mx_all) - logf(s_all);
+    }
+    if (dead || bidx == 0x7fffffff) {  // as the greedy kernel: token 0 with score -inf
+      bidx = 0;
+      lp = -INFINITY;
+    }
+    tok[b * tok_stride] = bidx;
+    score[b * score_stride] = lp;
+    if (pen.counts) pen.counts[(int64_t)b * V + bidx] += 1;
+    if (finished) {
+      bool f = bidx == eos;
+      for (int j = 0; j < stop.n; ++j) f |= (stop.id[j] == bidx);
+      if (f) finished[b] = 1;
+    }
+  }
+}
+
 }  // namespace
 
 int msa_launch_select_combine(const SelectPartial* partials, int n_parts, int B,
@@ -322,5 +558,47 @@ extern "C" int msa_target_logprob_f16(const void* logits, int64_t ld_logits, int
                      (hipStream_t)stream, (const half_t*)logits, ld_logits, V, temperature, scale,
                      target, out);
   MSA_CHECK_LAUNCH("msa_target_logprob_f16");
+  return MSA_OK;
+}
+
+extern "C" int msa_sample_topp_f16(const void* logits, int64_t ld_logits, int B, int V,
+                                   float temperature, const int32_t* banned_host, int n_banned,
+                                   const int32_t* stop_host, int n_stop, uint8_t* finished,
+                                   const uint8_t* row_mode, int force_eos_all, int eos_idx,
+                                   const float* topp_rows, float topp_all, const float* noise,
+                                   int64_t* counts, const int64_t* counts_src,
+                                   float alpha_presence, float alpha_frequency,
+                                   float alpha_presence_src, float alpha_frequency_src,
+                                   int64_t* tok, int64_t tok_stride, float* score,
+                                   int64_t score_stride, void* stream) {
+  const char* name = "msa_sample_topp_f16";
+  MSA_REQUIRE(logits && tok && score, MSA_ERR_INVALID_ARG, "%s: null pointer", name);
+  MSA_REQUIRE(B > 0 && V > 0 && ld_logits >= V, MSA_ERR_INVALID_ARG,
+              "%s: bad shape B=%d V=%d ld=%lld", name, B, V, (long long)ld_logits);
+  MSA_REQUIRE(n_banned >= 0 && n_banned <= 16 && (n_banned == 0 || banned_host),
+              MSA_ERR_INVALID_ARG, "%s: n_banned=%d (0..16)", name, n_banned);
+  MSA_REQUIRE(n_stop >= 0 && n_stop <= 16 && (n_stop == 0 || stop_host), MSA_ERR_INVALID_ARG,
+              "%s: n_stop=%d (0..16)", name, n_stop);
+  MSA_REQUIRE(eos_idx >= 0 && eos_idx < V, MSA_ERR_INVALID_ARG,
+              "%s: eos_idx=%d outside the vocabulary", name, eos_idx);
+  MSA_REQUIRE(temperature >= 0.f, MSA_ERR_INVALID_ARG, "%s: temperature < 0", name);
+  const bool scale = temperature > 0.f && temperature != 1.0f;
+  IdList banned{}, stop{};
+  banned.n = n_banned;
+  for (int i = 0; i < n_banned; ++i) banned.id[i] = banned_host[i];
+  stop.n = n_stop;
+  for (int i = 0; i < n_stop; ++i) stop.id[i] = stop_host[i];
+  Penalties pen{};
+  pen.counts = counts;
+  pen.counts_src = counts_src;
+  pen.presence = alpha_presence;
+  pen.frequency = alpha_frequency;
+  pen.presence_src = alpha_presence_src;
+  pen.frequency_src = alpha_frequency_src;
+  hipLaunchKernelGGL(sample_topp_kernel, dim3(B), dim3(SP_THREADS), 0, (hipStream_t)stream,
+                     (const half_t*)logits, ld_logits, V, temperature, scale, banned, stop,
+                     finished, row_mode, force_eos_all, eos_idx, topp_rows, topp_all, noise, pen,
+                     tok, tok_stride, score, score_stride);
+  MSA_CHECK_LAUNCH(name);
   return MSA_OK;
 }

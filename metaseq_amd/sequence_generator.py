@@ -7,9 +7,11 @@ token/score write-back and the finished-row update on the device, and the host o
 once end-of-sequence becomes possible (step >= min_len).
 
 Nucleus (top-p) sampling, factual-nucleus decay and the repetition penalties take the general
-path: the step's masked fp32 log-probabilities are materialised with device tensor ops in
-the reference's order (:271-308) and the draw is ``torch.multinomial`` on the device, as in
-the reference (:431).  Factual-nucleus state is kept per row (the reference's indexing only
+path: one kernel per step (msa_sample_topp_f16) applies the reference's masks and penalties
+(:271-293, :478-523), finds the nucleus without sorting and draws from it; only when the
+per-step distributions are wanted (``need_logprobs``) are the masked fp32 log-probabilities
+materialised with device tensor ops and the draw made by ``torch.multinomial``, as in the
+reference (:431).  Factual-nucleus state is kept per row (the reference's indexing only
 works at beam_size 1, where the two agree), and prompt-token counts of a replica row come from
 its own prompt (the reference indexes past the prompt batch when beam_size > 1).
 """
@@ -247,11 +249,16 @@ class SequenceGenerator(nn.Module):
                     step = nxt
             for step in range(start_step, max_len if not fused else start_step):
                 if general:
-                    lprobs = self._masked_lprobs(step_logits, step, min_len, max_len, finished,
-                                                 gs)
-                    if all_lprobs is not None:
-                        all_lprobs[:, step] = lprobs
-                    self._choose(lprobs, step, gs, finished, tokens, scores)
+                    if all_lprobs is None and step_logits.dtype == torch.float16:
+                        # masks, penalties, nucleus and draw in one kernel per step
+                        self._sample_step(lib, step_logits, step, min_len, max_len, finished, gs,
+                                          tokens, scores)
+                    else:  # the distributions are wanted: materialise them with tensor ops
+                        lprobs = self._masked_lprobs(step_logits, step, min_len, max_len,
+                                                     finished, gs)
+                        if all_lprobs is not None:
+                            all_lprobs[:, step] = lprobs
+                        self._choose(lprobs, step, gs, finished, tokens, scores)
                     if bool(finished.all()) or step + 1 >= max_len:
                         break
                     out = decoder(tokens[:, :step + 1], incremental_state=incremental_states)[0]
@@ -338,7 +345,34 @@ class SequenceGenerator(nn.Module):
         gs["toks_since_reset"] = torch.zeros(BB, 1, device=dev)
         gs["full_stop"] = torch.tensor(self.full_stop_list, device=dev)
         gs["rows"] = torch.arange(BB, device=dev)
+        gs["noise"] = (torch.empty(BB, V, dtype=torch.float32, device=dev) if self.sampling
+                       else None)
         return gs
+
+    def _sample_step(self, lib, step_logits, step, min_len, max_len, finished, gs, tokens,
+                     scores):
+        """One step of the general path on the device (metaseq/sequence_generator.py:272-308,
+        399-441, 478-534): msa_sample_topp_f16 applies the masks and the repetition penalties,
+        finds the nucleus and draws from it.  The draw consumes one Exp(1) number per row and
+        token from torch's device generator (an exponential race, the way torch.multinomial
+        itself draws), so ``torch.manual_seed`` fixes the samples."""
+        BB, V = step_logits.shape
+        banned = self._banned(step, min_len)
+        ba = (ctypes.c_int32 * len(banned))(*banned)
+        sa = (ctypes.c_int32 * max(1, len(self.stop)))(*self.stop)
+        noise = gs["noise"].exponential_() if self.sampling else None
+        topp_rows = gs["topp"] if (self.sampling and self.lambda_decay > 0) else None
+        tok, sc = tokens[:, step], scores[:, step]
+        check(lib.msa_sample_topp_f16(
+            ptr(step_logits), step_logits.stride(0), BB, V, float(self.temperature), ba,
+            len(banned), sa, len(self.stop), ptr(finished), None, int(step >= max_len - 1),
+            self.eos, ptr(topp_rows), float(self.sampling_topp) if self.sampling else 0.0,
+            ptr(noise), ptr(gs["count_tokens"]), ptr(gs["count_tokens_src"]),
+            float(self.alpha_presence), float(self.alpha_frequency),
+            float(self.alpha_presence_src), float(self.alpha_frequency_src), ptr(tok),
+            tokens.stride(0), ptr(sc), scores.stride(0), _capi.stream_ptr()))
+        if self.sampling and self.lambda_decay > 0:
+            self._update_sampling_topp(tokens[:, step], gs)
 
     def _apply_repetition_penalties(self, lprobs, count_tokens, count_tokens_src):
         """mu[j] - c[j] * alpha_frequency - [c[j] > 0] * alpha_presence (:478-523)."""

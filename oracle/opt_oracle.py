@@ -327,10 +327,16 @@ class OracleDecoder:
     __call__ = forward
 
 
-def sample_topp(lprobs: torch.Tensor, topp, generator=None):
+def sample_topp(lprobs: torch.Tensor, topp, generator=None, noise=None):
     """Nucleus choice of SequenceGenerator._sample_topp (metaseq/sequence_generator.py:399-441)
     for ``topp`` a float or a [rows, 1] tensor.  Returns (scores, token ids, the truncated
-    renormalised distribution in sorted order, the sort indices)."""
+    renormalised distribution in sorted order, the sort indices).
+
+    The reference draws with ``torch.multinomial``.  With ``noise`` ([rows, vocab] independent
+    Exp(1) numbers, one per token id) the same categorical draw is made as an exponential race
+    instead - the arg-max of probability / noise, which is how multinomial itself draws one
+    sample, there over sorted ranks - so that two implementations fed the same noise must pick
+    the same token."""
     probs = torch.softmax(lprobs, dim=-1)  # :416
     sprobs, sinds = probs.sort(dim=-1, descending=True)
     if torch.is_tensor(topp):
@@ -339,8 +345,12 @@ def sample_topp(lprobs: torch.Tensor, topp, generator=None):
     trunc = sprobs.clone()
     trunc[mask] = 0
     trunc = trunc / trunc.sum(dim=-1, keepdim=True)  # :430
-    choices = torch.multinomial(trunc, 1, generator=generator)[:, 0]  # :431
     rows = torch.arange(lprobs.size(0), device=lprobs.device)
+    if noise is not None:
+        by_id = torch.zeros_like(trunc).scatter_(1, sinds, trunc)
+        toks = (by_id / noise).argmax(dim=-1)
+        return probs[rows, toks].log(), toks, trunc, sinds
+    choices = torch.multinomial(trunc, 1, generator=generator)[:, 0]  # :431
     return sprobs[rows, choices].log(), sinds[rows, choices], trunc, sinds  # :433-434
 
 
@@ -381,14 +391,15 @@ def generate(decoder, src_tokens: torch.Tensor, max_len_b: int, min_len: int = 1
              alpha_presence: float = 0.0, alpha_frequency: float = 0.0,
              alpha_presence_src: float = 0.0, alpha_frequency_src: float = 0.0,
              alpha_src_penalty_end_idx: int = -1, need_logprobs: bool = False,
-             generator=None):
+             generator=None, noise_fn=None):
     """SequenceGenerator._generate (metaseq/sequence_generator.py:142-344; buffers :345-397;
     selection :399-441; factual nucleus :443-476; penalties :478-534).
 
     ``decoder(tokens, incremental_state=dict)`` must return ``(logits[B, T, V], extra)``.
     ``full_stop_list`` holds the ids the dictionary gives ".", "?" and "!" (:116; the unk id for
     a dictionary of BPE ids).  Factual-nucleus state is kept per row, which is what the
-    reference does at beam_size 1 (its indexing fails for more).
+    reference does at beam_size 1 (its indexing fails for more).  ``noise_fn(shape)``, if
+    given, supplies the Exp(1) numbers of each sampling step's draw (see ``sample_topp``).
     Returns {"tokens": [B, beam, max_len], "scores": [B, beam, max_len]} (+ "distributions"
     with ``need_logprobs``) and, on request, the logits tensors seen by the loop.
     """
@@ -463,7 +474,8 @@ def generate(decoder, src_tokens: torch.Tensor, max_len_b: int, min_len: int = 1
             next_scores, next_toks = lprobs.max(dim=-1)  # :413-415
         else:
             p = topp if lambda_decay <= 0 else topp_rows.unsqueeze(1)
-            next_scores, next_toks, _, _ = sample_topp(lprobs, p, generator)
+            noise = noise_fn(lprobs.shape) if noise_fn is not None else None
+            next_scores, next_toks, _, _ = sample_topp(lprobs, p, generator, noise)
             if lambda_decay > 0:
                 topp_rows = update_sampling_topp(next_toks, toks_since_reset, init_p,
                                                  list(full_stop_list), lambda_decay, omega_bound)

@@ -816,3 +816,123 @@ def test_stream_read_probe_runs_and_validates(lib):
     assert lib.msa_probe_stream_read(P(buf), 24, None) == -1
     assert lib.msa_probe_stream_read(ctypes.c_void_p(buf.data_ptr() + 2), 32, None) == -1
     assert lib.msa_probe_stream_read(None, 32, None) == -1
+
+
+# ---- nucleus sampling kernel ------------------------------------------------------------------
+def _sample(lib, logits, *, temperature=1.0, banned=(1,), stop=(), finished=None, row_mode=None,
+            force=0, eos=2, topp_rows=None, topp_all=0.0, noise=None, counts=None,
+            counts_src=None, alphas=(0.0, 0.0, 0.0, 0.0)):
+    B, V = logits.shape
+    ba = (ctypes.c_int32 * max(1, len(banned)))(*banned)
+    sa = (ctypes.c_int32 * max(1, len(stop)))(*stop)
+    tok = torch.full((B,), -7, dtype=torch.long, device=DEV)
+    sc = torch.zeros(B, dtype=torch.float32, device=DEV)
+    ok(lib.msa_sample_topp_f16(P(logits), logits.stride(0), B, V, temperature, ba, len(banned), sa,
+                               len(stop), P(finished), P(row_mode), force, eos, P(topp_rows),
+                               topp_all, P(noise), P(counts), P(counts_src), alphas[0], alphas[1],
+                               alphas[2], alphas[3], P(tok), 1, P(sc), 1, None), lib)
+    torch.cuda.synchronize()
+    return tok.cpu(), sc.cpu()
+
+
+def _reference_lprobs(logits, temperature, banned, early, only_eos, eos, counts, counts_src,
+                      alphas):
+    """The masked, penalised fp32 log-probabilities of the reference's loop
+    (sequence_generator.py:272-293, 478-523), in its order."""
+    z = logits.float().cpu()
+    if temperature != 1.0:
+        z = z / temperature
+    lp = torch.log_softmax(z, -1)
+    for r in range(lp.shape[0]):
+        lp[r, list(banned) + (list(early[r]) if early else [])] = float("-inf")
+    lp = O.apply_repetition_penalties(lp, counts, counts_src, *alphas)
+    for r in range(lp.shape[0]):
+        if only_eos[r]:
+            keep = lp[r, eos].clone()
+            lp[r] = float("-inf")
+            lp[r, eos] = keep
+    return lp
+
+
+@pytest.mark.parametrize("V,B", [(50272, 8), (4001, 5), (96, 16)])
+def test_nucleus_sampling_kernel_matches_oracle_given_the_same_noise(lib, V, B):
+    """Masks, per-row regimes, both repetition penalties, temperature, one top-p per row: the
+    kernel's token must be the oracle's (arg-max of truncated probability / noise over the same
+    nucleus), its score the log-probability among the eligible ids, and the generated-token
+    counts go up by one."""
+    print("sample_topp", V, B, flush=True)
+    g = torch.Generator().manual_seed(V)
+    logits = (torch.randn(B, V, generator=g) * 2.0).half()
+    counts = torch.randint(0, 3, (B, V), generator=g)
+    counts_src = torch.randint(0, 2, (B, V), generator=g)
+    alphas = (0.7, 0.2, 0.4, 0.1)
+    eos, stop = 2, [7, 11]
+    modes = torch.tensor([(i % 4) for i in range(B)], dtype=torch.uint8)   # 0, early, only, both
+    fin = torch.tensor([i == 5 for i in range(B)], dtype=torch.uint8)
+    topp = torch.tensor([0.05 + 0.9 * i / max(1, B - 1) for i in range(B)])
+    noise = torch.empty(B, V).exponential_(generator=g)
+    early = [[eos] + stop if int(m) & 1 else [] for m in modes]
+    only = [bool(int(m) & 2) or bool(f) for m, f in zip(modes, fin)]
+    lp = _reference_lprobs(logits, 0.8, [1], early, only, eos, counts, counts_src, alphas)
+    want_sc, want_tok, _, _ = O.sample_topp(lp, topp.unsqueeze(1), noise=noise)
+    cd = G(counts.clone())
+    tok, sc = _sample(lib, G(logits), temperature=0.8, banned=[1], stop=stop, finished=G(fin.clone()),
+                      row_mode=G(modes), eos=eos, topp_rows=G(topp), noise=G(noise), counts=cd,
+                      counts_src=G(counts_src), alphas=alphas)
+    dead = ~torch.isfinite(lp).any(-1)      # eos banned and alone eligible: (0, -inf)
+    assert bool(dead[3]) and int(tok[3]) == 0 and float(sc[3]) == float("-inf")
+    live = ~dead
+    assert torch.equal(tok[live], want_tok[live]), (tok, want_tok)
+    assert torch.allclose(sc[live], want_sc[live], atol=2e-5)
+    bumped = counts.clone()
+    bumped[torch.arange(B), tok] += 1
+    assert torch.equal(cd.cpu(), bumped)
+
+
+def test_nucleus_sampling_kernel_closed_forms(lib):
+    """Hand-made distributions.  (i) p = 1/2, 1/4, 1/8, ...: with top-p 0.6 the nucleus is the
+    first two ids (the third has 0.75 before it) and the race picks them 2 : 1; (ii) eight equal
+    ids with top-p 0.3: ties are cut by id, the first three belong (0, 0.125, 0.25 before them);
+    (iii) top-p >= 1 keeps everything; (iv) without noise the choice is greedy and the score the
+    penalised log-softmax value, as the reference's max() over lprobs gives."""
+    V = 16
+    pr = torch.tensor([2.0 ** -(i + 1) for i in range(V)])
+    pr[-1] = pr[-2]
+    order = torch.randperm(V, generator=torch.Generator().manual_seed(3))
+    probs = torch.zeros(V)
+    probs[order] = pr                          # the big ones are not the low ids
+    N = 4096
+    logits = probs.log().half().unsqueeze(0).repeat(N, 1)
+    noise = torch.empty(N, V).exponential_(generator=torch.Generator().manual_seed(4))
+    tok, sc = _sample(lib, G(logits), banned=[], topp_all=0.6, noise=G(noise))
+    a, b2 = int(order[0]), int(order[1])
+    assert set(tok.tolist()) == {a, b2}
+    frac = float((tok == a).float().mean())
+    assert abs(frac - 2 / 3) < 0.03, frac
+    assert torch.allclose(sc[tok == a], torch.tensor(0.5).log(), atol=2e-3)
+    # (ii) ties cut by id
+    flat = torch.zeros(N, V, dtype=torch.float16)
+    flat[:, 8:] = float("-inf")
+    tok, _ = _sample(lib, G(flat), banned=[], topp_all=0.3, noise=G(noise))
+    assert set(tok.tolist()) == {0, 1, 2}
+    for t in (0, 1, 2):
+        assert abs(float((tok == t).float().mean()) - 1 / 3) < 0.03
+    # (iii) the whole distribution
+    tok, _ = _sample(lib, G(logits), banned=[], topp_all=1.0, noise=G(noise))
+    freq = torch.bincount(tok, minlength=V).float() / N
+    assert torch.allclose(freq, probs / probs.sum(), atol=0.03)
+    # (iv) greedy with penalties: the arg-max of lprobs - penalties, score = that value
+    counts = torch.zeros(N, V, dtype=torch.long)
+    counts[:, a] = 5                           # pushes the best id below the second best
+    cd = G(counts.clone())
+    tok, sc = _sample(lib, G(logits), banned=[], counts=cd, alphas=(0.3, 0.2, 0.0, 0.0))
+    lp = torch.log_softmax(logits[0].float(), -1)
+    lp[a] -= 5 * 0.2 + 0.3
+    assert int(tok[0]) == int(lp.argmax()) == b2 and bool((tok == b2).all())
+    assert abs(float(sc[0]) - float(lp[b2])) < 2e-5
+    assert int(cd[0, b2]) == 1
+    # a NaN logit: token 0 with score -inf, whatever the mode
+    bad = logits[:2].clone()
+    bad[0, 3] = float("nan")
+    tok, sc = _sample(lib, G(bad), banned=[], topp_all=0.9, noise=G(noise[:2]))
+    assert int(tok[0]) == 0 and float(sc[0]) == float("-inf") and float(sc[1]) > float("-inf")

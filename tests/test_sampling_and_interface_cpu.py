@@ -197,3 +197,18 @@ def test_factual_nucleus_needs_resolvable_full_stops():
                             lambda_decay=0.8)
     assert gen.full_stop_list == [7, 8, 9]
     SequenceGenerator([dec], Dictionary(12), topp=0.9)  # no decay: nothing to resolve
+
+
+def test_exponential_race_draws_from_the_truncated_distribution():
+    """sample_topp with noise: the arg-max of probability / Exp(1) noise over the nucleus picks
+    every id with its renormalised nucleus probability (frequencies over 20 000 draws), never an
+    id outside the nucleus, and scores it with its untruncated log-probability."""
+    probs = torch.tensor([0.05, 0.4, 0.1, 0.25, 0.2])
+    n = 20000
+    lprobs = probs.log().unsqueeze(0).repeat(n, 1)
+    noise = torch.empty(n, 5).exponential_(generator=torch.Generator().manual_seed(5))
+    sc, tok, _, _ = O.sample_topp(lprobs, 0.7, noise=noise)   # nucleus: 0.4, 0.25, 0.2
+    assert set(tok.tolist()) == {1, 3, 4}
+    freq = torch.bincount(tok, minlength=5).float() / n
+    assert torch.allclose(freq, torch.tensor([0, 0.4, 0, 0.25, 0.2]) / 0.85, atol=0.012)
+    assert torch.allclose(sc, probs[tok].log(), atol=1e-6)
