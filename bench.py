@@ -274,6 +274,9 @@ def main():
     ap.add_argument("--unfused-select", action="store_true",
                     help="store the logits and run the stand-alone selection kernel instead of "
                          "selecting inside the vocabulary projection (for comparison)")
+    ap.add_argument("--python-step", action="store_true",
+                    help="drive every kernel of a decode step from Python instead of the one-call "
+                         "msa_decoder_step (same kernels, same results; for comparison)")
     ap.add_argument("--pmc-calibration", action="store_true",
                     help="also run a plain 1 GiB device copy, the known-size kernel that "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE readings are scaled by")
@@ -328,6 +331,7 @@ def main():
     lib = _capi.load()
     decoder = model.decoder
     decoder.kv_cache_capacity = max_len
+    decoder.native_step = not args.python_step
 
     tokens = torch.full((B, max_len), 1, dtype=torch.long, device=dev)
     scores = torch.zeros(B, max_len, dtype=torch.float32, device=dev)

@@ -293,6 +293,81 @@ int msa_lm_head_greedy_select_noalloc_f16(const void* x, const void* Ep, void* l
                                           int64_t score_stride, const int32_t* len_dev,
                                           void* stream);
 
+/* ---- one decode step of the whole decoder in one call ------------------------------------------
+ * msa_decoder_create copies a table of device pointers (it allocates host memory only and
+ * touches no GPU); msa_decoder_step then launches, on `stream`, exactly the sequence a caller
+ * would issue entry point by entry point for T == 1 and at most 64 rows: msa_embed_f16,
+ * msa_layernorm_f16, per layer msa_qkv_proj_* / msa_attention_f16 / msa_linear_partial_* /
+ * msa_residual_layernorm_f16 / msa_linear_* (ReLU) / msa_linear_partial_* /
+ * msa_residual_layernorm_f16, then msa_lm_head_greedy_select_f16 (if `tok` is given; `logits`
+ * optional) or msa_linear_f16 into `logits` - same arguments, same order, so bit-identical
+ * results.  Every linear weight is in the packed layout, int8 with scales if cfg.int8 (the
+ * embedding tables stay row-major fp16, lm_head_packed is the packed copy of embed_tokens).
+ * With len_dev (per-row lengths, see above) the rows that took part are advanced by one at the
+ * end of the step unless MSA_STEP_NO_ADVANCE; MSA_EMBED_COL_FROM_LEN as for msa_embed_f16.
+ * k_cache / v_cache are HOST arrays of cfg.layers device pointers ([B, H, S_cap, hd] each).
+ * workspace: msa_decoder_step_workspace_bytes(dec, B) bytes of device memory (scratch).
+ * Replaces one pass of ModelParallelTransformerDecoder.forward with a non-empty
+ * incremental_state (metaseq/models/transformer_decoder.py:494-537) plus, with `tok`, the
+ * per-step vocabulary passes of SequenceGenerator._generate
+ * (metaseq/sequence_generator.py:272-308, :319-323). */
+#define MSA_STEP_NO_ADVANCE 16u
+
+typedef struct {
+  int layers, d_model, heads, ffn, vocab;
+  int n_pos_rows; /* rows of the positional table */
+  int pad_idx;
+  int int8;       /* the four per-layer matrices are packed int8 with fp16 scales */
+} msa_decoder_config;
+
+typedef struct {
+  const void *ln1_gamma, *ln1_beta;                 /* self_attn_layer_norm */
+  const void *qkv_weight, *qkv_scales, *qkv_bias;   /* rows K | V | Q */
+  const void *out_weight, *out_scales, *out_bias;
+  const void *ln2_gamma, *ln2_beta;                 /* final_layer_norm */
+  const void *fc1_weight, *fc1_scales, *fc1_bias;
+  const void *fc2_weight, *fc2_scales, *fc2_bias;
+} msa_layer_weights;
+
+typedef struct {
+  const int64_t* tokens;  /* [B, n] ids; the new token of row b is column n - 1 */
+  int64_t tok_stride;
+  int n, B;
+  void* const* k_cache;
+  void* const* v_cache;
+  int S0, S_cap;
+  int32_t* len_dev;             /* optional int32 [B] */
+  const uint8_t* key_pad_mask;  /* optional uint8 [B, mask_stride] */
+  int64_t mask_stride;
+  unsigned flags;
+  void* workspace;
+  int64_t workspace_bytes;
+  void* logits;                 /* optional fp16 [B, vocab] */
+  int64_t* tok;                 /* optional: greedy selection, as msa_lm_head_greedy_select_f16 */
+  int64_t tok_stride_out;
+  float* score;
+  int64_t score_stride;
+  float temperature;
+  const int32_t* banned;
+  int n_banned;
+  const int32_t* stop;
+  int n_stop;
+  uint8_t* finished;
+  const uint8_t* row_mode;
+  int force_eos_all, eos_idx;
+  const int32_t* col_dev;
+} msa_step_args;
+
+typedef struct msa_decoder msa_decoder;
+
+int msa_decoder_create(const msa_decoder_config* cfg, const void* embed_tokens,
+                       const void* embed_positions, const void* lm_head_packed,
+                       const void* final_ln_gamma, const void* final_ln_beta,
+                       const msa_layer_weights* layers, msa_decoder** out);
+void msa_decoder_destroy(msa_decoder* dec);
+int64_t msa_decoder_step_workspace_bytes(msa_decoder* dec, int B);
+int msa_decoder_step(msa_decoder* dec, const msa_step_args* args, void* stream);
+
 /* Measurement aid with no counterpart in the reference: reads `bytes` bytes (a multiple of 16,
  * 16-byte aligned) of device memory once with 16-byte streaming loads and discards them.  The
  * benchmark times it to report the read rate this GPU actually sustains beside the published

@@ -20,6 +20,37 @@ MSA_ROW_BAN_EARLY = 1
 MSA_ROW_ONLY_EOS = 2
 
 _P = c_void_p
+MSA_STEP_NO_ADVANCE = 16
+
+
+class DecoderConfig(ctypes.Structure):
+    """msa_decoder_config"""
+    _fields_ = [(n, c_int) for n in ("layers", "d_model", "heads", "ffn", "vocab", "n_pos_rows",
+                                     "pad_idx", "int8")]
+
+
+class LayerWeights(ctypes.Structure):
+    """msa_layer_weights: device pointers of one layer's parameters."""
+    _fields_ = [(n, c_void_p) for n in (
+        "ln1_gamma", "ln1_beta", "qkv_weight", "qkv_scales", "qkv_bias", "out_weight",
+        "out_scales", "out_bias", "ln2_gamma", "ln2_beta", "fc1_weight", "fc1_scales",
+        "fc1_bias", "fc2_weight", "fc2_scales", "fc2_bias")]
+
+
+class StepArgs(ctypes.Structure):
+    """msa_step_args"""
+    _fields_ = [("tokens", c_void_p), ("tok_stride", c_int64), ("n", c_int), ("B", c_int),
+                ("k_cache", ctypes.POINTER(c_void_p)), ("v_cache", ctypes.POINTER(c_void_p)),
+                ("S0", c_int), ("S_cap", c_int), ("len_dev", c_void_p),
+                ("key_pad_mask", c_void_p), ("mask_stride", c_int64), ("flags", c_uint),
+                ("workspace", c_void_p), ("workspace_bytes", c_int64), ("logits", c_void_p),
+                ("tok", c_void_p), ("tok_stride_out", c_int64), ("score", c_void_p),
+                ("score_stride", c_int64), ("temperature", c_float),
+                ("banned", ctypes.POINTER(c_int32)), ("n_banned", c_int),
+                ("stop", ctypes.POINTER(c_int32)), ("n_stop", c_int), ("finished", c_void_p),
+                ("row_mode", c_void_p), ("force_eos_all", c_int), ("eos_idx", c_int),
+                ("col_dev", c_void_p)]
+
 
 # name -> argtypes, in the order of include/metaseq_amd.h
 SIGNATURES = {
@@ -57,9 +88,13 @@ SIGNATURES = {
     "msa_lm_head_greedy_select_noalloc_f16": [_P, _P, _P, c_int, c_int, c_int, c_float, _P, c_int,
                                               _P, c_int, _P, _P, c_int, c_int, _P, c_int64, _P,
                                               c_int64, _P, _P],
+    "msa_decoder_create": [ctypes.POINTER(DecoderConfig), _P, _P, _P, _P, _P,
+                           ctypes.POINTER(LayerWeights), ctypes.POINTER(c_void_p)],
+    "msa_decoder_step": [_P, ctypes.POINTER(StepArgs), _P],
     "msa_probe_stream_read": [_P, c_int64, _P],
 }
-OTHER_SYMBOLS = ["msa_last_error", "msa_version", "msa_lm_head_select_workspace_bytes"]
+OTHER_SYMBOLS = ["msa_last_error", "msa_version", "msa_lm_head_select_workspace_bytes",
+                 "msa_decoder_destroy", "msa_decoder_step_workspace_bytes"]
 
 _lib = None
 
@@ -84,6 +119,10 @@ def load():
     lib.msa_version.restype = c_int
     lib.msa_lm_head_select_workspace_bytes.argtypes = [c_int]
     lib.msa_lm_head_select_workspace_bytes.restype = c_int64
+    lib.msa_decoder_destroy.argtypes = [_P]
+    lib.msa_decoder_destroy.restype = None
+    lib.msa_decoder_step_workspace_bytes.argtypes = [_P, c_int]
+    lib.msa_decoder_step_workspace_bytes.restype = c_int64
     _lib = lib
     return lib
 

@@ -10,7 +10,7 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB = os.path.join(HERE, "libmetaseq_amd.so")
 SOURCES = ["capi.hip", "layernorm.hip", "embed.hip", "gemm.hip", "attention.hip", "attention_prefill.hip",
-           "sampling.hip", "probe.hip"]
+           "sampling.hip", "probe.hip", "decoder_step.hip"]
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17", "-Wall", "-Wno-unused-function",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",

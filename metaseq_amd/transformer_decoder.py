@@ -124,6 +124,10 @@ class TransformerDecoder(nn.Module):
         self.layer_norm = _Affine((D,), (D,), device)
         self.inference = True
         self.return_inner_states = False
+        # decode steps of at most 64 rows go through msa_decoder_step (one C call per token);
+        # False drives the same kernels entry point by entry point from Python
+        self.native_step = True
+        self._native = None  # (handle, keep-alive references)
         # capacity (positions) of the KV cache the next prefill allocates; None = grow on demand
         self.kv_cache_capacity: Optional[int] = None
         self._state_key = str(uuid.uuid4()) + ".kv_cache"
@@ -156,6 +160,7 @@ class TransformerDecoder(nn.Module):
                                               device=lin.bias.device)
                 lin.packed, lin.qweight, lin.scales = False, None, None
         self._lm_head = None
+        self._drop_native()
         return super().load_state_dict(sd, strict=strict, **kw)
 
     def load_tensors(self, named_tensors, quantize_int8=False):
@@ -173,6 +178,7 @@ class TransformerDecoder(nn.Module):
             if lin.packed or lin.qweight is not None:
                 raise RuntimeError("load_tensors needs a freshly constructed decoder")
         self._lm_head = None
+        self._drop_native()
         seen = set()
         for name, t in named_tensors:
             if name.startswith("decoder."):
@@ -294,6 +300,97 @@ class TransformerDecoder(nn.Module):
                                        ptr(vc), B, T, H, hd, S0, cap, D, flags, ptr(len_dev),
                                        stream))
 
+    def __del__(self):
+        self._drop_native()
+
+    def _apply(self, fn, *args, **kwargs):
+        self._drop_native()  # .to() / .half() move the tensors the handle points at
+        return super()._apply(fn, *args, **kwargs)
+
+    def _drop_native(self):
+        native = self.__dict__.get("_native")
+        lib = self.__dict__.get("_lib")
+        if native is not None and lib is not None:
+            lib.msa_decoder_destroy(native[0])
+        self.__dict__["_native"] = None
+
+    def _native_handle(self, lib):
+        """The msa_decoder handle over this model's packed weights (created on first use; the
+        table holds raw device pointers, so it is rebuilt when the weights are reloaded)."""
+        if self._native is None:
+            cfg = self.cfg
+            int8 = self.layers[0].fc2.qweight is not None
+            conf = _capi.DecoderConfig(cfg.decoder_layers, cfg.decoder_embed_dim,
+                                       cfg.decoder_attention_heads, cfg.decoder_ffn_embed_dim,
+                                       cfg.vocab_size, self.embed_positions.weight.shape[0],
+                                       self.padding_idx, int(int8))
+            table = (_capi.LayerWeights * cfg.decoder_layers)()
+            for i, layer in enumerate(self.layers):
+                t = table[i]
+                t.ln1_gamma = layer.self_attn_layer_norm.weight.data_ptr()
+                t.ln1_beta = layer.self_attn_layer_norm.bias.data_ptr()
+                t.ln2_gamma = layer.final_layer_norm.weight.data_ptr()
+                t.ln2_beta = layer.final_layer_norm.bias.data_ptr()
+                for name, lin in (("qkv", layer.self_attn.qkv_proj),
+                                  ("out", layer.self_attn.out_proj), ("fc1", layer.fc1),
+                                  ("fc2", layer.fc2)):
+                    w = lin.qweight if int8 else lin.weight
+                    setattr(t, name + "_weight", w.data_ptr())
+                    setattr(t, name + "_scales", lin.scales.data_ptr() if int8 else None)
+                    setattr(t, name + "_bias", lin.bias.data_ptr())
+            handle = ctypes.c_void_p()
+            check(lib.msa_decoder_create(ctypes.byref(conf), ptr(self.embed_tokens.weight),
+                                         ptr(self.embed_positions.weight), ptr(self._lm_head),
+                                         ptr(self.layer_norm.weight), ptr(self.layer_norm.bias),
+                                         table, ctypes.byref(handle)))
+            self._native = (handle, table)
+        return self._native[0]
+
+    def _native_step(self, lib, stream, tokens, n, B, cache, mask, len_dev, S0, out,
+                     col_from_len=False, advance=True):
+        """One decode step through msa_decoder_step.  ``out``: dict with ``logits`` ([B, V] fp16
+        tensor or None) and / or ``select`` (the keyword arguments of ``_select_from``)."""
+        handle = self._native_handle(lib)
+        ws = getattr(cache, "native_ws", None)
+        need = lib.msa_decoder_step_workspace_bytes(handle, B)
+        if ws is None or ws.numel() < need:
+            ws = cache.native_ws = torch.empty(need, dtype=torch.uint8, device=cache.device)
+            L = self.cfg.decoder_layers
+            cache.native_kv = ((ctypes.c_void_p * L)(*[cache.k(i).data_ptr() for i in range(L)]),
+                               (ctypes.c_void_p * L)(*[cache.v(i).data_ptr() for i in range(L)]),
+                               cache.capacity)
+        if cache.native_kv[2] != cache.capacity:  # the cache was re-allocated (grown)
+            L = self.cfg.decoder_layers
+            cache.native_kv = ((ctypes.c_void_p * L)(*[cache.k(i).data_ptr() for i in range(L)]),
+                               (ctypes.c_void_p * L)(*[cache.v(i).data_ptr() for i in range(L)]),
+                               cache.capacity)
+        a = _capi.StepArgs()
+        a.tokens, a.tok_stride, a.n, a.B = tokens.data_ptr(), tokens.stride(0), n, B
+        a.k_cache, a.v_cache = cache.native_kv[0], cache.native_kv[1]
+        a.S0, a.S_cap = S0, cache.capacity
+        a.len_dev = ptr(len_dev)
+        a.key_pad_mask = ptr(mask)
+        a.mask_stride = mask.stride(0) if mask is not None else 0
+        a.flags = ((MSA_EMBED_COL_FROM_LEN if col_from_len else 0)
+                   | (0 if advance else _capi.MSA_STEP_NO_ADVANCE))
+        a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel()
+        a.logits = ptr(out.get("logits"))
+        sel = out.get("select")
+        keep = None
+        if sel is not None:
+            banned, stop = list(sel["banned"]), list(sel["stop"])
+            ba = (ctypes.c_int32 * max(1, len(banned)))(*banned)
+            sa = (ctypes.c_int32 * max(1, len(stop)))(*stop)
+            keep = (ba, sa)
+            a.tok, a.tok_stride_out = ptr(sel["tok_out"]), sel["tok_stride"]
+            a.score, a.score_stride = ptr(sel["score_out"]), sel["score_stride"]
+            a.temperature = float(sel["temperature"])
+            a.banned, a.n_banned, a.stop, a.n_stop = ba, len(banned), sa, len(stop)
+            a.finished, a.row_mode = ptr(sel.get("finished")), ptr(sel.get("row_mode"))
+            a.force_eos_all, a.eos_idx = int(sel["force_eos"]), int(sel["eos"])
+        check(lib.msa_decoder_step(handle, ctypes.byref(a), stream))
+        del keep
+
     def _step_buffers(self, cache, B):
         """Work buffers of a decode step (<= 64 rows), allocated once per KV cache so that their
         addresses stay fixed (a captured graph replays against them)."""
@@ -394,6 +491,10 @@ class TransformerDecoder(nn.Module):
         B = tokens.shape[0]
         if B > 64 or cache.has_pads:
             raise ValueError("static decode steps need at most 64 rows and no padding")
+        if self.native_step and not self.return_inner_states:
+            self._native_step(lib, stream, tokens, tokens.shape[1], B, cache, None, len_dev, 0,
+                              {"logits": logits_out}, col_from_len=True, advance=False)
+            return logits_out
         bufs = self._step_buffers(cache, B)
         feat, _ = self._decode_core(lib, stream, tokens, tokens.shape[1], B, cache, None, bufs,
                                     len_dev, 0, True, col_from_len=True)
@@ -409,7 +510,7 @@ class TransformerDecoder(nn.Module):
 
     # ------------------------------------------------------------------ forward
     def _forward_features(self, prev_output_tokens, incremental_state, token_embeddings,
-                          self_attn_padding_mask, want_packed):
+                          self_attn_padding_mask, want_packed, native_out=None):
         """Embedding, L pre-LN layers and the final LayerNorm.  Returns (features, packed,
         extra): features are ``[B, T, D]`` row-major, or - for a decode step of at most 64 rows
         when ``want_packed`` - the packed activation buffer the vocabulary projection reads."""
@@ -489,6 +590,15 @@ class TransformerDecoder(nn.Module):
             cache.grow(min(max(self.max_positions(), S0 + 1), int(cache.capacity * 1.5) + 64))
 
         M = B * T
+        if (T == 1 and M <= 64 and native_out is not None and self.native_step
+                and not self.return_inner_states):
+            # the whole step (vocabulary projection / selection included) in one C call
+            self._native_step(lib, stream, tokens, n, B, cache, mask, lens, S0, native_out)
+            cache.length = S0 + T
+            if incremental_state is not None:
+                incremental_state[self._state_key] = cache
+            return None, True, (B, T), {"inner_states": [{"tok": None, "pos": None, "emb": None},
+                                                         None]}
         if T == 1 and M <= 64:
             bufs = self._step_buffers(cache, B)
             feat, x_last = self._decode_core(lib, stream, tokens, n, B, cache, mask, bufs, lens,
@@ -640,6 +750,13 @@ class TransformerDecoder(nn.Module):
         B = cache.batch
         if last_tokens.shape != (B,) or last_tokens.dtype != torch.long:
             raise AssertionError("last_tokens must be int64 [%d]" % B)
+        if self.native_step and not self.return_inner_states:
+            select = dict(temperature=temperature, banned=banned, stop=stop, finished=finished,
+                          row_mode=row_mode, force_eos=False, eos=eos, tok_out=tok_out,
+                          tok_stride=1, score_out=score_out, score_stride=1)
+            self._native_step(lib, stream, last_tokens.view(B, 1), 1, B, cache, None, cache.lens,
+                              0, {"logits": logits_out, "select": select})
+            return
         bufs = self._step_buffers(cache, B)
         feat, _ = self._decode_core(lib, stream, last_tokens.view(B, 1), 1, B, cache, None, bufs,
                                     cache.lens, 0, True)
@@ -675,11 +792,20 @@ class TransformerDecoder(nn.Module):
                 features_only: bool = False, src_lengths=None, token_embeddings=None,
                 self_attn_padding_mask=None):
         """metaseq/models/transformer_decoder.py:494-537."""
+        native_out = None
+        if (not features_only and self.native_step and incremental_state
+                and prev_output_tokens.dim() == 2 and prev_output_tokens.shape[0] <= 64
+                and prev_output_tokens.is_cuda):
+            native_out = {"logits": torch.empty(prev_output_tokens.shape[0], self.cfg.vocab_size,
+                                                dtype=torch.float16,
+                                                device=prev_output_tokens.device)}
         f, packed, (B, T), extra = self._forward_features(
             prev_output_tokens, incremental_state, token_embeddings, self_attn_padding_mask,
-            want_packed=not features_only)
+            want_packed=not features_only, native_out=native_out)
         if features_only:
             return f, extra
+        if f is None:  # the native step wrote the logits
+            return native_out["logits"].view(B, T, -1), extra
         return self._project(f, packed, B, T), extra
 
     def forward_select(self, prev_output_tokens, incremental_state, *, temperature, banned, stop,
@@ -694,10 +820,16 @@ class TransformerDecoder(nn.Module):
         ``finished`` the uint8 row flags the call updates."""
         if not incremental_state:
             raise AssertionError("forward_select is a decode step: prefill first")
-        f, packed, (B, T), _ = self._forward_features(prev_output_tokens, incremental_state, None,
-                                                      None, want_packed=True)
+        select = dict(temperature=temperature, banned=banned, stop=stop, finished=finished,
+                      row_mode=row_mode, force_eos=force_eos, eos=eos, tok_out=tok_out,
+                      tok_stride=tok_stride, score_out=score_out, score_stride=score_stride)
+        f, packed, (B, T), _ = self._forward_features(
+            prev_output_tokens, incremental_state, None, None, want_packed=True,
+            native_out={"logits": logits_out, "select": select})
         if not packed:
             raise ValueError("forward_select needs at most 64 rows")
+        if f is None:
+            return  # the native step selected
         self._select_from(self._lib, f, B, temperature, banned, stop, finished, row_mode,
                           force_eos, eos, tok_out, tok_stride, score_out, score_stride, logits_out)
 

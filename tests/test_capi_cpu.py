@@ -67,3 +67,31 @@ def test_argument_validation_needs_no_gpu():
     assert b"leaves a K range empty" in lib.msa_last_error()
     assert lib.msa_linear_partial_w8a16(one, one, one, one, 52, 8000, 768, 8, 2, None) == -1
     assert b"leaves a K range empty" in lib.msa_last_error()
+
+
+def test_decoder_handle_is_host_only_bookkeeping():
+    """msa_decoder_create validates and copies a pointer table without touching a GPU; the
+    workspace size grows with the row count; a bad configuration or a missing pointer is
+    refused."""
+    lib = _capi.load()
+    conf = _capi.DecoderConfig(2, 128, 2, 512, 64, 40, 1, 0)
+    table = (_capi.LayerWeights * 2)()
+    for t in table:
+        for name, _ in _capi.LayerWeights._fields_:
+            setattr(t, name, 4096)
+    h = ctypes.c_void_p()
+    one = ctypes.c_void_p(4096)
+    assert lib.msa_decoder_create(ctypes.byref(conf), one, one, one, one, one, table,
+                                  ctypes.byref(h)) == 0
+    w8, w40 = (lib.msa_decoder_step_workspace_bytes(h, b) for b in (8, 40))
+    assert 0 < w8 < w40 and lib.msa_decoder_step_workspace_bytes(h, 65) == 0
+    args = _capi.StepArgs()
+    assert lib.msa_decoder_step(h, ctypes.byref(args), None) == -1     # nothing filled in
+    lib.msa_decoder_destroy(h)
+    table[1].fc2_bias = None
+    assert lib.msa_decoder_create(ctypes.byref(conf), one, one, one, one, one, table,
+                                  ctypes.byref(h)) == -1
+    assert b"layer 1" in lib.msa_last_error()
+    bad = _capi.DecoderConfig(2, 160, 2, 512, 64, 40, 1, 0)            # head_dim 80
+    assert lib.msa_decoder_create(ctypes.byref(bad), one, one, one, one, one, table,
+                                  ctypes.byref(h)) == -1

@@ -273,3 +273,53 @@ def test_batch_above_64_rows_generates_like_the_oracle():
     same = (got["tokens"].cpu() == want["tokens"]).all(dim=-1).flatten()
     print("70-row generation: %d / 70 rows identical" % int(same.sum()), flush=True)
     assert int(same.sum()) >= 68  # tiny random models have near-tied logits now and then
+
+
+@pytest.mark.parametrize("int8", [False, True])
+def test_one_call_decode_step_equals_the_step_driven_entry_point_by_entry_point(int8):
+    """msa_decoder_step launches the same kernels with the same arguments as the Python-driven
+    sequence: logits, selected tokens, scores and the cache contents are bit-identical, for a
+    plain batch, a ragged one (per-row lengths) and the fused selection."""
+    cfg = opt_config("125m", max_target_positions=96)
+    model, _ = build(cfg, seed=12, int8=int8)
+    dec = model.decoder
+    src = random_prompts(cfg, 5, 20, seed=6).to(DEV)
+    ragged = src.clone()
+    ragged[1, 9:] = 1
+    ragged[4, 15:] = 1
+    nxt = torch.randint(4, cfg.vocab_size, (5, 6), generator=torch.Generator().manual_seed(1)).to(DEV)
+    for prompt in (src, ragged):
+        outs = []
+        for native in (True, False):
+            dec.native_step = native
+            inc = {}
+            model(prompt, incremental_state=inc)
+            toks = prompt
+            steps = []
+            for t in range(3):
+                toks = torch.cat([toks, nxt[:, t:t + 1]], 1)
+                steps.append(dec(toks, incremental_state=inc)[0].clone())
+            # fused selection on the next step
+            toks = torch.cat([toks, nxt[:, 3:4]], 1)
+            tok = torch.zeros(5, dtype=torch.long, device=DEV)
+            sc = torch.zeros(5, dtype=torch.float32, device=DEV)
+            fin = torch.zeros(5, dtype=torch.uint8, device=DEV)
+            lg = torch.zeros(5, cfg.vocab_size, dtype=torch.float16, device=DEV)
+            dec.forward_select(toks, inc, temperature=1.0, banned=[1, 2], stop=[], finished=fin,
+                               force_eos=False, eos=2, tok_out=tok, tok_stride=1, score_out=sc,
+                               score_stride=1, logits_out=lg)
+            cache = dec.get_cache(inc)
+            torch.cuda.synchronize()
+            # the valid part of one layer's keys (the rest of the buffer is never written)
+            lens = ([cache.length] * 5 if cache.lens is None else cache.lens.tolist())
+            keys = torch.cat([cache.k(3)[b, :, :lens[b]].reshape(-1) for b in range(5)])
+            outs.append((steps, tok.clone(), sc.clone(), lg.clone(), keys,
+                         None if cache.lens is None else cache.lens.clone(), cache.length))
+        dec.native_step = True
+        a, b = outs
+        for x, y in zip(a[0], b[0]):
+            assert torch.equal(x, y)
+        for x, y in zip(a[1:5], b[1:5]):
+            assert torch.equal(x, y)
+        assert (a[5] is None and b[5] is None) or torch.equal(a[5], b[5])
+        assert a[6] == b[6]
