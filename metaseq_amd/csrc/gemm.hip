@@ -477,27 +477,32 @@ __global__ __launch_bounds__(KG * 64) void linear_stream_kernel(
 // A tile group is NG * NT tiles, dealt round robin to the tile lanes; one barrier per stage;
 // activations are fetched two stages ahead and parked in LDS one stage ahead, weights (and int8
 // scales) one stage ahead.  The K lanes are summed through LDS in fixed order.
-constexpr int SH_THREADS = 512;
-
-template <int MB, bool W8, int NG, int NT, int U>
+// KL K lanes x NG tile lanes of one wave each (8 waves as 2 x 4, or 12 waves as 4 x 3 for
+// workgroups whose tile count is a multiple of 3: nine tiles fill 4 x 3 slots only to three
+// quarters, but 3 x 3 exactly).
+template <int MB, bool W8, int KL, int NG, int NT, int U>
 struct ShareCfg {
-  static constexpr int KL = 8 / NG, SK = KL * U, UA = W8 ? U / 2 : U;
+  static constexpr int THREADS = KL * NG * 64;
+  static constexpr int SK = KL * U, UA = W8 ? U / 2 : U;
   static constexpr int XH = SK * MB * 512;  // halves of activations per stage
-  static constexpr int XP = SK * MB / 8;    // 16-byte pieces per thread and stage
-  static constexpr int LDS_BYTES = 2 * XH * 2 + (KL - 1) * NG * NT * MB * 1024;
-  static_assert(SK * MB % 8 == 0 && U % 2 == 0, "stage must split evenly over the threads");
+  static constexpr int PIECES = XH / 8;     // 16-byte pieces per stage
+  static constexpr int XP = (PIECES + THREADS - 1) / THREADS;  // pieces per thread and stage
+  // activations double buffered, then one tile slot's partial sums of the other K lanes
+  static constexpr int LDS_BYTES = 2 * XH * 2 + (KL - 1) * NG * MB * 1024;
+  static_assert(U % 2 == 0, "a stage holds whole int8 blocks");
 };
 
-template <int MB, bool W8, int MODE, int NG, int NT, int U>
-__global__ __launch_bounds__(SH_THREADS) void linear_share_kernel(
+template <int MB, bool W8, int MODE, int KL, int NG, int NT, int U>
+__global__ __launch_bounds__(KL * NG * 64) void linear_share_kernel(
     const half_t* __restrict__ xp, const void* __restrict__ Wp, const half_t* __restrict__ scales,
     float* __restrict__ part, int M, int N, int K, int tiles_per_wg, int ks_per_split,
     Epilogue epi) {
   static_assert(MODE != MODE_SELECT, "selection runs in the plain stream kernel");
-  using C = ShareCfg<MB, W8, NG, NT, U>;
-  constexpr int KL = C::KL, SK = C::SK, UA = C::UA, XH = C::XH, XP = C::XP;
+  using C = ShareCfg<MB, W8, KL, NG, NT, U>;
+  constexpr int SK = C::SK, UA = C::UA, XH = C::XH, XP = C::XP, THREADS = C::THREADS;
+  constexpr int PIECES = C::PIECES;
   extern __shared__ __attribute__((aligned(16))) half_t lx_share[];  // [2][XH], then red
-  float4_t* red = reinterpret_cast<float4_t*>(lx_share + 2 * XH);    // [KL-1][NG][NT*MB][64]
+  float4_t* red = reinterpret_cast<float4_t*>(lx_share + 2 * XH);    // [KL-1][NG][MB][64]
   const int lane = threadIdx.x & 63;
   // the wave number as a scalar: everything derived from it stays out of the vector registers
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -520,7 +525,8 @@ __global__ __launch_bounds__(SH_THREADS) void linear_share_kernel(
     const int kb = ks_begin + (idx % nstages) * SK;
 #pragma unroll
     for (int i = 0; i < XP; ++i) {
-      const int p = tid + SH_THREADS * i, f = p >> 6;
+      // a stage need not split evenly over the threads: surplus slots re-read the last piece
+      const int p = min(tid + THREADS * i, PIECES - 1), f = p >> 6;
       const int kk = min(kb + f / MB, ks_end - 1);
       xr[i] = *reinterpret_cast<const half8_t*>(
           xp + (((int64_t)kk * MB + f % MB) * 64 + (p & 63)) * 8);
@@ -531,9 +537,10 @@ __global__ __launch_bounds__(SH_THREADS) void linear_share_kernel(
     half_t* l = lx_share + (idx & 1) * XH;
 #pragma unroll
     for (int i = 0; i < XP; ++i) {
-      const int p = tid + SH_THREADS * i;
+      const int p = tid + THREADS * i;
       const bool live = kb + (p >> 6) / MB < ks_end;
-      *reinterpret_cast<half8_t*>(l + p * 8) = live ? xr[i] : zero8();
+      if (PIECES % THREADS == 0 || p < PIECES)
+        *reinterpret_cast<half8_t*>(l + p * 8) = live ? xr[i] : zero8();
     }
   };
   struct Wst {
@@ -567,7 +574,8 @@ __global__ __launch_bounds__(SH_THREADS) void linear_share_kernel(
   auto compute = [&](const Wst& w, int idx) {
     const half_t* l = lx_share + (idx & 1) * XH + kl * U * MB * 512 + lane * 8;
     constexpr int F = U * MB;  // fragment f = K step f / MB, row block f % MB
-    constexpr int PD = 4;      // LDS fragment reads in flight
+    constexpr int PD = KL * NG > 8 ? 2 : 4;  // LDS fragment reads in flight (registers are
+                                             // scarcer at three waves per SIMD)
     half8_t bx[PD];
 #pragma unroll
     for (int p = 0; p < PD; ++p) bx[p] = *reinterpret_cast<const half8_t*>(l + p * 512);
@@ -608,24 +616,21 @@ __global__ __launch_bounds__(SH_THREADS) void linear_share_kernel(
   };
   auto finish = [&](int idx) {  // after the last stage of a tile group
     const int grp = idx / nstages;
-    if (kl > 0) {
 #pragma unroll
-      for (int j = 0; j < NT; ++j)
+    for (int j = 0; j < NT; ++j) {  // one tile slot per round through the reduction buffer
+      if (kl > 0) {
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb)
-          red[((((kl - 1) * NG + ng) * NT + j) * MB + mb) * 64 + lane] = acc[j][mb];
-    }
-    __syncthreads();
-    if (kl == 0) {
-#pragma unroll
-      for (int j = 0; j < NT; ++j) {
-        const int t = tile_begin + (grp * NT + j) * NG + ng;
-        if (t >= tile_end) continue;
+          red[(((kl - 1) * NG + ng) * MB + mb) * 64 + lane] = acc[j][mb];
+      }
+      __syncthreads();
+      const int t = tile_begin + (grp * NT + j) * NG + ng;
+      if (kl == 0 && t < tile_end) {
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb) {
           float4_t sum = acc[j][mb];
 #pragma unroll
-          for (int k = 1; k < KL; ++k) sum += red[((((k - 1) * NG + ng) * NT + j) * MB + mb) * 64 + lane];
+          for (int k = 1; k < KL; ++k) sum += red[(((k - 1) * NG + ng) * MB + mb) * 64 + lane];
           const int m = mb * 16 + (lane & 15);
           const int n = t * 16 + ((lane >> 4) << 2);
           if (m >= M) continue;
@@ -635,6 +640,7 @@ __global__ __launch_bounds__(SH_THREADS) void linear_share_kernel(
             epilogue4<MODE>(epi, m, n, sum);
         }
       }
+      if (j + 1 < NT) __syncthreads();  // the buffer is rewritten by the next slot
     }
     clear();
   };
@@ -997,7 +1003,7 @@ void launch_stream_mb(const void* xp, const void* W, const void* scales, float* 
                      ks_per_split, epi, m_off);
 }
 
-constexpr int SH_GROUP = 12;  // tiles per pass of the shared-activation kernel (4 lanes x 3)
+constexpr int SH_GROUP = 12;  // most tiles per pass of the shared-activation kernel (4 lanes x 3)
 
 // The shared-activation kernel sweeps K once per pass of SH_GROUP tiles: it is used when the
 // workgroup's tiles fill their passes to at least three quarters.
@@ -1010,21 +1016,21 @@ bool share_fits(int N, int S) {
   return 4 * tpw >= 3 * passes * SH_GROUP;
 }
 
-template <int MB, bool W8, int MODE, int NG, int NT, int U>
+template <int MB, bool W8, int MODE, int KL, int NG, int NT, int U>
 void launch_share_cfg(const void* xp, const void* W, const void* scales, float* part, int S, int M,
                       int N, int K, int tiles_per_wg, int gx, int ks_per_split, const Epilogue& epi,
                       hipStream_t s) {
-  using C = ShareCfg<MB, W8, NG, NT, U>;
+  using C = ShareCfg<MB, W8, KL, NG, NT, U>;
   static bool attr_set = false;  // one flag per instantiation
   if (!attr_set) {
-    if (hipFuncSetAttribute((const void*)linear_share_kernel<MB, W8, MODE, NG, NT, U>,
+    if (hipFuncSetAttribute((const void*)linear_share_kernel<MB, W8, MODE, KL, NG, NT, U>,
                             hipFuncAttributeMaxDynamicSharedMemorySize,
                             C::LDS_BYTES) != hipSuccess)
       return;  // the caller's launch check reports the error
     attr_set = true;
   }
-  hipLaunchKernelGGL((linear_share_kernel<MB, W8, MODE, NG, NT, U>), dim3(gx, S),
-                     dim3(SH_THREADS), C::LDS_BYTES, s, (const half_t*)xp, W,
+  hipLaunchKernelGGL((linear_share_kernel<MB, W8, MODE, KL, NG, NT, U>), dim3(gx, S),
+                     dim3(C::THREADS), C::LDS_BYTES, s, (const half_t*)xp, W,
                      (const half_t*)scales, part, M, N, K, tiles_per_wg, ks_per_split, epi);
 }
 
@@ -1039,16 +1045,24 @@ void launch_share(const void* xp, const void* W, const void* scales, float* part
   const int gx = (ntiles + tiles_per_wg - 1) / tiles_per_wg;
   int ks_per_split = (nks + S - 1) / S;
   if (W8) ks_per_split = (ks_per_split + 1) & ~1;  // int8 blocks cover two steps
-  // tiles per wave and pass: the fewest that take the workgroup's tiles in one pass, at most 3
+  // the wave grid and tiles per wave whose slots the workgroup's tiles fill best in one pass
+  if constexpr (W8) {
+    if (tiles_per_wg == 5 || tiles_per_wg == 6)
+      return launch_share_cfg<MB, W8, MODE, 4, 3, 2, 2>(xp, W, scales, part, S, M, N, K,
+                                                        tiles_per_wg, gx, ks_per_split, epi, s);
+    if (tiles_per_wg == 9)
+      return launch_share_cfg<MB, W8, MODE, 4, 3, 3, 2>(xp, W, scales, part, S, M, N, K,
+                                                        tiles_per_wg, gx, ks_per_split, epi, s);
+  }
   if (tiles_per_wg <= 4)
-    launch_share_cfg<MB, W8, MODE, 4, 1, 8>(xp, W, scales, part, S, M, N, K, tiles_per_wg, gx,
-                                            ks_per_split, epi, s);
+    launch_share_cfg<MB, W8, MODE, 2, 4, 1, 8>(xp, W, scales, part, S, M, N, K, tiles_per_wg, gx,
+                                               ks_per_split, epi, s);
   else if (tiles_per_wg <= 8)
-    launch_share_cfg<MB, W8, MODE, 4, 2, 4>(xp, W, scales, part, S, M, N, K, tiles_per_wg, gx,
-                                            ks_per_split, epi, s);
+    launch_share_cfg<MB, W8, MODE, 2, 4, 2, 4>(xp, W, scales, part, S, M, N, K, tiles_per_wg, gx,
+                                               ks_per_split, epi, s);
   else
-    launch_share_cfg<MB, W8, MODE, 4, 3, 4>(xp, W, scales, part, S, M, N, K, tiles_per_wg, gx,
-                                            ks_per_split, epi, s);
+    launch_share_cfg<MB, W8, MODE, 2, 4, 3, 4>(xp, W, scales, part, S, M, N, K, tiles_per_wg, gx,
+                                               ks_per_split, epi, s);
 }
 
 template <bool W8, int MODE, bool XR = false>
