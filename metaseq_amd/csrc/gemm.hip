@@ -492,7 +492,7 @@ struct ShareCfg {
   static_assert(U % 2 == 0, "a stage holds whole int8 blocks");
 };
 
-template <int MB, bool W8, int MODE, int KL, int NG, int NT, int U>
+template <int MB, bool W8, int MODE, int KL, int NG, int NT, int U, int PF>
 __global__ __launch_bounds__(KL * NG * 64) void linear_share_kernel(
     const half_t* __restrict__ xp, const void* __restrict__ Wp, const half_t* __restrict__ scales,
     float* __restrict__ part, int M, int N, int K, int tiles_per_wg, int ks_per_split,
@@ -545,7 +545,14 @@ __global__ __launch_bounds__(KL * NG * 64) void linear_share_kernel(
   };
   struct Wst {
     half8_t a[UA][NT];  // fp16: one A fragment; int8: 16 raw bytes = two A fragments
-    uint32_t sc[NT];    // int8: the row's fp16 scale in the low half
+  };
+  uint32_t sc[NT];  // int8: the row's fp16 scale in the low half, one per tile of the group
+  auto gload_sc = [&](int grp) {
+#pragma unroll
+    for (int j = 0; j < NT; ++j) {
+      const int t = min(tile_begin + (grp * NT + j) * NG + ng, tile_end - 1);
+      sc[j] = W8 ? reinterpret_cast<const uint16_t*>(scales)[t * 16 + (lane & 15)] : 0u;
+    }
   };
   auto gload_w = [&](Wst& w, int idx) {
     const int grp = idx / nstages, st = idx - grp * nstages;
@@ -560,7 +567,6 @@ __global__ __launch_bounds__(KL * NG * 64) void linear_share_kernel(
         w.a[u][j] = __builtin_nontemporal_load(
             reinterpret_cast<const half8_t*>((const half_t*)Wp + blk * 512 + lane * 8));
       }
-      w.sc[j] = W8 ? reinterpret_cast<const uint16_t*>(scales)[t * 16 + (lane & 15)] : 0u;
     }
   };
 
@@ -579,25 +585,27 @@ __global__ __launch_bounds__(KL * NG * 64) void linear_share_kernel(
     half8_t bx[PD];
 #pragma unroll
     for (int p = 0; p < PD; ++p) bx[p] = *reinterpret_cast<const half8_t*>(l + p * 512);
-    // the A fragments of K step u
-    half8_t a[2][NT];
+    // the A fragments of K step u (one set only where registers are scarce: the other waves of
+    // the SIMD then cover the expansion)
+    constexpr int AB = PF > 2 ? 1 : 2;
+    half8_t a[AB][NT];
     auto expand = [&](int u) {
 #pragma unroll
       for (int j = 0; j < NT; ++j) {
         if (W8) {
           typedef uint32_t u4 __attribute__((ext_vector_type(4)));
           const u4 raw = __builtin_bit_cast(u4, w.a[u / 2][j]);
-          const half_t sc = __builtin_bit_cast(half2_t, w.sc[j])[0];
-          a[u & 1][j] = (u & 1) ? dequant8(raw[2], raw[3], sc) : dequant8(raw[0], raw[1], sc);
+          const half_t scj = __builtin_bit_cast(half2_t, sc[j])[0];
+          a[u % AB][j] = (u & 1) ? dequant8(raw[2], raw[3], scj) : dequant8(raw[0], raw[1], scj);
         } else {
-          a[u & 1][j] = w.a[W8 ? 0 : u][j];
+          a[u % AB][j] = w.a[W8 ? 0 : u][j];
         }
       }
     };
     // the stage's LDS stores and global loads go out first, then LDS reads and MFMAs alternate
     __builtin_amdgcn_sched_group_barrier(0x200, XP, 0);
     __builtin_amdgcn_sched_group_barrier(0x020, XP, 0);  // activations first: needed first
-    __builtin_amdgcn_sched_group_barrier(0x020, UA * NT + (W8 ? NT : 0), 0);
+    __builtin_amdgcn_sched_group_barrier(0x020, UA * NT, 0);
     __builtin_amdgcn_sched_group_barrier(0x100, PD, 0);
 #pragma unroll
     for (int f = 0; f < F; ++f) {
@@ -606,7 +614,7 @@ __global__ __launch_bounds__(KL * NG * 64) void linear_share_kernel(
       const half8_t cur = bx[f % PD];
 #pragma unroll
       for (int j = 0; j < NT; ++j)
-        acc[j][mb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[u & 1][j], cur, acc[j][mb], 0, 0, 0);
+        acc[j][mb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[u % AB][j], cur, acc[j][mb], 0, 0, 0);
       __builtin_amdgcn_sched_group_barrier(0x008, NT, 0);
       if (f + PD < F) {
         bx[f % PD] = *reinterpret_cast<const half8_t*>(l + (f + PD) * 512);
@@ -643,12 +651,13 @@ __global__ __launch_bounds__(KL * NG * 64) void linear_share_kernel(
       if (j + 1 < NT) __syncthreads();  // the buffer is rewritten by the next slot
     }
     clear();
+    if (W8 && grp + 1 < ngroups) gload_sc(grp + 1);
   };
 
-  // PF weight stages in flight (a third int8 stage measured no faster than two)
-  constexpr int PF = 2;
+  // PF - 1 weight stages in flight beyond the one being consumed
   Wst w[PF];
   clear();
+  if (W8) gload_sc(0);
   // same issue order as in the loop (activations of the next stage, then weights), so that the
   // wait before the loop's first LDS store does not cover the weight loads
   gload_x(0);
@@ -1004,32 +1013,34 @@ void launch_stream_mb(const void* xp, const void* W, const void* scales, float* 
 }
 
 constexpr int SH_GROUP = 12;  // most tiles per pass of the shared-activation kernel (4 lanes x 3)
+constexpr int SH_GROUP_W8 = 18;  // int8 only: 6 lanes x 3
 
 // The shared-activation kernel sweeps K once per pass of SH_GROUP tiles: it is used when the
 // workgroup's tiles fill their passes to at least three quarters.
-bool share_fits(int N, int S) {
+bool share_fits(int N, int S, bool w8) {
   int G = num_cus() / S;
   if (G < 1) G = 1;
   const int tpw = (N / 16 + G - 1) / G;
   if (tpw <= SH_GROUP) return true;  // one pass, with the tile count per wave chosen to fit
+  if (w8 && tpw <= SH_GROUP_W8 && 4 * tpw >= 3 * SH_GROUP_W8) return true;  // one pass of 18
   const int passes = (tpw + SH_GROUP - 1) / SH_GROUP;
   return 4 * tpw >= 3 * passes * SH_GROUP;
 }
 
-template <int MB, bool W8, int MODE, int KL, int NG, int NT, int U>
+template <int MB, bool W8, int MODE, int KL, int NG, int NT, int U, int PF = 2>
 void launch_share_cfg(const void* xp, const void* W, const void* scales, float* part, int S, int M,
                       int N, int K, int tiles_per_wg, int gx, int ks_per_split, const Epilogue& epi,
                       hipStream_t s) {
   using C = ShareCfg<MB, W8, KL, NG, NT, U>;
   static bool attr_set = false;  // one flag per instantiation
   if (!attr_set) {
-    if (hipFuncSetAttribute((const void*)linear_share_kernel<MB, W8, MODE, KL, NG, NT, U>,
+    if (hipFuncSetAttribute((const void*)linear_share_kernel<MB, W8, MODE, KL, NG, NT, U, PF>,
                             hipFuncAttributeMaxDynamicSharedMemorySize,
                             C::LDS_BYTES) != hipSuccess)
       return;  // the caller's launch check reports the error
     attr_set = true;
   }
-  hipLaunchKernelGGL((linear_share_kernel<MB, W8, MODE, KL, NG, NT, U>), dim3(gx, S),
+  hipLaunchKernelGGL((linear_share_kernel<MB, W8, MODE, KL, NG, NT, U, PF>), dim3(gx, S),
                      dim3(C::THREADS), C::LDS_BYTES, s, (const half_t*)xp, W,
                      (const half_t*)scales, part, M, N, K, tiles_per_wg, ks_per_split, epi);
 }
@@ -1048,10 +1059,13 @@ void launch_share(const void* xp, const void* W, const void* scales, float* part
   // the wave grid and tiles per wave whose slots the workgroup's tiles fill best in one pass
   if constexpr (W8) {
     if (tiles_per_wg == 5 || tiles_per_wg == 6)
-      return launch_share_cfg<MB, W8, MODE, 4, 3, 2, 2>(xp, W, scales, part, S, M, N, K,
+      return launch_share_cfg<MB, W8, MODE, 4, 3, 2, 2, 2>(xp, W, scales, part, S, M, N, K,
                                                         tiles_per_wg, gx, ks_per_split, epi, s);
     if (tiles_per_wg == 9)
-      return launch_share_cfg<MB, W8, MODE, 4, 3, 3, 2>(xp, W, scales, part, S, M, N, K,
+      return launch_share_cfg<MB, W8, MODE, 4, 3, 3, 2, 2>(xp, W, scales, part, S, M, N, K,
+                                                        tiles_per_wg, gx, ks_per_split, epi, s);
+    if (tiles_per_wg > 12 && tiles_per_wg <= 18)
+      return launch_share_cfg<MB, W8, MODE, 2, 6, 3, 2, 3>(xp, W, scales, part, S, M, N, K,
                                                         tiles_per_wg, gx, ks_per_split, epi, s);
   }
   if (tiles_per_wg <= 4)
@@ -1068,7 +1082,7 @@ void launch_share(const void* xp, const void* W, const void* scales, float* part
 template <bool W8, int MODE, bool XR = false>
 void launch_stream(const void* xp, const void* W, const void* scales, float* part, int S, int M,
                    int N, int K, const Epilogue& epi, hipStream_t s, int64_t m_off = 0) {
-  if (!XR && MODE != MODE_SELECT && M > 32 && share_fits(N, S)) {
+  if (!XR && MODE != MODE_SELECT && M > 32 && share_fits(N, S, W8)) {
     constexpr int PM = MODE == MODE_SELECT ? MODE_PLAIN : MODE;
     if (M > 48)
       launch_share<4, W8, PM>(xp, W, scales, part, S, M, N, K, epi, s);
@@ -1399,8 +1413,9 @@ namespace {
 int pick_splits(int64_t M, int N, int K, int wbytes) {
   if (M < 1 || M > 64 || N % 16 || K % 64) return 1;
   const int MB = (int)((M + 15) / 16), ntiles = N / 16, nks = K / 32;
-  // tiles that share one sweep over the activations, and K steps per stage of the workgroup
-  const int NT = MB > 2 ? SH_GROUP : ST_NT;
+  // tiles that share one sweep over the activations (int8 has a 2 x 6 x 3 shape of the
+  // shared-activation kernel for up to 18), and K steps per stage of the workgroup
+  const int NT = MB > 2 ? (wbytes == 1 ? SH_GROUP_W8 : SH_GROUP) : ST_NT;
   const int stage = MB > 2 ? 16 : ST_KG * 4;
   int best = 1;
   double best_cost = 0;

@@ -439,6 +439,9 @@ def test_linear_rejects_bad_shapes(lib):
 @pytest.mark.parametrize("M,N,K", [(8, 768, 768), (64, 3072, 768), (32, 768, 3072),
                                    (200, 2304, 768), (48, 4096, 4096), (64, 24576, 256),
                                    (40, 73728, 128),
+                                   # 9 tiles per workgroup (12 waves as 4 x 3), the last
+                                   # workgroup short of tiles and a K range of 1.5 stages
+                                   (64, 36864, 256), (50, 36784, 192),
                                    (1000, 16400, 128), (1124, 16400, 128)])   # large tiled kernel
 def test_linear_w8a16(lib, M, N, K):
     print("w8a16", M, N, K, flush=True)
@@ -462,7 +465,10 @@ def test_linear_w8a16(lib, M, N, K):
 
 @pytest.mark.parametrize("M,N,K,S", [(32, 768, 768, 1), (32, 768, 3072, 4), (8, 4096, 4096, 4),
                                      (33, 2048, 8192, 8), (64, 768, 3072, 3),
-                                     (48, 4608, 2048, 4)])
+                                     (48, 4608, 2048, 4),
+                                     # int8: 18 and 9 tiles per workgroup (12 waves as 2 x 6
+                                     # and 4 x 3), the second with a ragged last K slice
+                                     (64, 9216, 1024, 8), (64, 9216, 1152, 4)])
 @pytest.mark.parametrize("w8", [False, True])
 def test_split_k_partials_and_fused_layernorm(lib, M, N, K, S, w8):
     """msa_linear_partial_* followed by msa_residual_layernorm_f16 equals the oracle's
