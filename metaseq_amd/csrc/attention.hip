@@ -63,8 +63,12 @@ __global__ void attention_kernel(const half_t* __restrict__ q, const half_t* __r
     if (sub == 0) sc[kk] = s;
     lmax = fmaxf(lmax, s);
   };
+  // U rows per lane group are requested before the first is used, also in the last (or only)
+  // round, where rows past the end re-read the last key and are not scored: a short history
+  // (few rounds, or less than one) is one memory latency, not one per row
+  const int last = n_keys - 1;
   int key = wave * RPW + rsel;
-  for (; key + (U - 1) * kstride < n_keys; key += U * kstride) {
+  for (; key + (U - 1) * kstride < n_keys; key += U * kstride) {  // whole rounds
     half8_t kv[U];
 #pragma unroll
     for (int u = 0; u < U; ++u)
@@ -73,20 +77,24 @@ __global__ void attention_kernel(const half_t* __restrict__ q, const half_t* __r
 #pragma unroll
     for (int u = 0; u < U; ++u) score(kv[u], key + u * kstride);
   }
-  for (; key < n_keys; key += kstride)
-    score(__builtin_nontemporal_load(reinterpret_cast<const half8_t*>(kbase + (int64_t)key * HD)),
-          key);
+  if (key < n_keys) {
+    half8_t kv[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+      kv[u] = __builtin_nontemporal_load(reinterpret_cast<const half8_t*>(
+          kbase + (int64_t)min(key + u * kstride, last) * HD));
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+      if (key + u * kstride < n_keys) score(kv[u], key + u * kstride);
+  }
 
   // the first V rows are requested before the softmax so that HBM stays busy through it
   half8_t vpre[U];
   const int vkey0 = wave * RPW + rsel;
-  const bool have_pre = vkey0 + (U - 1) * kstride < n_keys;
-  if (have_pre) {
 #pragma unroll
-    for (int u = 0; u < U; ++u)
-      vpre[u] = __builtin_nontemporal_load(
-          reinterpret_cast<const half8_t*>(vbase + (int64_t)(vkey0 + u * kstride) * HD));
-  }
+  for (int u = 0; u < U; ++u)
+    vpre[u] = __builtin_nontemporal_load(reinterpret_cast<const half8_t*>(
+        vbase + (int64_t)min(vkey0 + u * kstride, last) * HD));
   const float m = block_max(lmax, red);  // barriers inside also publish sc[]
 
   // ---- softmax in fp32, probabilities rounded to fp16 ----
@@ -104,17 +112,18 @@ __global__ void attention_kernel(const half_t* __restrict__ q, const half_t* __r
   float acc[8];
 #pragma unroll
   for (int i = 0; i < 8; ++i) acc[i] = 0.f;
-  key = vkey0;
-  if (have_pre) {
+  // rows past the end are skipped, not weighted by zero: what a clamped load returns is a real
+  // row, but a probability read past the end of sc[] is not a number to multiply with
+  auto weigh = [&](const half8_t& vv, int kk) {
+    if (kk < n_keys) {
+      const float p = sc[kk];
 #pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const float p = sc[key + u * kstride];
-#pragma unroll
-      for (int i = 0; i < 8; ++i) acc[i] = fmaf(p, (float)vpre[u][i], acc[i]);
+      for (int i = 0; i < 8; ++i) acc[i] = fmaf(p, (float)vv[i], acc[i]);
     }
-    key += U * kstride;
-  }
-  for (; key + (U - 1) * kstride < n_keys; key += U * kstride) {
+  };
+#pragma unroll
+  for (int u = 0; u < U; ++u) weigh(vpre[u], vkey0 + u * kstride);
+  for (key = vkey0 + U * kstride; key + (U - 1) * kstride < n_keys; key += U * kstride) {
     half8_t vv[U];
 #pragma unroll
     for (int u = 0; u < U; ++u)
@@ -127,12 +136,14 @@ __global__ void attention_kernel(const half_t* __restrict__ q, const half_t* __r
       for (int i = 0; i < 8; ++i) acc[i] = fmaf(p, (float)vv[u][i], acc[i]);
     }
   }
-  for (; key < n_keys; key += kstride) {
-    const half8_t vv =
-        __builtin_nontemporal_load(reinterpret_cast<const half8_t*>(vbase + (int64_t)key * HD));
-    const float p = sc[key];
+  if (key < n_keys) {
+    half8_t vv[U];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) acc[i] = fmaf(p, (float)vv[i], acc[i]);
+    for (int u = 0; u < U; ++u)
+      vv[u] = __builtin_nontemporal_load(reinterpret_cast<const half8_t*>(
+          vbase + (int64_t)min(key + u * kstride, last) * HD));
+#pragma unroll
+    for (int u = 0; u < U; ++u) weigh(vv[u], key + u * kstride);
   }
   // combine the RPW row groups of a wave, then the waves, in a fixed order
 #pragma unroll
