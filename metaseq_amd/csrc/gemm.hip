@@ -506,8 +506,8 @@ __global__ __launch_bounds__(KL * NG * 64) void linear_share_kernel(
   const int lane = threadIdx.x & 63;
   // the wave number as a scalar: everything derived from it stays out of the vector registers
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int tid = wave * 64 + lane;
   const int kl = wave / NG, ng = wave - kl * NG;
+  const uint32_t lane_off = (uint32_t)lane * 16u;  // the lane's 16 bytes of a 1 KB fragment
   const int ntiles = N >> 4, nks = K >> 5;
   const int tile_begin = blockIdx.x * tiles_per_wg;
   const int tile_end = min(ntiles, tile_begin + tiles_per_wg);
@@ -525,11 +525,13 @@ __global__ __launch_bounds__(KL * NG * 64) void linear_share_kernel(
     const int kb = ks_begin + (idx % nstages) * SK;
 #pragma unroll
     for (int i = 0; i < XP; ++i) {
-      // a stage need not split evenly over the threads: surplus slots re-read the last piece
-      const int p = min(tid + THREADS * i, PIECES - 1), f = p >> 6;
+      // Piece p = 64 * f + lane: fragment f is the same for the whole wave, so the address is a
+      // scalar base plus the lane's 16 bytes.  A stage need not split evenly over the waves:
+      // surplus slots re-read the last fragment.
+      const int f = min(wave + (THREADS / 64) * i, PIECES / 64 - 1);
       const int kk = min(kb + f / MB, ks_end - 1);
-      xr[i] = *reinterpret_cast<const half8_t*>(
-          xp + (((int64_t)kk * MB + f % MB) * 64 + (p & 63)) * 8);
+      const half_t* frag = xp + ((int64_t)kk * MB + f % MB) * 512;
+      xr[i] = *reinterpret_cast<const half8_t*>(reinterpret_cast<const char*>(frag) + lane_off);
     }
   };
   auto lstore = [&](int idx) {
@@ -537,10 +539,10 @@ __global__ __launch_bounds__(KL * NG * 64) void linear_share_kernel(
     half_t* l = lx_share + (idx & 1) * XH;
 #pragma unroll
     for (int i = 0; i < XP; ++i) {
-      const int p = tid + THREADS * i;
-      const bool live = kb + (p >> 6) / MB < ks_end;
-      if (PIECES % THREADS == 0 || p < PIECES)
-        *reinterpret_cast<half8_t*>(l + p * 8) = live ? xr[i] : zero8();
+      const int f = wave + (THREADS / 64) * i;  // wave-uniform, as are the two conditions
+      const bool live = kb + f / MB < ks_end;
+      if (PIECES % THREADS == 0 || f < PIECES / 64)
+        *reinterpret_cast<half8_t*>(l + f * 512 + lane * 8) = live ? xr[i] : zero8();
     }
   };
   struct Wst {
@@ -564,8 +566,9 @@ __global__ __launch_bounds__(KL * NG * 64) void linear_share_kernel(
         const int ks = ks_begin + st * SK + kl * U + (W8 ? 2 * u : u);
         const int ksc = min(ks, ks_end - (W8 ? 2 : 1));
         const int64_t blk = W8 ? (int64_t)t * (nks >> 1) + (ksc >> 1) : (int64_t)t * nks + ksc;
+        const half_t* block = (const half_t*)Wp + blk * 512;  // wave-uniform
         w.a[u][j] = __builtin_nontemporal_load(
-            reinterpret_cast<const half8_t*>((const half_t*)Wp + blk * 512 + lane * 8));
+            reinterpret_cast<const half8_t*>(reinterpret_cast<const char*>(block) + lane_off));
       }
     }
   };

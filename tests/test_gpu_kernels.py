@@ -441,7 +441,7 @@ def test_linear_rejects_bad_shapes(lib):
                                    (40, 73728, 128),
                                    # 9 tiles per workgroup (12 waves as 4 x 3), the last
                                    # workgroup short of tiles and a K range of 1.5 stages
-                                   (64, 36864, 256), (50, 36784, 192),
+                                   (64, 36864, 256), (50, 36784, 192), (40, 36864, 256),
                                    (1000, 16400, 128), (1124, 16400, 128)])   # large tiled kernel
 def test_linear_w8a16(lib, M, N, K):
     print("w8a16", M, N, K, flush=True)
