@@ -29,8 +29,8 @@ HBM_PEAK = 8.0e12  # MI355X HBM3E, bytes/s
 MFMA_PEAK = 2.5e15  # dense fp16 MFMA, flop/s
 # HBM bytes per decode-attention launch over its algorithmic bytes, from rocprofv3 FETCH_SIZE +
 # WRITE_SIZE scaled by a 1 GiB copy (profiles/decode_attention_opt6.7b_bs32_pmc_traffic.txt):
-# 540.1 MB measured for 540.0 MB algorithmic.
-ATTN_TRAFFIC_RATIO = 540.1 / 540.0
+# 540.4 MB measured for 540.0 MB algorithmic.
+ATTN_TRAFFIC_RATIO = 540.4 / 540.0
 
 CONFIGS = {
     # name: (size, batch, prompt, generate)
