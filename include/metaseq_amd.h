@@ -8,6 +8,9 @@
  *   - all pointers are DEVICE pointers unless the name ends in _host; the library never
  *     allocates or frees device memory on behalf of these calls; `stream` is a hipStream_t
  *     (NULL = the default stream).  Nothing synchronises: work is enqueued on `stream`.
+ *   - the calls act on the calling thread's current device and may be made from several
+ *     threads and for several devices of one process; a msa_decoder handle (below) is used
+ *     by one thread at a time.
  *   - fp16 tensors are IEEE binary16, row-major, innermost dimension contiguous.
  *   - "round" below means round-to-nearest-even to fp16.  Every kernel accumulates in fp32
  *     and rounds at exactly the points where the reference materialises an fp16 tensor.

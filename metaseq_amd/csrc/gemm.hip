@@ -24,6 +24,7 @@
 // that scatters K/V into the per-layer cache and scales Q.
 #include <math.h>
 
+#include <atomic>
 #include <mutex>
 
 #include "common.h"
@@ -976,17 +977,37 @@ __global__ __launch_bounds__(TB_THREADS) void linear_tiled_big_kernel(
 }
 
 // ---- host side ------------------------------------------------------------------------------
-int g_num_cus = 0;
-int num_cus() {
-  if (g_num_cus == 0) {
-    int dev = 0, n = 0;
-    if (hipGetDevice(&dev) != hipSuccess ||
+// Per-device facts are kept per device: a process may drive several GPUs, from several threads.
+constexpr int MAX_DEVICES = 64;
+int current_device() {
+  int dev = 0;
+  return hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < MAX_DEVICES ? dev : -1;
+}
+
+std::atomic<int> g_num_cus[MAX_DEVICES];
+int num_cus() {  // compute units of the current device
+  const int dev = current_device();
+  int n = dev >= 0 ? g_num_cus[dev].load(std::memory_order_relaxed) : 0;
+  if (n == 0) {
+    if (dev < 0 ||
         hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
         n <= 0)
       n = 256;
-    g_num_cus = n;
+    if (dev >= 0) g_num_cus[dev].store(n, std::memory_order_relaxed);
   }
-  return g_num_cus;
+  return n;
+}
+
+// Raises a kernel's dynamic LDS limit once per device (one mask per kernel instantiation; a
+// second thread that gets here at the same time only repeats the call).
+bool allow_lds(const void* kernel, int bytes, std::atomic<uint64_t>& done) {
+  const int dev = current_device();
+  const uint64_t bit = dev >= 0 ? 1ull << dev : 0;
+  if (bit && (done.load(std::memory_order_acquire) & bit)) return true;
+  if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes) != hipSuccess)
+    return false;
+  if (bit) done.fetch_or(bit, std::memory_order_release);
+  return true;
 }
 
 template <int MB, bool W8, int MODE, bool XR = false>
@@ -1035,14 +1056,10 @@ void launch_share_cfg(const void* xp, const void* W, const void* scales, float* 
                       int N, int K, int tiles_per_wg, int gx, int ks_per_split, const Epilogue& epi,
                       hipStream_t s) {
   using C = ShareCfg<MB, W8, KL, NG, NT, U>;
-  static bool attr_set = false;  // one flag per instantiation
-  if (!attr_set) {
-    if (hipFuncSetAttribute((const void*)linear_share_kernel<MB, W8, MODE, KL, NG, NT, U, PF>,
-                            hipFuncAttributeMaxDynamicSharedMemorySize,
-                            C::LDS_BYTES) != hipSuccess)
-      return;  // the caller's launch check reports the error
-    attr_set = true;
-  }
+  static std::atomic<uint64_t> lds_allowed{0};  // one mask per instantiation
+  if (!allow_lds((const void*)linear_share_kernel<MB, W8, MODE, KL, NG, NT, U, PF>, C::LDS_BYTES,
+                 lds_allowed))
+    return;  // the caller's launch check reports the error
   hipLaunchKernelGGL((linear_share_kernel<MB, W8, MODE, KL, NG, NT, U, PF>), dim3(gx, S),
                      dim3(C::THREADS), C::LDS_BYTES, s, (const half_t*)xp, W,
                      (const half_t*)scales, part, M, N, K, tiles_per_wg, ks_per_split, epi);
@@ -1115,14 +1132,9 @@ void launch_tiled(const void* x, const void* W, const void* scales, int64_t M, i
   // the 256 x 256 kernel once it fills the chip; the 128 x 128 one for the shapes in between
   const int64_t big_tiles = ((M + TB_BM - 1) / TB_BM) * ((N + TB_BN - 1) / TB_BN);
   if (K % (2 * TB_BK) == 0 && big_tiles >= num_cus()) {
-    static bool attr_set = false;  // one flag per instantiation
-    if (!attr_set) {
-      if (hipFuncSetAttribute((const void*)linear_tiled_big_kernel<W8, MODE>,
-                              hipFuncAttributeMaxDynamicSharedMemorySize,
-                              TB_LDS_BYTES) != hipSuccess)
-        return;  // the launch check below reports the error
-      attr_set = true;
-    }
+    static std::atomic<uint64_t> lds_allowed{0};  // one mask per instantiation
+    if (!allow_lds((const void*)linear_tiled_big_kernel<W8, MODE>, TB_LDS_BYTES, lds_allowed))
+      return;  // the launch check below reports the error
     // A ragged bottom block would cost a full extra round of workgroups for a few rows (a
     // prompt of 2^k tokens plus the leading end-of-sentence token always has one): up to 128
     // leftover rows go through the weight-streaming kernel instead, 64 rows at a time.
