@@ -200,6 +200,24 @@ int msa_attention_f16(const void* q, const void* Kcache, const void* Vcache,
                       int hd, int T, int S0, int S_cap, unsigned flags, const int32_t* len_dev,
                       void* stream);
 
+/* The decode step's attention (T == 1) in two launches, for few (batch row, head) pairs over long
+ * histories (batch-1 serving, a nearly empty slot cache): one workgroup per pair leaves most
+ * CUs idle and pulls the pair's K and V rows through a single CU.  Launch 1 writes the rounded
+ * scores of 8 key ranges per pair to `workspace` (fp32 [B*H, S_cap],
+ * msa_attention_split_workspace_bytes); launch 2, one workgroup per pair and 32-column slice of
+ * the head, repeats the softmax over all scores and streams its slice of the V rows.  Every sum
+ * is formed in the order msa_attention_f16 uses for B*H < 512, so the two give identical bits
+ * and a caller may choose per step; msa_attention_prefers_split says when the split form pays
+ * (measured: B*H <= 64 and n_keys*hd >= 512 K, i.e. histories beyond OPT's 2048 positions; below
+ * that the second launch costs more than the idle CUs).  Arguments and reference as for
+ * msa_attention_f16 with T == 1. */
+int64_t msa_attention_split_workspace_bytes(int B, int H, int S_cap);
+int msa_attention_prefers_split(int B, int H, int hd, int n_keys);
+int msa_attention_split_f16(const void* q, const void* Kcache, const void* Vcache,
+                            const uint8_t* key_pad_mask, int64_t mask_stride, void* out,
+                            void* workspace, int B, int H, int hd, int S0, int S_cap,
+                            unsigned flags, const int32_t* len_dev, void* stream);
+
 /* One step of greedy selection over fp16 logits[B, V] (row stride ld_logits), with the
  * generator's bookkeeping fused in:
  *   z = logits / temperature (only if temperature > 0 and != 1);
@@ -338,7 +356,8 @@ typedef struct {
   int n, B;
   void* const* k_cache;
   void* const* v_cache;
-  int S0, S_cap;
+  int S0, S_cap;                /* with len_dev: S0 = the caller's bound on the lengths, 0 if
+                                   it has none (it only steers the choice of attention form) */
   int32_t* len_dev;             /* optional int32 [B] */
   const uint8_t* key_pad_mask;  /* optional uint8 [B, mask_stride] */
   int64_t mask_stride;

@@ -76,6 +76,9 @@ SIGNATURES = {
                            c_int, c_uint, _P, _P],
     "msa_attention_f16": [_P, _P, _P, _P, c_int64, _P, c_int, c_int, c_int, c_int, c_int, c_int,
                           c_uint, _P, _P],
+    "msa_attention_split_f16": [_P, _P, _P, _P, c_int64, _P, _P, c_int, c_int, c_int, c_int, c_int,
+                                c_uint, _P, _P],
+    "msa_attention_prefers_split": [c_int, c_int, c_int, c_int],
     "msa_greedy_select_f16": [_P, c_int64, c_int, c_int, c_float, _P, c_int, _P, c_int, _P, _P,
                               c_int, c_int, _P, c_int64, _P, c_int64, _P, _P],
     "msa_sample_topp_f16": [_P, c_int64, c_int, c_int, c_float, _P, c_int, _P, c_int, _P, _P,
@@ -94,7 +97,8 @@ SIGNATURES = {
     "msa_probe_stream_read": [_P, c_int64, _P],
 }
 OTHER_SYMBOLS = ["msa_last_error", "msa_version", "msa_lm_head_select_workspace_bytes",
-                 "msa_decoder_destroy", "msa_decoder_step_workspace_bytes"]
+                 "msa_decoder_destroy", "msa_decoder_step_workspace_bytes",
+                 "msa_attention_split_workspace_bytes"]
 
 _lib = None
 
@@ -123,6 +127,8 @@ def load():
     lib.msa_decoder_destroy.restype = None
     lib.msa_decoder_step_workspace_bytes.argtypes = [_P, c_int]
     lib.msa_decoder_step_workspace_bytes.restype = c_int64
+    lib.msa_attention_split_workspace_bytes.argtypes = [c_int, c_int, c_int]
+    lib.msa_attention_split_workspace_bytes.restype = c_int64
     _lib = lib
     return lib
 

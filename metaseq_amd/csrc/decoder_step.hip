@@ -28,9 +28,18 @@ int64_t align256(int64_t n) { return (n + 255) & ~(int64_t)255; }
 
 // workspace layout for B rows
 struct StepBuffers {
-  char *x, *q, *h, *o, *u, *part, *positions, *step_len, *select_ws;
+  char *x, *q, *h, *o, *u, *part, *positions, *step_len, *select_ws, *attn_ws;
+  int64_t attn_keys;  // key positions per (b, h) that attn_ws holds scores for (0: none)
   int64_t bytes;
 };
+
+// most keys the split attention's score buffer is sized for
+int64_t split_attention_keys(const msa_decoder* d, int B) {
+  const int hd = d->cfg.d_model / d->cfg.heads;
+  const int64_t keys = d->cfg.n_pos_rows < 8192 ? d->cfg.n_pos_rows : 8192;
+  // the form can only ever be chosen for few (b, h) pairs; ask with the longest history
+  return msa_attention_prefers_split(B, d->cfg.heads, hd, (int)keys) ? keys : 0;
+}
 
 void pick_splits(msa_decoder* d, int B) {
   if (d->splits_rows == B) return;
@@ -61,6 +70,8 @@ StepBuffers carve(const msa_decoder* d, int B, char* base) {
   w.positions = take(B * 8);
   w.step_len = take(B * 4);
   w.select_ws = take(msa_lm_head_select_workspace_bytes(B));
+  w.attn_keys = split_attention_keys(d, B);
+  w.attn_ws = take(msa_attention_split_workspace_bytes(B, d->cfg.heads, (int)w.attn_keys));
   w.bytes = off;
   return w;
 }
@@ -158,6 +169,11 @@ extern "C" int msa_decoder_step(msa_decoder* d, const msa_step_args* a, void* st
   rc = msa_layernorm_f16(w.x, d->layers[0].ln1_gamma, d->layers[0].ln1_beta, w.h, B, D, eps, OUT,
                          stream);
   if (rc) return rc;
+  // few (b, h) pairs over a long history: the two-launch attention (same bits).  With lengths
+  // on the device S0 is the caller's bound on them if it has one (0: only the capacity is known).
+  const int keys_bound = a->len_dev && a->S0 == 0 ? a->S_cap : a->S0 + 1;
+  const bool split_attention =
+      a->S_cap <= w.attn_keys && msa_attention_prefers_split(B, H, hd, keys_bound);
   for (int i = 0; i < c.layers; ++i) {
     const msa_layer_weights& l = d->layers[i];
     void* kc = a->k_cache[i];
@@ -169,8 +185,12 @@ extern "C" int msa_decoder_step(msa_decoder* d, const msa_step_args* a, void* st
       rc = msa_qkv_proj_f16(w.h, l.qkv_weight, l.qkv_bias, w.q, kc, vc, B, 1, H, hd, a->S0,
                             a->S_cap, D, IN, len, stream);
     if (rc) return rc;
-    rc = msa_attention_f16(w.q, kc, vc, a->key_pad_mask, a->mask_stride, w.o, B, H, hd, 1, a->S0,
-                           a->S_cap, OUT, len, stream);
+    if (split_attention)
+      rc = msa_attention_split_f16(w.q, kc, vc, a->key_pad_mask, a->mask_stride, w.o, w.attn_ws, B,
+                                   H, hd, a->S0, a->S_cap, OUT, len, stream);
+    else
+      rc = msa_attention_f16(w.q, kc, vc, a->key_pad_mask, a->mask_stride, w.o, B, H, hd, 1, a->S0,
+                             a->S_cap, OUT, len, stream);
     if (rc) return rc;
     if (c.int8)
       rc = msa_linear_partial_w8a16(w.o, (const int8_t*)l.out_weight, l.out_scales,

@@ -323,3 +323,31 @@ def test_one_call_decode_step_equals_the_step_driven_entry_point_by_entry_point(
             assert torch.equal(x, y)
         assert (a[5] is None and b[5] is None) or torch.equal(a[5], b[5])
         assert a[6] == b[6]
+
+
+def test_one_call_step_with_split_attention_equals_the_one_launch_form():
+    """One request over a history of more than 4096 positions at head_dim 128:
+    msa_decoder_step takes the two-launch attention, the Python-driven step the one-launch
+    kernel; logits are bit-identical."""
+    cfg = OPTConfig(decoder_layers=2, decoder_embed_dim=256, decoder_attention_heads=2,
+                    vocab_size=512, max_target_positions=4400)
+    model, _ = build(cfg, seed=13)
+    dec = model.decoder
+    lib = dec.prepare_()
+    prompt = random_prompts(cfg, 1, 4200, seed=8).to(DEV)
+    assert lib.msa_attention_prefers_split(1, 2, 128, 4201) == 1
+    nxt = torch.randint(4, cfg.vocab_size, (1, 3), generator=torch.Generator().manual_seed(2)).to(DEV)
+    outs = []
+    for native in (True, False):
+        dec.native_step = native
+        inc = {}
+        model(prompt, incremental_state=inc)
+        toks, steps = prompt, []
+        for t in range(3):
+            toks = torch.cat([toks, nxt[:, t:t + 1]], 1)
+            steps.append(dec(toks, incremental_state=inc)[0].clone())
+        torch.cuda.synchronize()
+        outs.append(steps)
+    dec.native_step = True
+    for x, y in zip(*outs):
+        assert torch.equal(x, y)

@@ -652,6 +652,65 @@ def test_attention(lib, B, H, hd, T, S0, masked):
                       what="attention")
 
 
+@pytest.mark.parametrize("B,H,hd,S0,mode", [
+    (1, 12, 64, 1100, "plain"), (1, 12, 64, 37, "plain"), (2, 5, 128, 700, "mask"),
+    (3, 7, 128, 2049, "lens"), (2, 9, 64, 1500, "lens"), (1, 32, 128, 4, "plain"),
+    (1, 3, 128, 8191, "plain")])
+def test_split_attention_gives_the_bits_of_the_one_launch_form(lib, B, H, hd, S0, mode):
+    """msa_attention_split_f16 (scores of 8 key ranges, then one workgroup per 32-column slice)
+    forms every sum in the order of msa_attention_f16 at B*H < 512: the outputs are equal bit for
+    bit, row-major and packed, with a padding mask, with per-row lengths and an inactive row, for
+    histories shorter than one round of loads and at the 8192-key limit."""
+    print("split attention", B, H, hd, S0, mode, flush=True)
+    D = H * hd
+    S_cap = S0 + 1 + (0 if S0 + 1 == 8192 else 3)
+    q = G(rnd(B, D, seed=1, std=0.3))
+    Kc, Vc = G(rnd(B, H, S_cap, hd, seed=2)), G(rnd(B, H, S_cap, hd, seed=3))
+    dm, stride, ln = None, 0, None
+    if mode == "mask":
+        m = torch.zeros(B, S0 + 1, dtype=torch.uint8)
+        m[0, 1:40] = 1
+        m[B - 1, S0 // 2] = 1
+        dm, stride = m.to(DEV), S0 + 1
+    if mode == "lens":
+        lens = [S0, S0 // 3, -1][:B] if B >= 3 else [S0 // 2, S0]
+        ln = torch.tensor(lens, dtype=torch.int32, device=DEV)
+        for b, n in enumerate(lens):  # nothing past a row's own length may be read
+            Kc[b, :, max(n, -1) + 1:] = float("nan")
+            Vc[b, :, max(n, -1) + 1:] = float("nan")
+    ws = torch.empty(lib.msa_attention_split_workspace_bytes(B, H, S_cap), dtype=torch.uint8,
+                     device=DEV)
+    MB = (B + 15) // 16
+    for flags in (0, OUT_PACKED):
+        n_out = MB * 16 * D if flags else B * D
+        one = torch.full((n_out,), 7.0, dtype=torch.float16, device=DEV)
+        two = torch.full((n_out,), 7.0, dtype=torch.float16, device=DEV)
+        ok(lib.msa_attention_f16(P(q), P(Kc), P(Vc), P(dm), stride, P(one), B, H, hd, 1, S0, S_cap,
+                                 flags, P(ln), None), lib)
+        ok(lib.msa_attention_split_f16(P(q), P(Kc), P(Vc), P(dm), stride, P(two), P(ws), B, H, hd,
+                                       S0, S_cap, flags, P(ln), None), lib)
+        torch.cuda.synchronize()
+        assert torch.equal(one.view(torch.int16), two.view(torch.int16)), (
+            "split attention differs in %d of %d values"
+            % (int((one.view(torch.int16) != two.view(torch.int16)).sum()), n_out))
+        live = one.float()
+        assert bool(torch.isfinite(live).all())
+
+
+def test_split_attention_rejects_and_preference(lib):
+    x = torch.zeros(64, 128, dtype=torch.float16, device=DEV)
+    ws = torch.zeros(1 << 16, dtype=torch.uint8, device=DEV)
+    bad = lib.msa_attention_split_f16
+    assert bad(P(x), P(x), P(x), None, 0, P(x), None, 1, 1, 64, 0, 4, 0, None, None) == -1
+    assert bad(P(x), P(x), P(x), None, 0, P(x), P(ws), 1, 1, 96, 0, 4, 0, None, None) == -1
+    assert bad(P(x), P(x), P(x), None, 0, P(x), P(ws), 1, 1, 64, 4, 4, 0, None, None) == -2
+    assert lib.msa_attention_split_workspace_bytes(2, 3, 100) == 2 * 3 * 100 * 4
+    # very few pairs over a very long history: yes; a batch or OPT's 2048 positions: no
+    assert lib.msa_attention_prefers_split(1, 32, 128, 4097) == 1
+    assert lib.msa_attention_prefers_split(4, 32, 128, 8000) == 0
+    assert lib.msa_attention_prefers_split(1, 32, 128, 2049) == 0
+
+
 def test_attention_rejects(lib):
     x = torch.zeros(64, 96, dtype=torch.float16, device=DEV)
     assert lib.msa_attention_f16(P(x), P(x), P(x), None, 0, P(x), 1, 1, 96, 1, 0, 4, 0, None, None) == -1
