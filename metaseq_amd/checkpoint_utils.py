@@ -1,6 +1,7 @@
 """State-dict level ingest of the reference's checkpoints: gluing the tensor-parallel parts of
 a `reshard-model_part-{r}.pt` set into the single-part state dict this decoder loads, the
-inverse split, and key normalisation.
+inverse split, key normalisation, and the raw training form: FSDP shards
+(`checkpoint_last-model_part-{r}-shard{s}.pt`) whose parameters are flat, padded slices.
 
 Gluing rules (metaseq/distributed/stitch_fsdp_ckpt.py:203-214, 246-339):
 * `qkv_proj` weight and bias: every part holds its own heads as local thirds K_r | V_r | Q_r;
@@ -10,6 +11,14 @@ Gluing rules (metaseq/distributed/stitch_fsdp_ckpt.py:203-214, 246-339):
 * row-parallel `fc2` / `out_proj` weights: concatenated along dim 1, their biases replicated;
 * LayerNorms, positional table, everything else: replicated (taken from part 0; copies that
   drifted apart are reported, as the reference does, not refused).
+
+Flat FSDP shards (metaseq/scripts/reshard_fsdp.py:142-209; the same data-parallel
+consolidation metaseq/distributed/stitch_fsdp_ckpt.py:96-109 asks of fairscale): every wrapped
+module's parameters were flattened in order into one vector, cut into equal slices, one per
+data-parallel rank, the short ones padded at the end; a file's "shard_metadata" lists, per
+wrapped module, the flat vector's name and the names / shapes / element counts inside it and
+that file's padding.  Undoing it: drop each slice's padding, join the slices in shard order, cut at
+the element counts, reshape; buffers come from shard 0; shared parameters are aliases.
 
 Only tensors are read from files: `torch.load(..., weights_only=True)` executes nothing from the
 pickle, so a file whose "cfg" entry holds arbitrary Python objects is refused by the loader;
@@ -141,6 +150,103 @@ def load_model_state(paths: List[str]) -> "OrderedDict[str, torch.Tensor]":
             raise ValueError("%s does not hold a state dict of tensors" % path)
         parts.append(obj)
     return normalize_state_dict(glue_model_parts(parts) if len(parts) > 1 else parts[0])
+
+
+_WRAPPER_PREFIXES = ("_fsdp_wrapped_module.", "_fpw_module.")
+
+
+def _join(path, name):
+    full = path + "." + name if path else name
+    for w in _WRAPPER_PREFIXES:
+        full = full.replace(w, "")
+    return full
+
+
+def unflatten_fsdp_shards(shards: List[dict]) -> "OrderedDict[str, torch.Tensor]":
+    """The data-parallel shards of one model part (shard order; each
+    {"model": flat slices, "shard_metadata": ...}) -> that part's state dict with named, shaped
+    parameters.  Refuses slices whose joined length does not match the recorded element counts."""
+    if not shards:
+        raise ValueError("no shards")
+    for s in shards:
+        if "model" not in s or "shard_metadata" not in s:
+            raise ValueError("an FSDP shard holds 'model' and 'shard_metadata'")
+    layout = shards[0]["shard_metadata"]
+    out = OrderedDict()
+    for idx, group in enumerate(layout["param_metadata"]):
+        path = group["fsdp_path"]
+        for flat_name, info in group["params"].items():
+            key = path + "." + flat_name if path else flat_name
+            pieces = []
+            for r, s in enumerate(shards):
+                if key not in s["model"]:
+                    raise KeyError("shard %d holds no flat parameter %s" % (r, key))
+                piece = s["model"][key].reshape(-1)
+                pad = int(s["shard_metadata"]["param_metadata"][idx]["params"][flat_name]["padding"])
+                if pad < 0 or pad > piece.numel():
+                    raise ValueError("shard %d: padding %d of %s exceeds its %d elements"
+                                     % (r, pad, key, piece.numel()))
+                pieces.append(piece[:piece.numel() - pad])
+            flat = torch.cat(pieces)
+            numels = [int(n) for n in info["numels"]]
+            if sum(numels) != flat.numel():
+                raise ValueError("%s: shards join to %d elements, metadata lists %d"
+                                 % (key, flat.numel(), sum(numels)))
+            for name, shape, t in zip(info["names"], info["shapes"], flat.split(numels)):
+                out[_join(path, name)] = t.view(tuple(shape)).clone()
+    for src, dest in layout.get("shared_param_info", []) or []:
+        out[_join("", dest)] = out[_join("", src)]
+    for name in layout.get("buffer_names", []) or []:
+        if name not in shards[0]["model"]:
+            raise KeyError("shard 0 holds no buffer %s" % name)
+        out[_join("", name)] = shards[0]["model"][name].clone()
+    return out
+
+
+def is_flat_fsdp_shard(obj) -> bool:
+    """A raw training shard: has shard metadata and no named embedding table
+    (metaseq/distributed/stitch_fsdp_ckpt.py:84-93 tells the two forms apart the same way)."""
+    return (isinstance(obj, dict) and isinstance(obj.get("model"), dict)
+            and "shard_metadata" in obj and "decoder.embed_tokens.weight" not in obj["model"])
+
+
+def group_fsdp_files(names: List[str]) -> List[List[str]]:
+    """File names of one raw checkpoint -> [model part][shard], both in numeric order
+    (`...-model_part-{r}-shard{s}.pt`; no `model_part` in the names means one part).  Every part
+    must hold the same shard numbers 0..n-1."""
+    table = {}
+    for n in names:
+        s = re.search(r"shard(\d+)\.pt$", n)
+        if s is None:
+            raise ValueError("%s is not named ...shard<N>.pt" % n)
+        p = re.search(r"-model_part-(\d+)", n)
+        table.setdefault(int(p.group(1)) if p else 0, {})[int(s.group(1))] = n
+    parts = sorted(table)
+    if parts != list(range(len(parts))):
+        raise ValueError("model parts are not numbered 0..%d" % (len(parts) - 1))
+    width = len(table[0])
+    grouped = []
+    for r in parts:
+        if sorted(table[r]) != list(range(width)):
+            raise ValueError("model part %d does not hold shards 0..%d" % (r, width - 1))
+        grouped.append([table[r][i] for i in range(width)])
+    return grouped
+
+
+def load_fsdp_checkpoint(paths: List[str]) -> "OrderedDict[str, torch.Tensor]":
+    """Reads a raw training checkpoint (every `-model_part-{r}-shard{s}.pt` file of it, any
+    order): consolidates each part's data-parallel shards, glues the parts, normalises.  Files
+    that already hold named parameters (training without flattening) are taken as they are, one
+    per part, as metaseq/distributed/stitch_fsdp_ckpt.py:84-93,114-115 does."""
+    states = []
+    for files in group_fsdp_files(list(paths)):
+        shards = [torch.load(f, map_location="cpu", weights_only=True) for f in files]
+        if is_flat_fsdp_shard(shards[0]):
+            states.append(unflatten_fsdp_shards(shards))
+        else:
+            first = shards[0]
+            states.append(first["model"] if "model" in first else first)
+    return normalize_state_dict(glue_model_parts(states) if len(states) > 1 else states[0])
 
 
 def find_model_parts(names: List[str]) -> List[str]:

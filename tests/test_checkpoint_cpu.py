@@ -152,3 +152,137 @@ def test_load_model_state_reads_parts_from_files(tmp_path):
     torch.save({"model": {"a": 1}}, bad)
     with pytest.raises(ValueError):
         C.load_model_state([bad])
+
+
+# --- raw training checkpoints: flat, padded FSDP shards ------------------------------------
+#
+# The reference has no test or fixture for this form ("parity unpinned" by the reference); what
+# pins the consolidation is the sharding it undoes, written out here the way fairscale's FSDP
+# defines it (flatten the wrapped module's parameters in order, `chunk` over the data-parallel
+# ranks, pad every short or missing slice at the end to the first slice's length) and the
+# requirement that undoing it returns every parameter bit for bit.
+
+def _fsdp_shard(state, groups, world, buffers=(), shared=()):
+    """state dict -> `world` shard dicts.  groups: [(fsdp_path, [names relative to it])]."""
+    import torch.nn.functional as F
+    shards = [{"model": {}, "shard_metadata": {"param_metadata": [], "buffer_names": list(buffers),
+                                                "shared_param_info": list(shared)}}
+              for _ in range(world)]
+    for path, names in groups:
+        full = [(path + "." + n) if path else n for n in names]
+        flat = torch.cat([state[k].reshape(-1) for k in full])
+        chunks = list(flat.chunk(world))
+        size = chunks[0].numel()
+        key = (path + "." if path else "") + "flat_param_0"
+        for r in range(world):
+            c = chunks[r] if r < len(chunks) else flat.new_empty(0)
+            pad = size - c.numel()
+            shards[r]["model"][key] = F.pad(c, [0, pad]).clone()
+            shards[r]["shard_metadata"]["param_metadata"].append({
+                "fsdp_path": path,
+                "params": {"flat_param_0": {"names": list(names),
+                                            "shapes": [state[k].shape for k in full],
+                                            "numels": [state[k].numel() for k in full],
+                                            "padding": pad}}})
+    for r in range(world):
+        for b in buffers:
+            shards[r]["model"][b] = state[b].clone()
+    return shards
+
+
+def _fsdp_groups(state, shared=()):
+    skip = {"decoder.version"} | {d for _, d in shared}
+    groups = []
+    for i in range(L):
+        p = "decoder.layers.%d" % i
+        groups.append((p, [k[len(p) + 1:] for k in state if k.startswith(p + ".")]))
+    rest = [k for k in state if not k.startswith("decoder.layers.") and k not in skip]
+    groups.append(("", rest))
+    return groups
+
+
+@pytest.mark.parametrize("world", [1, 2, 3, 7])
+def test_flat_fsdp_shards_consolidate_to_the_sharded_state(world):
+    [sd] = _parts(1, seed=5)
+    sd["decoder.output_projection.weight"] = sd["decoder.embed_tokens.weight"]
+    shared = [("decoder.embed_tokens.weight", "decoder.output_projection.weight")]
+    shards = _fsdp_shard(sd, _fsdp_groups(sd, shared), world, buffers=["decoder.version"],
+                         shared=shared)
+    if world == 7:   # slices really are padded, and unevenly named parameters straddle them
+        assert any(g["params"]["flat_param_0"]["padding"] > 0
+                   for g in shards[-1]["shard_metadata"]["param_metadata"])
+    back = C.unflatten_fsdp_shards(shards)
+    assert set(back) == set(sd)
+    for k in sd:
+        assert back[k].shape == sd[k].shape and torch.equal(back[k], sd[k]), k
+
+
+def test_flat_fsdp_more_ranks_than_elements_leaves_empty_all_padding_slices():
+    sd = {"a.w": torch.arange(3.0), "a.b": torch.arange(2.0) + 10}
+    shards = _fsdp_shard(sd, [("a", ["w", "b"])], 8)
+    assert shards[7]["shard_metadata"]["param_metadata"][0]["params"]["flat_param_0"]["padding"] == 1
+    back = C.unflatten_fsdp_shards(shards)
+    assert torch.equal(back["a.w"], sd["a.w"]) and torch.equal(back["a.b"], sd["a.b"])
+
+
+def test_flat_fsdp_refuses_lengths_that_do_not_add_up_and_missing_vectors():
+    sd = {"a.w": torch.arange(6.0).view(2, 3)}
+    shards = _fsdp_shard(sd, [("a", ["w"])], 2)
+    shards[1]["shard_metadata"]["param_metadata"][0]["params"]["flat_param_0"]["padding"] = 1
+    with pytest.raises(ValueError, match="join to 5 elements, metadata lists 6"):
+        C.unflatten_fsdp_shards(shards)
+    shards = _fsdp_shard(sd, [("a", ["w"])], 2)
+    del shards[1]["model"]["a.flat_param_0"]
+    with pytest.raises(KeyError, match="shard 1 holds no flat parameter"):
+        C.unflatten_fsdp_shards(shards)
+
+
+def test_wrapper_prefixes_are_dropped_from_names():
+    sd = {"m.w": torch.arange(4.0)}
+    shards = _fsdp_shard(sd, [("m", ["w"])], 2)
+    for s in shards:
+        s["shard_metadata"]["param_metadata"][0]["params"]["flat_param_0"]["names"] = [
+            "_fsdp_wrapped_module._fpw_module.w"]
+    assert list(C.unflatten_fsdp_shards(shards)) == ["m.w"]
+
+
+def test_raw_checkpoint_files_two_parts_three_shards_give_the_glued_models_logits(tmp_path):
+    """File level: `-model_part-{r}-shard{s}.pt` of two tensor-parallel parts, each cut into
+    three data-parallel shards, listed out of order -> the state dict of the glued model."""
+    parts = _parts(2, seed=9)
+    names = []
+    for r, sd in enumerate(parts):
+        for s, shard in enumerate(_fsdp_shard(sd, _fsdp_groups(sd), 3, buffers=["decoder.version"])):
+            f = tmp_path / ("checkpoint_last-model_part-%d-shard%d.pt" % (r, s))
+            torch.save(shard, f)
+            names.append(str(f))
+    loaded = C.load_fsdp_checkpoint(names[::-1])
+    glued = C.normalize_state_dict(C.glue_model_parts(parts))
+    assert set(loaded) == set(glued)
+    for k in glued:
+        assert torch.equal(loaded[k], glued[k]), k
+    assert torch.allclose(_single_logits(loaded, TOKENS), tp_forward(parts, TOKENS, H), atol=1e-5)
+
+
+def test_raw_checkpoint_grouping_checks_numbering(tmp_path):
+    assert C.group_fsdp_files(["c-shard1.pt", "c-shard0.pt", "c-shard10.pt"][:2]) == [
+        ["c-shard0.pt", "c-shard1.pt"]]
+    with pytest.raises(ValueError, match="does not hold shards"):
+        C.group_fsdp_files(["c-model_part-0-shard0.pt", "c-model_part-0-shard1.pt",
+                            "c-model_part-1-shard0.pt", "c-model_part-1-shard2.pt"])
+    with pytest.raises(ValueError, match="not numbered"):
+        C.group_fsdp_files(["c-model_part-1-shard0.pt"])
+    with pytest.raises(ValueError, match="not named"):
+        C.group_fsdp_files(["reshard-model_part-0.pt"])
+
+
+def test_unflattened_training_files_are_taken_as_they_are(tmp_path):
+    parts = _parts(2, seed=11)
+    names = []
+    for r, sd in enumerate(parts):
+        f = tmp_path / ("checkpoint_last-model_part-%d-shard0.pt" % r)
+        torch.save({"model": sd, "shard_metadata": {"param_metadata": []}}, f)
+        names.append(str(f))
+    loaded = C.load_fsdp_checkpoint(names)
+    glued = C.normalize_state_dict(C.glue_model_parts(parts))
+    assert all(torch.equal(loaded[k], glued[k]) for k in glued)
