@@ -824,12 +824,16 @@ __global__ __launch_bounds__(TL_THREADS) void linear_tiled_kernel(
 // features (two weight tiles) for all 256 activation rows.  Weight fragments come straight from
 // the packed layout in global memory into registers (one KB per wave instruction, no LDS round
 // trip, no two waves read the same weights); only the row-major activations are staged through
-// LDS, double buffered, one barrier per 64-wide K stage.  The stage is software pipelined by
+// LDS, double buffered, one barrier per 64-wide K stage.  A staged row is 128 bytes, unpadded, and
+// its eight 16-byte chunks are stored XOR-swizzled by (row / 2) % 8: this part's LDS serves 256
+// bytes per clock only when the 16 lanes it takes together hit 16 different 16-byte bank groups,
+// which rows padded to 144 bytes do not (measured: 128 bytes per clock, i.e. the fragment reads of a
+// stage alone took as long as its MFMAs).  The stage is software pipelined by
 // hand: activations are fetched two stages ahead and parked in LDS one stage ahead, weights
 // are fetched one stage ahead, LDS fragment reads run TB_PD fragments ahead of the MFMAs, and
 // sched_group_barrier pins that order.  The main loop is branch free: rows and tiles past the
 // edge read clamped addresses and are dropped in the epilogue.  Needs K % 128 == 0.
-constexpr int TB_BM = 256, TB_BN = 256, TB_BK = 64, TB_LD = TB_BK + 8, TB_THREADS = 512;
+constexpr int TB_BM = 256, TB_BN = 256, TB_BK = 64, TB_LD = TB_BK, TB_THREADS = 512;
 constexpr int TB_MF = TB_BM / 16;       // activation fragments per wave and 32-wide step
 constexpr int TB_NT = TB_BN / 8 / 16;   // weight tiles per wave
 constexpr int TB_PD = 4;                // LDS fragment reads in flight
@@ -861,7 +865,7 @@ __global__ __launch_bounds__(TB_THREADS) void linear_tiled_big_kernel(
     const int row = c >> 3, ch = c & 7;
     const int64_t m = min(m0 + row, M - 1);
     xsrc[i] = x + m * K + ch * 8;
-    xdst[i] = row * TB_LD + ch * 8;
+    xdst[i] = row * TB_LD + ((ch ^ ((row >> 1) & 7)) * 8);
   }
   const char* wsrc[TB_NT];
   half_t wscale[TB_NT];
@@ -903,8 +907,16 @@ __global__ __launch_bounds__(TB_THREADS) void linear_tiled_big_kernel(
     for (int b = 0; b < TB_NT; ++b) acc[a][b] = float4_t{0.f, 0.f, 0.f, 0.f};
 
   auto compute = [&](const BigW<W8>& w, int buf) {
-    const half_t* l = lx_big + buf * (TB_BM * TB_LD) + lr * TB_LD + lg * 8;
-    constexpr int F = 2 * TB_MF;  // fragment f = 32-wide step f / TB_MF, row block f % TB_MF
+    // fragment f = 32-wide step f / TB_MF, row block f % TB_MF: chunk 4 * step + lg of row
+    // 16 * block + lr, whose swizzle is (lr / 2) % 8 for every block
+    const half_t* lb = lx_big + buf * (TB_BM * TB_LD) + lr * TB_LD;
+    const int sw = (lr >> 1) & 7;
+    const half_t* l0 = lb + ((lg ^ sw) * 8);
+    const half_t* l1 = lb + ((lg ^ sw ^ 4) * 8);
+    auto frag = [&](int f) {
+      return *reinterpret_cast<const half8_t*>((f / TB_MF ? l1 : l0) + (f % TB_MF) * 16 * TB_LD);
+    };
+    constexpr int F = 2 * TB_MF;
     half8_t a[2][TB_NT];
 #pragma unroll
     for (int ks = 0; ks < 2; ++ks)
@@ -920,7 +932,7 @@ __global__ __launch_bounds__(TB_THREADS) void linear_tiled_big_kernel(
     half8_t bx[TB_PD];
 #pragma unroll
     for (int p = 0; p < TB_PD; ++p)
-      bx[p] = *reinterpret_cast<const half8_t*>(l + (p % TB_MF) * 16 * TB_LD + (p / TB_MF) * 32);
+      bx[p] = frag(p);
     __builtin_amdgcn_sched_group_barrier(0x200, 4, 0);                         // LDS stores
     __builtin_amdgcn_sched_group_barrier(0x020, 4 + (W8 ? 1 : 2) * TB_NT, 0);  // global loads
     __builtin_amdgcn_sched_group_barrier(0x100, TB_PD, 0);                     // leading LDS reads
@@ -933,9 +945,7 @@ __global__ __launch_bounds__(TB_THREADS) void linear_tiled_big_kernel(
         acc[mf][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[ks][j], cur, acc[mf][j], 0, 0, 0);
       __builtin_amdgcn_sched_group_barrier(0x008, TB_NT, 0);
       if (f + TB_PD < F) {
-        const int g = f + TB_PD;
-        bx[f % TB_PD] =
-            *reinterpret_cast<const half8_t*>(l + (g % TB_MF) * 16 * TB_LD + (g / TB_MF) * 32);
+        bx[f % TB_PD] = frag(f + TB_PD);
         __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
       }
     }
