@@ -6,6 +6,14 @@
 // softmax statistics (QK^T only), pass 2 recomputing the same scores (bit-identical MFMAs)
 // and accumulating P*V.  QK^T runs twice, 1.5x the MFMA work of one-pass flash attention.
 //
+// Query tiles are aligned to the END of the new positions: a ragged tile (T % 128 queries) comes
+// first, where it sees the fewest keys (a prompt of 2^k tokens plus the leading EOS would
+// otherwise spend a whole extra sweep over all keys on its single last query).
+//
+// Scores are kept as packed fp16 pairs (they are fp16 values at this point of the reference);
+// the softmax reads them through mixed-precision FMAs: exp(s - m) / l is evaluated as
+// exp2(s * log2(e) - (m * log2(e) + log2(l))), one FMA and one exp2 per element.
+//
 // Workgroup = 128 queries of one (batch row, head); 4 waves x 32 queries.  Everything is kept
 // transposed so that softmax rows live in lanes: S^T = K * Q^T puts query j = lane & 31 in each
 // lane with 16 keys in registers (plus the other half-wave), which is already the B-operand
@@ -41,11 +49,12 @@ __global__ __launch_bounds__(PF_THREADS) void prefill_attention_kernel(
   const int D = H * HD;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int j = lane & 31, hl = lane >> 5;
-  const int q0 = qt * PF_BM + wave * 32;  // first query of this wave
-  const int tq = q0 + j;                  // this lane's query
-  const int tqc = tq < T ? tq : T - 1;
-  const int pq = S0 + tq;                 // its position = last key it may see
-  const int wg_last_q = min(T, qt * PF_BM + PF_BM) - 1;
+  const int lead = (PF_BM - T % PF_BM) % PF_BM;   // queries missing from the first tile
+  const int q0 = qt * PF_BM - lead + wave * 32;   // first query of this wave (may be negative)
+  const int tq = q0 + j;                          // this lane's query
+  const int tqc = tq < 0 ? 0 : tq;                // lanes before the first query repeat query 0
+  const int pq = S0 + tqc;                        // its position = last key it may see
+  const int wg_last_q = qt * PF_BM - lead + PF_BM - 1;
   const int n_keys = S0 + wg_last_q + 1;  // keys this workgroup needs
   const int ntiles = (n_keys + PF_BN - 1) / PF_BN;
   const half_t* kbase = Kc + (int64_t)bh * S_cap * HD;
@@ -112,34 +121,50 @@ __global__ __launch_bounds__(PF_THREADS) void prefill_attention_kernel(
     }
   };
 
-  // S^T tile of this wave: 64 keys x 32 queries = 2 accumulators; rounded to fp16 and masked
-  float16_t s[2];
+  // S^T tile of this wave: 64 keys x 32 queries = 2 accumulators, rounded to fp16, masked and kept
+  // as packed pairs: pair v2 of block ib holds keys 32*ib + 8*(v2/2) + 4*hl + 2*(v2%2) + {0, 1}
+  constexpr float LOG2E = 1.4426950408889634f;
+  const float16_t zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  half2_t sh[2][8];
   auto scores = [&](int tile) {
+    float16_t s[2];
+    // the two key blocks alternate so that no MFMA waits for the one just issued; the first
+    // step takes a literal zero as its addend (no accumulator clearing)
 #pragma unroll
-    for (int ib = 0; ib < 2; ++ib) {
+    for (int ks = 0; ks < KSTEPS; ++ks) {
 #pragma unroll
-      for (int v = 0; v < 16; ++v) s[ib][v] = 0.f;
-#pragma unroll
-      for (int ks = 0; ks < KSTEPS; ++ks) {
+      for (int ib = 0; ib < 2; ++ib) {
         const half8_t a =
             *reinterpret_cast<const half8_t*>(&lk[(ib * 32 + j) * KLD + ks * 16 + hl * 8]);
-        s[ib] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, qf[ks], s[ib], 0, 0, 0);
+        s[ib] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, qf[ks], ks == 0 ? zero16 : s[ib], 0, 0, 0);
       }
     }
-    const int kt0 = tile * PF_BN;
-    const bool need_mask = (kt0 + PF_BN - 1 > S0 + q0) || mrow != nullptr;  // wave-uniform
 #pragma unroll
     for (int ib = 0; ib < 2; ++ib)
 #pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        float x = round_h(s[ib][v]);
-        if (need_mask) {
+      for (int v2 = 0; v2 < 8; ++v2)
+        sh[ib][v2] = half2_t{(half_t)s[ib][2 * v2], (half_t)s[ib][2 * v2 + 1]};
+    const int kt0 = tile * PF_BN;
+    if (kt0 + PF_BN - 1 > S0 + max(q0, 0)) {  // wave-uniform: the tile reaches past a query's position
+#pragma unroll
+      for (int ib = 0; ib < 2; ++ib)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
           const int key = kt0 + ib * 32 + 8 * (v >> 2) + 4 * hl + (v & 3);
-          if (key > pq || (mrow && mrow[key < n_keys ? key : n_keys - 1])) x = -INFINITY;
+          if (key > pq) sh[ib][v >> 1][v & 1] = (half_t)(-INFINITY);
         }
-        s[ib][v] = x;
-      }
+    }
+    if (mrow != nullptr) {  // uniform: padded keys
+#pragma unroll
+      for (int ib = 0; ib < 2; ++ib)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          const int key = kt0 + ib * 32 + 8 * (v >> 2) + 4 * hl + (v & 3);
+          if (mrow[key < n_keys ? key : n_keys - 1]) sh[ib][v >> 1][v & 1] = (half_t)(-INFINITY);
+        }
+    }
   };
+  auto xor32 = [&](float v) { return __shfl_xor(v, 32, MSA_WAVE); };
 
   // ---------------- pass 1: row maximum and sum of exp ----------------
   float m = -INFINITY, l = 0.f;
@@ -150,25 +175,31 @@ __global__ __launch_bounds__(PF_THREADS) void prefill_attention_kernel(
     __syncthreads();
     if (tile + 1 < ntiles) load_k(tile + 1);  // the branch also pins the loads ahead of the MFMAs
     scores(tile);
-    float tm = -INFINITY;
+    half2_t t2 = sh[0][0];
 #pragma unroll
     for (int ib = 0; ib < 2; ++ib)
 #pragma unroll
-      for (int v = 0; v < 16; ++v) tm = fmaxf(tm, s[ib][v]);
-    tm = fmaxf(tm, __shfl_xor(tm, 32, MSA_WAVE));
+      for (int v2 = 0; v2 < 8; ++v2) t2 = __builtin_elementwise_max(t2, sh[ib][v2]);
+    float tm = fmaxf((float)t2[0], (float)t2[1]);
+    tm = fmaxf(tm, xor32(tm));
     if (tm > -INFINITY) {
       const float mn = fmaxf(m, tm);
+      const float c = mn * LOG2E;
       float ts = 0.f;
 #pragma unroll
       for (int ib = 0; ib < 2; ++ib)
 #pragma unroll
-        for (int v = 0; v < 16; ++v) ts += __expf(s[ib][v] - mn);  // -inf - finite = -inf -> 0
-      ts += __shfl_xor(ts, 32, MSA_WAVE);
-      l = l * __expf(m - mn) + ts;
+        for (int v2 = 0; v2 < 8; ++v2) {  // exp(s - mn); -inf gives 0
+          ts += __builtin_amdgcn_exp2f(__builtin_fmaf((float)sh[ib][v2][0], LOG2E, -c));
+          ts += __builtin_amdgcn_exp2f(__builtin_fmaf((float)sh[ib][v2][1], LOG2E, -c));
+        }
+      ts += xor32(ts);
+      l = l * __builtin_amdgcn_exp2f(m * LOG2E - c) + ts;
       m = mn;
     }
   }
-  const float inv_l = 1.0f / l;
+  // exp(s - m) / l = exp2(s * log2(e) - c2)
+  const float c2 = m * LOG2E + __builtin_amdgcn_logf(l);
 
   // ---------------- pass 2: O^T += V^T * P^T ----------------
   float16_t o[DBLK];
@@ -189,15 +220,18 @@ __global__ __launch_bounds__(PF_THREADS) void prefill_attention_kernel(
     }
     scores(tile);
     // k step c of S^T block ib covers keys 32*ib + 16*c + {4*hl + 0..3, 8 + 4*hl + 0..3}:
-    // exactly registers 8c .. 8c+7 of this lane, i.e. P^T is already a B operand
+    // exactly pairs 4c .. 4c+3 of this lane, i.e. P^T is already a B operand
 #pragma unroll
     for (int ib = 0; ib < 2; ++ib)
 #pragma unroll
       for (int c = 0; c < 2; ++c) {
         half8_t p;
 #pragma unroll
-        for (int e = 0; e < 8; ++e)
-          p[e] = (half_t)(__expf(s[ib][8 * c + e] - m) * inv_l);
+        for (int e = 0; e < 4; ++e) {
+          const half2_t h = sh[ib][4 * c + e];
+          p[2 * e] = (half_t)__builtin_amdgcn_exp2f(__builtin_fmaf((float)h[0], LOG2E, -c2));
+          p[2 * e + 1] = (half_t)__builtin_amdgcn_exp2f(__builtin_fmaf((float)h[1], LOG2E, -c2));
+        }
         const int kp = (ib * 32 + c * 16 + 4 * hl) >> 1;  // first key pair of this lane's group
 #pragma unroll
         for (int db = 0; db < DBLK; ++db) {
@@ -214,7 +248,7 @@ __global__ __launch_bounds__(PF_THREADS) void prefill_attention_kernel(
       }
   }
   // O^T accumulator: lane holds query j and d = 32*db + 8*blk + 4*hl + r
-  if (tq < T) {
+  if (tq >= 0) {
     half_t* orow = out + ((int64_t)b * T + tq) * D + h * HD;
 #pragma unroll
     for (int db = 0; db < DBLK; ++db)

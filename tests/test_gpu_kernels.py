@@ -611,6 +611,9 @@ def _oracle_core(dtype=torch.float16):
     (32, 12, 64, 1, 65, False), (2, 2, 128, 9, 0, False), (2, 2, 64, 33, 0, True),
     (1, 4, 128, 130, 0, False), (8, 32, 64, 1, 513, False), (2, 2, 64, 5, 11, False),
     (2, 3, 128, 257, 0, True), (1, 2, 64, 200, 56, False), (3, 1, 128, 129, 127, True),
+    # query tiles are aligned to the end: exact multiples, one query over, one query short
+    (1, 2, 128, 128, 0, False), (1, 1, 128, 1025, 0, False), (2, 1, 64, 127, 3, True),
+    (1, 2, 64, 384, 130, False),
 ])
 def test_attention(lib, B, H, hd, T, S0, masked):
     print("attention", B, H, hd, T, S0, masked, flush=True)
