@@ -185,14 +185,15 @@ __global__ __launch_bounds__(PF_THREADS) void prefill_attention_kernel(
     if (tm > -INFINITY) {
       const float mn = fmaxf(m, tm);
       const float c = mn * LOG2E;
-      float ts = 0.f;
+      float t4[4] = {0.f, 0.f, 0.f, 0.f};  // four chains: the adds do not wait for each other
 #pragma unroll
       for (int ib = 0; ib < 2; ++ib)
 #pragma unroll
         for (int v2 = 0; v2 < 8; ++v2) {  // exp(s - mn); -inf gives 0
-          ts += __builtin_amdgcn_exp2f(__builtin_fmaf((float)sh[ib][v2][0], LOG2E, -c));
-          ts += __builtin_amdgcn_exp2f(__builtin_fmaf((float)sh[ib][v2][1], LOG2E, -c));
+          t4[(2 * v2) & 3] += __builtin_amdgcn_exp2f(__builtin_fmaf((float)sh[ib][v2][0], LOG2E, -c));
+          t4[(2 * v2 + 1) & 3] += __builtin_amdgcn_exp2f(__builtin_fmaf((float)sh[ib][v2][1], LOG2E, -c));
         }
+      float ts = (t4[0] + t4[1]) + (t4[2] + t4[3]);
       ts += xor32(ts);
       l = l * __builtin_amdgcn_exp2f(m * LOG2E - c) + ts;
       m = mn;

@@ -17,6 +17,12 @@ FLAGS = [
 ]
 
 
+# per-source extras.  The prefill attention kernel keeps its MFMA results in ordinary vector
+# registers (its softmax reads every score; by default hipcc parks them in the accumulator bank
+# and copies each one out)
+EXTRA_FLAGS = {"attention_prefill.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"]}
+
+
 def _hipcc():
     for c in (os.environ.get("HIPCC"), "/opt/rocm/bin/hipcc", "hipcc"):
         if c and (os.path.sep not in c or os.path.exists(c)):
@@ -42,7 +48,7 @@ def build(force=True, verbose=True):
 
     def compile_one(src):
         obj = os.path.join(objdir, src.replace(".hip", ".o"))
-        cmd = [hipcc] + FLAGS + ["-c", os.path.join(HERE, src), "-o", obj]
+        cmd = [hipcc] + FLAGS + EXTRA_FLAGS.get(src, []) + ["-c", os.path.join(HERE, src), "-o", obj]
         r = subprocess.run(cmd, capture_output=True, text=True)
         err = "\n".join(l for l in r.stderr.splitlines()
                         if "packed-fp32-ops" not in l)  # host pass does not know the feature
