@@ -18,9 +18,8 @@
 // transposed so that softmax rows live in lanes: S^T = K * Q^T puts query j = lane & 31 in each
 // lane with 16 keys in registers (plus the other half-wave), which is already the B-operand
 // layout of O^T = V^T * P^T.  K tiles are staged row-major in LDS (A operand: 8 consecutive d
-// per lane); V tiles are staged by key quads ([key/4][d][4 keys]) so that the A operand of the
-// second product (8 keys of one d: two quads) is two conflict-free 64-bit LDS reads that land in
-// consecutive registers.
+// per lane); V tiles are staged with key pairs interleaved ([key/2][d][2]) so that the A
+// operand of the second product (8 keys of one d) is four conflict-free 32-bit LDS reads.
 #include <math.h>
 
 #include "common.h"
@@ -39,11 +38,10 @@ __global__ __launch_bounds__(PF_THREADS) void prefill_attention_kernel(
   constexpr int KSTEPS = HD / 16;  // MFMA k steps over the head dimension
   constexpr int DBLK = HD / 32;    // 32-row blocks of O^T
   constexpr int KLD = HD + 8;      // K tile row stride (halves)
-  constexpr int QLD = HD + 4;      // V tile stride between key quads (64-bit words, one = 4 keys of a d)
-  constexpr int VQ = (PF_BN / 4) * (HD / 8);  // staging pieces of a V tile: 4 keys x 8 d each
+  constexpr int VLD = HD + 16;     // V tile row stride (32-bit words, one word = a key pair)
   constexpr int PIECES = PF_BN * HD / 8 / PF_THREADS;  // 16-byte pieces per thread and tile
   __shared__ __attribute__((aligned(16))) half_t lk[PF_BN * KLD];
-  __shared__ __attribute__((aligned(16))) uint2 lv[(PF_BN / 4) * QLD];
+  __shared__ __attribute__((aligned(16))) uint32_t lv[(PF_BN / 2) * VLD];
 
   // query tiles are issued last-first: the tiles with the most keys start earliest
   const int bh = blockIdx.x, qt = gridDim.y - 1 - blockIdx.y;
@@ -75,7 +73,7 @@ __global__ __launch_bounds__(PF_THREADS) void prefill_attention_kernel(
   // staging: piece c = tid + 256*i of a tile: key c / (HD/8), d offset 8*(c % (HD/8)).
   // V pieces are taken as key pairs: pair p = c / (HD/8) (c < PF_BN/2 * HD/8 per half), so a
   // thread loads the same d range of keys 2p and 2p+1 and writes them interleaved.
-  half8_t rk[PIECES];
+  half8_t rk[PIECES], rv[PIECES];
   auto load_k = [&](int tile) {
 #pragma unroll
     for (int i = 0; i < PIECES; ++i) {
@@ -92,32 +90,34 @@ __global__ __launch_bounds__(PF_THREADS) void prefill_attention_kernel(
       *reinterpret_cast<half8_t*>(&lk[(c / (HD / 8)) * KLD + (c % (HD / 8)) * 8]) = rk[i];
     }
   };
-  // V: piece tid (of VQ) = key quad tid / (HD/8), d offset 8 * (tid % (HD/8)): four 16-byte loads
-  // (the same 8 d of 4 consecutive keys), stored as 8 quads = 64 contiguous bytes
-  half8_t rv[4];
+  // V: PIECES/2 pairs per thread; pair index pc = tid + 256*i, key pair pc / (HD/8)
   auto load_v = [&](int tile) {
-    if (tid < VQ) {
-      const int kq = tid / (HD / 8), dcol = (tid % (HD / 8)) * 8;
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        int key = tile * PF_BN + 4 * kq + r;
-        if (key >= n_keys) key = n_keys - 1;
-        rv[r] = *reinterpret_cast<const half8_t*>(vbase + (int64_t)key * HD + dcol);
-      }
+    for (int i = 0; i < PIECES / 2; ++i) {
+      const int pc = tid + PF_THREADS * i;
+      const int kp = pc / (HD / 8), dcol = (pc % (HD / 8)) * 8;
+      int k0 = tile * PF_BN + 2 * kp, k1 = k0 + 1;
+      if (k0 >= n_keys) k0 = n_keys - 1;
+      if (k1 >= n_keys) k1 = n_keys - 1;
+      rv[2 * i] = *reinterpret_cast<const half8_t*>(vbase + (int64_t)k0 * HD + dcol);
+      rv[2 * i + 1] = *reinterpret_cast<const half8_t*>(vbase + (int64_t)k1 * HD + dcol);
     }
   };
   auto store_v = [&]() {
-    if (tid < VQ) {
-      const int kq = tid / (HD / 8), dcol = (tid % (HD / 8)) * 8;
 #pragma unroll
-      for (int e2 = 0; e2 < 4; ++e2) {  // two d per 16-byte store
-        half8_t w;
+    for (int i = 0; i < PIECES / 2; ++i) {
+      const int pc = tid + PF_THREADS * i;
+      const int kp = pc / (HD / 8), dcol = (pc % (HD / 8)) * 8;
+      half8_t lo, hi;  // words d..d+3 and d+4..d+7, each word = (key 2p, key 2p+1)
 #pragma unroll
-        for (int h = 0; h < 2; ++h)
-#pragma unroll
-          for (int r = 0; r < 4; ++r) w[4 * h + r] = rv[r][2 * e2 + h];
-        *reinterpret_cast<half8_t*>(&lv[kq * QLD + dcol + 2 * e2]) = w;
+      for (int e = 0; e < 4; ++e) {
+        lo[2 * e] = rv[2 * i][e];
+        lo[2 * e + 1] = rv[2 * i + 1][e];
+        hi[2 * e] = rv[2 * i][4 + e];
+        hi[2 * e + 1] = rv[2 * i + 1][4 + e];
       }
+      *reinterpret_cast<half8_t*>(&lv[kp * VLD + dcol]) = lo;
+      *reinterpret_cast<half8_t*>(&lv[kp * VLD + dcol + 4]) = hi;
     }
   };
 
@@ -233,13 +233,16 @@ __global__ __launch_bounds__(PF_THREADS) void prefill_attention_kernel(
           p[2 * e] = (half_t)__builtin_amdgcn_exp2f(__builtin_fmaf((float)h[0], LOG2E, -c2));
           p[2 * e + 1] = (half_t)__builtin_amdgcn_exp2f(__builtin_fmaf((float)h[1], LOG2E, -c2));
         }
-        const int q4 = ib * 8 + c * 4 + hl;  // key quad of this lane's first four keys; the other is q4 + 2
+        const int kp = (ib * 32 + c * 16 + 4 * hl) >> 1;  // first key pair of this lane's group
 #pragma unroll
         for (int db = 0; db < DBLK; ++db) {
           const int d = db * 32 + j;
-          const uint2 lo = lv[q4 * QLD + d], hi = lv[(q4 + 2) * QLD + d];
           typedef uint32_t u4 __attribute__((ext_vector_type(4)));
-          const u4 w = {lo.x, lo.y, hi.x, hi.y};
+          u4 w;
+          w[0] = lv[(kp + 0) * VLD + d];
+          w[1] = lv[(kp + 1) * VLD + d];
+          w[2] = lv[(kp + 4) * VLD + d];
+          w[3] = lv[(kp + 5) * VLD + d];
           o[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, w), p, o[db],
                                                          0, 0, 0);
         }
