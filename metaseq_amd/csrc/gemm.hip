@@ -25,6 +25,7 @@
 #include <math.h>
 
 #include <atomic>
+#include <type_traits>
 #include <mutex>
 
 #include "common.h"
@@ -986,6 +987,196 @@ __global__ __launch_bounds__(TB_THREADS) void linear_tiled_big_kernel(
   }
 }
 
+// ---- large tiled kernel, fp16 weights: four waves of 128 x 128 ---------------------------------
+// 256 x 256 per workgroup of 4 waves (2 x 2), one wave per SIMD, each wave 128 rows x 128 features
+// on v_mfma_f32_16x16x32_f16: 64 accumulator tiles = 256 registers, kept in the AGPR bank.  hipcc
+// copies such accumulators in and out of the bank around every MFMA, so the MFMAs are issued from
+// inline assembly with the accumulator tied in place ("+a").  Both operands go global -> LDS
+// directly (global_load_lds_dwordx4: LDS address = M0 + 16 * lane, the lane's global address is
+// free), so no load ever targets a register and the only hand-placed waits are the vmcnt before
+// each barrier:
+//   * activations in 64-wide stages (whole 128-byte lines), rows unpadded with their eight 16-byte
+//     chunks XOR-swizzled by (row / 2) % 8, ring of 3 x 32 KB;
+//   * weights in 32-wide steps, the packed 16 x 32 blocks as they lie in memory (lane order, so the
+//     fragment reads are linear), ring of 3 x 16 KB.
+// One barrier per 32-wide step.  Behind the barrier of step t the weights of step t+1 (and, every
+// other step, the activations of the next stage) are complete and the buffers of step t are free:
+// the loads of step t+3 / stage S+2 are issued there, one between every few MFMAs, and the 16
+// fragments of step t+1 are read under the 64 MFMAs of step t (one ds_read_b128 per 4 MFMAs, a
+// quarter of the LDS traffic per MFMA of the 8-wave kernel above).  Nothing else sits between two
+// MFMAs: scalar bases are loop invariant, the lane offsets advance by a constant per step.
+// Workgroup -> tile: consecutive workgroups land on consecutive XCDs; where the default order would
+// give an XCD a long thin strip of a round's tiles, the 256 tiles of a round are regrouped so that
+// every XCD's L2 serves a compact a x b block (rm_a, rm_b, rm_r from the host).
+// Needs K % 64 == 0, K >= 128, M >= 256 (a ragged last row tile is moved up to end at M and stores
+// only the rows no other tile owns).
+constexpr int TQ_BM = 256, TQ_BN = 256, TQ_THREADS = 256;
+constexpr int TQ_RX = 3, TQ_RW = 3;
+constexpr int TQ_XBYTES = TQ_BM * 64 * 2;       // one 64-wide stage of activations
+constexpr int TQ_WBYTES = (TQ_BN / 16) * 1024;  // one 32-wide step of weights
+constexpr int TQ_WOFF = TQ_RX * TQ_XBYTES;
+constexpr int TQ_LDS_BYTES = TQ_RX * TQ_XBYTES + TQ_RW * TQ_WBYTES;  // 144 KB
+typedef __attribute__((address_space(3))) void tq_lds_void;
+
+#define TQ_MFMA(ACC, A, B) \
+  asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(ACC) : "v"(A), "v"(B))
+#define TQ_LOAD_LDS(VOFF, SBASE, LDSADDR)                                   \
+  asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(VOFF), \
+               "s"(SBASE), "s"(LDSADDR)                                     \
+               : "memory", "m0")
+
+template <int MODE>
+__global__ __launch_bounds__(TQ_THREADS) void linear_quad_kernel(
+    const half_t* __restrict__ x, const void* __restrict__ Wp, int64_t M, int N, int K,
+    int rm_a, int rm_b, int rm_r, Epilogue epi) {
+  extern __shared__ __attribute__((aligned(16))) char tq_lds[];
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int lr = lane & 15, lg = lane >> 4;
+  const int wm = wave >> 1, wn = wave & 1;
+  int bx = blockIdx.x, by = blockIdx.y;
+  if (rm_a > 0) {
+    const int ncol = gridDim.x, L = by * ncol + bx, round = L >> 8, i = L & 255;
+    if ((round + 1) * rm_r <= (int)gridDim.y) {  // a full round of 256 tiles
+      const int xcd = i & 7, k = i >> 3, gx = ncol / rm_a;
+      bx = (xcd % gx) * rm_a + k % rm_a;
+      by = round * rm_r + (xcd / gx) * rm_b + k / rm_a;
+    }
+  }
+  const int64_t m_own = (int64_t)by * TQ_BM;  // first row this tile owns
+  const int64_t m0 = m_own + TQ_BM > M ? M - TQ_BM : m_own;
+  const int n0 = bx * TQ_BN;
+  const int nst = K / 64, nks = K / 32;
+  const int ntiles = N / 16;
+
+  // direct loads.  Activations, per stage: instruction i (0..7) of the wave fills rows
+  // 64 * wave + 8 * i .. + 7 (lane l: row l / 8, chunk position l % 8, which must hold chunk
+  // (l % 8) ^ ((row / 2) % 8) = (l % 8) ^ (4 * (i % 2) + l / 16)).  Weights, per step: the wave
+  // copies the blocks of tiles 4 * wave .. 4 * wave + 3.
+  const char* xb[8];
+  const char* wb[4];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) xb[i] = (const char*)(x + (m0 + wave * 64 + i * 8) * K);
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int tt = min(n0 / 16 + wave * 4 + j, ntiles - 1);
+    wb[j] = (const char*)Wp + (int64_t)tt * K * 32;
+  }
+  const uint32_t xrow = (uint32_t)(lane >> 3) * (uint32_t)K * 2;
+  const uint32_t xlane0 = xrow + (((lane & 7) ^ (lane >> 4)) * 16);
+  const uint32_t xlane1 = xrow + (((lane & 7) ^ (4 + (lane >> 4))) * 16);
+  const uint32_t wlane = lane * 16;
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(tq_lds_void*)tq_lds;
+  auto issue_x = [&](int i, int slot, int st) {
+    st = min(st, nst - 1);
+    TQ_LOAD_LDS((i & 1 ? xlane1 : xlane0) + st * 128, xb[i],
+                lds0 + slot * TQ_XBYTES + wave * (64 * 128) + i * 1024);
+  };
+  auto issue_w = [&](int j, int slot, int ks) {
+    ks = min(ks, nks - 1);
+    TQ_LOAD_LDS(wlane + ks * 1024, wb[j], lds0 + TQ_WOFF + slot * TQ_WBYTES + wave * 4096 + j * 1024);
+  };
+
+  // fragment reads.  Activation fragment i of half h of a stage: row 128 * wm + 16 * i + lr, chunk
+  // 4 * h + lg at position (4 * h + lg) ^ ((lr / 2) % 8); weight fragment j: tile 8 * wn + j.
+  const int sw = (lr >> 1) & 7;
+  const uint32_t xoff0 = (uint32_t)(wm * 128 + lr) * 128 + ((lg ^ sw) * 16);
+  const uint32_t xoff1 = (uint32_t)(wm * 128 + lr) * 128 + ((lg ^ sw ^ 4) * 16);
+  const uint32_t woff = TQ_WOFF + (uint32_t)(wn * 8) * 1024 + lane * 16;
+  auto xfrag = [&](int slot, int h, int i) {
+    return *reinterpret_cast<const half8_t*>(tq_lds + slot * TQ_XBYTES + (h ? xoff1 : xoff0) +
+                                             i * (16 * 128));
+  };
+  auto wfrag = [&](int slot, int j) {
+    return *reinterpret_cast<const half8_t*>(tq_lds + slot * TQ_WBYTES + woff + j * 1024);
+  };
+
+  float4_t acc[8][8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      acc[i][j] = float4_t{0.f, 0.f, 0.f, 0.f};
+      asm volatile("" : "+a"(acc[i][j]));
+    }
+
+  // prologue: activation stages 0 and 1, weight steps 0, 1, 2 requested; stage 0 and step 0 landed
+  half8_t xf[2][8], wf[2][8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) issue_x(i, 0, 0);
+#pragma unroll
+  for (int j = 0; j < 4; ++j) issue_w(j, 0, 0);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) issue_x(i, 1, 1);
+#pragma unroll
+  for (int j = 0; j < 4; ++j) issue_w(j, 1, 1);
+#pragma unroll
+  for (int j = 0; j < 4; ++j) issue_w(j, 2, 2);
+  asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    xf[0][i] = xfrag(0, 0, i);
+    wf[0][i] = wfrag(0, i);
+  }
+
+  // step t = 2 S + H; xs, ws: ring slots of stage S and step t.  An even step issues 12 loads
+  // (stage S + 2, step t + 3), an odd one 4 (step t + 3); loads complete in order, so at the
+  // barrier of an even step at most the 4 loads of the step before may be outstanding for step
+  // t + 1's weights to have landed, at the barrier of an odd step the 12 of the step before.
+  auto step = [&](int t, int xs, int ws, auto hc) {
+    constexpr int H = decltype(hc)::value;
+    if (H == 0)
+      asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+    else
+      asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
+    __syncthreads();
+    const int S = t >> 1;
+    const int xfree = xs == 0 ? TQ_RX - 1 : xs - 1;  // slot of stage S - 1 = slot of stage S + 2
+    const int xnext = xs == TQ_RX - 1 ? 0 : xs + 1;  // slot of stage S + 1
+    const int wnext = ws == TQ_RW - 1 ? 0 : ws + 1;  // slot of step t + 1
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        TQ_MFMA(acc[i][j], wf[H][j], xf[H][i]);
+        if (j == 1) xf[H ^ 1][i] = H == 0 ? xfrag(xs, 1, i) : xfrag(xnext, 0, i);
+        if (j == 5) wf[H ^ 1][i] = wfrag(wnext, i);
+        if (H == 0) {
+          if (j == 3) issue_x(i, xfree, S + 2);
+          if (j == 7 && i >= 4) issue_w(i - 4, ws, t + 3);
+        } else {
+          if (j == 3 && (i & 1)) issue_w(i >> 1, ws, t + 3);
+        }
+      }
+    }
+  };
+  int xs = 0, ws = 0;
+  for (int t = 0; t < nks; t += 2) {
+    step(t, xs, ws, std::integral_constant<int, 0>{});
+    ws = ws == TQ_RW - 1 ? 0 : ws + 1;
+    step(t + 1, xs, ws, std::integral_constant<int, 1>{});
+    ws = ws == TQ_RW - 1 ? 0 : ws + 1;
+    xs = xs == TQ_RX - 1 ? 0 : xs + 1;
+  }
+  // no direct load may outlive the workgroup's LDS; the last MFMAs must have written their
+  // accumulators before these are read (the compiler does not see MFMAs inside the asm)
+  asm volatile("s_waitcnt vmcnt(0)\n\ts_nop 15\n\ts_nop 15" ::: "memory");
+
+  // D tile (i, j): lane holds activation row 128 * wm + 16 * i + lr and the 4 consecutive features
+  // 16 * (8 * wn + j) + 4 * lg ..
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int64_t m = m0 + wm * 128 + i * 16 + lr;
+    if (m < m_own) continue;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int n = n0 + wn * 128 + j * 16;
+      if (n >= N) continue;
+      epilogue4<MODE>(epi, m, n + lg * 4, acc[i][j]);
+    }
+  }
+}
+
 // ---- host side ------------------------------------------------------------------------------
 // Per-device facts are kept per device: a process may drive several GPUs, from several threads.
 constexpr int MAX_DEVICES = 64;
@@ -1141,6 +1332,36 @@ void launch_tiled(const void* x, const void* W, const void* scales, int64_t M, i
                   const Epilogue& epi, hipStream_t s) {
   // the 256 x 256 kernel once it fills the chip; the 128 x 128 one for the shapes in between
   const int64_t big_tiles = ((M + TB_BM - 1) / TB_BM) * ((N + TB_BN - 1) / TB_BN);
+  if constexpr (!W8) {
+    if (K % 64 == 0 && K >= 128 && big_tiles >= num_cus() && M >= 2 * TQ_BM) {
+      static std::atomic<uint64_t> lds_allowed_q{0};
+      if (!allow_lds((const void*)linear_quad_kernel<MODE>, TQ_LDS_BYTES, lds_allowed_q)) return;
+      // up to 128 leftover rows go through the weight-streaming kernel (see below); more than
+      // that get a last row tile moved up to end at the last row
+      int64_t M_main = M;
+      const int64_t rem = M % TQ_BM;
+      if (rem > 0 && rem <= 128) M_main = M - rem;
+      const int ncol = (N + TQ_BN - 1) / TQ_BN, nrow = (int)((M_main + TQ_BM - 1) / TQ_BM);
+      // regrouping of a round's 256 tiles: a x b per XCD with a * b = 32, (ncol / a) * (r / b) = 8
+      // for r = 256 / ncol rows per round; taken when it beats the default strip (ncol / 8) x r
+      int rm_a = 0, rm_b = 0, rm_r = 0;
+      if (ncol >= 8 && 256 % ncol == 0) {
+        const int r = 256 / ncol;
+        int best = ncol / 8 + r;
+        for (int a = 1; a <= 32; a *= 2) {
+          const int b = 32 / a;
+          if (ncol % a || r % b || (ncol / a) * (r / b) != 8) continue;
+          if (a + b < best) best = a + b, rm_a = a, rm_b = b, rm_r = r;
+        }
+      }
+      hipLaunchKernelGGL((linear_quad_kernel<MODE>), dim3(ncol, nrow), dim3(TQ_THREADS),
+                         TQ_LDS_BYTES, s, (const half_t*)x, W, M_main, N, K, rm_a, rm_b, rm_r, epi);
+      for (int64_t m0 = M_main; m0 < M; m0 += 64)
+        launch_stream<W8, MODE, true>(x, W, scales, nullptr, 1, (int)min((int64_t)64, M - m0), N,
+                                      K, epi, s, m0);
+      return;
+    }
+  }
   if (K % (2 * TB_BK) == 0 && big_tiles >= num_cus()) {
     static std::atomic<uint64_t> lds_allowed{0};  // one mask per instantiation
     if (!allow_lds((const void*)linear_tiled_big_kernel<W8, MODE>, TB_LDS_BYTES, lds_allowed))

@@ -361,6 +361,9 @@ LINEAR_SHAPES = [
     # enough 256 x 256 tiles to take the large tiled kernel, with ragged M and N edges; a bottom
     # block of at most 128 rows goes through the streaming kernel on row-major activations
     (1000, 16400, 128), (4099, 4096, 256), (1124, 16400, 128),
+    # 8 tiles across: the tiles of a full round of 256 are regrouped per XCD, those of the last,
+    # partial round (with a ragged bottom tile) are not
+    (9160, 2048, 128),
 ]
 
 
@@ -371,6 +374,18 @@ def _linear_want(x, W, b, res, relu):
     if res is not None:
         want = r16(want + res.float())
     return want
+
+
+def test_linear_f16_residual_in_place_ragged_rows(lib):
+    """y aliasing the residual on the large tiled kernel with a ragged bottom tile: the rows that
+    the moved-up last tile shares with its neighbour must be added to exactly once."""
+    M, N, K = 1000, 16384, 128
+    x, W, res = rnd(M, K, seed=7), rnd(N, K, seed=8, std=0.05), rnd(M, N, seed=10)
+    want = _linear_want(x, W, None, res, False).half()
+    y = G(res).clone()
+    ok(lib.msa_linear_f16(P(G(x)), P(pack_w(lib, G(W))), None, P(y), P(y), M, N, K, 0, None), lib)
+    torch.cuda.synchronize()
+    assert_fp16_close(y, want, atol=float(want.abs().max()) * 2 ** -10, what="in-place residual")
 
 
 @pytest.mark.parametrize("M,N,K", LINEAR_SHAPES)
