@@ -26,6 +26,7 @@
 
 #include <atomic>
 #include <type_traits>
+#include <utility>
 #include <mutex>
 
 #include "common.h"
@@ -992,38 +993,99 @@ __global__ __launch_bounds__(TB_THREADS) void linear_tiled_big_kernel(
 // on v_mfma_f32_16x16x32_f16: 64 accumulator tiles = 256 registers, kept in the AGPR bank.  hipcc
 // copies such accumulators in and out of the bank around every MFMA, so the MFMAs are issued from
 // inline assembly with the accumulator tied in place ("+a").  Both operands go global -> LDS
-// directly (global_load_lds_dwordx4: LDS address = M0 + 16 * lane, the lane's global address is
-// free), so no load ever targets a register and the only hand-placed waits are the vmcnt before
-// each barrier:
+// directly (global_load_lds_dwordx4: LDS address = M0 + instruction offset + 16 * lane, global
+// address = scalar base + lane offset + the same instruction offset), so no load ever targets a
+// register and the only hand-placed waits are the vmcnt before each barrier:
 //   * activations in 64-wide stages (whole 128-byte lines), rows unpadded with their eight 16-byte
 //     chunks XOR-swizzled by (row / 2) % 8, ring of 3 x 32 KB;
 //   * weights in 32-wide steps, the packed 16 x 32 blocks as they lie in memory (lane order, so the
-//     fragment reads are linear), ring of 3 x 16 KB.
+//     fragment reads are linear), ring of 4 x 16 KB.
+// A group of loads (the 8 of a wave's share of a stage, the 4 of its share of a step) shares one
+// M0 and one lane offset; the instruction offset picks the 1 KB piece, and the scalar bases, which
+// are loop invariant, are moved back by it.
 // One barrier per 32-wide step.  Behind the barrier of step t the weights of step t+1 (and, every
 // other step, the activations of the next stage) are complete and the buffers of step t are free:
-// the loads of step t+3 / stage S+2 are issued there, one between every few MFMAs, and the 16
+// the loads of step t+4 / stage S+2 are issued there, one between every few MFMAs, and the 16
 // fragments of step t+1 are read under the 64 MFMAs of step t (one ds_read_b128 per 4 MFMAs, a
-// quarter of the LDS traffic per MFMA of the 8-wave kernel above).  Nothing else sits between two
-// MFMAs: scalar bases are loop invariant, the lane offsets advance by a constant per step.
+// quarter of the LDS traffic per MFMA of the 8-wave kernel above).
+// Epilogue through LDS: a lane holds 4 features of 16 different rows per tile, which as stores are
+// 32-byte pieces; the rounded tile rows are parked in LDS and read back as 16 bytes per lane, whole
+// 256-byte row pieces per 16 lanes.
 // Workgroup -> tile: consecutive workgroups land on consecutive XCDs; where the default order would
 // give an XCD a long thin strip of a round's tiles, the 256 tiles of a round are regrouped so that
 // every XCD's L2 serves a compact a x b block (rm_a, rm_b, rm_r from the host).
 // Needs K % 64 == 0, K >= 128, M >= 256 (a ragged last row tile is moved up to end at M and stores
 // only the rows no other tile owns).
 constexpr int TQ_BM = 256, TQ_BN = 256, TQ_THREADS = 256;
-constexpr int TQ_RX = 3, TQ_RW = 3;
+constexpr int TQ_RX = 3, TQ_RW = 4;
 constexpr int TQ_XBYTES = TQ_BM * 64 * 2;       // one 64-wide stage of activations
 constexpr int TQ_WBYTES = (TQ_BN / 16) * 1024;  // one 32-wide step of weights
 constexpr int TQ_WOFF = TQ_RX * TQ_XBYTES;
-constexpr int TQ_LDS_BYTES = TQ_RX * TQ_XBYTES + TQ_RW * TQ_WBYTES;  // 144 KB
+constexpr int TQ_LDS_BYTES = TQ_RX * TQ_XBYTES + TQ_RW * TQ_WBYTES;  // 160 KB
 typedef __attribute__((address_space(3))) void tq_lds_void;
 
 #define TQ_MFMA(ACC, A, B) \
   asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(ACC) : "v"(A), "v"(B))
-#define TQ_LOAD_LDS(VOFF, SBASE, LDSADDR)                                   \
-  asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(VOFF), \
-               "s"(SBASE), "s"(LDSADDR)                                     \
-               : "memory", "m0")
+
+template <int... I, class F>
+__device__ __forceinline__ void tq_static_for_impl(std::integer_sequence<int, I...>, F&& f) {
+  (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, class F>
+__device__ __forceinline__ void tq_static_for(F&& f) {
+  tq_static_for_impl(std::make_integer_sequence<int, N>{}, f);
+}
+
+// 8 consecutive output columns n..n+7 of row m; v holds the accumulators rounded to fp16
+template <int MODE>
+__device__ __forceinline__ void epilogue8(const Epilogue& e, int64_t m, int n, half8_t v) {
+  float t[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) t[i] = (float)v[i];
+  if (e.bias) {
+    const half8_t b = *reinterpret_cast<const half8_t*>(e.bias + n);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) t[i] = round_h(t[i] + (float)b[i]);
+  }
+  half8_t o;
+  if (MODE == MODE_PLAIN) {
+    if (e.flags & MSA_EPI_RELU) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) t[i] = fmaxf(t[i], 0.f);
+    }
+    if (e.residual) {
+      const half8_t r = *reinterpret_cast<const half8_t*>(e.residual + m * e.N + n);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) t[i] = round_h(t[i] + (float)r[i]);
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) o[i] = (half_t)t[i];
+    if (e.out_mb > 0)
+      *reinterpret_cast<half8_t*>(e.y + packed_act_offset((int)m, n, e.out_mb)) = o;
+    else
+      *reinterpret_cast<half8_t*>(e.y + m * e.N + n) = o;
+  } else {
+    const int D = e.H * e.hd;
+    const int part = (n >= D) + (n >= 2 * D), c = n - part * D;  // 0 = K, 1 = V, 2 = Q
+    if (part == 2) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) o[i] = (half_t)(t[i] * e.qscale);
+      *reinterpret_cast<half8_t*>(e.q_out + m * D + c) = o;
+    } else {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) o[i] = (half_t)t[i];
+      const int h = e.hd_shift >= 0 ? c >> e.hd_shift : c / e.hd, d = c - h * e.hd;
+      const int mi = (int)m;
+      const int b = e.T == 1 ? mi : mi / e.T, tt = mi - b * e.T;
+      const int s0 = e.len_dev ? e.len_dev[b] : e.S0;
+      if (s0 >= 0 && s0 + tt < e.S_cap) {
+        half_t* dst = (part == 0 ? e.Kc : e.Vc) +
+                      (((int64_t)b * e.H + h) * e.S_cap + s0 + tt) * e.hd + d;
+        *reinterpret_cast<half8_t*>(dst) = o;
+      }
+    }
+  }
+}
 
 template <int MODE>
 __global__ __launch_bounds__(TQ_THREADS) void linear_quad_kernel(
@@ -1050,30 +1112,60 @@ __global__ __launch_bounds__(TQ_THREADS) void linear_quad_kernel(
 
   // direct loads.  Activations, per stage: instruction i (0..7) of the wave fills rows
   // 64 * wave + 8 * i .. + 7 (lane l: row l / 8, chunk position l % 8, which must hold chunk
-  // (l % 8) ^ ((row / 2) % 8) = (l % 8) ^ (4 * (i % 2) + l / 16)).  Weights, per step: the wave
-  // copies the blocks of tiles 4 * wave .. 4 * wave + 3.
+  // (l % 8) ^ ((row / 2) % 8) = (l % 8) ^ (4 * (i % 2) + l / 16)), with M0 at the wave's piece
+  // + 4 KB and instruction offset 1024 * (i - 4).  Weights, per step: the wave copies the blocks
+  // of tiles 4 * wave .. 4 * wave + 3, instruction offset 1024 * j.
   const char* xb[8];
   const char* wb[4];
 #pragma unroll
-  for (int i = 0; i < 8; ++i) xb[i] = (const char*)(x + (m0 + wave * 64 + i * 8) * K);
+  for (int i = 0; i < 8; ++i)
+    xb[i] = (const char*)(x + (m0 + wave * 64 + i * 8) * K) - (i - 4) * 1024;
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
     const int tt = min(n0 / 16 + wave * 4 + j, ntiles - 1);
-    wb[j] = (const char*)Wp + (int64_t)tt * K * 32;
+    wb[j] = (const char*)Wp + (int64_t)tt * K * 32 - j * 1024;
   }
   const uint32_t xrow = (uint32_t)(lane >> 3) * (uint32_t)K * 2;
   const uint32_t xlane0 = xrow + (((lane & 7) ^ (lane >> 4)) * 16);
   const uint32_t xlane1 = xrow + (((lane & 7) ^ (4 + (lane >> 4))) * 16);
   const uint32_t wlane = lane * 16;
   const uint32_t lds0 = (uint32_t)(uintptr_t)(tq_lds_void*)tq_lds;
-  auto issue_x = [&](int i, int slot, int st) {
+  uint32_t xv0 = 0, xv1 = 0, wv = 0;  // lane offsets of the group being issued
+  auto set_x = [&](int slot, int st) {
     st = min(st, nst - 1);
-    TQ_LOAD_LDS((i & 1 ? xlane1 : xlane0) + st * 128, xb[i],
-                lds0 + slot * TQ_XBYTES + wave * (64 * 128) + i * 1024);
+    xv0 = xlane0 + st * 128;
+    xv1 = xlane1 + st * 128;
+    asm volatile("s_mov_b32 m0, %0" ::"s"(lds0 + slot * TQ_XBYTES + wave * (64 * 128) + 4096)
+                 : "memory");
   };
-  auto issue_w = [&](int j, int slot, int ks) {
+  auto set_w = [&](int slot, int ks) {
     ks = min(ks, nks - 1);
-    TQ_LOAD_LDS(wlane + ks * 1024, wb[j], lds0 + TQ_WOFF + slot * TQ_WBYTES + wave * 4096 + j * 1024);
+    wv = wlane + ks * 1024;
+    asm volatile("s_mov_b32 m0, %0" ::"s"(lds0 + TQ_WOFF + slot * TQ_WBYTES + wave * 4096)
+                 : "memory");
+  };
+  auto issue_x = [&](auto ic) {
+    constexpr int i = decltype(ic)::value;
+    const uint32_t vo = i & 1 ? xv1 : xv0;
+    const char* sb = xb[i];
+    asm volatile("global_load_lds_dwordx4 %0, %1 offset:%2" ::"v"(vo), "s"(sb),
+                 "n"((i - 4) * 1024)
+                 : "memory");
+  };
+  auto issue_w = [&](auto jc) {
+    constexpr int j = decltype(jc)::value;
+    const uint32_t vo = wv;
+    const char* sb = wb[j];
+    asm volatile("global_load_lds_dwordx4 %0, %1 offset:%2" ::"v"(vo), "s"(sb), "n"(j * 1024)
+                 : "memory");
+  };
+  auto group_x = [&](int slot, int st) {
+    set_x(slot, st);
+    tq_static_for<8>([&](auto ic) { issue_x(ic); });
+  };
+  auto group_w = [&](int slot, int ks) {
+    set_w(slot, ks);
+    tq_static_for<4>([&](auto jc) { issue_w(jc); });
   };
 
   // fragment reads.  Activation fragment i of half h of a stage: row 128 * wm + 16 * i + lr, chunk
@@ -1099,19 +1191,16 @@ __global__ __launch_bounds__(TQ_THREADS) void linear_quad_kernel(
       asm volatile("" : "+a"(acc[i][j]));
     }
 
-  // prologue: activation stages 0 and 1, weight steps 0, 1, 2 requested; stage 0 and step 0 landed
+  // prologue: activation stages 0 and 1, weight steps 0..3 requested; stages 0, 1 and steps 0, 1
+  // landed
   half8_t xf[2][8], wf[2][8];
-#pragma unroll
-  for (int i = 0; i < 8; ++i) issue_x(i, 0, 0);
-#pragma unroll
-  for (int j = 0; j < 4; ++j) issue_w(j, 0, 0);
-#pragma unroll
-  for (int i = 0; i < 8; ++i) issue_x(i, 1, 1);
-#pragma unroll
-  for (int j = 0; j < 4; ++j) issue_w(j, 1, 1);
-#pragma unroll
-  for (int j = 0; j < 4; ++j) issue_w(j, 2, 2);
-  asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+  group_x(0, 0);
+  group_w(0, 0);
+  group_x(1, 1);
+  group_w(1, 1);
+  group_w(2, 2);
+  group_w(3, 3);
+  asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
   __syncthreads();
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
@@ -1120,35 +1209,37 @@ __global__ __launch_bounds__(TQ_THREADS) void linear_quad_kernel(
   }
 
   // step t = 2 S + H; xs, ws: ring slots of stage S and step t.  An even step issues 12 loads
-  // (stage S + 2, step t + 3), an odd one 4 (step t + 3); loads complete in order, so at the
-  // barrier of an even step at most the 4 loads of the step before may be outstanding for step
-  // t + 1's weights to have landed, at the barrier of an odd step the 12 of the step before.
+  // (stage S + 2, then step t + 4), an odd one 4 (step t + 4).  Loads complete in order; the
+  // weights of step t + 1 were requested in step t - 3, and the 16 loads of steps t - 2 and t - 1
+  // may still be outstanding at the barrier.  The activations an odd step starts to read (stage
+  // S + 1) were requested in step t - 3 as well.
   auto step = [&](int t, int xs, int ws, auto hc) {
     constexpr int H = decltype(hc)::value;
-    if (H == 0)
-      asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
-    else
-      asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
+    asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
     __syncthreads();
     const int S = t >> 1;
     const int xfree = xs == 0 ? TQ_RX - 1 : xs - 1;  // slot of stage S - 1 = slot of stage S + 2
     const int xnext = xs == TQ_RX - 1 ? 0 : xs + 1;  // slot of stage S + 1
     const int wnext = ws == TQ_RW - 1 ? 0 : ws + 1;  // slot of step t + 1
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
+    tq_static_for<8>([&](auto ic) {
+      constexpr int i = decltype(ic)::value;
+      tq_static_for<8>([&](auto jc) {
+        constexpr int j = decltype(jc)::value;
         TQ_MFMA(acc[i][j], wf[H][j], xf[H][i]);
         if (j == 1) xf[H ^ 1][i] = H == 0 ? xfrag(xs, 1, i) : xfrag(xnext, 0, i);
         if (j == 5) wf[H ^ 1][i] = wfrag(wnext, i);
-        if (H == 0) {
-          if (j == 3) issue_x(i, xfree, S + 2);
-          if (j == 7 && i >= 4) issue_w(i - 4, ws, t + 3);
+        if constexpr (H == 0) {  // the 8 activation loads under rows 0..3, the 4 weight loads after
+          if (i == 0 && j == 0) set_x(xfree, S + 2);
+          if constexpr (i < 4 && j == 3) issue_x(std::integral_constant<int, (i & 3) * 2>{});
+          if constexpr (i < 4 && j == 7) issue_x(std::integral_constant<int, (i & 3) * 2 + 1>{});
+          if (i == 4 && j == 0) set_w(ws, t + TQ_RW);
+          if constexpr (i >= 4 && j == 3) issue_w(std::integral_constant<int, (i & 3)>{});
         } else {
-          if (j == 3 && (i & 1)) issue_w(i >> 1, ws, t + 3);
+          if (i == 0 && j == 0) set_w(ws, t + TQ_RW);
+          if constexpr (j == 3 && (i & 1)) issue_w(std::integral_constant<int, (i >> 1)>{});
         }
-      }
-    }
+      });
+    });
   };
   int xs = 0, ws = 0;
   for (int t = 0; t < nks; t += 2) {
@@ -1158,21 +1249,35 @@ __global__ __launch_bounds__(TQ_THREADS) void linear_quad_kernel(
     ws = ws == TQ_RW - 1 ? 0 : ws + 1;
     xs = xs == TQ_RX - 1 ? 0 : xs + 1;
   }
-  // no direct load may outlive the workgroup's LDS; the last MFMAs must have written their
-  // accumulators before these are read (the compiler does not see MFMAs inside the asm)
+  // no direct load may still be in flight when the rings are reused below (or when the workgroup's
+  // LDS is released); the last MFMAs must have written their accumulators before these are read
+  // (the compiler does not see MFMAs inside the asm)
   asm volatile("s_waitcnt vmcnt(0)\n\ts_nop 15\n\ts_nop 15" ::: "memory");
+  __syncthreads();  // every wave is done with the operand rings
 
-  // D tile (i, j): lane holds activation row 128 * wm + 16 * i + lr and the 4 consecutive features
-  // 16 * (8 * wn + j) + 4 * lg ..
+  // D tile (i, j): the lane holds activation row 16 * i + lr of the wave's 128 and the 4 features
+  // 16 * j + 4 * lg ...  Per i the wave's 16 rows x 128 features (4 KB, two buffers per wave) are
+  // written as the lanes hold them (16-byte chunk 2 j + lg / 2 of the row, swizzled by the row) and
+  // read back as lane l -> row 4 r + l / 16, chunk l % 16, for r = 0..3.
+  char* mine = tq_lds + wave * 8192;
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
-    const int64_t m = m0 + wm * 128 + i * 16 + lr;
-    if (m < m_own) continue;
+    char* buf = mine + (i & 1) * 4096;
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
-      const int n = n0 + wn * 128 + j * 16;
-      if (n >= N) continue;
-      epilogue4<MODE>(epi, m, n + lg * 4, acc[i][j]);
+      half4_t o;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) o[e] = (half_t)(acc[i][j][e]);
+      const int c = (2 * j + (lg >> 1)) ^ lr;
+      *reinterpret_cast<half4_t*>(buf + lr * 256 + c * 16 + (lg & 1) * 8) = o;
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int row = 4 * r + (lane >> 4), c = lane & 15;
+      const half8_t v = *reinterpret_cast<const half8_t*>(buf + row * 256 + ((c ^ row) * 16));
+      const int64_t m = m0 + wm * 128 + i * 16 + row;
+      const int n = n0 + wn * 128 + c * 8;
+      if (n < N && m >= m_own) epilogue8<MODE>(epi, m, n, v);
     }
   }
 }
