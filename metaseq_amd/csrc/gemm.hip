@@ -1438,7 +1438,7 @@ void launch_tiled(const void* x, const void* W, const void* scales, int64_t M, i
   // the 256 x 256 kernel once it fills the chip; the 128 x 128 one for the shapes in between
   const int64_t big_tiles = ((M + TB_BM - 1) / TB_BM) * ((N + TB_BN - 1) / TB_BN);
   if constexpr (!W8) {
-    if (K % 64 == 0 && K >= 128 && big_tiles >= num_cus() && M >= 2 * TQ_BM) {
+    if (K % 64 == 0 && K >= 128 && big_tiles >= num_cus() && M >= TQ_BM) {
       static std::atomic<uint64_t> lds_allowed_q{0};
       if (!allow_lds((const void*)linear_quad_kernel<MODE>, TQ_LDS_BYTES, lds_allowed_q)) return;
       // up to 128 leftover rows go through the weight-streaming kernel (see below); more than

@@ -364,6 +364,9 @@ LINEAR_SHAPES = [
     # 8 tiles across: the tiles of a full round of 256 are regrouped per XCD, those of the last,
     # partial round (with a ragged bottom tile) are not
     (9160, 2048, 128),
+    # few rows under a wide output: one row tile of the four-wave kernel plus a bottom block for
+    # the streaming kernel; two row tiles, the second moved up over most of the first
+    (300, 32768, 128), (420, 32768, 128),
 ]
 
 
