@@ -1,5 +1,6 @@
 """Seeded random shapes through the C ABI: the decode GEMM paths (1 .. 64 packed rows, fp16 and
-int8 weights, with and without split-K) and both attention kernels (one query per row over a
+int8 weights, with and without split-K), the prefill GEMM paths (hundreds to thousands of
+row-major rows, enough 256 x 256 tiles for the large tiled kernels) and both attention kernels (one query per row over a
 history; a block of queries, causal, optionally appended to a history, optionally with a key
 padding mask), each against the same arithmetic written with torch ops on the device.  The fixed
 shapes of test_gpu_kernels.py pin the layouts and rounding points; these cases sweep the launch
@@ -81,6 +82,62 @@ def test_decode_gemm_random_shapes(lib):
         err = float((got - want).abs().max())
         assert err <= max(1e-3, float(want.abs().max()) * 2e-3), (it, err)
     assert ran >= 40
+
+
+def test_prefill_gemm_random_shapes(lib):
+    """Row-major activations with enough output tiles for the large tiled kernels: ragged bottom
+    row tiles (moved up, or handed to the streaming kernel), ragged right tiles, 8 / 16 tiles
+    across (regrouped per XCD), K a multiple of 64 but not of 128, every epilogue, y aliasing the
+    residual."""
+    rng = random.Random(23)
+    for it in range(18):
+        w8 = it % 3 == 2
+        ncol = rng.choice([8, 16, 16, 33, 48, 65, 100])
+        N = 256 * ncol - 16 * rng.choice([0, 0, 1, 5, 15])
+        nrow = -(-256 // ncol) + rng.choice([0, 1, 3])
+        M = max(256, 256 * nrow - rng.choice([0, 0, 1, 100, 128, 129, 200, 255]))
+        K = 64 * rng.choice([2, 3, 4, 5, 8, 12])
+        relu, use_res = rng.random() < 0.4, rng.random() < 0.6
+        in_place = use_res and rng.random() < 0.5
+        print("prefill gemm case", it, M, N, K, "int8" if w8 else "fp16", relu, use_res, in_place,
+              flush=True)
+        g = torch.Generator(device=DEV).manual_seed(100 + it)
+        x = (torch.randn(M, K, generator=g, device=DEV) * 0.5).half()
+        b = (torch.randn(N, generator=g, device=DEV) * 0.1).half()
+        res = torch.randn(M, N, generator=g, device=DEV).half() if use_res else None
+        if w8:
+            q = torch.randint(-127, 128, (N, K), generator=g, device=DEV, dtype=torch.int8)
+            sc = (torch.rand(N, generator=g, device=DEV) * 0.01 + 0.001).half()
+            Wd = (q.float() * sc.float()[:, None]).half()
+            Wp = torch.empty_like(q)
+            assert lib.msa_pack_weight_i8(q.data_ptr(), Wp.data_ptr(), N, K, None) == 0
+        else:
+            Wd = (torch.randn(N, K, generator=g, device=DEV) * 0.05).half()
+            Wp = torch.empty_like(Wd)
+            assert lib.msa_pack_weight_f16(Wd.data_ptr(), Wp.data_ptr(), N, K, None) == 0
+        want = r16(r16(x.float() @ Wd.float().t()) + b.float())
+        if relu:
+            want = want.clamp_min(0)
+        if use_res:
+            want = r16(want + res.float())
+        y = res.clone() if in_place else torch.full((M, N), float("nan"), dtype=torch.float16,
+                                                    device=DEV)
+        rp = None if res is None else (y.data_ptr() if in_place else res.data_ptr())
+        flags = 1 if relu else 0
+        if w8:
+            rc = lib.msa_linear_w8a16(x.data_ptr(), Wp.data_ptr(), sc.data_ptr(), b.data_ptr(), rp,
+                                      y.data_ptr(), M, N, K, flags, None)
+        else:
+            rc = lib.msa_linear_f16(x.data_ptr(), Wp.data_ptr(), b.data_ptr(), rp, y.data_ptr(), M,
+                                    N, K, flags, None)
+        assert rc == 0, lib.msa_last_error()
+        torch.cuda.synchronize()
+        got = y.float()
+        assert torch.isfinite(got).all(), (it, "unwritten or non-finite output")
+        err = float((got - want).abs().max())
+        # one fp16 ulp of the largest intermediate (a 1-ulp difference of the rounded product
+        # survives the bias / residual additions at the product's magnitude)
+        assert err <= float(want.abs().max()) * 2 ** -9 + 2e-3, (it, err)
 
 
 def test_attention_random_shapes(lib):
