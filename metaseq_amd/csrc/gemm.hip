@@ -1036,14 +1036,15 @@ __device__ __forceinline__ void tq_static_for(F&& f) {
   tq_static_for_impl(std::make_integer_sequence<int, N>{}, f);
 }
 
-// 8 consecutive output columns n..n+7 of row m; v holds the accumulators rounded to fp16
+// 8 consecutive output columns n..n+7 of row m; v holds the accumulators rounded to fp16, b the
+// bias and r the residual values of those columns (read only where the epilogue has them)
 template <int MODE>
-__device__ __forceinline__ void epilogue8(const Epilogue& e, int64_t m, int n, half8_t v) {
+__device__ __forceinline__ void epilogue8(const Epilogue& e, int64_t m, int n, half8_t v,
+                                          half8_t b, half8_t r) {
   float t[8];
 #pragma unroll
   for (int i = 0; i < 8; ++i) t[i] = (float)v[i];
   if (e.bias) {
-    const half8_t b = *reinterpret_cast<const half8_t*>(e.bias + n);
 #pragma unroll
     for (int i = 0; i < 8; ++i) t[i] = round_h(t[i] + (float)b[i]);
   }
@@ -1054,7 +1055,6 @@ __device__ __forceinline__ void epilogue8(const Epilogue& e, int64_t m, int n, h
       for (int i = 0; i < 8; ++i) t[i] = fmaxf(t[i], 0.f);
     }
     if (e.residual) {
-      const half8_t r = *reinterpret_cast<const half8_t*>(e.residual + m * e.N + n);
 #pragma unroll
       for (int i = 0; i < 8; ++i) t[i] = round_h(t[i] + (float)r[i]);
     }
@@ -1076,11 +1076,11 @@ __device__ __forceinline__ void epilogue8(const Epilogue& e, int64_t m, int n, h
       for (int i = 0; i < 8; ++i) o[i] = (half_t)t[i];
       const int h = e.hd_shift >= 0 ? c >> e.hd_shift : c / e.hd, d = c - h * e.hd;
       const int mi = (int)m;
-      const int b = e.T == 1 ? mi : mi / e.T, tt = mi - b * e.T;
-      const int s0 = e.len_dev ? e.len_dev[b] : e.S0;
+      const int bb = e.T == 1 ? mi : mi / e.T, tt = mi - bb * e.T;
+      const int s0 = e.len_dev ? e.len_dev[bb] : e.S0;
       if (s0 >= 0 && s0 + tt < e.S_cap) {
         half_t* dst = (part == 0 ? e.Kc : e.Vc) +
-                      (((int64_t)b * e.H + h) * e.S_cap + s0 + tt) * e.hd + d;
+                      (((int64_t)bb * e.H + h) * e.S_cap + s0 + tt) * e.hd + d;
         *reinterpret_cast<half8_t*>(dst) = o;
       }
     }
@@ -1259,7 +1259,28 @@ __global__ __launch_bounds__(TQ_THREADS) void linear_quad_kernel(
   // 16 * j + 4 * lg ...  Per i the wave's 16 rows x 128 features (4 KB, two buffers per wave) are
   // written as the lanes hold them (16-byte chunk 2 j + lg / 2 of the row, swizzled by the row) and
   // read back as lane l -> row 4 r + l / 16, chunk l % 16, for r = 0..3.
+  // The lane's column group is the same in every iteration, so the bias is read once; the residual
+  // rows are requested four iterations ahead (the fragment registers are free now), so that their
+  // latency is paid once per workgroup and not once per iteration.
   char* mine = tq_lds + wave * 8192;
+  const int ec = lane & 15, erow = lane >> 4;
+  const int en = n0 + wn * 128 + ec * 8;
+  const bool col_ok = en < N;
+  half8_t bias8 = zero8();
+  if (epi.bias && col_ok) bias8 = *reinterpret_cast<const half8_t*>(epi.bias + en);
+  constexpr int TQ_RES_AHEAD = 4;
+  half8_t res8[TQ_RES_AHEAD][4];
+  auto load_res = [&](int i, half8_t(&dst)[4]) {
+    if (MODE != MODE_PLAIN || !epi.residual) return;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int64_t m = m0 + wm * 128 + i * 16 + 4 * r + erow;
+      if (col_ok && m >= m_own)
+        dst[r] = *reinterpret_cast<const half8_t*>(epi.residual + m * epi.N + en);
+    }
+  };
+#pragma unroll
+  for (int i = 0; i < TQ_RES_AHEAD; ++i) load_res(i, res8[i]);
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
     char* buf = mine + (i & 1) * 4096;
@@ -1273,12 +1294,13 @@ __global__ __launch_bounds__(TQ_THREADS) void linear_quad_kernel(
     }
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
-      const int row = 4 * r + (lane >> 4), c = lane & 15;
-      const half8_t v = *reinterpret_cast<const half8_t*>(buf + row * 256 + ((c ^ row) * 16));
+      const int row = 4 * r + erow;
+      const half8_t v = *reinterpret_cast<const half8_t*>(buf + row * 256 + ((ec ^ row) * 16));
       const int64_t m = m0 + wm * 128 + i * 16 + row;
-      const int n = n0 + wn * 128 + c * 8;
-      if (n < N && m >= m_own) epilogue8<MODE>(epi, m, n, v);
+      if (col_ok && m >= m_own)
+        epilogue8<MODE>(epi, m, en, v, bias8, res8[i % TQ_RES_AHEAD][r]);
     }
+    if (i + TQ_RES_AHEAD < 8) load_res(i + TQ_RES_AHEAD, res8[i % TQ_RES_AHEAD]);
   }
 }
 
