@@ -17,9 +17,17 @@
 // Workgroup = 128 queries of one (batch row, head); 4 waves x 32 queries.  Everything is kept
 // transposed so that softmax rows live in lanes: S^T = K * Q^T puts query j = lane & 31 in each
 // lane with 16 keys in registers (plus the other half-wave), which is already the B-operand
-// layout of O^T = V^T * P^T.  K tiles are staged row-major in LDS (A operand: 8 consecutive d
-// per lane); V tiles are staged with key pairs interleaved ([key/2][d][2]) so that the A
-// operand of the second product (8 keys of one d) is four conflict-free 32-bit LDS reads.
+// layout of O^T = V^T * P^T.
+//
+// K and V tiles (64 keys) go global -> LDS directly (global_load_lds_dwordx4: the LDS address is
+// M0 + 16 * lane, the lane's global address is free), row-major as the cache holds them, with the
+// 16-byte chunks of a row XOR-swizzled so that the fragment reads are conflict free; no staging
+// registers, no LDS stores, one barrier per tile.  The A operand of S^T (8 consecutive d of one
+// key) is one 128-bit read.  The A operand of O^T needs 8 keys of one d, a column of the
+// row-major tile: ds_read_b64_tr_b16 delivers it (within 16 lanes, lane 4 r + c loads 4
+// consecutive d of key r; lane i then receives element i % 4 of the loads of lanes i / 4,
+// 4 + i / 4, 8 + i / 4, 12 + i / 4, i.e. 4 consecutive keys of d = i), two reads per MFMA.
+// Pass 1 keeps three K tiles in a ring (requests two tiles ahead), pass 2 two K and two V tiles.
 #include <math.h>
 
 #include "common.h"
@@ -29,25 +37,35 @@ namespace {
 constexpr int PF_BM = 128;  // queries per workgroup
 constexpr int PF_BN = 64;   // keys per tile
 constexpr int PF_THREADS = 256;
+typedef __fp16 pf_fp16x4 __attribute__((__vector_size__(4 * sizeof(__fp16))));
+typedef __attribute__((address_space(3))) pf_fp16x4 pf_lds_fp16x4;
+typedef __attribute__((address_space(3))) void pf_lds_void;
 
 template <int HD>
 __global__ __launch_bounds__(PF_THREADS) void prefill_attention_kernel(
     const half_t* __restrict__ q, const half_t* __restrict__ Kc, const half_t* __restrict__ Vc,
     const uint8_t* __restrict__ key_pad_mask, int64_t mask_stride, half_t* __restrict__ out,
-    int H, int T, int S0, int S_cap) {
-  constexpr int KSTEPS = HD / 16;  // MFMA k steps over the head dimension
-  constexpr int DBLK = HD / 32;    // 32-row blocks of O^T
-  constexpr int KLD = HD + 8;      // K tile row stride (halves)
-  constexpr int VLD = HD + 16;     // V tile row stride (32-bit words, one word = a key pair)
-  constexpr int PIECES = PF_BN * HD / 8 / PF_THREADS;  // 16-byte pieces per thread and tile
-  __shared__ __attribute__((aligned(16))) half_t lk[PF_BN * KLD];
-  __shared__ __attribute__((aligned(16))) uint32_t lv[(PF_BN / 2) * VLD];
+    int BH, int n_qt, int H, int T, int S0, int S_cap) {
+  constexpr int KSTEPS = HD / 16;           // MFMA k steps over the head dimension
+  constexpr int DBLK = HD / 32;             // 32-row blocks of O^T
+  constexpr int ROWB = HD * 2;              // bytes of a key row
+  constexpr int CH = HD / 8;                // 16-byte chunks of a key row
+  constexpr int TILEB = PF_BN * ROWB;       // bytes of a tile
+  constexpr int RPI = 1024 / ROWB;          // key rows per 1 KB load instruction
+  constexpr int IPW = TILEB / 1024 / 4;     // load instructions per wave and tile
+  __shared__ __attribute__((aligned(16))) char lds[4 * TILEB];
 
-  // query tiles are issued last-first: the tiles with the most keys start earliest
-  const int bh = blockIdx.x, qt = gridDim.y - 1 - blockIdx.y;
+  // Workgroup -> (batch row and head, query tile).  Consecutive workgroups land on consecutive
+  // XCDs, each with its own L2; all query tiles of one (row, head) share its K and V rows, so they
+  // are given to one XCD, back to back (workgroups i, i + 8, i + 16, ...), the tile with the most
+  // keys first: the rows are then fetched from memory once instead of once per query tile.
+  const int L = blockIdx.x, xcd = L & 7, seq = L >> 3;
+  const int bh = (seq / n_qt) * 8 + xcd, qt = n_qt - 1 - seq % n_qt;
+  if (bh >= BH) return;  // the last group of 8 may be incomplete (uniform per workgroup)
   const int b = bh / H, h = bh - b * H;
   const int D = H * HD;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int j = lane & 31, hl = lane >> 5;
   const int lead = (PF_BM - T % PF_BM) % PF_BM;   // queries missing from the first tile
   const int q0 = qt * PF_BM - lead + wave * 32;   // first query of this wave (may be negative)
@@ -70,63 +88,59 @@ __global__ __launch_bounds__(PF_THREADS) void prefill_attention_kernel(
       qf[ks] = *reinterpret_cast<const half8_t*>(qrow + ks * 16);
   }
 
-  // staging: piece c = tid + 256*i of a tile: key c / (HD/8), d offset 8*(c % (HD/8)).
-  // V pieces are taken as key pairs: pair p = c / (HD/8) (c < PF_BN/2 * HD/8 per half), so a
-  // thread loads the same d range of keys 2p and 2p+1 and writes them interleaved.
-  half8_t rk[PIECES], rv[PIECES];
-  auto load_k = [&](int tile) {
+  // chunk swizzles: K rows are read 16 keys at a time at one chunk index (swizzle by the key),
+  // V rows 4 keys at a time at two neighbouring chunks (swizzle the chunk pair by key % 4)
+  auto fk = [](int row) { return HD == 128 ? (row & 15) : ((row >> 1) & 7); };
+  auto fv = [](int row) { return 2 * (row & 3); };
+
+  // direct loads: instruction u of this wave covers tile rows (IPW * wave + u) * RPI ..; lane l
+  // lands at row l / CH, chunk position l % CH, which must hold chunk (l % CH) ^ f(row)
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(pf_lds_void*)lds;
+  int drow[IPW];
+  uint32_t kchunk[IPW], vchunk[IPW];
 #pragma unroll
-    for (int i = 0; i < PIECES; ++i) {
-      const int c = tid + PF_THREADS * i;
-      int key = tile * PF_BN + c / (HD / 8);
-      if (key >= n_keys) key = n_keys - 1;  // clamped rows are masked out below
-      rk[i] = *reinterpret_cast<const half8_t*>(kbase + (int64_t)key * HD + (c % (HD / 8)) * 8);
+  for (int u = 0; u < IPW; ++u) {
+    drow[u] = (wave * IPW + u) * RPI + lane / CH;
+    kchunk[u] = ((lane % CH) ^ fk(drow[u])) * 16;
+    vchunk[u] = ((lane % CH) ^ fv(drow[u])) * 16;
+  }
+  // keys past the last needed one repeat it (they are masked out below); a tile past the last
+  // one loads that key 64 times, which keeps the number of loads in flight the same everywhere
+  auto issue_tile = [&](const half_t* base, const uint32_t(&chunk)[IPW], int slot, int tile) {
+#pragma unroll
+    for (int u = 0; u < IPW; ++u) {
+      const int key = min(tile * PF_BN + drow[u], n_keys - 1);
+      const uint32_t vo = (uint32_t)key * ROWB + chunk[u];
+      const uint32_t la = lds0 + slot * TILEB + (wave * IPW + u) * 1024;
+      asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(vo), "s"(base),
+                   "s"(la)
+                   : "memory");
     }
   };
-  auto store_k = [&]() {
+  // K fragment of step ks (block ib adds 32 rows): row j, chunk 2 ks + hl
+  uint32_t kfo[KSTEPS];
 #pragma unroll
-    for (int i = 0; i < PIECES; ++i) {
-      const int c = tid + PF_THREADS * i;
-      *reinterpret_cast<half8_t*>(&lk[(c / (HD / 8)) * KLD + (c % (HD / 8)) * 8]) = rk[i];
+  for (int ks = 0; ks < KSTEPS; ++ks) kfo[ks] = j * ROWB + (((2 * ks + hl) ^ fk(j)) * 16);
+  // V, this lane as a source of the transposing read: key row 4 * (lane / 32) + (lane % 16) / 4
+  // of a 16-key step (+ 8 for the second read), d = 32 db + 16 * ((lane / 16) % 2) + 4 * (lane % 4)
+  uint32_t vfo[DBLK];
+  {
+    const int g = lane >> 4, i = lane & 15;
+    const int vrow = 4 * (g >> 1) + (i >> 2);
+#pragma unroll
+    for (int db = 0; db < DBLK; ++db) {
+      const int chunk = 4 * db + 2 * (g & 1) + ((i & 3) >> 1);
+      vfo[db] = vrow * ROWB + ((chunk ^ fv(vrow)) * 16) + (i & 1) * 8;
     }
-  };
-  // V: PIECES/2 pairs per thread; pair index pc = tid + 256*i, key pair pc / (HD/8)
-  auto load_v = [&](int tile) {
-#pragma unroll
-    for (int i = 0; i < PIECES / 2; ++i) {
-      const int pc = tid + PF_THREADS * i;
-      const int kp = pc / (HD / 8), dcol = (pc % (HD / 8)) * 8;
-      int k0 = tile * PF_BN + 2 * kp, k1 = k0 + 1;
-      if (k0 >= n_keys) k0 = n_keys - 1;
-      if (k1 >= n_keys) k1 = n_keys - 1;
-      rv[2 * i] = *reinterpret_cast<const half8_t*>(vbase + (int64_t)k0 * HD + dcol);
-      rv[2 * i + 1] = *reinterpret_cast<const half8_t*>(vbase + (int64_t)k1 * HD + dcol);
-    }
-  };
-  auto store_v = [&]() {
-#pragma unroll
-    for (int i = 0; i < PIECES / 2; ++i) {
-      const int pc = tid + PF_THREADS * i;
-      const int kp = pc / (HD / 8), dcol = (pc % (HD / 8)) * 8;
-      half8_t lo, hi;  // words d..d+3 and d+4..d+7, each word = (key 2p, key 2p+1)
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        lo[2 * e] = rv[2 * i][e];
-        lo[2 * e + 1] = rv[2 * i + 1][e];
-        hi[2 * e] = rv[2 * i][4 + e];
-        hi[2 * e + 1] = rv[2 * i + 1][4 + e];
-      }
-      *reinterpret_cast<half8_t*>(&lv[kp * VLD + dcol]) = lo;
-      *reinterpret_cast<half8_t*>(&lv[kp * VLD + dcol + 4]) = hi;
-    }
-  };
+  }
 
   // S^T tile of this wave: 64 keys x 32 queries = 2 accumulators, rounded to fp16, masked and kept
   // as packed pairs: pair v2 of block ib holds keys 32*ib + 8*(v2/2) + 4*hl + 2*(v2%2) + {0, 1}
   constexpr float LOG2E = 1.4426950408889634f;
   const float16_t zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
   half2_t sh[2][8];
-  auto scores = [&](int tile) {
+  auto scores = [&](int tile, int slot) {
+    const char* kt = lds + slot * TILEB;
     float16_t s[2];
     // the two key blocks alternate so that no MFMA waits for the one just issued; the first
     // step takes a literal zero as its addend (no accumulator clearing)
@@ -134,8 +148,7 @@ __global__ __launch_bounds__(PF_THREADS) void prefill_attention_kernel(
     for (int ks = 0; ks < KSTEPS; ++ks) {
 #pragma unroll
       for (int ib = 0; ib < 2; ++ib) {
-        const half8_t a =
-            *reinterpret_cast<const half8_t*>(&lk[(ib * 32 + j) * KLD + ks * 16 + hl * 8]);
+        const half8_t a = *reinterpret_cast<const half8_t*>(kt + ib * 32 * ROWB + kfo[ks]);
         s[ib] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, qf[ks], ks == 0 ? zero16 : s[ib], 0, 0, 0);
       }
     }
@@ -168,13 +181,15 @@ __global__ __launch_bounds__(PF_THREADS) void prefill_attention_kernel(
 
   // ---------------- pass 1: row maximum and sum of exp ----------------
   float m = -INFINITY, l = 0.f;
-  load_k(0);
-  for (int tile = 0; tile < ntiles; ++tile) {
-    __syncthreads();  // previous tile fully consumed
-    store_k();
-    __syncthreads();
-    if (tile + 1 < ntiles) load_k(tile + 1);  // the branch also pins the loads ahead of the MFMAs
-    scores(tile);
+  issue_tile(kbase, kchunk, 0, 0);
+  issue_tile(kbase, kchunk, 1, 1);
+  for (int tile = 0, slot = 0; tile < ntiles; ++tile) {
+    // all but this wave's newest IPW loads have landed: its part of this tile is there
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(IPW) : "memory");
+    __syncthreads();  // the tile is complete, and the slot of the previous tile is free
+    issue_tile(kbase, kchunk, slot == 0 ? 2 : slot - 1, tile + 2);
+    scores(tile, slot);
+    slot = slot == 2 ? 0 : slot + 1;
     half2_t t2 = sh[0][0];
 #pragma unroll
     for (int ib = 0; ib < 2; ++ib)
@@ -208,18 +223,18 @@ __global__ __launch_bounds__(PF_THREADS) void prefill_attention_kernel(
   for (int db = 0; db < DBLK; ++db)
 #pragma unroll
     for (int v = 0; v < 16; ++v) o[db][v] = 0.f;
-  load_k(0);
-  load_v(0);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();  // pass 1's last loads have landed and its last tile is consumed
+  issue_tile(kbase, kchunk, 0, 0);
+  issue_tile(vbase, vchunk, 2, 0);
   for (int tile = 0; tile < ntiles; ++tile) {
+    const int slot = tile & 1;
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
-    store_k();
-    store_v();
-    __syncthreads();
-    if (tile + 1 < ntiles) {
-      load_k(tile + 1);
-      load_v(tile + 1);
-    }
-    scores(tile);
+    issue_tile(kbase, kchunk, slot ^ 1, tile + 1);
+    issue_tile(vbase, vchunk, 2 + (slot ^ 1), tile + 1);
+    scores(tile, slot);
+    const char* vt = lds + (2 + slot) * TILEB;
     // k step c of S^T block ib covers keys 32*ib + 16*c + {4*hl + 0..3, 8 + 4*hl + 0..3}:
     // exactly pairs 4c .. 4c+3 of this lane, i.e. P^T is already a B operand
 #pragma unroll
@@ -233,16 +248,16 @@ __global__ __launch_bounds__(PF_THREADS) void prefill_attention_kernel(
           p[2 * e] = (half_t)__builtin_amdgcn_exp2f(__builtin_fmaf((float)h[0], LOG2E, -c2));
           p[2 * e + 1] = (half_t)__builtin_amdgcn_exp2f(__builtin_fmaf((float)h[1], LOG2E, -c2));
         }
-        const int kp = (ib * 32 + c * 16 + 4 * hl) >> 1;  // first key pair of this lane's group
 #pragma unroll
         for (int db = 0; db < DBLK; ++db) {
-          const int d = db * 32 + j;
+          const char* vp = vt + (ib * 32 + c * 16) * ROWB + vfo[db];
+          typedef uint32_t u2 __attribute__((ext_vector_type(2)));
           typedef uint32_t u4 __attribute__((ext_vector_type(4)));
-          u4 w;
-          w[0] = lv[(kp + 0) * VLD + d];
-          w[1] = lv[(kp + 1) * VLD + d];
-          w[2] = lv[(kp + 4) * VLD + d];
-          w[3] = lv[(kp + 5) * VLD + d];
+          const u2 lo = __builtin_bit_cast(
+              u2, __builtin_amdgcn_ds_read_tr16_b64_v4f16((pf_lds_fp16x4*)vp));
+          const u2 hi = __builtin_bit_cast(
+              u2, __builtin_amdgcn_ds_read_tr16_b64_v4f16((pf_lds_fp16x4*)(vp + 8 * ROWB)));
+          const u4 w = {lo[0], lo[1], hi[0], hi[1]};
           o[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, w), p, o[db],
                                                          0, 0, 0);
         }
@@ -269,14 +284,15 @@ int msa_launch_prefill_attention(const void* q, const void* Kc, const void* Vc,
                                  const uint8_t* key_pad_mask, int64_t mask_stride, void* out,
                                  int B, int H, int hd, int T, int S0, int S_cap,
                                  hipStream_t stream) {
-  const dim3 grid((unsigned)(B * H), (unsigned)((T + PF_BM - 1) / PF_BM));
+  const int n_qt = (T + PF_BM - 1) / PF_BM, BH = B * H;
+  const dim3 grid((unsigned)(((BH + 7) / 8) * 8 * n_qt));
   if (hd == 64)
     hipLaunchKernelGGL(prefill_attention_kernel<64>, grid, dim3(PF_THREADS), 0, stream,
                        (const half_t*)q, (const half_t*)Kc, (const half_t*)Vc, key_pad_mask,
-                       mask_stride, (half_t*)out, H, T, S0, S_cap);
+                       mask_stride, (half_t*)out, BH, n_qt, H, T, S0, S_cap);
   else
     hipLaunchKernelGGL(prefill_attention_kernel<128>, grid, dim3(PF_THREADS), 0, stream,
                        (const half_t*)q, (const half_t*)Kc, (const half_t*)Vc, key_pad_mask,
-                       mask_stride, (half_t*)out, H, T, S0, S_cap);
+                       mask_stride, (half_t*)out, BH, n_qt, H, T, S0, S_cap);
   return 0;
 }
