@@ -88,10 +88,12 @@ __global__ __launch_bounds__(PF_THREADS) void prefill_attention_kernel(
       qf[ks] = *reinterpret_cast<const half8_t*>(qrow + ks * 16);
   }
 
-  // chunk swizzles: K rows are read 16 keys at a time at one chunk index (swizzle by the key),
-  // V rows 4 keys at a time at two neighbouring chunks (swizzle the chunk pair by key % 4)
+  // chunk swizzles: K rows are read 16 keys at a time at one chunk index (swizzle by the key).
+  // V rows are read by 32 lanes at a time as 4 keys x two neighbouring 32-byte chunk pairs: the
+  // pair index is XORed with 2 * (key % 4), which sends the 8 pieces to the 8 pair positions of
+  // the 256 bytes the banks span (128-byte rows: two rows span the banks, XOR with 2 * (key / 2 % 2))
   auto fk = [](int row) { return HD == 128 ? (row & 15) : ((row >> 1) & 7); };
-  auto fv = [](int row) { return 2 * (row & 3); };
+  auto fv = [](int row) { return HD == 128 ? 4 * (row & 3) : 4 * ((row >> 1) & 1); };
 
   // direct loads: instruction u of this wave covers tile rows (IPW * wave + u) * RPI ..; lane l
   // lands at row l / CH, chunk position l % CH, which must hold chunk (l % CH) ^ f(row)
