@@ -45,7 +45,7 @@ template <int HD>
 __global__ __launch_bounds__(PF_THREADS) void prefill_attention_kernel(
     const half_t* __restrict__ q, const half_t* __restrict__ Kc, const half_t* __restrict__ Vc,
     const uint8_t* __restrict__ key_pad_mask, int64_t mask_stride, half_t* __restrict__ out,
-    int BH, int n_qt, int H, int T, int S0, int S_cap) {
+    int BH, int n_qt, int grouped, int H, int T, int S0, int S_cap) {
   constexpr int KSTEPS = HD / 16;           // MFMA k steps over the head dimension
   constexpr int DBLK = HD / 32;             // 32-row blocks of O^T
   constexpr int ROWB = HD * 2;              // bytes of a key row
@@ -59,8 +59,19 @@ __global__ __launch_bounds__(PF_THREADS) void prefill_attention_kernel(
   // XCDs, each with its own L2; all query tiles of one (row, head) share its K and V rows, so they
   // are given to one XCD, back to back (workgroups i, i + 8, i + 16, ...), the tile with the most
   // keys first: the rows are then fetched from memory once instead of once per query tile.
-  const int L = blockIdx.x, xcd = L & 7, seq = L >> 3;
-  const int bh = (seq / n_qt) * 8 + xcd, qt = n_qt - 1 - seq % n_qt;
+  // Small problems (all K and V rows fit the caches anyway) keep the plain order instead, every
+  // (row, head)'s longest tile first, which balances the tail better.
+  const int L = blockIdx.x;
+  int bh, qt;
+  if (grouped) {
+    const int xcd = L & 7, seq = L >> 3;
+    bh = (seq / n_qt) * 8 + xcd;
+    qt = n_qt - 1 - seq % n_qt;
+  } else {
+    const int BHp = gridDim.x / n_qt;
+    bh = L % BHp;
+    qt = n_qt - 1 - L / BHp;
+  }
   if (bh >= BH) return;  // the last group of 8 may be incomplete (uniform per workgroup)
   const int b = bh / H, h = bh - b * H;
   const int D = H * HD;
@@ -288,13 +299,15 @@ int msa_launch_prefill_attention(const void* q, const void* Kc, const void* Vc,
                                  hipStream_t stream) {
   const int n_qt = (T + PF_BM - 1) / PF_BM, BH = B * H;
   const dim3 grid((unsigned)(((BH + 7) / 8) * 8 * n_qt));
+  // K and V rows of all (row, head) pairs against the 32 MB of L2 + part of the memory-side cache
+  const int grouped = (int64_t)BH * (S0 + T) * hd * 4 > (int64_t)64 * 1024 * 1024;
   if (hd == 64)
     hipLaunchKernelGGL(prefill_attention_kernel<64>, grid, dim3(PF_THREADS), 0, stream,
                        (const half_t*)q, (const half_t*)Kc, (const half_t*)Vc, key_pad_mask,
-                       mask_stride, (half_t*)out, BH, n_qt, H, T, S0, S_cap);
+                       mask_stride, (half_t*)out, BH, n_qt, grouped, H, T, S0, S_cap);
   else
     hipLaunchKernelGGL(prefill_attention_kernel<128>, grid, dim3(PF_THREADS), 0, stream,
                        (const half_t*)q, (const half_t*)Kc, (const half_t*)Vc, key_pad_mask,
-                       mask_stride, (half_t*)out, BH, n_qt, H, T, S0, S_cap);
+                       mask_stride, (half_t*)out, BH, n_qt, grouped, H, T, S0, S_cap);
   return 0;
 }

@@ -632,6 +632,9 @@ def _oracle_core(dtype=torch.float16):
     # query tiles are aligned to the end: exact multiples, one query over, one query short
     (1, 2, 128, 128, 0, False), (1, 1, 128, 1025, 0, False), (2, 1, 64, 127, 3, True),
     (1, 2, 64, 384, 130, False),
+    # enough K and V rows (> 64 MiB) for the XCD-grouped order of the query tiles, with a number of
+    # (row, head) pairs that is no multiple of 8
+    (2, 33, 128, 1990, 10, True),
 ])
 def test_attention(lib, B, H, hd, T, S0, masked):
     print("attention", B, H, hd, T, S0, masked, flush=True)
