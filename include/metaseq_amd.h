@@ -68,6 +68,15 @@ int msa_pack_weight_f16(const void* src, void* dst, int N, int K, void* stream);
 int msa_unpack_weight_f16(const void* src, void* dst, int N, int K, void* stream);
 int msa_pack_weight_i8(const int8_t* src, int8_t* dst, int N, int K, void* stream);
 int msa_unpack_weight_i8(const int8_t* src, int8_t* dst, int N, int K, void* stream);
+/* Tile-packed int8 weights Wq with per-output-channel fp16 scales[N] -> tile-packed fp16 weights
+ * Wp (N*K halves), every element round(Wq[n,k] * scales[n]): exactly the values the w8a16 kernels
+ * form in registers, so msa_linear_f16 / msa_qkv_proj_f16 on Wp compute the product
+ * msa_linear_w8a16 / msa_qkv_proj_w8a16 compute on Wq.  For products of thousands of rows
+ * (prefill), where expanding a matrix once (3 bytes moved per weight) and running the fp16 kernel
+ * beats dequantising every fragment in every workgroup.  K % 64 == 0.  No reference counterpart
+ * (see msa_linear_w8a16). */
+int msa_expand_weight_w8_f16(const int8_t* Wq, const void* scales, void* Wp, int N, int K,
+                             void* stream);
 
 /* ---- device-resident per-row sequence lengths -------------------------------------------------
  * The entry points of a decode step (T == 1) take an optional `len_dev`: int32 [B] on the device,

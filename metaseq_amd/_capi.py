@@ -58,6 +58,7 @@ SIGNATURES = {
     "msa_unpack_weight_f16": [_P, _P, c_int, c_int, _P],
     "msa_pack_weight_i8": [_P, _P, c_int, c_int, _P],
     "msa_unpack_weight_i8": [_P, _P, c_int, c_int, _P],
+    "msa_expand_weight_w8_f16": [_P, _P, _P, c_int, c_int, _P],
     "msa_layernorm_f16": [_P, _P, _P, _P, c_int64, c_int, c_float, c_uint, _P],
     "msa_residual_layernorm_f16": [_P, c_int, _P, _P, _P, _P, _P, c_int64, c_int, c_float, c_uint,
                                    _P],

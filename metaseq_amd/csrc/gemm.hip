@@ -240,6 +240,27 @@ __global__ __launch_bounds__(256) void pack_i8_kernel(const int8_t* __restrict__
   *reinterpret_cast<uint2*>(unpack ? dst + rm : dst + piece * 8) = v;
 }
 
+// packed int8 -> packed fp16, each element round(q * scale): int8 block (t, ks8) becomes the fp16
+// blocks (t, 2 ks8) and (t, 2 ks8 + 1), and a lane's bytes 0..7 / 8..15 become its 8 halves in
+// the first / second of them (the lane index is the same in both layouts).  One thread per lane
+// and int8 block.
+__global__ __launch_bounds__(256) void expand_w8_kernel(const uint8_t* __restrict__ Wq,
+                                                        const half_t* __restrict__ scales,
+                                                        half_t* __restrict__ dst, int N, int K) {
+  const int64_t id = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (id >= (int64_t)N * K / 16) return;
+  const int lane = (int)(id & 63);
+  const int64_t blk = id >> 6;
+  const int nks8 = K >> 6;
+  const int t = (int)(blk / nks8);
+  typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+  const u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(Wq) + id);
+  const half_t sc = scales[t * 16 + (lane & 15)];
+  half8_t* out = reinterpret_cast<half8_t*>(dst) + (blk * 2) * 64 + lane;
+  out[0] = dequant8(v[0], v[1], sc);
+  out[64] = dequant8(v[2], v[3], sc);
+}
+
 // ---- stream kernel (M <= 64) --------------------------------------------------------------
 // MFMA fragments: lane l supplies 8 consecutive K elements (offset 8*(l>>4)) of row (l&15) of
 // its operand; A rows are output features n, B rows are activation rows m.  The accumulator
@@ -1649,6 +1670,20 @@ extern "C" int msa_pack_weight_i8(const int8_t* src, int8_t* dst, int N, int K, 
 }
 extern "C" int msa_unpack_weight_i8(const int8_t* src, int8_t* dst, int N, int K, void* stream) {
   return pack_entry("msa_unpack_weight_i8", src, dst, N, K, true, true, stream);
+}
+
+extern "C" int msa_expand_weight_w8_f16(const int8_t* Wq, const void* scales, void* Wp, int N,
+                                        int K, void* stream) {
+  MSA_REQUIRE(Wq && scales && Wp && (const void*)Wq != Wp, MSA_ERR_INVALID_ARG,
+              "msa_expand_weight_w8_f16: null or aliased pointers");
+  MSA_REQUIRE(N > 0 && K > 0 && N % 16 == 0 && K % 64 == 0, MSA_ERR_INVALID_ARG,
+              "msa_expand_weight_w8_f16: N=%d must be a multiple of 16 and K=%d of 64", N, K);
+  const int64_t n = (int64_t)N * K / 16;
+  hipLaunchKernelGGL(expand_w8_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0,
+                     (hipStream_t)stream, (const uint8_t*)Wq, (const half_t*)scales, (half_t*)Wp,
+                     N, K);
+  MSA_CHECK_LAUNCH("msa_expand_weight_w8_f16");
+  return MSA_OK;
 }
 
 extern "C" int64_t msa_lm_head_select_workspace_bytes(int M) {

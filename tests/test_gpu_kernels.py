@@ -612,6 +612,24 @@ def test_qkv_proj_scatter_large_tiled_kernel(lib, w8):
     assert float(Kc[:, :, :S0].abs().sum()) == 0 and float(Kc[:, :, S0 + T:].abs().sum()) == 0
 
 
+@pytest.mark.parametrize("N,K", [(16, 64), (48, 192), (1008, 4096)])
+def test_expand_weight_w8_f16(lib, N, K):
+    """Packed int8 + scales -> packed fp16: bit for bit the packed form of the dequantised matrix
+    round(q * scale), including the extreme bytes and a zero scale."""
+    g = torch.Generator().manual_seed(5)
+    q = torch.randint(-127, 128, (N, K), generator=g, dtype=torch.int8)
+    q[0, :4] = torch.tensor([-128, -127, 127, 0], dtype=torch.int8)
+    sc = (torch.rand(N, generator=g) * 0.02 + 1e-4).half()
+    sc[N - 1] = 0
+    want = pack_w(lib, G(O.dequantize_int8(q, sc).half()))
+    got = torch.full((N, K), float("nan"), dtype=torch.float16, device=DEV)
+    ok(lib.msa_expand_weight_w8_f16(P(pack_w8(lib, G(q))), P(G(sc)), P(got), N, K, None), lib)
+    torch.cuda.synchronize()
+    assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+    assert lib.msa_expand_weight_w8_f16(P(got), P(G(sc)), P(got), N, K, None) == -1
+    assert lib.msa_expand_weight_w8_f16(P(G(q)), P(G(sc)), P(got), N, 96, None) == -1
+
+
 def test_qkv_proj_capacity_error(lib):
     x = torch.zeros(2, 128, dtype=torch.float16, device=DEV)
     rc = lib.msa_qkv_proj_f16(P(x), P(x), P(x), P(x), P(x), P(x), 2, 1, 2, 64, 10, 10, 128, 0,
