@@ -117,6 +117,79 @@ __global__ __launch_bounds__(THREADS) void layernorm_f16_kernel(
   }
 }
 
+// Plain LayerNorm over thousands of rows: a workgroup walks rows blockIdx.x, + gridDim.x, ...
+// with gamma and beta held in registers (read once per workgroup, not once per row) and the next
+// row requested before the current one is reduced.  Per row the same threads do the same
+// arithmetic in the same order as layernorm_f16_kernel<0, THREADS>: the results are its bits.
+template <int THREADS>
+__global__ __launch_bounds__(THREADS) void layernorm_rows_kernel(
+    const half_t* __restrict__ x, const half_t* __restrict__ gamma,
+    const half_t* __restrict__ beta, half_t* __restrict__ y, int M, int D, float eps) {
+  __shared__ float red[16];
+  const int nchunk = D >> 3;
+  half8_t v[LN_MAX_CHUNKS], nx[LN_MAX_CHUNKS], gv[LN_MAX_CHUNKS], bv[LN_MAX_CHUNKS];
+  auto load_row = [&](int row, half8_t(&dst)[LN_MAX_CHUNKS]) {
+#pragma unroll
+    for (int c = 0; c < LN_MAX_CHUNKS; ++c) {
+      const int idx = threadIdx.x + c * THREADS;
+      if (idx < nchunk)
+        dst[c] = __builtin_nontemporal_load(
+            reinterpret_cast<const half8_t*>(x + (int64_t)row * D + (idx << 3)));
+    }
+  };
+#pragma unroll
+  for (int c = 0; c < LN_MAX_CHUNKS; ++c) {
+    const int idx = threadIdx.x + c * THREADS;
+    if (idx < nchunk) {
+      gv[c] = *reinterpret_cast<const half8_t*>(gamma + (idx << 3));
+      bv[c] = *reinterpret_cast<const half8_t*>(beta + (idx << 3));
+    }
+  }
+  int row = blockIdx.x;
+  if (row < M) load_row(row, v);
+  for (; row < M; row += gridDim.x) {
+    const int next = row + gridDim.x;
+    if (next < M) load_row(next, nx);  // uniform
+    float s = 0.f;
+#pragma unroll
+    for (int c = 0; c < LN_MAX_CHUNKS; ++c) {
+      const int idx = threadIdx.x + c * THREADS;
+      if (idx < nchunk) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) s += (float)v[c][i];
+      }
+    }
+    const float mean = block_sum(s, red) / (float)D;
+    float q = 0.f;
+#pragma unroll
+    for (int c = 0; c < LN_MAX_CHUNKS; ++c) {
+      const int idx = threadIdx.x + c * THREADS;
+      if (idx < nchunk) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          const float d = (float)v[c][i] - mean;
+          q += d * d;
+        }
+      }
+    }
+    const float var = block_sum(q, red) / (float)D;
+    const float rstd = rsqrtf(var + eps);
+#pragma unroll
+    for (int c = 0; c < LN_MAX_CHUNKS; ++c) {
+      const int idx = threadIdx.x + c * THREADS;
+      if (idx < nchunk) {
+        half8_t o;
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+          o[i] = (half_t)(((float)v[c][i] - mean) * rstd * (float)gv[c][i] + (float)bv[c][i]);
+        *reinterpret_cast<half8_t*>(y + (int64_t)row * D + (idx << 3)) = o;
+      }
+    }
+#pragma unroll
+    for (int c = 0; c < LN_MAX_CHUNKS; ++c) v[c] = nx[c];
+  }
+}
+
 int check(const char* name, int64_t rows, int D, unsigned flags) {
   MSA_REQUIRE(rows >= 0 && rows <= 0x7fffffff, MSA_ERR_INVALID_ARG, "%s: rows=%lld out of range",
               name, (long long)rows);
@@ -144,6 +217,23 @@ extern "C" int msa_layernorm_f16(const void* x, const void* gamma, const void* b
   const int threads = rows <= 64 || D > 256 * 8 * LN_MAX_CHUNKS ? LN_THREADS
                       : D > 128 * 8 * LN_MAX_CHUNKS             ? 256
                                                                 : 128;
+  if (rows > 64 && out_mb == 0) {
+    // up to 2048 threads per CU worth of workgroups, each walking its share of the rows
+    int dev = 0, cus = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
+        cus <= 0)
+      cus = 256;
+    const int64_t wgs = (int64_t)cus * (2048 / threads);
+    const dim3 grid((unsigned)(rows < wgs ? rows : wgs));
+    auto rk = threads == LN_THREADS ? layernorm_rows_kernel<LN_THREADS>
+              : threads == 256      ? layernorm_rows_kernel<256>
+                                    : layernorm_rows_kernel<128>;
+    hipLaunchKernelGGL(rk, grid, dim3(threads), 0, (hipStream_t)stream, (const half_t*)x,
+                       (const half_t*)gamma, (const half_t*)beta, (half_t*)y, (int)rows, D, eps);
+    MSA_CHECK_LAUNCH("msa_layernorm_f16");
+    return MSA_OK;
+  }
   auto kernel = threads == LN_THREADS ? layernorm_f16_kernel<0, LN_THREADS>
                 : threads == 256      ? layernorm_f16_kernel<0, 256>
                                       : layernorm_f16_kernel<0, 128>;

@@ -98,7 +98,9 @@ def rnd(*shape, seed=0, std=1.0):
 @pytest.mark.parametrize("rows,D", [(1, 64), (32, 768), (7, 2048), (32, 4096), (33, 7168),
                                     (32, 9216), (300, 1024),
                                     # many rows: 128-, 256- and 512-thread workgroups
-                                    (100, 4096), (200, 768), (70, 7168), (65, 9216)])
+                                    (100, 4096), (200, 768), (70, 7168), (65, 9216),
+                                    # more rows than workgroups: every workgroup walks several rows
+                                    (9001, 1024), (4500, 7168), (3000, 9216)])
 def test_layernorm(lib, rows, D):
     print("layernorm", rows, D, flush=True)
     x = rnd(rows, D, seed=1)
