@@ -1380,6 +1380,17 @@ void launch_stream_mb(const void* xp, const void* W, const void* scales, float* 
                        m_off);
     return;
   }
+  // The ragged bottom rows of a prefill-sized product (row-major activations, 33 .. 64 rows, fp16):
+  // the workgroup's few tiles would leave most of the 8 tile slots per activation fragment empty
+  // (their clamped loads still run), so groups of 4 are used when the tiles fit them.
+  if constexpr (XR && !W8 && MB > 2) {
+    if (tiles_per_wg <= ST_NT) {
+      hipLaunchKernelGGL((linear_stream_kernel<MB, W8, MODE, XR, ST_KG, ST_NT>), dim3(gx, S),
+                         dim3(ST_KG * 64), 0, s, (const half_t*)xp, W, (const half_t*)scales, part,
+                         M, N, K, tiles_per_wg, ks_per_split, epi, m_off);
+      return;
+    }
+  }
   hipLaunchKernelGGL((linear_stream_kernel<MB, W8, MODE, XR>), dim3(gx, S), dim3(ST_KG * 64), 0,
                      s, (const half_t*)xp, W, (const half_t*)scales, part, M, N, K, tiles_per_wg,
                      ks_per_split, epi, m_off);

@@ -369,6 +369,8 @@ LINEAR_SHAPES = [
     # few rows under a wide output: one row tile of the four-wave kernel plus a bottom block for
     # the streaming kernel; two row tiles, the second moved up over most of the first
     (300, 32768, 128), (420, 32768, 128),
+    # 64 and 44 bottom rows with few tiles per workgroup: the streaming kernel's four-tile groups
+    (4160, 4096, 256), (4140, 8192, 128),
 ]
 
 
