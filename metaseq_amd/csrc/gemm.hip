@@ -5,7 +5,7 @@
 // the order the 64 lanes read it, and the blocks of one 16-row tile follow each other along K.
 // A wave instruction therefore reads one whole KB and a tile's K sweep is one linear stream.
 //
-// Four kernels:
+// Five kernels:
 //   * stream (M <= 32 packed rows, the decode step; also the fused vocabulary projection +
 //     selection up to 64 rows): HBM-bound.  A workgroup of 8 waves owns a contiguous range of
 //     16-row tiles (and, with split-K, one K range); it walks the tiles 3 or 4 at a time, the
@@ -16,8 +16,10 @@
 //     the waves through LDS (fixed order: results are run-to-run deterministic).
 //   * shared-activation stream (33 .. 64 packed rows): the same weight streaming, with the
 //     activation fragments staged once per workgroup in LDS and shared by four waves.
-//   * large tiled (prefill-sized M): 256 x 256 x 64 per workgroup, weights straight from the
-//     packed layout into registers, activations through LDS, v_mfma_f32_16x16x32_f16.
+//   * large tiled, fp16 weights (prefill-sized M): 256 x 256 per workgroup of four waves of
+//     128 x 128 with their accumulators in the AGPR bank, both operands global -> LDS directly.
+//   * large tiled, int8 weights: 256 x 256 x 64 per workgroup of eight waves, weights straight
+//     from the packed layout into registers (dequantised there), activations through LDS.
 //   * tiled (shapes in between): 128 x 128 x 32 LDS double-buffered tiles, 4 waves of 64 x 64,
 //     v_mfma_f32_32x32x16_f16.
 // All share one epilogue that reproduces the reference's fp16 rounding points, and a QKV mode
