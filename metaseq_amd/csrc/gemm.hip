@@ -1494,15 +1494,22 @@ void launch_tiled(const void* x, const void* W, const void* scales, int64_t M, i
   // the 256 x 256 kernel once it fills the chip; the 128 x 128 one for the shapes in between
   const int64_t big_tiles = ((M + TB_BM - 1) / TB_BM) * ((N + TB_BN - 1) / TB_BN);
   if constexpr (!W8) {
-    if (K % 64 == 0 && K >= 128 && big_tiles >= num_cus() && M >= TQ_BM) {
+    // also below one tile per CU: down to 3/8 of the CUs a single round of these tiles beats the
+    // 128 x 128 kernel on the same product (which runs at a third of this kernel's rate per CU)
+    if (K % 64 == 0 && K >= 128 && big_tiles * 8 >= (int64_t)num_cus() * 3 && M >= TQ_BM) {
       static std::atomic<uint64_t> lds_allowed_q{0};
       if (!allow_lds((const void*)linear_quad_kernel<MODE>, TQ_LDS_BYTES, lds_allowed_q)) return;
       // up to 128 leftover rows go through the weight-streaming kernel (see below); more than
       // that get a last row tile moved up to end at the last row
+      // (unless one more row of tiles fits the last round of workgroups anyway)
+      const int ncol = (N + TQ_BN - 1) / TQ_BN;
       int64_t M_main = M;
       const int64_t rem = M % TQ_BM;
-      if (rem > 0 && rem <= 128) M_main = M - rem;
-      const int ncol = (N + TQ_BN - 1) / TQ_BN, nrow = (int)((M_main + TQ_BM - 1) / TQ_BM);
+      if (rem > 0 && rem <= 128) {
+        const int64_t cus = num_cus(), full = (M / TQ_BM) * ncol;
+        if ((full + ncol + cus - 1) / cus > (full + cus - 1) / cus) M_main = M - rem;
+      }
+      const int nrow = (int)((M_main + TQ_BM - 1) / TQ_BM);
       // regrouping of a round's 256 tiles: a x b per XCD with a * b = 32, (ncol / a) * (r / b) = 8
       // for r = 256 / ncol rows per round; taken when it beats the default strip (ncol / 8) x r
       int rm_a = 0, rm_b = 0, rm_r = 0;
