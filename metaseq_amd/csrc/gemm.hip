@@ -1039,12 +1039,14 @@ __global__ __launch_bounds__(TB_THREADS) void linear_tiled_big_kernel(
 // every XCD's L2 serves a compact a x b block (rm_a, rm_b, rm_r from the host).
 // Needs K % 64 == 0, K >= 128, M >= 256 (a ragged last row tile is moved up to end at M and stores
 // only the rows no other tile owns).
-constexpr int TQ_BM = 256, TQ_BN = 256, TQ_THREADS = 256;
+constexpr int TQ_BM = 256, TQ_THREADS = 256;
 constexpr int TQ_RX = 3, TQ_RW = 4;
 constexpr int TQ_XBYTES = TQ_BM * 64 * 2;       // one 64-wide stage of activations
-constexpr int TQ_WBYTES = (TQ_BN / 16) * 1024;  // one 32-wide step of weights
 constexpr int TQ_WOFF = TQ_RX * TQ_XBYTES;
-constexpr int TQ_LDS_BYTES = TQ_RX * TQ_XBYTES + TQ_RW * TQ_WBYTES;  // 160 KB
+// WF = weight fragments (16-feature tiles) per wave: 8 -> 256 features per workgroup, 4 -> 128
+constexpr int tq_bn(int WF) { return 32 * WF; }
+constexpr int tq_wbytes(int WF) { return 2 * WF * 1024; }  // one 32-wide step of weights
+constexpr int tq_lds_bytes(int WF) { return TQ_RX * TQ_XBYTES + TQ_RW * tq_wbytes(WF); }  // 160 / 128 KB
 typedef __attribute__((address_space(3))) void tq_lds_void;
 
 #define TQ_MFMA(ACC, A, B) \
@@ -1110,7 +1112,7 @@ __device__ __forceinline__ void epilogue8(const Epilogue& e, int64_t m, int n, h
   }
 }
 
-template <int MODE>
+template <int MODE, int WF>
 __global__ __launch_bounds__(TQ_THREADS) void linear_quad_kernel(
     const half_t* __restrict__ x, const void* __restrict__ Wp, int64_t M, int N, int K,
     int rm_a, int rm_b, int rm_r, Epilogue epi) {
@@ -1118,6 +1120,8 @@ __global__ __launch_bounds__(TQ_THREADS) void linear_quad_kernel(
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lr = lane & 15, lg = lane >> 4;
   const int wm = wave >> 1, wn = wave & 1;
+  constexpr int TQ_BN = tq_bn(WF), TQ_WBYTES = tq_wbytes(WF);
+  constexpr int WL = WF / 2;  // weight load instructions per wave and step
   int bx = blockIdx.x, by = blockIdx.y;
   if (rm_a > 0) {
     const int ncol = gridDim.x, L = by * ncol + bx, round = L >> 8, i = L & 255;
@@ -1139,13 +1143,13 @@ __global__ __launch_bounds__(TQ_THREADS) void linear_quad_kernel(
   // + 4 KB and instruction offset 1024 * (i - 4).  Weights, per step: the wave copies the blocks
   // of tiles 4 * wave .. 4 * wave + 3, instruction offset 1024 * j.
   const char* xb[8];
-  const char* wb[4];
+  const char* wb[WL];
 #pragma unroll
   for (int i = 0; i < 8; ++i)
     xb[i] = (const char*)(x + (m0 + wave * 64 + i * 8) * K) - (i - 4) * 1024;
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    const int tt = min(n0 / 16 + wave * 4 + j, ntiles - 1);
+  for (int j = 0; j < WL; ++j) {
+    const int tt = min(n0 / 16 + wave * WL + j, ntiles - 1);
     wb[j] = (const char*)Wp + (int64_t)tt * K * 32 - j * 1024;
   }
   const uint32_t xrow = (uint32_t)(lane >> 3) * (uint32_t)K * 2;
@@ -1164,7 +1168,7 @@ __global__ __launch_bounds__(TQ_THREADS) void linear_quad_kernel(
   auto set_w = [&](int slot, int ks) {
     ks = min(ks, nks - 1);
     wv = wlane + ks * 1024;
-    asm volatile("s_mov_b32 m0, %0" ::"s"(lds0 + TQ_WOFF + slot * TQ_WBYTES + wave * 4096)
+    asm volatile("s_mov_b32 m0, %0" ::"s"(lds0 + TQ_WOFF + slot * TQ_WBYTES + wave * (WL * 1024))
                  : "memory");
   };
   auto issue_x = [&](auto ic) {
@@ -1188,7 +1192,7 @@ __global__ __launch_bounds__(TQ_THREADS) void linear_quad_kernel(
   };
   auto group_w = [&](int slot, int ks) {
     set_w(slot, ks);
-    tq_static_for<4>([&](auto jc) { issue_w(jc); });
+    tq_static_for<WL>([&](auto jc) { issue_w(jc); });
   };
 
   // fragment reads.  Activation fragment i of half h of a stage: row 128 * wm + 16 * i + lr, chunk
@@ -1196,7 +1200,7 @@ __global__ __launch_bounds__(TQ_THREADS) void linear_quad_kernel(
   const int sw = (lr >> 1) & 7;
   const uint32_t xoff0 = (uint32_t)(wm * 128 + lr) * 128 + ((lg ^ sw) * 16);
   const uint32_t xoff1 = (uint32_t)(wm * 128 + lr) * 128 + ((lg ^ sw ^ 4) * 16);
-  const uint32_t woff = TQ_WOFF + (uint32_t)(wn * 8) * 1024 + lane * 16;
+  const uint32_t woff = TQ_WOFF + (uint32_t)(wn * WF) * 1024 + lane * 16;
   auto xfrag = [&](int slot, int h, int i) {
     return *reinterpret_cast<const half8_t*>(tq_lds + slot * TQ_XBYTES + (h ? xoff1 : xoff0) +
                                              i * (16 * 128));
@@ -1205,40 +1209,41 @@ __global__ __launch_bounds__(TQ_THREADS) void linear_quad_kernel(
     return *reinterpret_cast<const half8_t*>(tq_lds + slot * TQ_WBYTES + woff + j * 1024);
   };
 
-  float4_t acc[8][8];
+  float4_t acc[8][WF];
 #pragma unroll
   for (int i = 0; i < 8; ++i)
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
+    for (int j = 0; j < WF; ++j) {
       acc[i][j] = float4_t{0.f, 0.f, 0.f, 0.f};
       asm volatile("" : "+a"(acc[i][j]));
     }
 
   // prologue: activation stages 0 and 1, weight steps 0..3 requested; stages 0, 1 and steps 0, 1
   // landed
-  half8_t xf[2][8], wf[2][8];
+  half8_t xf[2][8], wf[2][WF];
   group_x(0, 0);
   group_w(0, 0);
   group_x(1, 1);
   group_w(1, 1);
   group_w(2, 2);
   group_w(3, 3);
-  asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * WL) : "memory");
   __syncthreads();
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    xf[0][i] = xfrag(0, 0, i);
-    wf[0][i] = wfrag(0, i);
-  }
+  for (int i = 0; i < 8; ++i) xf[0][i] = xfrag(0, 0, i);
+#pragma unroll
+  for (int j = 0; j < WF; ++j) wf[0][j] = wfrag(0, j);
 
-  // step t = 2 S + H; xs, ws: ring slots of stage S and step t.  An even step issues 12 loads
-  // (stage S + 2, then step t + 4), an odd one 4 (step t + 4).  Loads complete in order; the
-  // weights of step t + 1 were requested in step t - 3, and the 16 loads of steps t - 2 and t - 1
-  // may still be outstanding at the barrier.  The activations an odd step starts to read (stage
-  // S + 1) were requested in step t - 3 as well.
+  // step t = 2 S + H; xs, ws: ring slots of stage S and step t.  An even step issues 8 + WL loads
+  // (stage S + 2, then step t + 4), an odd one WL (step t + 4).  Loads complete in order; the
+  // weights of step t + 1 were requested in step t - 3, and the 8 + 2 WL loads of steps t - 2 and
+  // t - 1 may still be outstanding at the barrier.  The activations an odd step starts to read
+  // (stage S + 1) were requested in step t - 3 as well, ahead of that step's weights.
+  // The 8 x WF MFMAs of a step carry, one each: the 8 + WF fragment reads of step t + 1 and the
+  // loads (even steps: activations under rows 0..3, weights under rows 4..7).
   auto step = [&](int t, int xs, int ws, auto hc) {
     constexpr int H = decltype(hc)::value;
-    asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(8 + 2 * WL) : "memory");
     __syncthreads();
     const int S = t >> 1;
     const int xfree = xs == 0 ? TQ_RX - 1 : xs - 1;  // slot of stage S - 1 = slot of stage S + 2
@@ -1246,20 +1251,34 @@ __global__ __launch_bounds__(TQ_THREADS) void linear_quad_kernel(
     const int wnext = ws == TQ_RW - 1 ? 0 : ws + 1;  // slot of step t + 1
     tq_static_for<8>([&](auto ic) {
       constexpr int i = decltype(ic)::value;
-      tq_static_for<8>([&](auto jc) {
+      tq_static_for<WF>([&](auto jc) {
         constexpr int j = decltype(jc)::value;
         TQ_MFMA(acc[i][j], wf[H][j], xf[H][i]);
         if (j == 1) xf[H ^ 1][i] = H == 0 ? xfrag(xs, 1, i) : xfrag(xnext, 0, i);
-        if (j == 5) wf[H ^ 1][i] = wfrag(wnext, i);
-        if constexpr (H == 0) {  // the 8 activation loads under rows 0..3, the 4 weight loads after
+        if constexpr (WF == 8) {
+          if (j == 5) wf[H ^ 1][i % WF] = wfrag(wnext, i % WF);
+        } else {
+          if constexpr (j == 3 && (i & 1)) wf[H ^ 1][(i >> 1) % WF] = wfrag(wnext, (i >> 1) % WF);
+        }
+        if constexpr (H == 0) {
           if (i == 0 && j == 0) set_x(xfree, S + 2);
-          if constexpr (i < 4 && j == 3) issue_x(std::integral_constant<int, (i & 3) * 2>{});
-          if constexpr (i < 4 && j == 7) issue_x(std::integral_constant<int, (i & 3) * 2 + 1>{});
+          if constexpr (i < 4 && j == WF / 2 - 1) issue_x(std::integral_constant<int, (i & 3) * 2>{});
+          if constexpr (i < 4 && j == WF - 1) issue_x(std::integral_constant<int, (i & 3) * 2 + 1>{});
           if (i == 4 && j == 0) set_w(ws, t + TQ_RW);
-          if constexpr (i >= 4 && j == 3) issue_w(std::integral_constant<int, (i & 3)>{});
+          if constexpr (WF == 8) {
+            if constexpr (i >= 4 && j == 3) issue_w(std::integral_constant<int, (i & 3) % WL>{});
+          } else {
+            if constexpr ((i == 4 || i == 6) && j == 2)
+              issue_w(std::integral_constant<int, (i >> 1) & 1>{});
+          }
         } else {
           if (i == 0 && j == 0) set_w(ws, t + TQ_RW);
-          if constexpr (j == 3 && (i & 1)) issue_w(std::integral_constant<int, (i >> 1)>{});
+          if constexpr (WF == 8) {
+            if constexpr (j == 3 && (i & 1)) issue_w(std::integral_constant<int, (i >> 1) % WL>{});
+          } else {
+            if constexpr ((i == 2 || i == 6) && j == 2)
+              issue_w(std::integral_constant<int, (i >> 2) & 1>{});
+          }
         }
       });
     });
@@ -1279,25 +1298,29 @@ __global__ __launch_bounds__(TQ_THREADS) void linear_quad_kernel(
   __syncthreads();  // every wave is done with the operand rings
 
   // D tile (i, j): the lane holds activation row 16 * i + lr of the wave's 128 and the 4 features
-  // 16 * j + 4 * lg ...  Per i the wave's 16 rows x 128 features (4 KB, two buffers per wave) are
-  // written as the lanes hold them (16-byte chunk 2 j + lg / 2 of the row, swizzled by the row) and
-  // read back as lane l -> row 4 r + l / 16, chunk l % 16, for r = 0..3.
+  // 16 * j + 4 * lg ...  Per i the wave's 16 rows x 16 WF features (4 or 2 KB, two buffers per wave)
+  // are written as the lanes hold them (16-byte chunk 2 j + lg / 2 of the row, swizzled by the row)
+  // and read back 16 bytes per lane, whole rows per 16 (8) lanes.
   // The lane's column group is the same in every iteration, so the bias is read once; the residual
   // rows are requested four iterations ahead (the fragment registers are free now), so that their
   // latency is paid once per workgroup and not once per iteration.
   char* mine = tq_lds + wave * 8192;
-  const int ec = lane & 15, erow = lane >> 4;
-  const int en = n0 + wn * 128 + ec * 8;
+  constexpr int ECH = 2 * WF;        // 16-byte chunks of a staged row (16 WF features)
+  constexpr int ERB = 16 * ECH;      // bytes of a staged row
+  constexpr int ERPI = 64 / ECH;     // rows a 64-lane read covers
+  constexpr int ENR = 16 / ERPI;     // reads per 16 rows
+  const int ec = lane % ECH, erow = lane / ECH;
+  const int en = n0 + wn * (16 * WF) + ec * 8;
   const bool col_ok = en < N;
   half8_t bias8 = zero8();
   if (epi.bias && col_ok) bias8 = *reinterpret_cast<const half8_t*>(epi.bias + en);
   constexpr int TQ_RES_AHEAD = 4;
-  half8_t res8[TQ_RES_AHEAD][4];
-  auto load_res = [&](int i, half8_t(&dst)[4]) {
+  half8_t res8[TQ_RES_AHEAD][ENR];
+  auto load_res = [&](int i, half8_t(&dst)[ENR]) {
     if (MODE != MODE_PLAIN || !epi.residual) return;
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      const int64_t m = m0 + wm * 128 + i * 16 + 4 * r + erow;
+    for (int r = 0; r < ENR; ++r) {
+      const int64_t m = m0 + wm * 128 + i * 16 + ERPI * r + erow;
       if (col_ok && m >= m_own)
         dst[r] = *reinterpret_cast<const half8_t*>(epi.residual + m * epi.N + en);
     }
@@ -1308,17 +1331,18 @@ __global__ __launch_bounds__(TQ_THREADS) void linear_quad_kernel(
   for (int i = 0; i < 8; ++i) {
     char* buf = mine + (i & 1) * 4096;
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
+    for (int j = 0; j < WF; ++j) {
       half4_t o;
 #pragma unroll
       for (int e = 0; e < 4; ++e) o[e] = (half_t)(acc[i][j][e]);
-      const int c = (2 * j + (lg >> 1)) ^ lr;
-      *reinterpret_cast<half4_t*>(buf + lr * 256 + c * 16 + (lg & 1) * 8) = o;
+      const int c = (2 * j + (lg >> 1)) ^ (lr & (ECH - 1));
+      *reinterpret_cast<half4_t*>(buf + lr * ERB + c * 16 + (lg & 1) * 8) = o;
     }
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      const int row = 4 * r + erow;
-      const half8_t v = *reinterpret_cast<const half8_t*>(buf + row * 256 + ((ec ^ row) * 16));
+    for (int r = 0; r < ENR; ++r) {
+      const int row = ERPI * r + erow;
+      const half8_t v = *reinterpret_cast<const half8_t*>(buf + row * ERB +
+                                                          ((ec ^ (row & (ECH - 1))) * 16));
       const int64_t m = m0 + wm * 128 + i * 16 + row;
       if (col_ok && m >= m_own)
         epilogue8<MODE>(epi, m, en, v, bias8, res8[i % TQ_RES_AHEAD][r]);
@@ -1488,46 +1512,66 @@ void launch_stream(const void* xp, const void* W, const void* scales, float* par
   }
 }
 
+// One launch of the four-wave kernel (WF = 8: 256 x 256 tiles, WF = 4: 256 x 128) plus, for a
+// ragged bottom of at most 128 rows that does not fit the last round of workgroups, the streaming
+// kernel on those rows.
+template <int MODE, int WF>
+void launch_quad(const void* x, const void* W, const void* scales, int64_t M, int N, int K,
+                 const Epilogue& epi, hipStream_t s) {
+  static std::atomic<uint64_t> lds_allowed_q{0};
+  if (!allow_lds((const void*)linear_quad_kernel<MODE, WF>, tq_lds_bytes(WF), lds_allowed_q)) return;
+  // up to 128 leftover rows go through the weight-streaming kernel (see below); more than
+  // that get a last row tile moved up to end at the last row
+  // (unless one more row of tiles fits the last round of workgroups anyway)
+  const int ncol = (N + tq_bn(WF) - 1) / tq_bn(WF);
+  int64_t M_main = M;
+  const int64_t rem = M % TQ_BM;
+  if (rem > 0 && rem <= 128) {
+    const int64_t cus = num_cus(), full = (M / TQ_BM) * ncol;
+    if ((full + ncol + cus - 1) / cus > (full + cus - 1) / cus) M_main = M - rem;
+  }
+  const int nrow = (int)((M_main + TQ_BM - 1) / TQ_BM);
+  // regrouping of a round's 256 tiles: a x b per XCD with a * b = 32, (ncol / a) * (r / b) = 8
+  // for r = 256 / ncol rows per round; taken when it beats the default strip (ncol / 8) x r
+  int rm_a = 0, rm_b = 0, rm_r = 0;
+  if (ncol >= 8 && 256 % ncol == 0) {
+    const int r = 256 / ncol;
+    int best = ncol / 8 + r;
+    for (int a = 1; a <= 32; a *= 2) {
+      const int b = 32 / a;
+      if (ncol % a || r % b || (ncol / a) * (r / b) != 8) continue;
+      if (a + b < best) best = a + b, rm_a = a, rm_b = b, rm_r = r;
+    }
+  }
+  hipLaunchKernelGGL((linear_quad_kernel<MODE, WF>), dim3(ncol, nrow), dim3(TQ_THREADS),
+                     tq_lds_bytes(WF), s, (const half_t*)x, W, M_main, N, K, rm_a, rm_b, rm_r, epi);
+  for (int64_t m0 = M_main; m0 < M; m0 += 64)
+    launch_stream<false, MODE, true>(x, W, scales, nullptr, 1, (int)min((int64_t)64, M - m0), N,
+                                     K, epi, s, m0);
+}
+
 template <bool W8, int MODE>
 void launch_tiled(const void* x, const void* W, const void* scales, int64_t M, int N, int K,
                   const Epilogue& epi, hipStream_t s) {
   // the 256 x 256 kernel once it fills the chip; the 128 x 128 one for the shapes in between
   const int64_t big_tiles = ((M + TB_BM - 1) / TB_BM) * ((N + TB_BN - 1) / TB_BN);
   if constexpr (!W8) {
-    // also below one tile per CU: down to 3/8 of the CUs a single round of these tiles beats the
-    // 128 x 128 kernel on the same product (which runs at a third of this kernel's rate per CU)
-    if (K % 64 == 0 && K >= 128 && big_tiles * 8 >= (int64_t)num_cus() * 3 && M >= TQ_BM) {
-      static std::atomic<uint64_t> lds_allowed_q{0};
-      if (!allow_lds((const void*)linear_quad_kernel<MODE>, TQ_LDS_BYTES, lds_allowed_q)) return;
-      // up to 128 leftover rows go through the weight-streaming kernel (see below); more than
-      // that get a last row tile moved up to end at the last row
-      // (unless one more row of tiles fits the last round of workgroups anyway)
-      const int ncol = (N + TQ_BN - 1) / TQ_BN;
-      int64_t M_main = M;
-      const int64_t rem = M % TQ_BM;
-      if (rem > 0 && rem <= 128) {
-        const int64_t cus = num_cus(), full = (M / TQ_BM) * ncol;
-        if ((full + ncol + cus - 1) / cus > (full + cus - 1) / cus) M_main = M - rem;
+    // Two tile widths, 256 and 128 features.  A workgroup of the narrower one does half the MFMAs in
+    // about 0.8 of the time, so it pays only where all of its tiles run at once (the wide tiles
+    // would then fill less than half of the CUs).  Either is taken down to 3/8 of a tile per CU:
+    // below that a single round of these tiles no longer beats the 128 x 128 kernel on the same
+    // product (which runs at a third of this kernel's rate per CU).
+    if (K % 64 == 0 && K >= 128 && M >= TQ_BM) {
+      const int64_t cus = num_cus(), rows_t = (M + TQ_BM - 1) / TQ_BM;
+      const int64_t t8 = rows_t * ((N + 255) / 256), t4 = rows_t * ((N + 127) / 128);
+      const bool narrow = t4 <= cus;
+      if ((narrow ? t4 : t8) * 8 >= cus * 3) {
+        if (narrow)
+          launch_quad<MODE, 4>(x, W, scales, M, N, K, epi, s);
+        else
+          launch_quad<MODE, 8>(x, W, scales, M, N, K, epi, s);
+        return;
       }
-      const int nrow = (int)((M_main + TQ_BM - 1) / TQ_BM);
-      // regrouping of a round's 256 tiles: a x b per XCD with a * b = 32, (ncol / a) * (r / b) = 8
-      // for r = 256 / ncol rows per round; taken when it beats the default strip (ncol / 8) x r
-      int rm_a = 0, rm_b = 0, rm_r = 0;
-      if (ncol >= 8 && 256 % ncol == 0) {
-        const int r = 256 / ncol;
-        int best = ncol / 8 + r;
-        for (int a = 1; a <= 32; a *= 2) {
-          const int b = 32 / a;
-          if (ncol % a || r % b || (ncol / a) * (r / b) != 8) continue;
-          if (a + b < best) best = a + b, rm_a = a, rm_b = b, rm_r = r;
-        }
-      }
-      hipLaunchKernelGGL((linear_quad_kernel<MODE>), dim3(ncol, nrow), dim3(TQ_THREADS),
-                         TQ_LDS_BYTES, s, (const half_t*)x, W, M_main, N, K, rm_a, rm_b, rm_r, epi);
-      for (int64_t m0 = M_main; m0 < M; m0 += 64)
-        launch_stream<W8, MODE, true>(x, W, scales, nullptr, 1, (int)min((int64_t)64, M - m0), N,
-                                      K, epi, s, m0);
-      return;
     }
   }
   if (K % (2 * TB_BK) == 0 && big_tiles >= num_cus()) {

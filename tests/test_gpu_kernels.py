@@ -371,6 +371,11 @@ LINEAR_SHAPES = [
     (300, 32768, 128), (420, 32768, 128),
     # 64 and 44 bottom rows with few tiles per workgroup: the streaming kernel's four-tile groups
     (4160, 4096, 256), (4140, 8192, 128),
+    # exactly one full round of 256 x 256 tiles, also with a moved-up bottom tile
+    (2048, 8192, 128), (2000, 8192, 192),
+    # few enough tiles that the 256 x 128 ones all run at once: one row over four row tiles (moved-up
+    # tile in the same round), a moved-up tile over most of its neighbour, a ragged right tile
+    (1025, 4096, 256), (700, 6144, 128), (512, 16016, 192),
 ]
 
 
