@@ -1512,24 +1512,15 @@ void launch_stream(const void* xp, const void* W, const void* scales, float* par
   }
 }
 
-// One launch of the four-wave kernel (WF = 8: 256 x 256 tiles, WF = 4: 256 x 128) plus, for a
-// ragged bottom of at most 128 rows that does not fit the last round of workgroups, the streaming
-// kernel on those rows.
+// One launch of the four-wave kernel (WF = 8: 256 x 256 tiles, WF = 4: 256 x 128) on rows
+// 0 .. M_main - 1 (a ragged last row tile is moved up) plus the streaming kernel on the rows from
+// M_main on (at most 128).
 template <int MODE, int WF>
-void launch_quad(const void* x, const void* W, const void* scales, int64_t M, int N, int K,
-                 const Epilogue& epi, hipStream_t s) {
+void launch_quad(const void* x, const void* W, const void* scales, int64_t M, int64_t M_main, int N,
+                 int K, const Epilogue& epi, hipStream_t s) {
   static std::atomic<uint64_t> lds_allowed_q{0};
   if (!allow_lds((const void*)linear_quad_kernel<MODE, WF>, tq_lds_bytes(WF), lds_allowed_q)) return;
-  // up to 128 leftover rows go through the weight-streaming kernel (see below); more than
-  // that get a last row tile moved up to end at the last row
-  // (unless one more row of tiles fits the last round of workgroups anyway)
   const int ncol = (N + tq_bn(WF) - 1) / tq_bn(WF);
-  int64_t M_main = M;
-  const int64_t rem = M % TQ_BM;
-  if (rem > 0 && rem <= 128) {
-    const int64_t cus = num_cus(), full = (M / TQ_BM) * ncol;
-    if ((full + ncol + cus - 1) / cus > (full + cus - 1) / cus) M_main = M - rem;
-  }
   const int nrow = (int)((M_main + TQ_BM - 1) / TQ_BM);
   // regrouping of a round's 256 tiles: a x b per XCD with a * b = 32, (ncol / a) * (r / b) = 8
   // for r = 256 / ncol rows per round; taken when it beats the default strip (ncol / 8) x r
@@ -1556,20 +1547,36 @@ void launch_tiled(const void* x, const void* W, const void* scales, int64_t M, i
   // the 256 x 256 kernel once it fills the chip; the 128 x 128 one for the shapes in between
   const int64_t big_tiles = ((M + TB_BM - 1) / TB_BM) * ((N + TB_BN - 1) / TB_BN);
   if constexpr (!W8) {
-    // Two tile widths, 256 and 128 features.  A workgroup of the narrower one does half the MFMAs in
-    // about 0.8 of the time, so it pays only where all of its tiles run at once (the wide tiles
-    // would then fill less than half of the CUs).  Either is taken down to 3/8 of a tile per CU:
-    // below that a single round of these tiles no longer beats the 128 x 128 kernel on the same
-    // product (which runs at a third of this kernel's rate per CU).
+    // Two tile widths, 256 and 128 features (a workgroup of the narrower one does half the MFMAs in
+    // about 0.8 of the time), and two ways to take a ragged bottom of at most 128 rows: as one more,
+    // moved-up row of tiles, or through the streaming kernel (one sweep over the weights per 64
+    // rows).  The four combinations are priced in rounds of workgroups and the cheapest is taken,
+    // down to 3/8 of a tile per CU: below that a single round of these tiles no longer beats the
+    // 128 x 128 kernel on the same product (which runs at a third of this kernel's rate per CU).
     if (K % 64 == 0 && K >= 128 && M >= TQ_BM) {
-      const int64_t cus = num_cus(), rows_t = (M + TQ_BM - 1) / TQ_BM;
-      const int64_t t8 = rows_t * ((N + 255) / 256), t4 = rows_t * ((N + 127) / 128);
-      const bool narrow = t4 <= cus;
-      if ((narrow ? t4 : t8) * 8 >= cus * 3) {
-        if (narrow)
-          launch_quad<MODE, 4>(x, W, scales, M, N, K, epi, s);
-        else
-          launch_quad<MODE, 8>(x, W, scales, M, N, K, epi, s);
+      const int64_t cus = num_cus(), rem = M % TQ_BM;
+      const int64_t c8 = (N + 255) / 256, c4 = (N + 127) / 128;
+      const double unit = 63.0 * K / 4096;  // us per round of wide tiles
+      const double sweep = (double)N * K * 2 / 5e6 + 4;  // us per streaming launch
+      double best = 1e30;
+      int best_wf = 0;
+      int64_t best_main = M;
+      for (int opt = 0; opt < 4; ++opt) {
+        const bool narrow = opt & 1, stream = opt & 2;
+        if (stream && !(rem > 0 && rem <= 128)) continue;
+        const int64_t m_main = stream ? M - rem : M;
+        const int64_t tiles = ((m_main + TQ_BM - 1) / TQ_BM) * (narrow ? c4 : c8);
+        if (tiles * 8 < cus * 3) continue;
+        const double cost = (double)((tiles + cus - 1) / cus) * (narrow ? 0.8 : 1.0) * unit +
+                            (stream ? (double)((rem + 63) / 64) * sweep : 0.0);
+        if (cost < best) best = cost, best_wf = narrow ? 4 : 8, best_main = m_main;
+      }
+      if (best_wf == 4) {
+        launch_quad<MODE, 4>(x, W, scales, M, best_main, N, K, epi, s);
+        return;
+      }
+      if (best_wf == 8) {
+        launch_quad<MODE, 8>(x, W, scales, M, best_main, N, K, epi, s);
         return;
       }
     }
