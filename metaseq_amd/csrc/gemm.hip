@@ -1295,6 +1295,11 @@ __global__ __launch_bounds__(TQ_THREADS) void linear_quad_kernel(
   // LDS is released); the last MFMAs must have written their accumulators before these are read
   // (the compiler does not see MFMAs inside the asm)
   asm volatile("s_waitcnt vmcnt(0)\n\ts_nop 15\n\ts_nop 15" ::: "memory");
+  // ties every accumulator to this point: none of their reads may be scheduled above the wait
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+#pragma unroll
+    for (int j = 0; j < WF; ++j) asm volatile("" : "+a"(acc[i][j]));
   __syncthreads();  // every wave is done with the operand rings
 
   // D tile (i, j): the lane holds activation row 16 * i + lr of the wave's 128 and the 4 features
