@@ -639,6 +639,38 @@ def test_expand_weight_w8_f16(lib, N, K):
     assert lib.msa_expand_weight_w8_f16(P(G(q)), P(G(sc)), P(got), N, 96, None) == -1
 
 
+def test_qkv_proj_wide_decode_batch_with_row_lengths(lib):
+    """300 rows of one new position each (T = 1) with per-row cache lengths on the device, one
+    row inactive: a row-major product large enough for the four-wave tiled kernel, whose QKV
+    epilogue must append every row at its own length and leave the inactive row's cache alone."""
+    B, H, hd, K, S_cap = 300, 16, 128, 256, 40
+    D = H * hd
+    x, W, b = rnd(B, K, seed=1), rnd(3 * D, K, seed=2, std=0.05), rnd(3 * D, seed=3, std=0.1)
+    g = torch.Generator().manual_seed(4)
+    lens = torch.randint(0, S_cap, (B,), generator=g, dtype=torch.int32)
+    lens[7] = -1
+    kvq = O.linear(x.float(), W.float(), b.float(), r16)
+    k, v, q = kvq.split(D, dim=-1)
+    q = r16(q * (hd ** -0.5))
+    atol = float(kvq.abs().max()) * 2 ** -10
+    Kc = torch.zeros(B, H, S_cap, hd, dtype=torch.float16, device=DEV)
+    Vc = torch.zeros_like(Kc)
+    qo = torch.empty(B, D, dtype=torch.float16, device=DEV)
+    ok(lib.msa_qkv_proj_f16(P(G(x)), P(pack_w(lib, G(W))), P(G(b)), P(qo), P(Kc), P(Vc), B, 1, H,
+                            hd, 0, S_cap, K, 0, P(G(lens)), None), lib)
+    torch.cuda.synchronize()
+    assert_fp16_close(qo, q.half(), atol=atol, what="q")
+    Kh, Vh = Kc.cpu(), Vc.cpu()
+    wantK, wantV = torch.zeros_like(Kh), torch.zeros_like(Vh)
+    for r in range(B):
+        if lens[r] >= 0:
+            wantK[r, :, lens[r]] = k[r].view(H, hd).half()
+            wantV[r, :, lens[r]] = v[r].view(H, hd).half()
+    assert_fp16_close(Kh, wantK, atol=atol, what="K cache")
+    assert_fp16_close(Vh, wantV, atol=atol, what="V cache")
+    assert float(Kh[7].abs().sum()) == 0 and float(Vh[7].abs().sum()) == 0
+
+
 def test_qkv_proj_capacity_error(lib):
     x = torch.zeros(2, 128, dtype=torch.float16, device=DEV)
     rc = lib.msa_qkv_proj_f16(P(x), P(x), P(x), P(x), P(x), P(x), 2, 1, 2, 64, 10, 10, 128, 0,
