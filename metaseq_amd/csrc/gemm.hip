@@ -1063,9 +1063,10 @@ __device__ __forceinline__ void tq_static_for(F&& f) {
 
 // 8 consecutive output columns n..n+7 of row m; v holds the accumulators rounded to fp16, b the
 // bias and r the residual values of those columns (read only where the epilogue has them)
+// (QKV mode: qb, qt = the row's batch row and position, m = qb * T + qt)
 template <int MODE>
 __device__ __forceinline__ void epilogue8(const Epilogue& e, int64_t m, int n, half8_t v,
-                                          half8_t b, half8_t r) {
+                                          half8_t b, half8_t r, int qb, int qt) {
   float t[8];
 #pragma unroll
   for (int i = 0; i < 8; ++i) t[i] = (float)v[i];
@@ -1100,12 +1101,10 @@ __device__ __forceinline__ void epilogue8(const Epilogue& e, int64_t m, int n, h
 #pragma unroll
       for (int i = 0; i < 8; ++i) o[i] = (half_t)t[i];
       const int h = e.hd_shift >= 0 ? c >> e.hd_shift : c / e.hd, d = c - h * e.hd;
-      const int mi = (int)m;
-      const int bb = e.T == 1 ? mi : mi / e.T, tt = mi - bb * e.T;
-      const int s0 = e.len_dev ? e.len_dev[bb] : e.S0;
-      if (s0 >= 0 && s0 + tt < e.S_cap) {
+      const int s0 = e.len_dev ? e.len_dev[qb] : e.S0;
+      if (s0 >= 0 && s0 + qt < e.S_cap) {
         half_t* dst = (part == 0 ? e.Kc : e.Vc) +
-                      (((int64_t)bb * e.H + h) * e.S_cap + s0 + tt) * e.hd + d;
+                      (((int64_t)qb * e.H + h) * e.S_cap + s0 + qt) * e.hd + d;
         *reinterpret_cast<half8_t*>(dst) = o;
       }
     }
@@ -1332,6 +1331,14 @@ __global__ __launch_bounds__(TQ_THREADS) void linear_quad_kernel(
   };
 #pragma unroll
   for (int i = 0; i < TQ_RES_AHEAD; ++i) load_res(i, res8[i]);
+  // QKV mode: the lane's rows come ERPI apart, so (batch row, position) of a row follow from the
+  // previous row's without a division
+  int qb = 0, qt = 0;
+  if (MODE == MODE_QKV) {
+    const int mf = (int)(m0 + wm * 128 + erow);
+    qb = epi.T == 1 ? mf : mf / epi.T;
+    qt = mf - qb * epi.T;
+  }
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
     char* buf = mine + (i & 1) * 4096;
@@ -1350,7 +1357,11 @@ __global__ __launch_bounds__(TQ_THREADS) void linear_quad_kernel(
                                                           ((ec ^ (row & (ECH - 1))) * 16));
       const int64_t m = m0 + wm * 128 + i * 16 + row;
       if (col_ok && m >= m_own)
-        epilogue8<MODE>(epi, m, en, v, bias8, res8[i % TQ_RES_AHEAD][r]);
+        epilogue8<MODE>(epi, m, en, v, bias8, res8[i % TQ_RES_AHEAD][r], qb, qt);
+      if (MODE == MODE_QKV) {
+        qt += ERPI;
+        while (qt >= epi.T) qt -= epi.T, ++qb;
+      }
     }
     if (i + TQ_RES_AHEAD < 8) load_res(i + TQ_RES_AHEAD, res8[i % TQ_RES_AHEAD]);
   }
