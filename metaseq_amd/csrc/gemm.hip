@@ -1130,8 +1130,11 @@ __global__ __launch_bounds__(TQ_THREADS) void linear_quad_kernel(
       by = round * rm_r + (xcd / gx) * rm_b + k / rm_a;
     }
   }
+  // The narrowest form (WF = 2) also serves fewer than 256 rows: it does not move a ragged tile up
+  // but repeats the last row in its loads and drops the rows past it in the epilogue.
+  constexpr bool CLAMP = WF == 2;
   const int64_t m_own = (int64_t)by * TQ_BM;  // first row this tile owns
-  const int64_t m0 = m_own + TQ_BM > M ? M - TQ_BM : m_own;
+  const int64_t m0 = !CLAMP && m_own + TQ_BM > M ? M - TQ_BM : m_own;
   const int n0 = bx * TQ_BN;
   const int nst = K / 64, nks = K / 32;
   const int ntiles = N / 16;
@@ -1144,8 +1147,10 @@ __global__ __launch_bounds__(TQ_THREADS) void linear_quad_kernel(
   const char* xb[8];
   const char* wb[WL];
 #pragma unroll
-  for (int i = 0; i < 8; ++i)
-    xb[i] = (const char*)(x + (m0 + wave * 64 + i * 8) * K) - (i - 4) * 1024;
+  for (int i = 0; i < 8; ++i) {
+    const int64_t r = m0 + wave * 64 + i * 8;
+    xb[i] = (const char*)(x + (CLAMP ? min(r, M - 1) : r) * K) - (i - 4) * 1024;
+  }
 #pragma unroll
   for (int j = 0; j < WL; ++j) {
     const int tt = min(n0 / 16 + wave * WL + j, ntiles - 1);
@@ -1155,10 +1160,21 @@ __global__ __launch_bounds__(TQ_THREADS) void linear_quad_kernel(
   const uint32_t xlane0 = xrow + (((lane & 7) ^ (lane >> 4)) * 16);
   const uint32_t xlane1 = xrow + (((lane & 7) ^ (4 + (lane >> 4))) * 16);
   const uint32_t wlane = lane * 16;
+  // CLAMP: per instruction, the lane's row offset from the (clamped) scalar base row
+  uint32_t xl[CLAMP ? 8 : 1];
+  if (CLAMP) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int64_t r = m0 + wave * 64 + i * 8;
+      const int64_t d = min(r + (lane >> 3), M - 1) - min(r, M - 1);
+      xl[i] = (uint32_t)d * (uint32_t)K * 2 + ((i & 1 ? xlane1 : xlane0) - xrow);
+    }
+  }
   const uint32_t lds0 = (uint32_t)(uintptr_t)(tq_lds_void*)tq_lds;
-  uint32_t xv0 = 0, xv1 = 0, wv = 0;  // lane offsets of the group being issued
+  uint32_t xv0 = 0, xv1 = 0, wv = 0, xst = 0;  // lane offsets of the group being issued
   auto set_x = [&](int slot, int st) {
     st = min(st, nst - 1);
+    xst = st * 128;
     xv0 = xlane0 + st * 128;
     xv1 = xlane1 + st * 128;
     asm volatile("s_mov_b32 m0, %0" ::"s"(lds0 + slot * TQ_XBYTES + wave * (64 * 128) + 4096)
@@ -1172,7 +1188,7 @@ __global__ __launch_bounds__(TQ_THREADS) void linear_quad_kernel(
   };
   auto issue_x = [&](auto ic) {
     constexpr int i = decltype(ic)::value;
-    const uint32_t vo = i & 1 ? xv1 : xv0;
+    const uint32_t vo = CLAMP ? xl[CLAMP ? i : 0] + xst : (i & 1 ? xv1 : xv0);
     const char* sb = xb[i];
     asm volatile("global_load_lds_dwordx4 %0, %1 offset:%2" ::"v"(vo), "s"(sb),
                  "n"((i - 4) * 1024)
@@ -1256,8 +1272,10 @@ __global__ __launch_bounds__(TQ_THREADS) void linear_quad_kernel(
         if (j == 1) xf[H ^ 1][i] = H == 0 ? xfrag(xs, 1, i) : xfrag(xnext, 0, i);
         if constexpr (WF == 8) {
           if (j == 5) wf[H ^ 1][i % WF] = wfrag(wnext, i % WF);
-        } else {
+        } else if constexpr (WF == 4) {
           if constexpr (j == 3 && (i & 1)) wf[H ^ 1][(i >> 1) % WF] = wfrag(wnext, (i >> 1) % WF);
+        } else {
+          if constexpr (j == 0 && (i == 1 || i == 5)) wf[H ^ 1][(i >> 2) % WF] = wfrag(wnext, (i >> 2) % WF);
         }
         if constexpr (H == 0) {
           if (i == 0 && j == 0) set_x(xfree, S + 2);
@@ -1266,17 +1284,21 @@ __global__ __launch_bounds__(TQ_THREADS) void linear_quad_kernel(
           if (i == 4 && j == 0) set_w(ws, t + TQ_RW);
           if constexpr (WF == 8) {
             if constexpr (i >= 4 && j == 3) issue_w(std::integral_constant<int, (i & 3) % WL>{});
-          } else {
+          } else if constexpr (WF == 4) {
             if constexpr ((i == 4 || i == 6) && j == 2)
-              issue_w(std::integral_constant<int, (i >> 1) & 1>{});
+              issue_w(std::integral_constant<int, ((i >> 1) & 1) % WL>{});
+          } else {
+            if constexpr (i == 4 && j == 1) issue_w(std::integral_constant<int, 0>{});
           }
         } else {
           if (i == 0 && j == 0) set_w(ws, t + TQ_RW);
           if constexpr (WF == 8) {
             if constexpr (j == 3 && (i & 1)) issue_w(std::integral_constant<int, (i >> 1) % WL>{});
-          } else {
+          } else if constexpr (WF == 4) {
             if constexpr ((i == 2 || i == 6) && j == 2)
-              issue_w(std::integral_constant<int, (i >> 2) & 1>{});
+              issue_w(std::integral_constant<int, ((i >> 2) & 1) % WL>{});
+          } else {
+            if constexpr (i == 2 && j == 1) issue_w(std::integral_constant<int, 0>{});
           }
         }
       });
@@ -1325,7 +1347,7 @@ __global__ __launch_bounds__(TQ_THREADS) void linear_quad_kernel(
 #pragma unroll
     for (int r = 0; r < ENR; ++r) {
       const int64_t m = m0 + wm * 128 + i * 16 + ERPI * r + erow;
-      if (col_ok && m >= m_own)
+      if (col_ok && m >= m_own && m < M)
         dst[r] = *reinterpret_cast<const half8_t*>(epi.residual + m * epi.N + en);
     }
   };
@@ -1356,7 +1378,7 @@ __global__ __launch_bounds__(TQ_THREADS) void linear_quad_kernel(
       const half8_t v = *reinterpret_cast<const half8_t*>(buf + row * ERB +
                                                           ((ec ^ (row & (ECH - 1))) * 16));
       const int64_t m = m0 + wm * 128 + i * 16 + row;
-      if (col_ok && m >= m_own)
+      if (col_ok && m >= m_own && m < M)
         epilogue8<MODE>(epi, m, en, v, bias8, res8[i % TQ_RES_AHEAD][r], qb, qt);
       if (MODE == MODE_QKV) {
         qt += ERPI;
@@ -1563,38 +1585,38 @@ void launch_tiled(const void* x, const void* W, const void* scales, int64_t M, i
   // the 256 x 256 kernel once it fills the chip; the 128 x 128 one for the shapes in between
   const int64_t big_tiles = ((M + TB_BM - 1) / TB_BM) * ((N + TB_BN - 1) / TB_BN);
   if constexpr (!W8) {
-    // Two tile widths, 256 and 128 features (a workgroup of the narrower one does half the MFMAs in
-    // about 0.8 of the time), and two ways to take a ragged bottom of at most 128 rows: as one more,
-    // moved-up row of tiles, or through the streaming kernel (one sweep over the weights per 64
-    // rows).  The four combinations are priced in rounds of workgroups and the cheapest is taken,
-    // down to 3/8 of a tile per CU: below that a single round of these tiles no longer beats the
-    // 128 x 128 kernel on the same product (which runs at a third of this kernel's rate per CU).
-    if (K % 64 == 0 && K >= 128 && M >= TQ_BM) {
+    // Three tile widths, 256, 128 and 64 features (a workgroup of 128 does half the MFMAs of 256 in
+    // about 0.8 of the time, one of 64 a quarter in about 0.55), and two ways to take a ragged
+    // bottom of at most 128 rows: as one more, moved-up row of tiles, or through the streaming
+    // kernel (one sweep over the weights per 64 rows).  The combinations are priced in rounds of
+    // workgroups and the cheapest is taken.  The two wider forms go down to 3/8 of a tile per CU:
+    // below that a single round of their tiles no longer beats the narrowest form, which is taken
+    // down to 1/8 of a tile per CU and also serves 65 .. 255 rows (it repeats the last row instead
+    // of moving a tile up); below that the 128 x 128 kernel runs.
+    if (K % 64 == 0 && K >= 128 && M > 64) {
       const int64_t cus = num_cus(), rem = M % TQ_BM;
-      const int64_t c8 = (N + 255) / 256, c4 = (N + 127) / 128;
+      const int64_t cols[3] = {(N + 255) / 256, (N + 127) / 128, (N + 63) / 64};
+      const double factor[3] = {1.0, 0.8, 0.55};
       const double unit = 63.0 * K / 4096;  // us per round of wide tiles
       const double sweep = (double)N * K * 2 / 5e6 + 4;  // us per streaming launch
       double best = 1e30;
-      int best_wf = 0;
+      int best_w = -1;
       int64_t best_main = M;
-      for (int opt = 0; opt < 4; ++opt) {
-        const bool narrow = opt & 1, stream = opt & 2;
-        if (stream && !(rem > 0 && rem <= 128)) continue;
+      for (int opt = 0; opt < 6; ++opt) {
+        const int w = opt >> 1;
+        const bool stream = opt & 1;
+        if (w < 2 && M < TQ_BM) continue;
+        if (stream && !(w < 2 && rem > 0 && rem <= 128 && M - rem >= TQ_BM)) continue;
         const int64_t m_main = stream ? M - rem : M;
-        const int64_t tiles = ((m_main + TQ_BM - 1) / TQ_BM) * (narrow ? c4 : c8);
-        if (tiles * 8 < cus * 3) continue;
-        const double cost = (double)((tiles + cus - 1) / cus) * (narrow ? 0.8 : 1.0) * unit +
+        const int64_t tiles = ((m_main + TQ_BM - 1) / TQ_BM) * cols[w];
+        if (tiles * 8 < (w == 2 ? cus : cus * 3)) continue;
+        const double cost = (double)((tiles + cus - 1) / cus) * factor[w] * unit +
                             (stream ? (double)((rem + 63) / 64) * sweep : 0.0);
-        if (cost < best) best = cost, best_wf = narrow ? 4 : 8, best_main = m_main;
+        if (cost < best) best = cost, best_w = w, best_main = m_main;
       }
-      if (best_wf == 4) {
-        launch_quad<MODE, 4>(x, W, scales, M, best_main, N, K, epi, s);
-        return;
-      }
-      if (best_wf == 8) {
-        launch_quad<MODE, 8>(x, W, scales, M, best_main, N, K, epi, s);
-        return;
-      }
+      if (best_w == 0) return launch_quad<MODE, 8>(x, W, scales, M, best_main, N, K, epi, s);
+      if (best_w == 1) return launch_quad<MODE, 4>(x, W, scales, M, best_main, N, K, epi, s);
+      if (best_w == 2) return launch_quad<MODE, 2>(x, W, scales, M, best_main, N, K, epi, s);
     }
   }
   if (K % (2 * TB_BK) == 0 && big_tiles >= num_cus()) {

@@ -376,6 +376,9 @@ LINEAR_SHAPES = [
     # few enough tiles that the 256 x 128 ones all run at once: one row over four row tiles (moved-up
     # tile in the same round), a moved-up tile over most of its neighbour, a ragged right tile
     (1025, 4096, 256), (700, 6144, 128), (512, 16016, 192),
+    # the 256 x 64 form: fewer than 256 rows (the last row repeated in the loads), a ragged right
+    # tile, more than 256 rows with a ragged bottom that is not moved up
+    (128, 4096, 256), (100, 2304, 128), (65, 2064, 192), (255, 6144, 64), (300, 4096, 128),
 ]
 
 

@@ -97,6 +97,8 @@ def test_prefill_gemm_random_shapes(lib):
         N = 256 * ncol - 16 * rng.choice([0, 0, 1, 5, 15])
         nrow = max(1, 100 // ncol) if small else -(-256 // ncol) + rng.choice([0, 1, 3])
         M = max(256, 256 * nrow - rng.choice([0, 0, 1, 100, 128, 129, 200, 255]))
+        if it % 6 == 4:
+            M = rng.choice([65, 100, 128, 200, 255])  # fewer rows than a tile: the 256 x 64 form
         K = 64 * rng.choice([2, 3, 4, 5, 8, 12])
         relu, use_res = rng.random() < 0.4, rng.random() < 0.6
         in_place = use_res and rng.random() < 0.5
