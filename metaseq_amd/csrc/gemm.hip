@@ -1037,16 +1037,21 @@ __global__ __launch_bounds__(TB_THREADS) void linear_tiled_big_kernel(
 // Workgroup -> tile: consecutive workgroups land on consecutive XCDs; where the default order would
 // give an XCD a long thin strip of a round's tiles, the 256 tiles of a round are regrouped so that
 // every XCD's L2 serves a compact a x b block (rm_a, rm_b, rm_r from the host).
-// Needs K % 64 == 0, K >= 128, M >= 256 (a ragged last row tile is moved up to end at M and stores
-// only the rows no other tile owns).
+// Three widths of the workgroup's tile, by the number WF of 16-feature weight fragments per wave:
+// 8 -> 256 x 256 (as described), 4 -> 256 x 128, 2 -> 256 x 64 (fewer accumulators, weight loads and
+// MFMAs per step; the same activation stages).  The two wider forms need M >= 256: a ragged last
+// row tile is moved up to end at M and stores only the rows no other tile owns.  The narrowest
+// form repeats the last row in its loads instead and drops the rows past it, so it also serves
+// fewer than 256 rows.  All need K % 64 == 0, K >= 128.
 constexpr int TQ_BM = 256, TQ_THREADS = 256;
 constexpr int TQ_RX = 3, TQ_RW = 4;
 constexpr int TQ_XBYTES = TQ_BM * 64 * 2;       // one 64-wide stage of activations
 constexpr int TQ_WOFF = TQ_RX * TQ_XBYTES;
-// WF = weight fragments (16-feature tiles) per wave: 8 -> 256 features per workgroup, 4 -> 128
 constexpr int tq_bn(int WF) { return 32 * WF; }
 constexpr int tq_wbytes(int WF) { return 2 * WF * 1024; }  // one 32-wide step of weights
-constexpr int tq_lds_bytes(int WF) { return TQ_RX * TQ_XBYTES + TQ_RW * tq_wbytes(WF); }  // 160 / 128 KB
+constexpr int tq_lds_bytes(int WF) {  // 160 / 128 / 112 KB
+  return TQ_RX * TQ_XBYTES + TQ_RW * tq_wbytes(WF);
+}
 typedef __attribute__((address_space(3))) void tq_lds_void;
 
 #define TQ_MFMA(ACC, A, B) \
