@@ -642,11 +642,13 @@ def test_expand_weight_w8_f16(lib, N, K):
     assert lib.msa_expand_weight_w8_f16(P(G(q)), P(G(sc)), P(got), N, 96, None) == -1
 
 
-def test_qkv_proj_wide_decode_batch_with_row_lengths(lib):
-    """300 rows of one new position each (T = 1) with per-row cache lengths on the device, one
-    row inactive: a row-major product large enough for the four-wave tiled kernel, whose QKV
-    epilogue must append every row at its own length and leave the inactive row's cache alone."""
-    B, H, hd, K, S_cap = 300, 16, 128, 256, 40
+@pytest.mark.parametrize("B", [300, 130])
+def test_qkv_proj_wide_decode_batch_with_row_lengths(lib, B):
+    """300 (130) rows of one new position each (T = 1) with per-row cache lengths on the device,
+    one row inactive: a row-major product for the four-wave tiled kernel (more and fewer rows than
+    one of its tiles), whose QKV epilogue must append every row at its own length and leave the
+    inactive row's cache alone."""
+    H, hd, K, S_cap = 16, 128, 256, 40
     D = H * hd
     x, W, b = rnd(B, K, seed=1), rnd(3 * D, K, seed=2, std=0.05), rnd(3 * D, seed=3, std=0.1)
     g = torch.Generator().manual_seed(4)
