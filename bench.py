@@ -135,6 +135,8 @@ def cpu_baseline(warm=5, timed=5, seed=1234):
     return {
         "value": B * G / mean, "unit": "tokens/s", "cores": cores, "kind": "port",
         "timing": "measured",
+        # another model, batch and context than the GPU headline: not a speed-up denominator
+        "comparable_to_headline": False,
         "cpu": _cpu_model(),
         "sample": ("oracle restatement of the reference forward + greedy loop, fp32, on the "
                    "reference's CPU-runnable case: OPT-125m, batch %d, prompt EOS+%d, %d generated "
@@ -263,6 +265,10 @@ def main():
                     help="timed decode steps (default: the workload's generation length minus "
                          "the warm-up steps, so warm-up + timed = the configured decode length)")
     ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--repeats", type=int, default=5,
+                    help="how many times the window of exactly --steps timed steps is run (over "
+                         "the same contexts: the cache length is wound back); ms_per_step is "
+                         "their mean, reported with its standard deviation and minimum")
     ap.add_argument("--config", default="6.7b", choices=sorted(CONFIGS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-same-shape", action="store_true",
@@ -386,23 +392,36 @@ def main():
         step += 1
     torch.cuda.synchronize()
     S_first = step + 1  # positions attended by the first timed forward
+    cache = decoder.get_cache(inc)
+    start_step, start_len, start_logits = step, cache.length, step_logits
+    R = max(1, args.repeats) if st is None else 1  # a replayed graph keeps its length on the device
+    walls, gpus = [], []
     ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    wall0 = time.perf_counter()
-    ev0.record()
-    for _ in range(K):
-        step_logits = one_step(step, step_logits)
-        step += 1
-    ev1.record()
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - wall0
-    gpu_s = ev0.elapsed_time(ev1) / 1e3
-    t_step = wall / K
+    for _ in range(R):
+        # every window times exactly K steps over the same contexts: wind the history back (the
+        # steps are deterministic, so they rewrite the same tokens, keys and values)
+        step, cache.length, step_logits = start_step, start_len, start_logits
+        torch.cuda.synchronize()
+        wall0 = time.perf_counter()
+        ev0.record()
+        for _ in range(K):
+            step_logits = one_step(step, step_logits)
+            step += 1
+        ev1.record()
+        torch.cuda.synchronize()
+        walls.append((time.perf_counter() - wall0) / K)
+        gpus.append(ev0.elapsed_time(ev1) / 1e3 / K)
+    t_step = sum(walls) / R
+    t_std = (sum((w - t_step) ** 2 for w in walls) / R) ** 0.5
+    gpu_s = sum(gpus) / R * K
     S_last = step
     S_mean = (S_first + S_last) / 2.0
     bytes_mean = sum(step_bytes(cfg, B, s, int8) for s in range(S_first, S_last + 1)) / K
+    fracs = [bytes_mean / w / HBM_PEAK for w in walls]
+    frac_mean = sum(fracs) / R
+    frac_std = (sum((f - frac_mean) ** 2 for f in fracs) / R) ** 0.5
 
     # ---- live timing of the dominant kernel: decode attention over every layer's cache ----
-    cache = decoder.get_cache(inc)
     S_probe = cache.length
     D, H, hd = cfg.decoder_embed_dim, cfg.decoder_attention_heads, cfg.head_dim
     q = torch.randn(B, D, device=dev).half()
@@ -428,16 +447,93 @@ def main():
     achieved = ab / attn_s / 1e9
 
     # ---- what a plain streaming read reaches on this GPU (context for the fractions of the
-    # published peak): 4 GiB read once per launch by the library's probe kernel
+    # published peak): the library's probe kernel over slices of a 4 GiB region, one launch per
+    # slice so that every launch reads cold memory, as the step's kernels do
     probe = torch.empty(1 << 31, dtype=torch.float16, device=dev).zero_()
-    _capi.check(lib.msa_probe_stream_read(probe.data_ptr(), probe.numel() * 2, stream))
-    torch.cuda.synchronize()
-    a0.record()
-    for _ in range(5):
-        _capi.check(lib.msa_probe_stream_read(probe.data_ptr(), probe.numel() * 2, stream))
-    a1.record()
-    torch.cuda.synchronize()
-    stream_read = probe.numel() * 2 / (a0.elapsed_time(a1) / 1e3 / 5) / 1e9
+    probe_bytes = probe.numel() * 2
+
+    def loop_time(fn, n):
+        """Average seconds per call of fn(i), i = 0 .. n - 1, after one untimed round."""
+        for i in range(n):
+            fn(i)
+        torch.cuda.synchronize()
+        a0.record()
+        for i in range(n):
+            fn(i)
+        a1.record()
+        torch.cuda.synchronize()
+        return a0.elapsed_time(a1) / 1e3 / n
+
+    def plain_read_GBps(nbytes):
+        nbytes = max(16, min(probe_bytes, int(nbytes)) // 16 * 16)
+        slices = max(1, probe_bytes // nbytes)
+        n = max(5, min(slices, 64))
+        t = loop_time(lambda i: _capi.check(lib.msa_probe_stream_read(
+            probe.data_ptr() + (i % slices) * nbytes, nbytes, stream)), n)
+        return nbytes / t / 1e9
+
+    stream_read = plain_read_GBps(probe_bytes)
+    attn_ceiling = plain_read_GBps(ab)
+
+    # ---- the step's other kernels, each timed live over every layer's weights in turn (cold
+    # reads, as in the step) next to a plain read of the same number of bytes
+    kernels = {"attention": {"bytes": ab, "us": attn_s * 1e6, "GBps": achieved,
+                             "frac_of_peak": achieved * 1e9 / HBM_PEAK,
+                             "plain_read_GBps_at_size": attn_ceiling,
+                             "frac_of_plain_read": achieved / attn_ceiling}}
+    if B <= 64:
+        from metaseq_amd._capi import MSA_IN_PACKED, MSA_OUT_PACKED
+        F, L, V = cfg.decoder_ffn_embed_dim, cfg.decoder_layers, cfg.vocab_size
+        wb = 1 if int8 else 2
+        bufs = decoder._step_buffers(cache, B)
+        layers = decoder.layers
+        S0 = cache.length - 1
+        IN, OUT = MSA_IN_PACKED, MSA_OUT_PACKED
+        tok1 = torch.zeros(B, dtype=torch.long, device=dev)
+        sc1 = torch.zeros(B, dtype=torch.float32, device=dev)
+        fin1 = torch.zeros(B, dtype=torch.uint8, device=dev)
+
+        def lm_head(i):
+            decoder._select_from(lib, bufs["h"], B, 1.0, [1], [], fin1, None, False, 2, tok1, 1,
+                                 sc1, 1, None)
+        flush_bytes = 1 << 29  # evicts the one vocabulary matrix between its launches
+
+        def flush(i):
+            _capi.check(lib.msa_probe_stream_read(probe.data_ptr() + (i % 4) * flush_bytes,
+                                                  flush_bytes, stream))
+        t_flush = loop_time(flush, 8)
+        t_lm = loop_time(lambda i: (flush(i), lm_head(i)), 8) - t_flush
+        timed = {
+            "qkv_proj": (3 * D * D * wb, loop_time(lambda i: decoder._qkv(
+                lib, stream, bufs["h"], layers[i].self_attn.qkv_proj, bufs["q"], cache.k(i),
+                cache.v(i), B, 1, H, hd, S0, cache.capacity, D, IN, None), L)),
+            "out_proj (split-K partial sums)": (D * D * wb, loop_time(
+                lambda i: decoder._linear_partial(lib, stream, bufs["o"],
+                                                  layers[i].self_attn.out_proj, bufs["part"], B,
+                                                  D, D, bufs["S_o"]), L)),
+            "fc1": (F * D * wb, loop_time(lambda i: decoder._linear(
+                lib, stream, bufs["h"], layers[i].fc1, B, F, D, relu=True, out=bufs["u"],
+                flags=IN | OUT), L)),
+            "fc2 (split-K partial sums)": (D * F * wb, loop_time(
+                lambda i: decoder._linear_partial(lib, stream, bufs["u"], layers[i].fc2,
+                                                  bufs["part"], B, D, F, bufs["S_f"]), L)),
+            "vocabulary projection + selection": (V * D * 2, t_lm),
+        }
+        for name, (nbytes, t) in timed.items():
+            ceiling = plain_read_GBps(nbytes)
+            kernels[name] = {"bytes": nbytes, "us": t * 1e6, "GBps": nbytes / t / 1e9,
+                             "frac_of_peak": nbytes / t / HBM_PEAK,
+                             "plain_read_GBps_at_size": ceiling,
+                             "frac_of_plain_read": nbytes / t / 1e9 / ceiling}
+        t_ln = loop_time(lambda i: _capi.check(lib.msa_residual_layernorm_f16(
+            bufs["part"].data_ptr(), bufs["S_o"], layers[i].self_attn.out_proj.bias.data_ptr(),
+            bufs["x"].data_ptr(), layers[i].final_layer_norm.weight.data_ptr(),
+            layers[i].final_layer_norm.bias.data_ptr(), bufs["h"].data_ptr(), B, D, 1e-5, OUT,
+            stream)), L)
+        kernels["bias + residual + LayerNorm tail"] = {"bytes": 0, "us": t_ln * 1e6,
+                                                        "launches_per_layer": 2}
+        per_layer = (attn_s + sum(timed[k][1] for k in timed if "vocabulary" not in k) + 2 * t_ln)
+        kernels["sum_of_kernels_ms_per_step"] = (L * per_layer + t_lm + t_ln) * 1e3
     del probe
 
     result = {
@@ -450,6 +546,10 @@ def main():
         "steps": K,
         "warmup": W,
         "ms_per_step": t_step * 1e3,
+        "ms_per_step_std": t_std * 1e3,
+        "ms_per_step_min": min(walls) * 1e3,
+        "ms_per_step_windows": [w * 1e3 for w in walls],
+        "repeats": R,
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
@@ -460,7 +560,10 @@ def main():
                         "steps attend %d..%d positions" % (size, B, P, S_first, S_last),
             "layers": cfg.decoder_layers, "d_model": D, "heads": H, "vocab": cfg.vocab_size,
         },
-        "hbm_frac_step": bytes_mean / t_step / HBM_PEAK,
+        "hbm_frac_step": frac_mean,
+        "hbm_frac_step_std": frac_std,
+        "hbm_frac_step_mean_minus_std": frac_mean - frac_std,
+        "hbm_frac_step_best_window": max(fracs),
         "step_bytes_mean": bytes_mean,
         "gpu_ms_per_step": gpu_s / K * 1e3,
         "graph_replay": st is not None,
@@ -477,6 +580,7 @@ def main():
             "bytes_per_launch": ab, "avg_launch_us": attn_s * 1e6, "context": S_probe,
             "plain_stream_read_GBps": stream_read,
         },
+        "kernels": kernels,
     }
     if args.torch_eager and not int8:
         del inc, cache

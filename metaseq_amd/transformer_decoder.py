@@ -124,6 +124,10 @@ class TransformerDecoder(nn.Module):
         self.layer_norm = _Affine((D,), (D,), device)
         self.inference = True
         self.return_inner_states = False
+        # instrumentation: called as layer_probe(i, x) with the residual stream [B * T, D] after
+        # layer i of a pass over row-major activations (prefill); the tensor is overwritten by
+        # the next layer, so a probe that keeps it must copy
+        self.layer_probe = None
         # decode steps of at most 64 rows go through msa_decoder_step (one C call per token);
         # False drives the same kernels entry point by entry point from Python
         self.native_step = True
@@ -449,12 +453,9 @@ class TransformerDecoder(nn.Module):
         depends on the step, so the sequence can be captured once and replayed.  The new tokens
         are the last column of ``tokens`` (or column ``len_dev[b]`` with ``col_from_len``)."""
         cfg = self.cfg
-        D, H, hd = cfg.decoder_embed_dim, cfg.decoder_attention_heads, cfg.head_dim
-        F, L, M = cfg.decoder_ffn_embed_dim, cfg.decoder_layers, B
-        x, q, h, o, u, part = (bufs[k] for k in ("x", "q", "h", "o", "u", "part"))
-        S_o, S_f = bufs["S_o"], bufs["S_f"]
-        IN, OUT = MSA_IN_PACKED, MSA_OUT_PACKED
-        mask_stride = mask.stride(0) if mask is not None else 0
+        D, L, M = cfg.decoder_embed_dim, cfg.decoder_layers, B
+        x, h = bufs["x"], bufs["h"]
+        OUT = MSA_OUT_PACKED
         # a row whose new token is a pad sits this step out (step_len = -1), as does an
         # inactive row; under graph replay there are no pads and the lengths are used as is
         step_len = bufs["step_len"] if (len_dev is not None and not col_from_len) else None
@@ -466,44 +467,58 @@ class TransformerDecoder(nn.Module):
                                 MSA_EMBED_COL_FROM_LEN if col_from_len else 0, stream))
         if step_len is not None:
             len_dev = step_len
-        ld = ptr(len_dev)
         self._layernorm(lib, stream, x, self.layers[0].self_attn_layer_norm, M, D, h, OUT)
         x_last = None
         feat = h
         for i, layer in enumerate(self.layers):
-            kc, vc = cache.k(i), cache.v(i)
-            self._qkv(lib, stream, h, layer.self_attn.qkv_proj, q, kc, vc, B, 1, H, hd, S0,
-                      cache.capacity, D, IN, len_dev)
-            check(lib.msa_attention_f16(ptr(q), ptr(kc), ptr(vc), ptr(mask), mask_stride, ptr(o),
-                                        B, H, hd, 1, S0, cache.capacity, OUT, ld, stream))
-            op = layer.self_attn.out_proj
-            self._linear_partial(lib, stream, o, op, part, M, D, D, S_o)
-            ln = layer.final_layer_norm
-            check(lib.msa_residual_layernorm_f16(ptr(part), S_o, ptr(op.bias), ptr(x),
-                                                 ptr(ln.weight), ptr(ln.bias), ptr(h), M, D, 1e-5,
-                                                 OUT, stream))
-            self._linear(lib, stream, h, layer.fc1, M, F, D, relu=True, out=u, flags=IN | OUT)
-            self._linear_partial(lib, stream, u, layer.fc2, part, M, D, F, S_f)
             last = i + 1 == L
             ln = self.layer_norm if last else self.layers[i + 1].self_attn_layer_norm
-            b2 = layer.fc2.bias
             if last and self.return_inner_states:
-                check(lib.msa_residual_layernorm_f16(ptr(part), S_f, ptr(b2), ptr(x), None, None,
-                                                     None, M, D, 1e-5, 0, stream))
+                self._decode_layer(lib, stream, layer, cache.k(i), cache.v(i), cache.capacity,
+                                   bufs, B, S0, mask, len_dev, None, None, 0)
                 x_last = x.view(B, 1, D).transpose(0, 1).clone()
                 feat = h if want_packed else torch.empty(M, D, dtype=torch.float16,
                                                          device=x.device)
                 self._layernorm(lib, stream, x, ln, M, D, feat, OUT if want_packed else 0)
             elif last and not want_packed:
                 feat = torch.empty(M, D, dtype=torch.float16, device=x.device)
-                check(lib.msa_residual_layernorm_f16(ptr(part), S_f, ptr(b2), ptr(x),
-                                                     ptr(ln.weight), ptr(ln.bias), ptr(feat), M,
-                                                     D, 1e-5, 0, stream))
+                self._decode_layer(lib, stream, layer, cache.k(i), cache.v(i), cache.capacity,
+                                   bufs, B, S0, mask, len_dev, ln, feat, 0)
             else:
-                check(lib.msa_residual_layernorm_f16(ptr(part), S_f, ptr(b2), ptr(x),
-                                                     ptr(ln.weight), ptr(ln.bias), ptr(h), M, D,
-                                                     1e-5, OUT, stream))
+                self._decode_layer(lib, stream, layer, cache.k(i), cache.v(i), cache.capacity,
+                                   bufs, B, S0, mask, len_dev, ln, h, OUT)
         return feat, x_last
+
+    def _decode_layer(self, lib, stream, layer, kc, vc, cap, bufs, B, S0, mask, len_dev, tail_ln,
+                      tail_out, tail_flags):
+        """One layer of a decode step of at most 64 rows (transformer_decoder_layer.py:233-284).
+        In: the residual stream ``bufs["x"]`` (row-major) and its LayerNorm ``bufs["h"]``
+        (packed).  Out: ``x`` updated in place and, through the tail fused behind fc2,
+        ``tail_out = LayerNorm(x; tail_ln)`` - the next layer's input or the decoder's final
+        LayerNorm (``tail_ln`` None: the residual stream only)."""
+        cfg = self.cfg
+        D, H, hd, F = (cfg.decoder_embed_dim, cfg.decoder_attention_heads, cfg.head_dim,
+                       cfg.decoder_ffn_embed_dim)
+        x, q, h, o, u, part = (bufs[k] for k in ("x", "q", "h", "o", "u", "part"))
+        S_o, S_f = bufs["S_o"], bufs["S_f"]
+        IN, OUT = MSA_IN_PACKED, MSA_OUT_PACKED
+        mask_stride = mask.stride(0) if mask is not None else 0
+        self._qkv(lib, stream, h, layer.self_attn.qkv_proj, q, kc, vc, B, 1, H, hd, S0, cap, D,
+                  IN, len_dev)
+        check(lib.msa_attention_f16(ptr(q), ptr(kc), ptr(vc), ptr(mask), mask_stride, ptr(o), B,
+                                    H, hd, 1, S0, cap, OUT, ptr(len_dev), stream))
+        op = layer.self_attn.out_proj
+        self._linear_partial(lib, stream, o, op, part, B, D, D, S_o)
+        ln = layer.final_layer_norm
+        check(lib.msa_residual_layernorm_f16(ptr(part), S_o, ptr(op.bias), ptr(x), ptr(ln.weight),
+                                             ptr(ln.bias), ptr(h), B, D, 1e-5, OUT, stream))
+        self._linear(lib, stream, h, layer.fc1, B, F, D, relu=True, out=u, flags=IN | OUT)
+        self._linear_partial(lib, stream, u, layer.fc2, part, B, D, F, S_f)
+        check(lib.msa_residual_layernorm_f16(
+            ptr(part), S_f, ptr(layer.fc2.bias), ptr(x),
+            ptr(tail_ln.weight) if tail_ln is not None else None,
+            ptr(tail_ln.bias) if tail_ln is not None else None, ptr(tail_out), B, D, 1e-5,
+            tail_flags, stream))
 
     def decode_step_static(self, tokens, cache, len_dev, logits_out):
         """Graph-capturable decode step: embeds column ``len_dev[b]`` of the full ``tokens``
@@ -651,8 +666,7 @@ class TransformerDecoder(nn.Module):
         (anything with ``k(i)``, ``v(i)`` and ``capacity``).  Returns the normalised features
         [B * T, D] and the inner-states list."""
         cfg = self.cfg
-        D, H, hd = cfg.decoder_embed_dim, cfg.decoder_attention_heads, cfg.head_dim
-        F = cfg.decoder_ffn_embed_dim
+        D = cfg.decoder_embed_dim
         dev = tokens.device
         M = B * T
         x = torch.empty(M, D, dtype=torch.float16, device=dev)
@@ -665,30 +679,46 @@ class TransformerDecoder(nn.Module):
         inner_states = [{"tok": None, "pos": positions, "emb": None}]
         if self.return_inner_states:
             inner_states[0]["emb"] = x.view(B, T, D).transpose(0, 1).clone()
-        mask_stride = mask.stride(0) if mask is not None else 0
-        q = torch.empty(M, D, dtype=torch.float16, device=dev)
-        h = torch.empty_like(x)
-        o = torch.empty_like(x)
-        u = torch.empty(M, F, dtype=torch.float16, device=dev)
+        work = self._rows_buffers(M, dev)
         for i, layer in enumerate(self.layers):
-            self._layernorm(lib, stream, x, layer.self_attn_layer_norm, M, D, h)
-            kc, vc = kv.k(i), kv.v(i)
-            self._qkv(lib, stream, h, layer.self_attn.qkv_proj, q, kc, vc, B, T, H, hd, S0,
-                      kv.capacity, D, 0)
-            check(lib.msa_attention_f16(ptr(q), ptr(kc), ptr(vc), ptr(mask), mask_stride,
-                                        ptr(o), B, H, hd, T, S0, kv.capacity, 0, None,
-                                        stream))
-            # x = round(round(o Wo^T + bo) + x)   (transformer_decoder_layer.py:222-230)
-            self._linear(lib, stream, o, layer.self_attn.out_proj, M, D, D, residual=x, out=x)
-            self._layernorm(lib, stream, x, layer.final_layer_norm, M, D, h)
-            self._linear(lib, stream, h, layer.fc1, M, F, D, relu=True, out=u)
-            self._linear(lib, stream, u, layer.fc2, M, D, F, residual=x, out=x)
+            self._rows_layer(lib, stream, layer, x, work, B, T, S0, kv.k(i), kv.v(i),
+                             kv.capacity, mask)
+            if self.layer_probe is not None:
+                self.layer_probe(i, x)
         if self.return_inner_states:
             inner_states.append(x.view(B, T, D).transpose(0, 1).clone())
         else:
             inner_states.append(None)
+        h = work["h"]
         self._layernorm(lib, stream, x, self.layer_norm, M, D, h)
         return h, inner_states
+
+    def _rows_buffers(self, M, dev):
+        """Work buffers of ``_rows_layer`` for M row-major activation rows."""
+        D, F = self.cfg.decoder_embed_dim, self.cfg.decoder_ffn_embed_dim
+        f16 = dict(dtype=torch.float16, device=dev)
+        return {"q": torch.empty(M, D, **f16), "h": torch.empty(M, D, **f16),
+                "o": torch.empty(M, D, **f16), "u": torch.empty(M, F, **f16)}
+
+    def _rows_layer(self, lib, stream, layer, x, work, B, T, S0, kc, vc, cap, mask):
+        """One layer over B * T row-major rows (transformer_decoder_layer.py:233-284): ``x`` is
+        the residual stream, updated in place; keys and values of the T new positions of every
+        row go to positions S0 .. S0 + T - 1 of ``kc`` / ``vc``."""
+        cfg = self.cfg
+        D, H, hd, F = (cfg.decoder_embed_dim, cfg.decoder_attention_heads, cfg.head_dim,
+                       cfg.decoder_ffn_embed_dim)
+        M = B * T
+        q, h, o, u = work["q"], work["h"], work["o"], work["u"]
+        mask_stride = mask.stride(0) if mask is not None else 0
+        self._layernorm(lib, stream, x, layer.self_attn_layer_norm, M, D, h)
+        self._qkv(lib, stream, h, layer.self_attn.qkv_proj, q, kc, vc, B, T, H, hd, S0, cap, D, 0)
+        check(lib.msa_attention_f16(ptr(q), ptr(kc), ptr(vc), ptr(mask), mask_stride, ptr(o), B,
+                                    H, hd, T, S0, cap, 0, None, stream))
+        # x = round(round(o Wo^T + bo) + x)   (transformer_decoder_layer.py:222-230)
+        self._linear(lib, stream, o, layer.self_attn.out_proj, M, D, D, residual=x, out=x)
+        self._layernorm(lib, stream, x, layer.final_layer_norm, M, D, h)
+        self._linear(lib, stream, h, layer.fc1, M, F, D, relu=True, out=u)
+        self._linear(lib, stream, u, layer.fc2, M, D, F, residual=x, out=x)
 
     # ------------------------------------------------------------------ slot interface
     # A running batch whose rows belong to different requests (continuous batching): a fixed

@@ -153,11 +153,19 @@ class OracleDecoder:
     """
 
     def __init__(self, cfg: OracleConfig, state_dict: Dict[str, torch.Tensor],
-                 dtype=torch.float32, device="cpu", lean=False, native_matmul=False):
+                 dtype=torch.float32, device="cpu", lean=False, native_matmul=False,
+                 store_dtype=None):
         self.cfg = cfg
         self.dtype = dtype
         self.device = torch.device(device)
         self.lean = lean
+        # trace: None, or {layer index: []}; every pass through such a layer appends a dict of
+        # the tensors the reference materialises there (batch-major, in `dtype`), for tests that
+        # feed one op of another implementation the oracle's own input of that op
+        self.trace: Optional[Dict[int, list]] = None
+        # what to record: None = everything, a set of names, or {layer index: set or None}
+        self.trace_keys = None
+        self.trace_device = None  # where recorded tensors are kept (None = where they are)
         # native_matmul: matrix products are handed to torch in `dtype` itself (what the
         # reference does on a GPU: the BLAS accumulates in fp32 and rounds once on output)
         # instead of as fp32 products of `dtype` values that are rounded afterwards.  Same
@@ -166,8 +174,11 @@ class OracleDecoder:
         self.native_matmul = native_matmul and dtype != torch.float32
         # weights are values already rounded to `dtype`, held as fp32 copies - or, when lean, in
         # `dtype` itself (no copy if the caller's tensor already is) and upcast at each use
+        # store_dtype (lean only): the dtype the weights are kept in when it is narrower than the
+        # arithmetic `dtype` (fp16 weights evaluated in fp32 throughout: exact upcasts at each use)
+        store = store_dtype if (lean and store_dtype is not None) else dtype
         self.w = _Weights({
-            k: (v.detach().to(self.device).to(dtype) if lean
+            k: (v.detach().to(self.device).to(store) if lean
                 else v.detach().to(self.device).to(dtype).float())
             for k, v in state_dict.items()
             if v.is_floating_point()
@@ -247,6 +258,8 @@ class OracleDecoder:
         kvq = self._linear(x, p + "qkv_proj.weight", p + "qkv_proj.bias")
         k, v, q = kvq.split(D, dim=-1)  # :316-319, thirds are K | V | Q
         q = self._r(q * (hd ** -0.5))  # :429
+        tr = self._tr(i)
+        self._rec(tr, k=k, v=v, q=q)
         q = q.contiguous().view(T, B * H, hd).transpose(0, 1)  # :431-435
         k = k.contiguous().view(-1, B * H, hd).transpose(0, 1)
         v = v.contiguous().view(-1, B * H, hd).transpose(0, 1)
@@ -265,14 +278,39 @@ class OracleDecoder:
             incremental_state[key] = saved
         o = self._attention_rows(q, k, v, B, attn_mask, key_padding_mask)
         o = o.transpose(0, 1).contiguous().view(T, B, D)  # :552
+        self._rec(tr, o=o)
         return self._linear(o, p + "out_proj.weight", None), self.w[p + "out_proj.bias"]
+
+    def _tr(self, i):
+        """The dict the current pass through layer ``i`` records into, or None."""
+        if self.trace is None or not self.trace.get(i):
+            return None
+        return self.trace[i][-1]
+
+    def _rec(self, tr, **tensors):
+        """Records [T, B, D] tensors as batch-major [B * T, D] copies in the activation dtype
+        (the values are already rounded to it, so nothing is lost)."""
+        if tr is None:
+            return
+        keys = self.trace_keys
+        if isinstance(keys, dict):
+            keys = keys.get(tr["layer"])
+        for name, t in tensors.items():
+            if keys is None or name in keys:
+                t = t.transpose(0, 1).reshape(-1, t.shape[-1]).to(self.dtype)
+                tr[name] = t if self.trace_device is None else t.to(self.trace_device)
 
     def _layer(self, i, x, incremental_state, attn_mask, key_padding_mask):
         """transformer_decoder_layer.py:233-284 (pre-LN, ReLU FFN)."""
         p = f"decoder.layers.{i}."
+        tr = None
+        if self.trace is not None and i in self.trace:
+            tr = {"layer": i}
+            self.trace[i].append(tr)
         residual = x
         h = self._r(layer_norm(x, self.w[p + "self_attn_layer_norm.weight"],
                                self.w[p + "self_attn_layer_norm.bias"]))
+        self._rec(tr, x_in=x, h1=h)
         a, a_bias = self._attention(i, h, incremental_state, attn_mask, key_padding_mask)
         a = self._r(a + a_bias)  # :222-223
         x = self._r(a + residual)  # :230
@@ -280,8 +318,11 @@ class OracleDecoder:
         h = self._r(layer_norm(x, self.w[p + "final_layer_norm.weight"],
                                self.w[p + "final_layer_norm.bias"]))
         u = F.relu(self._linear(h, p + "fc1.weight", p + "fc1.bias"))  # feedforward.py:21
+        self._rec(tr, x_mid=x, h2=h, u=u)
         z = self._linear(u, p + "fc2.weight", p + "fc2.bias")
-        return self._r(residual + z)  # :283
+        x = self._r(residual + z)  # :283
+        self._rec(tr, x_out=x)
+        return x
 
     def extract_features(self, prev_output_tokens, incremental_state=None,
                          self_attn_padding_mask=None):

@@ -18,8 +18,9 @@ def oracle_cfg(cfg):
                         cfg.padding_idx, cfg.eos_idx)
 
 
-def make_oracle(cfg, sd, dtype=torch.float32, device="cpu", lean=False):
-    return OracleDecoder(oracle_cfg(cfg), sd, dtype=dtype, device=device, lean=lean)
+def make_oracle(cfg, sd, dtype=torch.float32, device="cpu", lean=False, store_dtype=None):
+    return OracleDecoder(oracle_cfg(cfg), sd, dtype=dtype, device=device, lean=lean,
+                         store_dtype=store_dtype)
 
 
 def assert_tokens_match_up_to_ties(got, want, step_logits, n0, ulps=2, pad=1, eos=2,
