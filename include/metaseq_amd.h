@@ -9,8 +9,9 @@
  *     allocates or frees device memory on behalf of these calls; `stream` is a hipStream_t
  *     (NULL = the default stream).  Nothing synchronises: work is enqueued on `stream`.
  *   - the calls act on the calling thread's current device and may be made from several
- *     threads and for several devices of one process; a msa_decoder handle (below) is used
- *     by one thread at a time.
+ *     threads and for several devices of one process, a msa_decoder handle (below) included:
+ *     the handle is read-only after msa_decoder_create, every call's state lives in its own
+ *     arguments and workspace.
  *   - fp16 tensors are IEEE binary16, row-major, innermost dimension contiguous.
  *   - "round" below means round-to-nearest-even to fp16.  Every kernel accumulates in fp32
  *     and rounds at exactly the points where the reference materialises an fp16 tensor.
@@ -313,7 +314,10 @@ int msa_lm_head_greedy_select_f16(const void* x, const void* Ep, void* logits, v
  * call allocates and frees nothing.  Limits: M <= 64 rows and at most 256 compute units
  * (MSA_ERR_CAPACITY beyond).  All calls on one GPU share that array: calls that overlap on one
  * GPU (different streams or threads) race; calls on one stream are ordered and safe.  Nothing
- * in the array needs to start at zero: every partial that is read is written by the same call. */
+ * in the array needs to start at zero: every partial that is read is written by the same call.
+ * The FIRST call on a device looks the array's address up (hipGetDevice, hipGetSymbolAddress,
+ * which may load the code object): make one call per device outside any stream capture before
+ * capturing calls into a graph; every later call issues kernel launches only. */
 int msa_lm_head_greedy_select_noalloc_f16(const void* x, const void* Ep, void* logits, int M,
                                           int V, int K, float temperature,
                                           const int32_t* banned_host, int n_banned,

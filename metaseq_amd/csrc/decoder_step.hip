@@ -19,7 +19,6 @@ struct msa_decoder {
   const void* final_ln_gamma;
   const void* final_ln_beta;
   msa_layer_weights* layers;
-  int splits_out, splits_fc2, splits_rows;  // split-K counts, chosen for splits_rows rows
 };
 
 namespace {
@@ -41,19 +40,25 @@ int64_t split_attention_keys(const msa_decoder* d, int B) {
   return msa_attention_prefers_split(B, d->cfg.heads, hd, (int)keys) ? keys : 0;
 }
 
-void pick_splits(msa_decoder* d, int B) {
-  if (d->splits_rows == B) return;
+// split-K counts of out_proj and fc2 for B rows.  Computed per call (a few integer operations) and
+// kept out of the handle: the handle holds nothing that a call writes.
+struct Splits {
+  int out, fc2;
+};
+
+Splits pick_splits(const msa_decoder* d, int B) {
   const int D = d->cfg.d_model, F = d->cfg.ffn;
-  d->splits_out = d->cfg.int8 ? msa_linear_default_splits_w8a16(B, D, D)
-                              : msa_linear_default_splits(B, D, D);
-  d->splits_fc2 = d->cfg.int8 ? msa_linear_default_splits_w8a16(B, D, F)
-                              : msa_linear_default_splits(B, D, F);
-  d->splits_rows = B;
+  Splits s;
+  s.out = d->cfg.int8 ? msa_linear_default_splits_w8a16(B, D, D)
+                      : msa_linear_default_splits(B, D, D);
+  s.fc2 = d->cfg.int8 ? msa_linear_default_splits_w8a16(B, D, F)
+                      : msa_linear_default_splits(B, D, F);
+  return s;
 }
 
-StepBuffers carve(const msa_decoder* d, int B, char* base) {
+StepBuffers carve(const msa_decoder* d, int B, const Splits& sp, char* base) {
   const int64_t D = d->cfg.d_model, F = d->cfg.ffn, MP = ((B + 15) / 16) * 16;
-  const int64_t S = d->splits_out > d->splits_fc2 ? d->splits_out : d->splits_fc2;
+  const int64_t S = sp.out > sp.fc2 ? sp.out : sp.fc2;
   StepBuffers w{};
   int64_t off = 0;
   auto take = [&](int64_t n) {
@@ -119,7 +124,6 @@ extern "C" int msa_decoder_create(const msa_decoder_config* cfg, const void* emb
   d->final_ln_gamma = final_ln_gamma;
   d->final_ln_beta = final_ln_beta;
   d->layers = lw;
-  d->splits_rows = -1;
   *out = d;
   return MSA_OK;
 }
@@ -132,8 +136,7 @@ extern "C" void msa_decoder_destroy(msa_decoder* d) {
 
 extern "C" int64_t msa_decoder_step_workspace_bytes(msa_decoder* d, int B) {
   if (!d || B < 1 || B > 64) return 0;
-  pick_splits(d, B);
-  return carve(d, B, nullptr).bytes;
+  return carve(d, B, pick_splits(d, B), nullptr).bytes;
 }
 
 extern "C" int msa_decoder_step(msa_decoder* d, const msa_step_args* a, void* stream) {
@@ -148,8 +151,8 @@ extern "C" int msa_decoder_step(msa_decoder* d, const msa_step_args* a, void* st
   MSA_REQUIRE(!a->tok || a->score, MSA_ERR_INVALID_ARG, "%s: tok needs score", name);
   MSA_REQUIRE((a->flags & ~(MSA_EMBED_COL_FROM_LEN | MSA_STEP_NO_ADVANCE)) == 0,
               MSA_ERR_INVALID_ARG, "%s: unsupported flags 0x%x", name, a->flags);
-  pick_splits(d, B);
-  const StepBuffers w = carve(d, B, (char*)a->workspace);
+  const Splits sp = pick_splits(d, B);
+  const StepBuffers w = carve(d, B, sp, (char*)a->workspace);
   MSA_REQUIRE(a->workspace_bytes >= w.bytes, MSA_ERR_CAPACITY,
               "%s: workspace of %lld bytes, %lld needed", name, (long long)a->workspace_bytes,
               (long long)w.bytes);
@@ -194,12 +197,12 @@ extern "C" int msa_decoder_step(msa_decoder* d, const msa_step_args* a, void* st
     if (rc) return rc;
     if (c.int8)
       rc = msa_linear_partial_w8a16(w.o, (const int8_t*)l.out_weight, l.out_scales,
-                                    (float*)w.part, B, D, D, d->splits_out, IN, stream);
+                                    (float*)w.part, B, D, D, sp.out, IN, stream);
     else
-      rc = msa_linear_partial_f16(w.o, l.out_weight, (float*)w.part, B, D, D, d->splits_out, IN,
+      rc = msa_linear_partial_f16(w.o, l.out_weight, (float*)w.part, B, D, D, sp.out, IN,
                                   stream);
     if (rc) return rc;
-    rc = msa_residual_layernorm_f16((const float*)w.part, d->splits_out, l.out_bias, w.x,
+    rc = msa_residual_layernorm_f16((const float*)w.part, sp.out, l.out_bias, w.x,
                                     l.ln2_gamma, l.ln2_beta, w.h, B, D, eps, OUT, stream);
     if (rc) return rc;
     if (c.int8)
@@ -211,13 +214,13 @@ extern "C" int msa_decoder_step(msa_decoder* d, const msa_step_args* a, void* st
     if (rc) return rc;
     if (c.int8)
       rc = msa_linear_partial_w8a16(w.u, (const int8_t*)l.fc2_weight, l.fc2_scales,
-                                    (float*)w.part, B, D, F, d->splits_fc2, IN, stream);
+                                    (float*)w.part, B, D, F, sp.fc2, IN, stream);
     else
-      rc = msa_linear_partial_f16(w.u, l.fc2_weight, (float*)w.part, B, D, F, d->splits_fc2, IN,
+      rc = msa_linear_partial_f16(w.u, l.fc2_weight, (float*)w.part, B, D, F, sp.fc2, IN,
                                   stream);
     if (rc) return rc;
     const bool last = i + 1 == c.layers;
-    rc = msa_residual_layernorm_f16((const float*)w.part, d->splits_fc2, l.fc2_bias, w.x,
+    rc = msa_residual_layernorm_f16((const float*)w.part, sp.fc2, l.fc2_bias, w.x,
                                     last ? d->final_ln_gamma : d->layers[i + 1].ln1_gamma,
                                     last ? d->final_ln_beta : d->layers[i + 1].ln1_beta, w.h, B, D,
                                     eps, OUT, stream);

@@ -1176,34 +1176,39 @@ __global__ __launch_bounds__(TQ_THREADS) void linear_quad_kernel(
     }
   }
   const uint32_t lds0 = (uint32_t)(uintptr_t)(tq_lds_void*)tq_lds;
-  uint32_t xv0 = 0, xv1 = 0, wv = 0, xst = 0;  // lane offsets of the group being issued
+  // Lane offsets and LDS base of the group being issued.  The LDS base travels in M0, which every
+  // load names as an explicit register operand: the compiler then knows that M0 is live between
+  // the loads of a group (ordinary code - fragment reads, MFMAs - runs between them) and writes
+  // it once per group.
+  uint32_t xv0 = 0, xv1 = 0, wv = 0, xst = 0, xm0 = 0, wm0 = 0;
   auto set_x = [&](int slot, int st) {
     st = min(st, nst - 1);
     xst = st * 128;
     xv0 = xlane0 + st * 128;
     xv1 = xlane1 + st * 128;
-    asm volatile("s_mov_b32 m0, %0" ::"s"(lds0 + slot * TQ_XBYTES + wave * (64 * 128) + 4096)
-                 : "memory");
+    xm0 = lds0 + slot * TQ_XBYTES + wave * (64 * 128) + 4096;
   };
   auto set_w = [&](int slot, int ks) {
     ks = min(ks, nks - 1);
     wv = wlane + ks * 1024;
-    asm volatile("s_mov_b32 m0, %0" ::"s"(lds0 + TQ_WOFF + slot * TQ_WBYTES + wave * (WL * 1024))
-                 : "memory");
+    wm0 = lds0 + TQ_WOFF + slot * TQ_WBYTES + wave * (WL * 1024);
   };
   auto issue_x = [&](auto ic) {
     constexpr int i = decltype(ic)::value;
     const uint32_t vo = CLAMP ? xl[CLAMP ? i : 0] + xst : (i & 1 ? xv1 : xv0);
     const char* sb = xb[i];
+    const uint32_t base = xm0;
     asm volatile("global_load_lds_dwordx4 %0, %1 offset:%2" ::"v"(vo), "s"(sb),
-                 "n"((i - 4) * 1024)
+                 "n"((i - 4) * 1024), "{m0}"(base)
                  : "memory");
   };
   auto issue_w = [&](auto jc) {
     constexpr int j = decltype(jc)::value;
     const uint32_t vo = wv;
     const char* sb = wb[j];
-    asm volatile("global_load_lds_dwordx4 %0, %1 offset:%2" ::"v"(vo), "s"(sb), "n"(j * 1024)
+    const uint32_t base = wm0;
+    asm volatile("global_load_lds_dwordx4 %0, %1 offset:%2" ::"v"(vo), "s"(sb), "n"(j * 1024),
+                 "{m0}"(base)
                  : "memory");
   };
   auto group_x = [&](int slot, int st) {

@@ -5,8 +5,8 @@ Both run the same kernels; only the home of the selection partials differs (a fi
 inside the library instead of the workspace), so tokens, finished flags, scores and stored
 logits must be bit-identical.  Two calls in a row, the second with fewer rows and a smaller
 vocabulary, so that stale partials of the first call sit in the shared array while the second
-runs.  The test also asserts that the call leaves torch's allocator statistics untouched and
-that sizes beyond the fixed array are refused."""
+runs.  The test also asserts that the call leaves torch's allocator statistics and the device's
+own count of free memory untouched, and that sizes beyond the fixed array are refused."""
 import ctypes
 
 import pytest
@@ -24,7 +24,7 @@ def _pack_act(x):
     return xp.view(MB, 16, K // 32, 4, 8).permute(2, 0, 3, 1, 4).contiguous().view(-1)
 
 
-def _case(lib, M, V, K, seed, banned, stop, temperature, finished_rows):
+def _case(lib, M, V, K, seed, banned, stop, temperature, finished_rows, device_memory=False):
     P = lambda t: None if t is None else t.data_ptr()
     g = torch.Generator().manual_seed(seed)
     x = torch.randn(M, K, generator=g).half()
@@ -44,10 +44,17 @@ def _case(lib, M, V, K, seed, banned, stop, temperature, finished_rows):
         torch.cuda.synchronize()
         if noalloc:
             before = torch.cuda.memory_stats()["allocation.all.allocated"]
+            free_before = torch.cuda.mem_get_info()[0]
             rc = lib.msa_lm_head_greedy_select_noalloc_f16(
                 P(xp), P(Ep), P(lg), M, V, K, temperature, ba, len(banned), sa, len(stop), P(fin),
                 None, 0, 2, P(tok[:, 1]), 3, P(sc[:, 1]), 3, None, None)
             assert torch.cuda.memory_stats()["allocation.all.allocated"] == before
+            if device_memory:
+                # torch's statistics cannot see a hipMalloc made inside the library; the
+                # device's own count of free bytes can (asked for on a call after the first on
+                # this device, which may load the code object)
+                torch.cuda.synchronize()
+                assert torch.cuda.mem_get_info()[0] == free_before, "device memory was allocated"
         else:
             rc = lib.msa_lm_head_greedy_select_f16(
                 P(xp), P(Ep), P(lg), P(ws), M, V, K, temperature, ba, len(banned), sa, len(stop),
@@ -79,7 +86,7 @@ def test_noalloc_entry_matches_workspace_entry_on_two_calls_in_a_row():
           finished_rows=[i % 5 == 0 for i in range(64)])
     # second call: fewer rows, fewer workgroups; the array still holds the first call's partials
     _case(lib, 5, 4000, 128, 12, banned=[1], stop=[], temperature=1.0,
-          finished_rows=[False] * 5)
+          finished_rows=[False] * 5, device_memory=True)
 
 
 def test_noalloc_entry_rejects_sizes_beyond_the_fixed_array():
