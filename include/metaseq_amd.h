@@ -45,6 +45,7 @@ typedef enum {
 #define MSA_ROW_BAN_EARLY 1u /* eos_idx and the stop ids are not eligible for this row (the row
                                 has not reached its minimum length)                             */
 #define MSA_ROW_ONLY_EOS 2u  /* only eos_idx is eligible for this row (its last allowed step)   */
+#define MSA_ROW_SKIP 4u      /* msa_sample_topp_f16: leave this row's outputs untouched          */
 
 const char* msa_last_error(void);
 int msa_version(void);
@@ -255,31 +256,49 @@ int msa_greedy_select_f16(const void* logits, int64_t ld_logits, int B, int V, f
 /* One step of nucleus (top-p) sampling over fp16 logits[B, V], with the same bookkeeping as
  * msa_greedy_select_f16 (masks, row_mode, finished rows, token / score write-back) plus the
  * repetition penalties:
- *   z = logits / temperature;  lp = log_softmax_fp32(z) over all ids (a NaN anywhere: the row
- *   gets token 0 with score -inf, as does a row with no eligible id);
+ *   z = logits / temperature (temperature_rows[b] if given, else `temperature`; no division for
+ *   0 or 1);  lp = log_softmax_fp32(z) over all ids (a NaN anywhere: the row gets token 0 with
+ *   score -inf, as does a row with no eligible id);
  *   banned / early / only-eos ids -> -inf;  lp[v] -= counts[b,v] * alpha_frequency +
  *   (counts[b,v] > 0) * alpha_presence, likewise counts_src (int64 [B, V] device, optional);
+ *   lprobs_out (optional, fp32, row stride ld_lprobs) receives that masked, penalised row: what
+ *   the reference stores as the step's distribution;
  *   p = softmax(lp);  with the ids in order of decreasing p (ties: increasing id), id k belongs
  *   to the nucleus iff the mass of the ids before it is < topp (topp_rows[b] if given, else
  *   topp_all);  the token is the arg-max over the nucleus of p[v] / noise[b, v], noise (fp32
  *   [B, V]) holding independent Exp(1) draws: an exponential race, which picks v with probability
  *   p[v] / mass(nucleus);  score = log p[tok].
- *   Without noise, or with topp <= 0, the choice is greedy: arg-max of lp (lowest id on ties),
- *   score = lp[tok].  counts[b, tok] += 1 when counts is given.
+ *   Without noise, or with topp <= 0 or temperature 0 for the row (the reference's greedy
+ *   cases, :412), the choice is greedy: arg-max of lp (lowest id on ties), score = lp[tok].
+ *   counts[b, tok] += 1 when counts is given.
+ *   A row whose row_mode has MSA_ROW_SKIP is left alone (no output is written for it): a batch
+ *   whose other rows were chosen by another entry point.
  * The nucleus is found without sorting (radix descent over the bit patterns of p with exact
  * fixed-point masses), so the result does not depend on the order of any summation.
  * Replaces SequenceGenerator._sample_topp and _apply_repetition_penalties
- * (metaseq/sequence_generator.py:399-441, :478-534) and the masking in front of them
- * (:272-293); the reference draws with torch.multinomial over the sorted, renormalised nucleus,
- * which is the same distribution. */
+ * (metaseq/sequence_generator.py:399-441, :478-534), the masking in front of them (:272-293)
+ * and the copy of the step's distribution (:301-303); the reference draws with
+ * torch.multinomial over the sorted, renormalised nucleus, which is the same distribution. */
 int msa_sample_topp_f16(const void* logits, int64_t ld_logits, int B, int V, float temperature,
-                        const int32_t* banned_host, int n_banned, const int32_t* stop_host,
-                        int n_stop, uint8_t* finished, const uint8_t* row_mode,
-                        int force_eos_all, int eos_idx, const float* topp_rows, float topp_all,
-                        const float* noise, int64_t* counts, const int64_t* counts_src,
-                        float alpha_presence, float alpha_frequency, float alpha_presence_src,
-                        float alpha_frequency_src, int64_t* tok, int64_t tok_stride, float* score,
-                        int64_t score_stride, void* stream);
+                        const float* temperature_rows, const int32_t* banned_host, int n_banned,
+                        const int32_t* stop_host, int n_stop, uint8_t* finished,
+                        const uint8_t* row_mode, int force_eos_all, int eos_idx,
+                        const float* topp_rows, float topp_all, const float* noise,
+                        int64_t* counts, const int64_t* counts_src, float alpha_presence,
+                        float alpha_frequency, float alpha_presence_src,
+                        float alpha_frequency_src, float* lprobs_out, int64_t ld_lprobs,
+                        int64_t* tok, int64_t tok_stride, float* score, int64_t score_stride,
+                        void* stream);
+
+/* fp32 log-softmax of n_outer x n_inner fp16 logits rows of V ids:
+ *   out[o*out_outer_stride + i*ld_out + v] = z[v] - max z - log(sum(exp(z - max z))),
+ *   z = logits[o*in_outer_stride + i*ld_logits + v] / temperature (no division for 0 or 1).
+ * The two-level strides let one call copy the rows of every prompt into a [B, max_len, V] buffer.
+ * Replaces BaseDecoder.get_normalized_probs over the prompt positions
+ * (metaseq/models/base_decoder.py:95-100 as called at metaseq/sequence_generator.py:235-250). */
+int msa_log_softmax_f16(const void* logits, int64_t in_outer_stride, int64_t ld_logits,
+                        int n_outer, int n_inner, int V, float temperature, float* out,
+                        int64_t out_outer_stride, int64_t ld_out, void* stream);
 
 /* Log-probabilities of given target ids under fp16 logits rows:
  *   out[r] = logits[r, target[r]]/temperature - logsumexp_fp32(logits[r,:]/temperature).

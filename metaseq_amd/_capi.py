@@ -18,6 +18,7 @@ MSA_OUT_PACKED = 4
 MSA_EMBED_COL_FROM_LEN = 8
 MSA_ROW_BAN_EARLY = 1
 MSA_ROW_ONLY_EOS = 2
+MSA_ROW_SKIP = 4
 
 _P = c_void_p
 MSA_STEP_NO_ADVANCE = 16
@@ -82,9 +83,11 @@ SIGNATURES = {
     "msa_attention_prefers_split": [c_int, c_int, c_int, c_int],
     "msa_greedy_select_f16": [_P, c_int64, c_int, c_int, c_float, _P, c_int, _P, c_int, _P, _P,
                               c_int, c_int, _P, c_int64, _P, c_int64, _P, _P],
-    "msa_sample_topp_f16": [_P, c_int64, c_int, c_int, c_float, _P, c_int, _P, c_int, _P, _P,
+    "msa_sample_topp_f16": [_P, c_int64, c_int, c_int, c_float, _P, _P, c_int, _P, c_int, _P, _P,
                             c_int, c_int, _P, c_float, _P, _P, _P, c_float, c_float, c_float,
-                            c_float, _P, c_int64, _P, c_int64, _P],
+                            c_float, _P, c_int64, _P, c_int64, _P, c_int64, _P],
+    "msa_log_softmax_f16": [_P, c_int64, c_int64, c_int, c_int, c_int, c_float, _P, c_int64,
+                            c_int64, _P],
     "msa_target_logprob_f16": [_P, c_int64, c_int64, c_int, c_float, _P, _P, _P],
     "msa_lm_head_greedy_select_f16": [_P, _P, _P, _P, c_int, c_int, c_int, c_float, _P, c_int, _P,
                                       c_int, _P, _P, c_int, c_int, _P, c_int64, _P, c_int64, _P,

@@ -268,6 +268,19 @@ __global__ __launch_bounds__(256) void select_combine_kernel(
 }
 
 
+// fp32 log-softmax of fp16 logits rows; row (o, i) is read at o * in_outer + i * ld and written
+// at o * out_outer + i * ld_out
+__global__ __launch_bounds__(SM_THREADS) void log_softmax_kernel(
+    const half_t* __restrict__ logits, int64_t in_outer, int64_t ld, int n_inner, int V,
+    float temperature, bool scale, float* __restrict__ out, int64_t out_outer, int64_t ld_out) {
+  __shared__ float red[16];
+  const int o = blockIdx.x / n_inner, i = blockIdx.x % n_inner;
+  const half_t* row = logits + o * in_outer + i * ld;
+  float* orow = out + o * out_outer + i * ld_out;
+  const RowStats st = row_logsumexp(row, V, temperature, scale, red);
+  for_each_z(row, V, temperature, scale, [&](int id, float z) { orow[id] = (z - st.max) - st.lse; });
+}
+
 // ---- nucleus (top-p) sampling --------------------------------------------------------------
 // One workgroup per row.  The nucleus boundary is found without sorting, by a radix descent over
 // the bit pattern of the probabilities (positive floats order like their bit patterns): four
@@ -295,12 +308,13 @@ __device__ __forceinline__ void argbest(float& v, int& i, float ov, int oi) {
 }
 
 __global__ __launch_bounds__(SP_THREADS) void sample_topp_kernel(
-    const half_t* __restrict__ logits, int64_t ld, int V, float temperature, bool scale,
-    IdList banned, IdList stop, uint8_t* __restrict__ finished,
-    const uint8_t* __restrict__ row_mode, int force_eos_all, int eos,
-    const float* __restrict__ topp_rows, float topp_all, const float* __restrict__ noise,
-    Penalties pen, int64_t* __restrict__ tok, int64_t tok_stride, float* __restrict__ score,
-    int64_t score_stride) {
+    const half_t* __restrict__ logits, int64_t ld, int V, float temperature_all,
+    const float* __restrict__ temperature_rows, IdList banned, IdList stop,
+    uint8_t* __restrict__ finished, const uint8_t* __restrict__ row_mode, int force_eos_all,
+    int eos, const float* __restrict__ topp_rows, float topp_all,
+    const float* __restrict__ noise, Penalties pen, float* __restrict__ lprobs_out,
+    int64_t ld_lprobs, int64_t* __restrict__ tok, int64_t tok_stride,
+    float* __restrict__ score, int64_t score_stride) {
   __shared__ float red[16];
   __shared__ float rbest[16], rprob[16];
   __shared__ int ridx[16];
@@ -310,9 +324,12 @@ __global__ __launch_bounds__(SP_THREADS) void sample_topp_kernel(
   const int b = blockIdx.x;
   const half_t* row = logits + (int64_t)b * ld;
   const unsigned rm = row_mode ? row_mode[b] : 0u;
+  if (rm & MSA_ROW_SKIP) return;  // the whole workgroup: this row is not part of the call
   const bool only_eos = force_eos_all || (finished && finished[b]) || (rm & MSA_ROW_ONLY_EOS);
   const bool ban_early = rm & MSA_ROW_BAN_EARLY;
   const float topp = topp_rows ? topp_rows[b] : topp_all;
+  const float temperature = temperature_rows ? temperature_rows[b] : temperature_all;
+  const bool scale = temperature > 0.f && temperature != 1.0f;
 
   // e(id) = z - penalties for an eligible id, -inf otherwise; nan_out collects NaN logits
   auto eligible = [&](int id) {
@@ -374,7 +391,7 @@ __global__ __launch_bounds__(SP_THREADS) void sample_topp_kernel(
   // ---- nucleus: ids in order of decreasing p (ties: increasing id) belong while the mass
   // before them is < topp.  T = the smallest probability whose strictly-greater mass is below
   // topp: everything above T is in, of the ids equal to T those below tie_limit.
-  const bool sampling = noise != nullptr && topp > 0.f && !dead;
+  const bool sampling = noise != nullptr && topp > 0.f && temperature > 0.f && !dead;
   unsigned tbits = 0;
   int tie_limit = V;
   if (sampling) {
@@ -438,15 +455,46 @@ __global__ __launch_bounds__(SP_THREADS) void sample_topp_kernel(
     }
   }
 
-  // ---- the draw: exponential race over the nucleus (the arg-max of p when not sampling)
-  float best = -1.f, bestp = 0.f;
+  // ---- the masked log-probabilities of the row, if asked for: log-softmax over all ids, the
+  // ineligible ones at -inf, then the penalties (frequency, then presence) - before the counts
+  // are updated below
+  if (lprobs_out) {
+    float* lrow = lprobs_out + (int64_t)b * ld_lprobs;
+    const float log_s = dead ? 0.f : logf(s_all);
+    for (int id = threadIdx.x; id < V; id += SP_THREADS) {
+      float v = -INFINITY;
+      if (!dead && eligible(id)) {
+        float z = (float)row[id];
+        if (scale) z = z / temperature;
+        v = (z - mx_all) - log_s;
+        if (pen.counts) {
+          const float cnt = (float)pen.counts[(int64_t)b * V + id];
+          v = v - cnt * pen.frequency;
+          v = v - (cnt > 0.f ? pen.presence : 0.f);
+        }
+        if (pen.counts_src) {
+          const float cnt = (float)pen.counts_src[(int64_t)b * V + id];
+          v = v - cnt * pen.frequency_src;
+          v = v - (cnt > 0.f ? pen.presence_src : 0.f);
+        }
+      }
+      lrow[id] = v;
+    }
+  }
+
+  // ---- the draw: exponential race over the nucleus; when not sampling, the arg-max of the
+  // penalised values themselves (exp() may map two close values to one probability)
+  float best = -INFINITY, bestp = 0.f;
   int bidx = 0x7fffffff;
   if (!dead) {
     for (int id = threadIdx.x; id < V; id += SP_THREADS) {
-      const float pv = p_of(id);
-      if (!(pv > 0.f)) continue;
-      float key = pv;
+      bool unused = false;
+      const float e = e_of(id, unused);
+      if (!(e > -INFINITY)) continue;
+      const float pv = expf(e - mx) * inv;
+      float key = e;
       if (sampling) {
+        if (!(pv > 0.f)) continue;
         const unsigned u = __float_as_uint(pv);
         if (!(u > tbits || (u == tbits && id < tie_limit))) continue;
         key = pv / noise[(int64_t)b * V + id];
@@ -562,19 +610,23 @@ extern "C" int msa_target_logprob_f16(const void* logits, int64_t ld_logits, int
 }
 
 extern "C" int msa_sample_topp_f16(const void* logits, int64_t ld_logits, int B, int V,
-                                   float temperature, const int32_t* banned_host, int n_banned,
+                                   float temperature, const float* temperature_rows,
+                                   const int32_t* banned_host, int n_banned,
                                    const int32_t* stop_host, int n_stop, uint8_t* finished,
                                    const uint8_t* row_mode, int force_eos_all, int eos_idx,
                                    const float* topp_rows, float topp_all, const float* noise,
                                    int64_t* counts, const int64_t* counts_src,
                                    float alpha_presence, float alpha_frequency,
                                    float alpha_presence_src, float alpha_frequency_src,
-                                   int64_t* tok, int64_t tok_stride, float* score,
-                                   int64_t score_stride, void* stream) {
+                                   float* lprobs_out, int64_t ld_lprobs, int64_t* tok,
+                                   int64_t tok_stride, float* score, int64_t score_stride,
+                                   void* stream) {
   const char* name = "msa_sample_topp_f16";
   MSA_REQUIRE(logits && tok && score, MSA_ERR_INVALID_ARG, "%s: null pointer", name);
   MSA_REQUIRE(B > 0 && V > 0 && ld_logits >= V, MSA_ERR_INVALID_ARG,
               "%s: bad shape B=%d V=%d ld=%lld", name, B, V, (long long)ld_logits);
+  MSA_REQUIRE(!lprobs_out || ld_lprobs >= V, MSA_ERR_INVALID_ARG,
+              "%s: log-probability rows of stride %lld < V=%d", name, (long long)ld_lprobs, V);
   MSA_REQUIRE(n_banned >= 0 && n_banned <= 16 && (n_banned == 0 || banned_host),
               MSA_ERR_INVALID_ARG, "%s: n_banned=%d (0..16)", name, n_banned);
   MSA_REQUIRE(n_stop >= 0 && n_stop <= 16 && (n_stop == 0 || stop_host), MSA_ERR_INVALID_ARG,
@@ -582,7 +634,6 @@ extern "C" int msa_sample_topp_f16(const void* logits, int64_t ld_logits, int B,
   MSA_REQUIRE(eos_idx >= 0 && eos_idx < V, MSA_ERR_INVALID_ARG,
               "%s: eos_idx=%d outside the vocabulary", name, eos_idx);
   MSA_REQUIRE(temperature >= 0.f, MSA_ERR_INVALID_ARG, "%s: temperature < 0", name);
-  const bool scale = temperature > 0.f && temperature != 1.0f;
   IdList banned{}, stop{};
   banned.n = n_banned;
   for (int i = 0; i < n_banned; ++i) banned.id[i] = banned_host[i];
@@ -596,9 +647,29 @@ extern "C" int msa_sample_topp_f16(const void* logits, int64_t ld_logits, int B,
   pen.presence_src = alpha_presence_src;
   pen.frequency_src = alpha_frequency_src;
   hipLaunchKernelGGL(sample_topp_kernel, dim3(B), dim3(SP_THREADS), 0, (hipStream_t)stream,
-                     (const half_t*)logits, ld_logits, V, temperature, scale, banned, stop,
-                     finished, row_mode, force_eos_all, eos_idx, topp_rows, topp_all, noise, pen,
-                     tok, tok_stride, score, score_stride);
+                     (const half_t*)logits, ld_logits, V, temperature, temperature_rows, banned,
+                     stop, finished, row_mode, force_eos_all, eos_idx, topp_rows, topp_all, noise,
+                     pen, lprobs_out, ld_lprobs, tok, tok_stride, score, score_stride);
+  MSA_CHECK_LAUNCH(name);
+  return MSA_OK;
+}
+
+extern "C" int msa_log_softmax_f16(const void* logits, int64_t in_outer_stride, int64_t ld_logits,
+                                   int n_outer, int n_inner, int V, float temperature,
+                                   float* out, int64_t out_outer_stride, int64_t ld_out,
+                                   void* stream) {
+  const char* name = "msa_log_softmax_f16";
+  MSA_REQUIRE(logits && out, MSA_ERR_INVALID_ARG, "%s: null pointer", name);
+  MSA_REQUIRE(n_outer >= 0 && n_inner >= 0 && V > 0 && ld_logits >= V && ld_out >= V &&
+                  (int64_t)n_outer * n_inner < (1ll << 31),
+              MSA_ERR_INVALID_ARG, "%s: bad shape %d x %d rows of V=%d", name, n_outer, n_inner,
+              V);
+  MSA_REQUIRE(temperature >= 0.f, MSA_ERR_INVALID_ARG, "%s: temperature < 0", name);
+  if (n_outer == 0 || n_inner == 0) return MSA_OK;
+  const bool scale = temperature > 0.f && temperature != 1.0f;
+  hipLaunchKernelGGL(log_softmax_kernel, dim3((unsigned)(n_outer * n_inner)), dim3(SM_THREADS), 0,
+                     (hipStream_t)stream, (const half_t*)logits, in_outer_stride, ld_logits,
+                     n_inner, V, temperature, scale, out, out_outer_stride, ld_out);
   MSA_CHECK_LAUNCH(name);
   return MSA_OK;
 }

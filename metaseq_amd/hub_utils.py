@@ -49,6 +49,8 @@ class GeneratorInterface:
         self.bpe = tokenizer if tokenizer is not None else _IdTokenizer()
         self.device = torch.device(device)
         self._max_positions = max_positions
+        # handed to every SequenceGenerator this interface builds (see its noise_fn)
+        self.noise_fn = None
         # hub_utils.py:184-191
         self._pad_token_ind = tgt_dict.pad_index
         self._special_token_inds = {tgt_dict.eos_index, tgt_dict.pad_index, tgt_dict.bos_index,
@@ -127,6 +129,7 @@ class GeneratorInterface:
             alpha_frequency=alpha_frequency, alpha_presence_src=alpha_presence_src,
             alpha_frequency_src=alpha_frequency_src,
             alpha_src_penalty_end_idx=alpha_src_penalty_end_idx)
+        generator.noise_fn = self.noise_fn
         sample = {"net_input": {"src_tokens": src_tokens.to(self.device),
                                 "src_lengths": src_lengths.to(self.device)}}
         t0 = time.time()

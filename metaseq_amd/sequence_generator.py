@@ -6,14 +6,14 @@ device-to-host syncs per step; here one kernel per step does log-sum-exp, maskin
 token/score write-back and the finished-row update on the device, and the host only syncs
 once end-of-sequence becomes possible (step >= min_len).
 
-Nucleus (top-p) sampling, factual-nucleus decay and the repetition penalties take the general
-path: one kernel per step (msa_sample_topp_f16) applies the reference's masks and penalties
-(:271-293, :478-523), finds the nucleus without sorting and draws from it; only when the
-per-step distributions are wanted (``need_logprobs``) are the masked fp32 log-probabilities
-materialised with device tensor ops and the draw made by ``torch.multinomial``, as in the
-reference (:431).  Factual-nucleus state is kept per row (the reference's indexing only
-works at beam_size 1, where the two agree), and prompt-token counts of a replica row come from
-its own prompt (the reference indexes past the prompt batch when beam_size > 1).
+Nucleus (top-p) sampling, factual-nucleus decay, the repetition penalties and ``need_logprobs``
+take the general path: one kernel per step (msa_sample_topp_f16) applies the reference's masks
+and penalties (:271-293, :478-523), writes the step's masked fp32 log-probabilities straight
+into the ``distributions`` buffer when they are wanted (:301-303), finds the nucleus without
+sorting and draws from it (or takes the arg-max).  Factual-nucleus state is kept per row (the
+reference's indexing only works at beam_size 1, where the two agree), and prompt-token counts of
+a replica row come from its own prompt (the reference indexes past the prompt batch when
+beam_size > 1).
 """
 import ctypes
 from typing import Dict, List, Optional
@@ -76,6 +76,9 @@ class SequenceGenerator(nn.Module):
         self.penalties_src = max(alpha_presence_src, alpha_frequency_src) > 0
         self.model.eval()
         self.profile = profile
+        # noise_fn(step, rows, vocab) -> fp32 [rows, vocab] device tensor of independent Exp(1)
+        # numbers for the draw of that step; None: torch's device generator (torch.manual_seed)
+        self.noise_fn = None
 
     def cuda(self):
         self.model.cuda()
@@ -206,10 +209,12 @@ class SequenceGenerator(nn.Module):
             # scores after each row's own prompt are reset (:262-266)
             col = torch.arange(max_len, device=dev).unsqueeze(0)
             scores.masked_fill_(col > rep_lengths.unsqueeze(1), 0.0)
-            if all_lprobs is not None:
-                full = self.model.get_normalized_probs(self._tempered(logits), log_probs=True)
-                all_lprobs[:, 1:start_step] = full[:, :-1]
-                del full
+            if all_lprobs is not None and start_step > 1:
+                # the distributions of the prompt positions (:247-250), fp32 rows written in place
+                dst = all_lprobs[:, 1]
+                check(lib.msa_log_softmax_f16(ptr(flat), T * flat.stride(0), flat.stride(0), BB,
+                                              start_step - 1, V, float(self.temperature), ptr(dst),
+                                              all_lprobs.stride(0), all_lprobs.stride(1), stream))
             # the row that predicts each sample's first free token (:262-267)
             if int(rep_lengths.max()) >= T:
                 # the reference indexes lprobs[i, prompt_len] out of range in this case: every
@@ -221,7 +226,8 @@ class SequenceGenerator(nn.Module):
 
             finished = torch.zeros(BB, dtype=torch.uint8, device=dev)
             cache = decoder.get_cache(incremental_states) if hasattr(decoder, "get_cache") else None
-            general = self.sampling or self.penalties or self.penalties_src
+            general = (self.sampling or self.penalties or self.penalties_src
+                       or all_lprobs is not None)
             gs = self._general_state(src_tokens, BB, V, dev) if general else None
             st = None
             if (self.use_graph and all_lprobs is None and cache is not None and BB <= 64
@@ -249,16 +255,10 @@ class SequenceGenerator(nn.Module):
                     step = nxt
             for step in range(start_step, max_len if not fused else start_step):
                 if general:
-                    if all_lprobs is None and step_logits.dtype == torch.float16:
-                        # masks, penalties, nucleus and draw in one kernel per step
-                        self._sample_step(lib, step_logits, step, min_len, max_len, finished, gs,
-                                          tokens, scores)
-                    else:  # the distributions are wanted: materialise them with tensor ops
-                        lprobs = self._masked_lprobs(step_logits, step, min_len, max_len,
-                                                     finished, gs)
-                        if all_lprobs is not None:
-                            all_lprobs[:, step] = lprobs
-                        self._choose(lprobs, step, gs, finished, tokens, scores)
+                    # masks, penalties, the step's distribution, nucleus and draw: one kernel
+                    self._sample_step(lib, step_logits, step, min_len, max_len, finished, gs,
+                                      tokens, scores,
+                                      all_lprobs[:, step] if all_lprobs is not None else None)
                     if bool(finished.all()) or step + 1 >= max_len:
                         break
                     out = decoder(tokens[:, :step + 1], incremental_state=incremental_states)[0]
@@ -270,9 +270,6 @@ class SequenceGenerator(nn.Module):
                         break
                     step_logits = st["logits"]
                     continue
-                if all_lprobs is not None:
-                    all_lprobs[:, step] = self._masked_lprobs(step_logits, step, min_len, max_len,
-                                                              finished)
                 self._select(lib, step_logits, step, min_len, max_len, finished, tokens, scores)
                 # rows can only finish once eos / stop tokens are allowed or forced
                 if (step >= min_len or step >= max_len - 1) and bool(finished.all()):
@@ -297,35 +294,6 @@ class SequenceGenerator(nn.Module):
                                                                       self.vocab_size)
         return retval
 
-    # ---- slow path used only with need_logprobs ----
-    def _tempered(self, logits):
-        x = logits.float()
-        if self.temperature > 0 and self.temperature != 1.0:
-            x = x / self.temperature
-        return x
-
-    def _masked_lprobs(self, step_logits, step, min_len, max_len, finished, gs=None):
-        """fp32 log-probabilities of one step with the reference's masks in the reference's
-        order (:272-293): min-length block, NaN, pad, forced eos, penalties, finished rows."""
-        import math
-        lprobs = self.model.get_normalized_probs(self._tempered(step_logits), log_probs=True)
-        if step < min_len:
-            lprobs[:, self.eos] = -math.inf
-            for t in self.stop:
-                lprobs[:, t] = -math.inf
-        lprobs[lprobs != lprobs] = -math.inf
-        lprobs[:, self.pad] = -math.inf
-        if step >= max_len - 1:
-            lprobs[:, :self.eos] = -math.inf
-            lprobs[:, self.eos + 1:] = -math.inf
-        if gs is not None:
-            lprobs = self._apply_repetition_penalties(lprobs, gs["count_tokens"],
-                                                      gs["count_tokens_src"])
-        fin = finished.bool()
-        lprobs[fin, :self.eos] = -math.inf
-        lprobs[fin, self.eos + 1:] = -math.inf
-        return lprobs
-
     # ---- general path: nucleus sampling, factual-nucleus decay, repetition penalties ----
     def _general_state(self, src_tokens, BB, V, dev):
         """Per-call buffers of the general path (:372-395)."""
@@ -344,69 +312,39 @@ class SequenceGenerator(nn.Module):
         gs["topp"] = gs["init_p"].clone()
         gs["toks_since_reset"] = torch.zeros(BB, 1, device=dev)
         gs["full_stop"] = torch.tensor(self.full_stop_list, device=dev)
-        gs["rows"] = torch.arange(BB, device=dev)
         gs["noise"] = (torch.empty(BB, V, dtype=torch.float32, device=dev) if self.sampling
                        else None)
         return gs
 
     def _sample_step(self, lib, step_logits, step, min_len, max_len, finished, gs, tokens,
-                     scores):
+                     scores, lprobs_out=None):
         """One step of the general path on the device (metaseq/sequence_generator.py:272-308,
         399-441, 478-534): msa_sample_topp_f16 applies the masks and the repetition penalties,
         finds the nucleus and draws from it.  The draw consumes one Exp(1) number per row and
         token from torch's device generator (an exponential race, the way torch.multinomial
-        itself draws), so ``torch.manual_seed`` fixes the samples."""
+        itself draws), so ``torch.manual_seed`` fixes the samples.  ``lprobs_out`` ([BB, V] fp32
+        view, any row stride) receives the step's masked, penalised log-probabilities."""
         BB, V = step_logits.shape
         banned = self._banned(step, min_len)
         ba = (ctypes.c_int32 * len(banned))(*banned)
         sa = (ctypes.c_int32 * max(1, len(self.stop)))(*self.stop)
-        noise = gs["noise"].exponential_() if self.sampling else None
+        noise = None
+        if self.sampling:
+            noise = (self.noise_fn(step, BB, V) if self.noise_fn is not None
+                     else gs["noise"].exponential_())
         topp_rows = gs["topp"] if (self.sampling and self.lambda_decay > 0) else None
         tok, sc = tokens[:, step], scores[:, step]
         check(lib.msa_sample_topp_f16(
-            ptr(step_logits), step_logits.stride(0), BB, V, float(self.temperature), ba,
+            ptr(step_logits), step_logits.stride(0), BB, V, float(self.temperature), None, ba,
             len(banned), sa, len(self.stop), ptr(finished), None, int(step >= max_len - 1),
             self.eos, ptr(topp_rows), float(self.sampling_topp) if self.sampling else 0.0,
             ptr(noise), ptr(gs["count_tokens"]), ptr(gs["count_tokens_src"]),
             float(self.alpha_presence), float(self.alpha_frequency),
-            float(self.alpha_presence_src), float(self.alpha_frequency_src), ptr(tok),
-            tokens.stride(0), ptr(sc), scores.stride(0), _capi.stream_ptr()))
+            float(self.alpha_presence_src), float(self.alpha_frequency_src), ptr(lprobs_out),
+            lprobs_out.stride(0) if lprobs_out is not None else 0, ptr(tok), tokens.stride(0),
+            ptr(sc), scores.stride(0), _capi.stream_ptr()))
         if self.sampling and self.lambda_decay > 0:
             self._update_sampling_topp(tokens[:, step], gs)
-
-    def _apply_repetition_penalties(self, lprobs, count_tokens, count_tokens_src):
-        """mu[j] - c[j] * alpha_frequency - [c[j] > 0] * alpha_presence (:478-523)."""
-        if self.penalties:
-            lprobs = (lprobs - count_tokens * self.alpha_frequency
-                      - count_tokens.gt(0) * self.alpha_presence)
-        if self.penalties_src:
-            lprobs = (lprobs - count_tokens_src * self.alpha_frequency_src
-                      - count_tokens_src.gt(0) * self.alpha_presence_src)
-        return lprobs
-
-    def _sample_topp(self, lprobs, gs):
-        """Draw among the smallest set of tokens whose probability mass reaches p (:399-441)."""
-        if not self.sampling:
-            return tuple(lprobs.max(dim=-1))
-        probs = torch.softmax(lprobs, dim=-1)
-        sprobs, sinds = probs.sort(dim=-1, descending=True)
-        p = self.sampling_topp if self.lambda_decay <= 0 else gs["topp"]
-        mask = (sprobs.cumsum(dim=-1) - sprobs) >= p
-        trunc = sprobs.masked_fill(mask, 0)
-        trunc.div_(trunc.sum(dim=-1, keepdim=True))
-        # A row with every token masked (min_len == max_len at the last step) has NaN
-        # probabilities: the reference's multinomial raises there, and on the device that check
-        # is an assertion that takes the GPU context down.  Such a row gets what the greedy
-        # branch's max() gives it: token 0 with score -inf.
-        dead = ~torch.isfinite(lprobs).any(dim=-1)
-        trunc = torch.nan_to_num(trunc, nan=0.0, posinf=0.0, neginf=0.0)
-        trunc[:, 0] += dead.to(trunc.dtype)
-        choices = torch.multinomial(trunc, 1)[:, 0]
-        tok_ids = sinds[gs["rows"], choices].masked_fill(dead, 0)
-        scores = sprobs[gs["rows"], choices].log().masked_fill(dead, float("-inf"))
-        if self.lambda_decay > 0:
-            self._update_sampling_topp(tok_ids, gs)
-        return scores, tok_ids
 
     def _update_sampling_topp(self, tok_ids, gs):
         """Factual-nucleus decay, vectorised over rows (:443-476): p restarts at its initial
@@ -418,15 +356,3 @@ class SequenceGenerator(nn.Module):
         gs["toks_since_reset"] = tsr
         decay = (tsr - 1).clamp_(min=0)
         gs["topp"] = torch.clamp(gs["init_p"] * self.lambda_decay ** decay, min=self.omega_bound)
-
-    def _choose(self, lprobs, step, gs, finished, tokens, scores):
-        """Selection and bookkeeping of one general-path step (:295-308)."""
-        next_scores, next_toks = self._sample_topp(lprobs, gs)
-        if gs["count_tokens"] is not None:
-            gs["count_tokens"][gs["rows"], next_toks] += 1
-        tokens[:, step] = next_toks
-        scores[:, step] = next_scores
-        done = next_toks == self.eos
-        for t in self.stop:
-            done |= next_toks == t
-        finished |= done.to(finished.dtype)

@@ -11,9 +11,10 @@ thread that drives the GPU, results delivered through a per-request queue):
   the sequence length, or when nothing arrives for ``timeout_ms``.
 * ``ContinuousBatcher`` - no reference counterpart: a fixed set of slots over one KV cache with
   per-row lengths; a request is prefilled into a free slot whenever one exists and leaves it the
-  moment it ends, while the other rows keep decoding.  Greedy requests only; each row follows
-  its own ``min_tokens`` / ``max_tokens`` / end-of-sequence rules, and gets the record a
-  single-request ``GeneratorInterface.generate`` call would give it.
+  moment it ends, while the other rows keep decoding.  Greedy and sampled requests share the
+  batch; each row follows its own temperature, nucleus and ``min_tokens`` / ``max_tokens`` /
+  end-of-sequence rules, and gets the record a single-request ``GeneratorInterface.generate``
+  call would give it.
 """
 import heapq
 import itertools
@@ -93,6 +94,22 @@ class Backlog:
             if not live:
                 return None
             return max(live, key=lambda e: e[0])[1]
+
+    def take_oldest(self, signature: str, due) -> Optional[Request]:
+        """The earliest-submitted request of one signature if ``due(request)`` holds, else
+        None (the request stays where it is)."""
+        with self._cv:
+            heap = self._heaps.get(signature) or []
+            if not heap:
+                return None
+            i = min(range(len(heap)), key=lambda j: heap[j][1].uid)
+            req = heap[i][1]
+            if not due(req):
+                return None
+            heap[i] = heap[-1]
+            heap.pop()
+            heapq.heapify(heap)
+            return req
 
     def take(self, signature: str, wait: float = 0.0) -> Optional[Request]:
         """Cheapest request of one signature; waits up to ``wait`` seconds for one to arrive."""
@@ -226,15 +243,18 @@ class BatchingService(_Front):
 
 
 class _Row:
-    """A request while it occupies a slot."""
+    """One replica of a request while it occupies a slot."""
 
-    __slots__ = ("req", "tokens", "scores", "n_new", "min_new", "max_new", "last", "done")
+    __slots__ = ("group", "replica", "tokens", "scores", "n_new", "min_new", "max_new", "last",
+                 "done")
 
-    def __init__(self, req: Request, tokens: List[int], scores: List[float], max_new: int):
-        self.req, self.tokens, self.scores = req, tokens, scores
+    def __init__(self, group: "_Group", replica: int, tokens: List[int], scores: List[float]):
+        req = group.req
+        self.group, self.replica = group, replica
+        self.tokens, self.scores = tokens, scores
         self.n_new = 0
         self.min_new = int(req.options.get("min_tokens", 0) or 0)
-        self.max_new = max_new
+        self.max_new = group.max_new
         self.last = tokens[-1]
         self.done = False
 
@@ -259,6 +279,30 @@ class _Row:
         return self.done
 
 
+class _Group:
+    """A request in flight: its replicas (``best_of`` rows that share the prompt), how they are
+    chosen, and the records of those that have ended."""
+
+    def __init__(self, req: Request, max_new: int):
+        o = req.options
+        self.req, self.max_new = req, max_new
+        self.n = int(o.get("n", 1) or 1)
+        self.replicas = int(o.get("best_of") or self.n)
+        # the reference's reading of the two options (metaseq/hub_utils.py:262-274): top_p <= 0
+        # or temperature 0 mean greedy; temperature 0 also means "do not scale"
+        temperature = o.get("temperature", 1.0)
+        temperature = 1.0 if temperature is None else float(temperature)
+        top_p = o.get("top_p", -1.0)
+        top_p = float(top_p) if (top_p is not None and top_p > 0) else 0.0
+        if temperature == 0:
+            temperature, top_p = 1.0, 0.0
+        self.temperature, self.topp = temperature, top_p
+        # rows chosen inside the vocabulary projection (greedy on the unscaled logits) or by the
+        # sampling kernel on the stored logits (any other temperature, nucleus sampling)
+        self.plain = temperature == 1.0 and top_p == 0.0
+        self.finished: Dict[int, "_Row"] = {}
+
+
 class SlotBatch:
     """The running batch of the continuous engine: which request sits in which slot, and the
     arithmetic that decides whether a request can be taken in."""
@@ -272,6 +316,9 @@ class SlotBatch:
             if r is None:
                 return i
         return None
+
+    def free_slots(self) -> List[int]:
+        return [i for i, r in enumerate(self.rows) if r is None]
 
     def active(self):
         return [(i, r) for i, r in enumerate(self.rows) if r is not None]
@@ -288,18 +335,26 @@ class SlotBatch:
 
 
 class ContinuousBatcher(_Front):
-    """Continuous batching of greedy requests over ``slots`` rows of one KV cache.
+    """Continuous batching over ``slots`` rows of one KV cache.
 
     ``interface`` is the ``GeneratorInterface`` whose model, dictionary and tokenizer are used;
-    ``capacity`` is the number of positions a slot can hold (prompt + continuation).  Requests
-    that need sampling, several replicas, penalties or ``logprobs`` are refused with a
-    ValueError delivered to the caller (serve them through ``BatchingService``)."""
+    ``capacity`` is the number of positions a slot can hold (prompt + continuation).  Greedy and
+    sampled requests (``temperature``, ``top_p``) share the running batch, each row under its own
+    temperature, nucleus and length rules; ``n`` / ``best_of`` replicas of a request are rows of
+    their own that share one prefill.  Requests that need penalties, the factual-nucleus decay
+    or ``logprobs`` are refused with a ValueError delivered to the caller (serve them through
+    ``BatchingService``).
+
+    ``noise_fn(request, replica, position, vocab)`` -> fp32 [vocab] device tensor, if given,
+    supplies the Exp(1) numbers of the draw that chooses the token at ``position`` of that
+    replica (tests hand both engines the same numbers); otherwise they come from torch's device
+    generator.  A request that has waited ``patience`` steps is served before cheaper ones."""
 
     UNSUPPORTED = ("lambda_decay", "alpha_presence", "alpha_frequency", "alpha_presence_src",
                    "alpha_frequency_src")
 
     def __init__(self, interface, slots: int = 32, capacity: int = MAX_SEQ_LEN,
-                 idle_ms: float = 2.0):
+                 idle_ms: float = 2.0, noise_fn=None, patience: int = 64):
         super().__init__(idle_ms / 1000.0)
         import torch
 
@@ -315,11 +370,16 @@ class ContinuousBatcher(_Front):
         self.backlog = Backlog()
         self.cache = None  # allocated with the first request
         self._stop: tuple = ()  # stop ids of the running batch
+        self.noise_fn, self.patience = noise_fn, int(patience)
         dev = self.device
         self._last = torch.full((slots,), self.dict.pad(), dtype=torch.long, device=dev)
         self._mode = torch.zeros(slots, dtype=torch.uint8, device=dev)
         self._tok = torch.zeros(slots, dtype=torch.long, device=dev)
         self._score = torch.zeros(slots, dtype=torch.float32, device=dev)
+        # state of the rows the sampling kernel chooses (allocated with the first such request)
+        self._smode = self._temp = self._topp = self._logits = self._noise = None
+        self._clock = 0         # step() calls so far; a request's arrival is stamped with it
+        self._arrived: Dict[int, int] = {}
         self.steps = 0          # decode steps run
         self.rows_stepped = 0   # active rows summed over those steps
 
@@ -330,16 +390,21 @@ class ContinuousBatcher(_Front):
         if problem:
             req.answer(ValueError(problem))
         else:
-            self.backlog.put(req, signature="")  # one queue: every greedy request can share
+            self._arrived[req.uid] = self._clock
+            self.backlog.put(req, signature="")  # one queue: all requests can share the batch
         return req.reply
 
     def _why_not(self, req: Request) -> Optional[str]:
         o = req.options
-        temperature, top_p = o.get("temperature", 1.0), o.get("top_p", -1.0)
-        if not (temperature == 0 or ((top_p is None or top_p <= 0) and temperature == 1.0)):
-            return "continuous batching serves greedy requests only (temperature 0, or top_p <= 0)"
-        if (o.get("n", 1) or 1) != 1 or (o.get("best_of") or 1) != 1:
-            return "continuous batching serves one replica per request"
+        temperature = o.get("temperature", 1.0)
+        if temperature is not None and temperature < 0:
+            return "temperature must be >= 0"
+        n, best_of = int(o.get("n", 1) or 1), int(o.get("best_of") or 0)
+        if n < 1 or (best_of and best_of < n):
+            return "best_of must be at least n, and n at least 1"
+        if max(n, best_of) > len(self.batch.rows):
+            return ("%d replicas do not fit the %d slots of the running batch"
+                    % (max(n, best_of), len(self.batch.rows)))
         if (o.get("logprobs", 0) or 0) > 0:
             return "continuous batching does not record distributions (logprobs > 0)"
         for k in self.UNSUPPORTED:
@@ -353,81 +418,155 @@ class ContinuousBatcher(_Front):
         return None
 
     # -- consumer side ------------------------------------------------------------------
-    def _admit(self, slot: int, req: Request):
-        """Prefill into the slot and choose the request's first token from the prompt's last
-        position."""
+    def _sampling_state(self):
+        """Per-slot state of the rows chosen by the sampling kernel, on first use."""
+        if self._smode is None:
+            torch, dev, slots = self._torch, self.device, len(self.batch.rows)
+            V = len(self.dict)
+            self._smode = torch.zeros(slots, dtype=torch.uint8, device=dev)
+            self._temp = torch.ones(slots, dtype=torch.float32, device=dev)
+            self._topp = torch.zeros(slots, dtype=torch.float32, device=dev)
+            self._logits = torch.empty(slots, V, dtype=torch.float16, device=dev)
+            self._noise = torch.empty(slots, V, dtype=torch.float32, device=dev)
+
+    def _draw_noise(self, out, rows):
+        """Exp(1) numbers for the draws of ``rows`` ((index into ``out``, row) pairs)."""
+        if self.noise_fn is None:
+            out.exponential_()
+            return
+        V = out.shape[1]
+        for i, row in rows:
+            out[i].copy_(self.noise_fn(row.group.req, row.replica, len(row.tokens), V))
+
+    def _admit(self, slots: List[int], req: Request):
+        """One prefill for the request, its keys and values copied to every replica's slot, and
+        each replica's first token chosen from the prompt's last position."""
         torch = self._torch
         eos, pad = self.dict.eos(), self.dict.pad()
         if self.cache is None:
             self.cache = self.decoder.new_slot_cache(len(self.batch.rows), self.batch.capacity,
                                                      self.device)
         ids = [eos] + req.prompt
-        row = _Row(req, ids, [], self.batch.room_for(req))
-        row.scores = self.decoder.admit_slot(
-            self.cache, slot, torch.tensor(ids, dtype=torch.long, device=self.device),
-            banned=[pad], stop=self._stop, eos=eos, mode=row.mode(),
-            tok_out=self._tok[slot:slot + 1], score_out=self._score[slot:slot + 1])
-        self.batch.rows[slot] = row
-        if row.take(int(self._tok[slot]), float(self._score[slot]), eos, self._stop):
-            self._retire(slot)
+        group = _Group(req, self.batch.room_for(req))
+        rows = [_Row(group, j, list(ids), []) for j in range(group.replicas)]
+        R = len(rows)
+        tok = torch.zeros(R, dtype=torch.long, device=self.device)
+        score = torch.zeros(R, dtype=torch.float32, device=self.device)
+        extra = {}
+        if not group.plain:
+            self._sampling_state()
+            noise = None
+            if group.topp > 0:
+                noise = self._noise[:R]
+                self._draw_noise(noise, list(enumerate(rows)))
+            extra = dict(temperature=group.temperature, topp=group.topp, noise=noise)
+        if R > 1:
+            extra["replicas"] = slots[1:]
+        prompt_scores = self.decoder.admit_slot(
+            self.cache, slots[0], torch.tensor(ids, dtype=torch.long, device=self.device),
+            banned=[pad], stop=self._stop, eos=eos, mode=rows[0].mode(), tok_out=tok,
+            score_out=score, **extra)
+        toks, scs = tok.tolist(), score.tolist()
+        for j, (slot, row) in enumerate(zip(slots, rows)):
+            row.scores = list(prompt_scores)
+            self.batch.rows[slot] = row
+            if row.take(toks[j], scs[j], eos, self._stop):
+                self._retire(slot)
 
     def _retire(self, slot: int):
         row = self.batch.rows[slot]
         self.batch.rows[slot] = None
         self.decoder.release_slot(self.cache, slot)
-        req = row.req
+        group = row.group
+        group.finished[row.replica] = row
+        if len(group.finished) < group.replicas:
+            return
+        req = group.req
         try:
-            # the row as the generation loop would return it: tokens up to the end, then eos
-            toks, scs = list(row.tokens), list(row.scores)
-            if toks[-1] != self.dict.eos():
-                toks.append(self.dict.eos())
-                scs.append(0.0)
-            rec = self.interface._record(toks, scs, None, len(req.prompt), row.max_new,
-                                         bool(req.options.get("echo", False)), 0)
-            req.answer([rec])
+            # replicas best cumulative score first (metaseq/sequence_generator.py:325-333), each
+            # as the generation loop would return it: tokens up to the end, then eos
+            ranked = sorted(group.finished.values(), key=lambda r: (-sum(r.scores), r.replica))
+            records = []
+            for r in ranked[:group.n]:
+                toks, scs = list(r.tokens), list(r.scores)
+                if toks[-1] != self.dict.eos():
+                    toks.append(self.dict.eos())
+                    scs.append(0.0)
+                records.append(self.interface._record(
+                    toks, scs, None, len(req.prompt), group.max_new,
+                    bool(req.options.get("echo", False)), 0))
+            req.answer(records)
         except Exception as e:  # noqa: BLE001 - delivered to the caller
             req.answer(e)
+
+    def _next_request(self) -> Optional[Request]:
+        """The cheapest waiting request, unless the oldest one has waited ``patience`` steps."""
+        old = self.backlog.take_oldest(
+            "", lambda r: self._clock - self._arrived.get(r.uid, self._clock) >= self.patience)
+        return old if old is not None else self.backlog.take("")
 
     def step(self) -> int:
         """Takes waiting requests into free slots, then runs one decode step over the occupied
         slots.  Returns the number of rows that were served (admitted or stepped).  The rows of
         the running batch share one stop list: a request with another one waits until the batch
-        has drained."""
+        has drained, and nothing is admitted past it while it waits."""
         torch = self._torch
+        self._clock += 1
         served = 0
         while True:
-            slot = self.batch.free_slot()
-            if slot is None:
+            free = self.batch.free_slots()
+            if not free:
                 break
-            req = self.backlog.take("")
+            req = self._next_request()
             if req is None:
                 break
+            need = int(req.options.get("best_of") or req.options.get("n", 1) or 1)
             stop = tuple(sorted(req.options.get("stop") or ()))
-            if self.batch.active() and stop != self._stop:
+            if (self.batch.active() and stop != self._stop) or need > len(free):
                 self.backlog.put(req, signature="")
                 break
             self._stop = stop
+            self._arrived.pop(req.uid, None)
             try:
-                self._admit(slot, req)
+                self._admit(free[:need], req)
             except RuntimeError:
                 raise
             except Exception as e:  # noqa: BLE001 - this request's own answer
-                self.batch.rows[slot] = None
+                for slot in free[:need]:
+                    self.batch.rows[slot] = None
+                    if self.cache is not None:
+                        self.decoder.release_slot(self.cache, slot)
                 req.answer(e)
-            served += 1
+            served += need
         active = self.batch.active()
         if not active:
             return served
         eos, pad = self.dict.eos(), self.dict.pad()
-        last = [pad] * len(self.batch.rows)
-        mode = [0] * len(self.batch.rows)
+        slots = len(self.batch.rows)
+        last, mode = [pad] * slots, [0] * slots
+        general = [(i, row) for i, row in active if not row.group.plain]
         for i, row in active:
             last[i], mode[i] = row.last, row.mode()
         self._last.copy_(torch.tensor(last, dtype=torch.long))
         self._mode.copy_(torch.tensor(mode, dtype=torch.uint8))
+        extra = {}
+        if general:
+            smode, temp, topp = [4] * slots, [1.0] * slots, [0.0] * slots  # 4 = MSA_ROW_SKIP
+            for i, row in general:
+                smode[i], temp[i], topp[i] = mode[i], row.group.temperature, row.group.topp
+            self._smode.copy_(torch.tensor(smode, dtype=torch.uint8))
+            self._temp.copy_(torch.tensor(temp, dtype=torch.float32))
+            self._topp.copy_(torch.tensor(topp, dtype=torch.float32))
+            noise = None
+            if any(t > 0 for t in topp):
+                noise = self._noise
+                self._draw_noise(noise, [(i, row) for i, row in general if row.group.topp > 0])
+            extra = dict(logits_out=self._logits,
+                         sampled=dict(row_mode=self._smode, temperature=self._temp,
+                                      topp=self._topp, noise=noise))
         self.decoder.decode_slots(self.cache, self._last, temperature=1.0, banned=[pad],
                                   stop=self._stop, eos=eos, row_mode=self._mode,
-                                  tok_out=self._tok, score_out=self._score)
+                                  tok_out=self._tok, score_out=self._score, **extra)
         toks, scs = self._tok.tolist(), self._score.tolist()
         self.steps += 1
         self.rows_stepped += len(active)

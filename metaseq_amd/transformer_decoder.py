@@ -760,12 +760,19 @@ class TransformerDecoder(nn.Module):
         return self._project(h, False, 1, T)[0]
 
     def admit_slot(self, cache: KVCache, slot: int, tokens: torch.Tensor, *, banned=(), stop=(),
-                   eos=2, mode=0, tok_out=None, score_out=None):
+                   eos=2, mode=0, tok_out=None, score_out=None, temperature=1.0, topp=0.0,
+                   noise=None, replicas=()):
         """``prefill_slot`` plus what a request needs from its prompt: the log-probability of
         every prompt token given its prefix (returned as a list, 0.0 for the first token) and
-        the greedy choice of the first new token from the last position, written to
-        ``tok_out`` / ``score_out`` (one-element int64 / fp32 device tensors) under the
-        selection regime ``mode`` (MSA_ROW_* bits)."""
+        the choice of the first new token from the last position, written to ``tok_out`` /
+        ``score_out`` (int64 / fp32 device tensors, one element per replica) under the selection
+        regime ``mode`` (MSA_ROW_* bits).
+
+        With the defaults the choice is greedy on the unscaled logits.  ``temperature`` scales
+        the logits (prompt scores included, as the reference's loop does); ``topp`` > 0 with
+        ``noise`` (fp32 [1 + len(replicas), V], independent Exp(1) numbers) draws from the
+        nucleus.  ``replicas``: further slots that receive a copy of the prompt's keys and values
+        and make their own choice (row r of ``noise``, element r of the outputs)."""
         lib = self.prepare_()
         logits = self.prefill_slot(cache, slot, tokens)
         T, V = logits.shape
@@ -774,49 +781,88 @@ class TransformerDecoder(nn.Module):
         if T > 1:
             lp = torch.empty(T - 1, dtype=torch.float32, device=logits.device)
             target = tokens.long()[1:].contiguous()
-            check(lib.msa_target_logprob_f16(ptr(logits), logits.stride(0), T - 1, V, 1.0,
-                                             ptr(target), ptr(lp), stream))
+            check(lib.msa_target_logprob_f16(ptr(logits), logits.stride(0), T - 1, V,
+                                             float(temperature), ptr(target), ptr(lp), stream))
             scores[1:] = lp.tolist()
+        for dst in replicas:
+            self.copy_slot(cache, slot, dst)
+        R = 1 + len(replicas)
+        plain = float(temperature) == 1.0 and not topp > 0 and noise is None
         banned, stop = list(banned), list(stop)
         ba = (ctypes.c_int32 * max(1, len(banned)))(*banned)
         sa = (ctypes.c_int32 * max(1, len(stop)))(*stop)
-        row_mode = torch.tensor([mode], dtype=torch.uint8, device=logits.device)
+        row_mode = torch.full((R,), mode, dtype=torch.uint8, device=logits.device)
         last = logits[T - 1:T]
-        check(lib.msa_greedy_select_f16(ptr(last), last.stride(0), 1, V, 1.0, ba, len(banned), sa,
-                                        len(stop), None, ptr(row_mode), 0, int(eos), ptr(tok_out),
-                                        1, ptr(score_out), 1, None, stream))
+        if R > 1:  # every replica reads its own copy of the row (a few hundred KB)
+            last = last.expand(R, V).contiguous()
+        if plain:
+            check(lib.msa_greedy_select_f16(ptr(last), last.stride(0), R, V, 1.0, ba, len(banned),
+                                            sa, len(stop), None, ptr(row_mode), 0, int(eos),
+                                            ptr(tok_out), 1, ptr(score_out), 1, None, stream))
+        else:
+            check(lib.msa_sample_topp_f16(
+                ptr(last), last.stride(0), R, V, float(temperature), None, ba, len(banned), sa,
+                len(stop), None, ptr(row_mode), 0, int(eos), None, float(topp), ptr(noise), None,
+                None, 0.0, 0.0, 0.0, 0.0, None, 0, ptr(tok_out), 1, ptr(score_out), 1, stream))
         return scores
+
+    def copy_slot(self, cache: KVCache, src: int, dst: int):
+        """Makes slot ``dst`` a copy of slot ``src``: keys, values and length (a replica of a
+        request starts from the same prompt)."""
+        n = int(cache.lens[src])
+        for layer in cache.layers:
+            layer[:, dst, :, :n].copy_(layer[:, src, :, :n])
+        cache.lens[dst] = n
 
     def release_slot(self, cache: KVCache, slot: int):
         cache.lens[slot] = -1
 
     def decode_slots(self, cache: KVCache, last_tokens: torch.Tensor, *, temperature=1.0,
                      banned=(), stop=(), eos=2, row_mode=None, tok_out=None, score_out=None,
-                     finished=None, logits_out=None):
+                     finished=None, logits_out=None, sampled=None):
         """One decode step over every active slot: ``last_tokens`` ([slots] ids on the device;
         what an inactive slot holds does not matter) are embedded at each row's own position,
         appended to its history and attended over it; the vocabulary projection selects the
         next token greedily into ``tok_out`` / ``score_out`` ([slots], int64 / fp32) under the
         per-row ``row_mode`` (uint8 [slots]: MSA_ROW_BAN_EARLY, MSA_ROW_ONLY_EOS).  Every active
-        row's length advances by one.  Outputs of inactive slots are undefined."""
+        row's length advances by one.  Outputs of inactive slots are undefined.
+
+        ``sampled``: rows that are not chosen that way (another temperature, nucleus sampling) -
+        a dict with ``row_mode`` (uint8 [slots]: the regime bits of those rows, MSA_ROW_SKIP for
+        all others), ``temperature`` and ``topp`` (fp32 [slots]; top-p 0 = greedy at that
+        temperature) and ``noise`` (fp32 [slots, V] Exp(1) numbers, or None).  The step then
+        also stores its logits (``logits_out``, [slots, V] fp16, required) and
+        msa_sample_topp_f16 overwrites the outputs of those rows."""
         lib = self.prepare_()
         stream = _capi.stream_ptr()
         B = cache.batch
         if last_tokens.shape != (B,) or last_tokens.dtype != torch.long:
             raise AssertionError("last_tokens must be int64 [%d]" % B)
+        if sampled is not None and logits_out is None:
+            raise AssertionError("sampled rows need logits_out")
         if self.native_step and not self.return_inner_states:
             select = dict(temperature=temperature, banned=banned, stop=stop, finished=finished,
                           row_mode=row_mode, force_eos=False, eos=eos, tok_out=tok_out,
                           tok_stride=1, score_out=score_out, score_stride=1)
             self._native_step(lib, stream, last_tokens.view(B, 1), 1, B, cache, None, cache.lens,
                               0, {"logits": logits_out, "select": select})
-            return
-        bufs = self._step_buffers(cache, B)
-        feat, _ = self._decode_core(lib, stream, last_tokens.view(B, 1), 1, B, cache, None, bufs,
-                                    cache.lens, 0, True)
-        check(lib.msa_advance_len(ptr(cache.lens), ptr(bufs["step_len"]), B, 1, stream))
-        self._select_from(lib, feat, B, temperature, banned, stop, finished, row_mode, False, eos,
-                          tok_out, 1, score_out, 1, logits_out)
+        else:
+            bufs = self._step_buffers(cache, B)
+            feat, _ = self._decode_core(lib, stream, last_tokens.view(B, 1), 1, B, cache, None,
+                                        bufs, cache.lens, 0, True)
+            check(lib.msa_advance_len(ptr(cache.lens), ptr(bufs["step_len"]), B, 1, stream))
+            self._select_from(lib, feat, B, temperature, banned, stop, finished, row_mode, False,
+                              eos, tok_out, 1, score_out, 1, logits_out)
+        if sampled is not None:
+            banned, stop = list(banned), list(stop)
+            ba = (ctypes.c_int32 * max(1, len(banned)))(*banned)
+            sa = (ctypes.c_int32 * max(1, len(stop)))(*stop)
+            V = self.cfg.vocab_size
+            check(lib.msa_sample_topp_f16(
+                ptr(logits_out), logits_out.stride(0), B, V, 1.0, ptr(sampled["temperature"]), ba,
+                len(banned), sa, len(stop), ptr(finished), ptr(sampled["row_mode"]), 0, int(eos),
+                ptr(sampled["topp"]), 0.0, ptr(sampled.get("noise")), None, None, 0.0, 0.0, 0.0,
+                0.0, None, 0, ptr(tok_out), 1, ptr(score_out), 1, stream))
 
     def extract_features(self, prev_output_tokens, incremental_state=None,
                          token_embeddings=None, self_attn_padding_mask=None):

@@ -974,16 +974,18 @@ def test_stream_read_probe_runs_and_validates(lib):
 # ---- nucleus sampling kernel ------------------------------------------------------------------
 def _sample(lib, logits, *, temperature=1.0, banned=(1,), stop=(), finished=None, row_mode=None,
             force=0, eos=2, topp_rows=None, topp_all=0.0, noise=None, counts=None,
-            counts_src=None, alphas=(0.0, 0.0, 0.0, 0.0)):
+            counts_src=None, alphas=(0.0, 0.0, 0.0, 0.0), temperature_rows=None, lprobs=None):
     B, V = logits.shape
     ba = (ctypes.c_int32 * max(1, len(banned)))(*banned)
     sa = (ctypes.c_int32 * max(1, len(stop)))(*stop)
     tok = torch.full((B,), -7, dtype=torch.long, device=DEV)
     sc = torch.zeros(B, dtype=torch.float32, device=DEV)
-    ok(lib.msa_sample_topp_f16(P(logits), logits.stride(0), B, V, temperature, ba, len(banned), sa,
-                               len(stop), P(finished), P(row_mode), force, eos, P(topp_rows),
-                               topp_all, P(noise), P(counts), P(counts_src), alphas[0], alphas[1],
-                               alphas[2], alphas[3], P(tok), 1, P(sc), 1, None), lib)
+    ok(lib.msa_sample_topp_f16(P(logits), logits.stride(0), B, V, temperature, P(temperature_rows),
+                               ba, len(banned), sa, len(stop), P(finished), P(row_mode), force,
+                               eos, P(topp_rows), topp_all, P(noise), P(counts), P(counts_src),
+                               alphas[0], alphas[1], alphas[2], alphas[3], P(lprobs),
+                               0 if lprobs is None else lprobs.stride(0), P(tok), 1, P(sc), 1,
+                               None), lib)
     torch.cuda.synchronize()
     return tok.cpu(), sc.cpu()
 
@@ -1029,9 +1031,11 @@ def test_nucleus_sampling_kernel_matches_oracle_given_the_same_noise(lib, V, B):
     lp = _reference_lprobs(logits, 0.8, [1], early, only, eos, counts, counts_src, alphas)
     want_sc, want_tok, _, _ = O.sample_topp(lp, topp.unsqueeze(1), noise=noise)
     cd = G(counts.clone())
+    # the step's distribution goes into rows of a wider buffer, as into all_lprobs[:, step]
+    stored = torch.full((B, 2, V + 3), 7.0, dtype=torch.float32, device=DEV)
     tok, sc = _sample(lib, G(logits), temperature=0.8, banned=[1], stop=stop, finished=G(fin.clone()),
                       row_mode=G(modes), eos=eos, topp_rows=G(topp), noise=G(noise), counts=cd,
-                      counts_src=G(counts_src), alphas=alphas)
+                      counts_src=G(counts_src), alphas=alphas, lprobs=stored[:, 1])
     dead = ~torch.isfinite(lp).any(-1)      # eos banned and alone eligible: (0, -inf)
     assert bool(dead[3]) and int(tok[3]) == 0 and float(sc[3]) == float("-inf")
     live = ~dead
@@ -1040,6 +1044,66 @@ def test_nucleus_sampling_kernel_matches_oracle_given_the_same_noise(lib, V, B):
     bumped = counts.clone()
     bumped[torch.arange(B), tok] += 1
     assert torch.equal(cd.cpu(), bumped)
+    # the stored rows are the reference's masked, penalised log-probabilities (-inf where they
+    # are), and nothing around them was touched
+    got_lp = stored[:, 1, :V].cpu()
+    assert torch.equal(torch.isinf(got_lp), torch.isinf(lp))
+    fin_ = torch.isfinite(lp)
+    assert torch.allclose(got_lp[fin_], lp[fin_], atol=1e-5, rtol=1e-6)
+    assert bool((stored[:, 0] == 7.0).all()) and bool((stored[:, 1, V:] == 7.0).all())
+
+
+def test_sampling_kernel_per_row_temperature_and_skipped_rows(lib):
+    """Rows of one call at their own temperature and top-p equal the same rows run one call
+    each; a row marked MSA_ROW_SKIP keeps whatever its outputs held; top-p 0 or temperature 0 for
+    a row makes that row greedy."""
+    B, V = 6, 4001
+    g = torch.Generator().manual_seed(11)
+    logits = (torch.randn(B, V, generator=g) * 2.0).half()
+    noise = torch.empty(B, V).exponential_(generator=g)
+    temps = torch.tensor([1.0, 0.7, 1.3, 0.0, 0.5, 0.9])
+    topp = torch.tensor([0.9, 0.5, 1.0, 0.8, 0.0, 0.3])
+    modes = torch.tensor([0, 0, 4, 0, 0, 1], dtype=torch.uint8)          # row 2 is skipped
+    ld, nd = G(logits), G(noise)
+    ba = (ctypes.c_int32 * 1)(1)
+    sa = (ctypes.c_int32 * 1)(9)
+    tok = torch.full((B,), -7, dtype=torch.long, device=DEV)
+    sc = torch.full((B,), 5.0, dtype=torch.float32, device=DEV)
+    ok(lib.msa_sample_topp_f16(P(ld), V, B, V, 1.0, P(G(temps)), ba, 1, sa, 1, None, P(G(modes)),
+                               0, 2, P(G(topp)), 0.0, P(nd), None, None, 0.0, 0.0, 0.0, 0.0, None,
+                               0, P(tok), 1, P(sc), 1, None), lib)
+    torch.cuda.synchronize()
+    assert int(tok[2]) == -7 and float(sc[2]) == 5.0
+    for r in (0, 1, 3, 4, 5):
+        t, p_ = float(temps[r]), float(topp[r])
+        greedy = t == 0.0 or p_ == 0.0
+        one_tok, one_sc = _sample(lib, ld[r:r + 1], temperature=t, banned=[1], stop=[9],
+                                  row_mode=G(modes[r:r + 1]), topp_all=0.0 if greedy else p_,
+                                  noise=None if greedy else nd[r:r + 1])
+        assert int(tok[r]) == int(one_tok[0]) and float(sc[r]) == float(one_sc[0]), r
+        if greedy:
+            z = logits[r].float() / (t if t > 0 else 1.0)
+            lp = torch.log_softmax(z, -1)
+            lp[1] = float("-inf")
+            assert int(tok[r]) == int(lp.argmax()) and abs(float(sc[r]) - float(lp.max())) < 2e-5
+
+
+def test_log_softmax_rows_into_a_strided_buffer(lib):
+    """msa_log_softmax_f16 against torch's fp32 log_softmax: rows (b, t), t < T - 1, of logits
+    [B, T, V] land at out[b, t + 1], as the generator stores the prompt's distributions."""
+    B, T, V, L = 3, 5, 4001, 9
+    g = torch.Generator().manual_seed(5)
+    logits = (torch.randn(B, T, V, generator=g) * 3.0).half()
+    out = torch.full((B, L, V), 7.0, dtype=torch.float32, device=DEV)
+    ld = G(logits)
+    for temperature in (1.0, 0.6):
+        ok(lib.msa_log_softmax_f16(P(ld), T * V, V, B, T - 1, V, temperature, P(out[:, 1]), L * V, V,
+                                   None), lib)
+        torch.cuda.synchronize()
+        want = torch.log_softmax(logits.float() / temperature, -1)[:, :-1]
+        assert torch.allclose(out[:, 1:T].cpu(), want, atol=2e-5, rtol=1e-6)
+        assert bool((out[:, 0] == 7.0).all()) and bool((out[:, T:] == 7.0).all())
+    assert lib.msa_log_softmax_f16(P(ld), T * V, V - 1, B, T, V, 1.0, P(out), L * V, V, None) == -1
 
 
 def test_nucleus_sampling_kernel_closed_forms(lib):

@@ -3,9 +3,9 @@ and the request front end on the GPU.
 
 Parity for sampling is exact, not statistical: with a scripted decoder both sides see identical
 log-probabilities, and the oracle (run on the same device) is handed the very Exp(1) numbers the
-product's sampling kernel draws with (or, with ``need_logprobs``, makes the same sequence of
-``torch.multinomial`` calls from the same seed), so the tokens must agree exactly.  The draw rule
-itself is pinned on the CPU (frequencies and nucleus membership).
+product's sampling kernel draws with, so the tokens must agree exactly - with ``need_logprobs``
+too, where the same kernel also writes every step's distribution.  The draw rule itself is
+pinned on the CPU (frequencies and nucleus membership).
 """
 import math
 
@@ -48,13 +48,9 @@ def _both(kw, B=3, seed=11, beam=1, max_len_b=16, min_len=6, src=None):
     got = gen.generate([dec], {"net_input": {"src_tokens": src.to(DEV)}})
     dec2 = ScriptedDecoder(script, V, device=DEV, dtype=torch.float16)
     torch.manual_seed(1234)
-    # the kernel path draws by an exponential race over token ids, one Exp(1) number per row
-    # and id and step from the device generator; the oracle is handed the same numbers.  With
-    # need_logprobs the product takes its tensor-op path and draws with torch.multinomial, as
-    # the oracle then does too.
-    noise_fn = None
-    if not kw.get("need_logprobs"):
-        noise_fn = lambda shape: torch.empty(shape, dtype=torch.float32, device=DEV).exponential_()
+    # the kernel draws by an exponential race over token ids, one Exp(1) number per row and id
+    # and step from the device generator; the oracle is handed the same numbers
+    noise_fn = lambda shape: torch.empty(shape, dtype=torch.float32, device=DEV).exponential_()
     want = O.generate(dec2, src.to(DEV), max_len_b=max_len_b, min_len=min_len, beam_size=beam,
                       full_stop_list=tuple(FULL_STOPS.values()), noise_fn=noise_fn, **kw)
     return got, want
@@ -70,19 +66,21 @@ def _both(kw, B=3, seed=11, beam=1, max_len_b=16, min_len=6, src=None):
     dict(alpha_presence_src=1.0, alpha_frequency_src=0.3),
     dict(topp=0.8, alpha_presence=0.5, alpha_presence_src=0.5, alpha_frequency_src=0.1,
          need_logprobs=True),
+    dict(need_logprobs=True, temperature=0.8, stop=[10]),            # greedy, distributions kept
 ], ids=lambda k: ",".join("%s=%s" % kv for kv in k.items()))
 def test_general_path_matches_oracle_bit_for_bit(kw):
     got, want = _both(kw)
     assert torch.equal(got["tokens"], want["tokens"]), (got["tokens"], want["tokens"])
     n0 = 4
-    # scores: the kernels' fp32 summation order differs from the tensor ops'; with need_logprobs
-    # the generated positions run the same device ops on both sides and agree to the last bit
-    if kw.get("need_logprobs"):
-        assert torch.equal(got["scores"][..., n0:], want["scores"][..., n0:])
+    # scores and distributions: the kernels' fp32 summation order differs from the tensor ops'
     assert torch.allclose(got["scores"], want["scores"], atol=2e-5)
     if kw.get("need_logprobs"):
-        assert torch.equal(got["distributions"][:, :, n0:], want["distributions"][:, :, n0:])
-        assert torch.allclose(got["distributions"], want["distributions"], atol=2e-5)
+        gd, wd = got["distributions"], want["distributions"]
+        assert gd.shape == wd.shape
+        assert torch.equal(torch.isinf(gd), torch.isinf(wd)), "masked ids differ"
+        ok = torch.isfinite(wd)
+        assert torch.allclose(gd[ok], wd[ok], atol=2e-5)
+        assert bool(torch.isfinite(gd[:, :, n0:]).any())
     # sampling really happened: some pick is not the arg-max of its distribution
     if kw.get("topp", 0) >= 0.8:
         greedy, _ = _both({k: v for k, v in kw.items() if k != "topp"})
@@ -280,3 +278,57 @@ def test_continuous_batcher_rows_equal_single_request_generation():
         assert got[0]["text"] == want[0][0]["text"]
     # every slot is free again and the cache holds no active row
     assert cb.cache.lens.tolist() == [-1, -1, -1]
+
+
+def _noise_for(prompt, replica, position, vocab):
+    """Exp(1) numbers that depend only on the request's prompt, the replica and the position of
+    the token being drawn, so that two engines can be handed the same ones."""
+    g = torch.Generator(device=DEV).manual_seed(7919 * sum(prompt) + 101 * replica + position)
+    return torch.empty(vocab, dtype=torch.float32, device=DEV).exponential_(generator=g)
+
+
+def test_continuous_batcher_sampled_rows_equal_single_request_generation():
+    """Sampled requests (each with its own temperature and top-p), greedy requests at another
+    temperature, plainly greedy ones and requests with several replicas share the slots of one
+    running batch.  Given the same noise per (request, replica, position), every request gets
+    the tokens and scores of a generation of its own: its rows run through the same kernels on
+    the same logits, whatever their neighbours are and however they are chosen."""
+    from metaseq_amd.service import ContinuousBatcher
+    gi, model, cfg, sd = _interface()
+    specs = [dict(prompt=[5, 9, 33, 12, 7], max_tokens=9, temperature=0.7, top_p=0.9),
+             dict(prompt=[40], max_tokens=5),
+             dict(prompt=[8, 8, 8, 21, 22, 23, 24, 25], min_tokens=5, max_tokens=12, top_p=0.5),
+             dict(prompt=[17, 4], max_tokens=6, temperature=0.5),
+             dict(prompt=[30, 31, 32], min_tokens=2, max_tokens=7, temperature=1.2, top_p=0.95,
+                  n=2, best_of=3),
+             dict(prompt=[11], max_tokens=10, temperature=0, top_p=0.9),
+             dict(prompt=[45, 46, 47, 48], max_tokens=6, top_p=1.0, echo=True)]
+    cb = ContinuousBatcher(gi, slots=5, capacity=40,
+                           noise_fn=lambda req, j, pos, V: _noise_for(req.prompt, j, pos, V))
+    replies = [cb.submit(s["prompt"], **{k: v for k, v in s.items() if k != "prompt"})
+               for s in specs]
+    n = 0
+    while cb.step():
+        n += 1
+        assert n < 300
+    assert cb.rows_stepped > cb.steps > 0
+    for s, r in zip(specs, replies):
+        _, got = r.get_nowait()
+        assert not isinstance(got, Exception), got
+        prompt = s["prompt"]
+        gi.noise_fn = lambda step, BB, V: torch.stack(
+            [_noise_for(prompt, j, step, V) for j in range(BB)])
+        want = gi.generate([prompt], max_tokens=[s["max_tokens"]],
+                           min_tokens=[s.get("min_tokens", 0)], echo=s.get("echo", False),
+                           temperature=s.get("temperature", 1.0), top_p=s.get("top_p", -1.0),
+                           n=s.get("n", 1), best_of=s.get("best_of"))[0]
+        gi.noise_fn = None
+        assert len(got) == len(want) == s.get("n", 1)
+        for g_rec, w_rec in zip(got, want):
+            assert g_rec["tokens"] == w_rec["tokens"], (s, g_rec["tokens"], w_rec["tokens"])
+            assert g_rec["token_scores"] == w_rec["token_scores"], s
+        if s is specs[0]:
+            # sampling happened: the continuation is not the request's greedy one
+            greedy = gi.generate([prompt], max_tokens=[9], min_tokens=[0])[0][0]
+            assert greedy["tokens"] != got[0]["tokens"]
+    assert cb.cache.lens.tolist() == [-1] * 5

@@ -128,8 +128,14 @@ def _rule(last, length):
     return EOS if t % 9 == 0 else max(t, 4)
 
 
-def _choose(last, length, mode, stop):
+def _choose(last, length, mode, stop, temperature=1.0, topp=0.0, noise=None):
+    """A row of the scripted model.  Rows that are not plainly greedy shift the rule's token by
+    a function of their temperature and, when they sample, of the largest noise entry: what
+    matters to these tests is that every parameter reaches the row it belongs to."""
     t = _rule(last, length)
+    if temperature != 1.0 or topp > 0:
+        shift = int(round(temperature * 10)) + (int(noise.argmax()) if topp > 0 else 0)
+        t = max((t + shift) % V, 4)
     if mode & 2:
         return EOS
     if mode & 1 and (t == EOS or t in stop):
@@ -154,17 +160,21 @@ class FakeSlotDecoder:
         self.capacity = capacity
         return self.Cache(slots)
 
-    def admit_slot(self, cache, slot, tokens, *, banned, stop, eos, mode, tok_out, score_out):
-        assert cache.lens[slot] == -1 and banned == [PAD] and eos == EOS
+    def admit_slot(self, cache, slot, tokens, *, banned, stop, eos, mode, tok_out, score_out,
+                   temperature=1.0, topp=0.0, noise=None, replicas=()):
+        assert banned == [PAD] and eos == EOS
         ids = tokens.tolist()
         self.prefills.append((slot, ids))
-        cache.lens[slot] = len(ids)
-        tok_out[0] = _choose(ids[-1], len(ids), mode, stop)
-        score_out[0] = -0.5
+        for r, s in enumerate([slot] + list(replicas)):
+            assert cache.lens[s] == -1
+            cache.lens[s] = len(ids)
+            tok_out[r] = _choose(ids[-1], len(ids), mode, stop, temperature, topp,
+                                 None if noise is None else noise[r])
+            score_out[r] = -0.5 - 0.01 * r
         return [0.0] + [-1.0] * (len(ids) - 1)
 
     def decode_slots(self, cache, last_tokens, *, temperature, banned, stop, eos, row_mode,
-                     tok_out, score_out):
+                     tok_out, score_out, logits_out=None, sampled=None):
         active = [i for i, n in enumerate(cache.lens) if n >= 0]
         self.steps.append(active)
         for i in active:
@@ -172,34 +182,48 @@ class FakeSlotDecoder:
             cache.lens[i] += 1
             tok_out[i] = _choose(int(last_tokens[i]), cache.lens[i], int(row_mode[i]), stop)
             score_out[i] = -0.25
+        if sampled is not None:
+            assert logits_out is not None
+            for i in active:
+                m = int(sampled["row_mode"][i])
+                if m & 4:
+                    continue
+                topp = float(sampled["topp"][i])
+                tok_out[i] = _choose(int(last_tokens[i]), cache.lens[i], m, stop,
+                                     round(float(sampled["temperature"][i]), 4), topp,
+                                     sampled["noise"][i] if topp > 0 else None)
+                score_out[i] = -0.125 * (i + 1)
 
     def release_slot(self, cache, slot):
         cache.lens[slot] = -1
 
 
-def _expected(prompt, min_tokens=0, max_tokens=0, stop=(), capacity=64):
-    """What one request generates on its own: the loop written out."""
+def _expected(prompt, min_tokens=0, max_tokens=0, stop=(), capacity=64, temperature=1.0,
+              topp=0.0, noise=None):
+    """What one request generates on its own: the loop written out.  ``noise(position)`` gives
+    the row's Exp(1) numbers for the draw of the token at that position."""
     ids = [EOS] + list(prompt)
     room = capacity - len(ids)
     max_new = max(1, min(max_tokens or room, room))
     out = []
     while True:
         mode = (1 if len(out) < min_tokens else 0) | (2 if len(out) >= max_new - 1 else 0)
-        t = _choose(ids[-1], len(ids), mode, stop)
+        t = _choose(ids[-1], len(ids), mode, stop, temperature, topp,
+                    noise(len(ids)) if (noise and topp > 0) else None)
         out.append(t)
         if t == EOS or t in stop or len(out) >= max_new:
             return out
         ids.append(t)
 
 
-def _batcher(slots=3, capacity=64):
+def _batcher(slots=3, capacity=64, **kw):
     class Model:
         pass
     model = Model()
     model.decoder = FakeSlotDecoder()
     model.max_positions = model.decoder.max_positions
     gi = GeneratorInterface(model, Dictionary(V), device="cpu")
-    return ContinuousBatcher(gi, slots=slots, capacity=capacity), model.decoder
+    return ContinuousBatcher(gi, slots=slots, capacity=capacity, **kw), model.decoder
 
 
 def _drain(cb, limit=500):
@@ -266,12 +290,92 @@ def test_continuous_batcher_echo_stop_lists_and_refusals():
         str(t) for t in _expected([8, 8, 8], max_tokens=5) if t != EOS]
     assert all(len(act) == 1 for act in dec.steps[-8:])   # the two never shared a step
     # what the engine does not serve is answered with an error, not queued
-    for bad in (dict(temperature=0.7, top_p=0.9), dict(n=2), dict(logprobs=3),
-                dict(alpha_presence=0.5)):
+    for bad in (dict(logprobs=3), dict(alpha_presence=0.5), dict(lambda_decay=0.9), dict(n=3),
+                dict(n=2, best_of=1), dict(temperature=-1)):
         res = cb.submit([5], **bad).get_nowait()[1]
         assert isinstance(res, ValueError), bad
     assert isinstance(cb.submit([5] * 70).get_nowait()[1], ValueError)    # longer than a slot
     assert cb.step() == 0
+
+
+def _noise(req, replica, position, vocab):
+    """Exp(1)-like numbers that depend on nothing but the request's prompt, the replica and the
+    position of the token being drawn."""
+    g = torch.Generator().manual_seed(1000 * sum(req.prompt) + 100 * replica + position)
+    return torch.empty(vocab).exponential_(generator=g)
+
+
+def test_continuous_batcher_mixes_greedy_and_sampled_rows_each_under_its_own_parameters():
+    """Sampled requests (their own temperature and top-p), greedy ones at another temperature
+    and plainly greedy ones share the running batch; every row is chosen with its own
+    parameters and noise, so each answer equals the request's own single-request loop."""
+    cb, dec = _batcher(slots=4, noise_fn=_noise)
+    specs = [dict(prompt=[5, 9, 4], max_tokens=12, temperature=0.7, top_p=0.9),
+             dict(prompt=[8], max_tokens=9),
+             dict(prompt=[6] * 7, min_tokens=4, max_tokens=15, temperature=1.3, top_p=0.5),
+             dict(prompt=[17, 4], max_tokens=8, temperature=0.5),                  # greedy, scaled
+             dict(prompt=[21, 30], max_tokens=10, temperature=0, top_p=0.9),      # plainly greedy
+             dict(prompt=[33, 13], max_tokens=11, top_p=0.3)]
+    replies = [cb.submit(s["prompt"], **{k: v for k, v in s.items() if k != "prompt"})
+               for s in specs]
+    _drain(cb)
+    assert max(len(a) for a in dec.steps) == 4
+    for s, r in zip(specs, replies):
+        res = r.get_nowait()[1]
+        assert not isinstance(res, Exception), res
+        t, p = s.get("temperature", 1.0), s.get("top_p", -1.0)
+        t, p = (1.0, 0.0) if t == 0 else (t, max(p, 0.0))
+        req = Request(0, s["prompt"], {})
+        want = _expected(s["prompt"], s.get("min_tokens", 0), s["max_tokens"], temperature=t,
+                         topp=p, noise=lambda pos: _noise(req, 0, pos, V))
+        assert res[0]["tokens"] == [str(x) for x in want if x != EOS], (s, res[0]["tokens"], want)
+
+
+def test_continuous_batcher_replicas_share_one_prefill_and_come_back_best_first():
+    cb, dec = _batcher(slots=4, noise_fn=_noise)
+    a = cb.submit([5, 9, 4], max_tokens=6, temperature=0.9, top_p=0.8, n=2, best_of=3)
+    b = cb.submit([8, 8], max_tokens=5)
+    _drain(cb)
+    assert len(dec.prefills) == 2                       # one prefill per request
+    res = a.get_nowait()[1]
+    assert len(res) == 2
+    req = Request(0, [5, 9, 4], {})
+    runs = []
+    for j in range(3):
+        toks = _expected([5, 9, 4], max_tokens=6, temperature=0.9, topp=0.8,
+                         noise=lambda pos: _noise(req, j, pos, V))
+        runs.append([str(x) for x in toks if x != EOS])
+    got = [r["tokens"] for r in res]
+    assert all(g in runs for g in got)
+    sums = [sum(r["token_scores"]) for r in res]
+    assert sums[0] >= sums[1]
+    assert b.get_nowait()[1][0]["tokens"] == [
+        str(t) for t in _expected([8, 8], max_tokens=5) if t != EOS]
+    # three replicas wait until three slots are free at once
+    cb, dec = _batcher(slots=3, noise_fn=_noise)
+    first = cb.submit([9] * 4, max_tokens=20)
+    second = cb.submit([7, 7, 7, 7, 7, 7, 7, 7], max_tokens=4, top_p=0.9, best_of=3)
+    _drain(cb)
+    assert len(second.get_nowait()[1]) == 1 and len(first.get_nowait()[1]) == 1
+    assert all(len(a) <= 3 for a in dec.steps)
+
+
+def test_continuous_batcher_serves_a_request_that_has_waited_before_cheaper_ones():
+    """Cheapest first is the rule, but a request that has waited ``patience`` steps goes first,
+    and a request whose stop list differs from the running batch's blocks later arrivals until
+    the batch has drained: neither can starve."""
+    cb, dec = _batcher(slots=1, patience=3)
+    long_one = cb.submit([9] * 12, max_tokens=2)
+    for _ in range(12):
+        cb.submit([8], max_tokens=2)                    # cheaper, keeps arriving first in rank
+    order = []
+    for _ in range(60):
+        before = len(dec.prefills)
+        if not cb.step():
+            break
+        order += [len(ids) - 1 for _, ids in dec.prefills[before:]]
+    assert long_one.get_nowait()[1][0] is not None
+    assert order.index(12) <= 3                         # not after all twelve cheap ones
 
 
 def test_continuous_batcher_serving_thread():
