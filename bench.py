@@ -270,6 +270,10 @@ def main():
                          "the same contexts: the cache length is wound back); ms_per_step is "
                          "their mean, reported with its standard deviation and minimum")
     ap.add_argument("--config", default="6.7b", choices=sorted(CONFIGS))
+    ap.add_argument("--batch", type=int, default=None,
+                    help="override the configuration's batch size (service-style batches)")
+    ap.add_argument("--prompt", type=int, default=None,
+                    help="override the configuration's prompt length")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-same-shape", action="store_true",
                     help="also time the oracle on the host at the GPU workload's own shape "
@@ -305,6 +309,7 @@ def main():
         build(force=True)
 
     size, B, P, G = CONFIGS[args.config]
+    B, P = args.batch or B, args.prompt or P
     int8 = args.config.endswith("int8")
     W = args.warmup
     K = args.steps if args.steps is not None else max(1, G - W)
@@ -358,12 +363,12 @@ def main():
     prefill_cold_s, prefill_s = prefill_times
 
     st = None
-    if args.graph and B <= 64:
+    if args.graph and B <= 64:  # (a captured step selects inside the vocabulary projection)
         st = gen.static_state(decoder, decoder.get_cache(inc), tokens, scores, finished,
                               step_logits)
 
     min_len = max_len - 1
-    fused = st is None and B <= 64 and not args.unfused_select
+    fused = st is None and B <= 128 and not args.unfused_select
     if fused:
         # the generator's fast path: the token at n0 comes from the prefill logits, every later
         # one is chosen inside the decode step's vocabulary projection
@@ -481,7 +486,7 @@ def main():
                              "frac_of_peak": achieved * 1e9 / HBM_PEAK,
                              "plain_read_GBps_at_size": attn_ceiling,
                              "frac_of_plain_read": achieved / attn_ceiling}}
-    if B <= 64:
+    if B <= 128:
         from metaseq_amd._capi import MSA_IN_PACKED, MSA_OUT_PACKED
         F, L, V = cfg.decoder_ffn_embed_dim, cfg.decoder_layers, cfg.vocab_size
         wb = 1 if int8 else 2
@@ -538,7 +543,7 @@ def main():
 
     result = {
         "metric": ("decode tokens/sec + % HBM roofline, OPT-6.7B-shape fp16 bs32, 1xMI355X"
-                   if args.config == "6.7b" else
+                   if args.config == "6.7b" and (B, P) == CONFIGS["6.7b"][1:3] else
                    "decode tokens/sec + %% HBM roofline, OPT-%s shape bs%d, 1xMI355X" % (size, B)),
         "value": B / t_step,
         "unit": "tokens/s",
@@ -576,7 +581,8 @@ def main():
             "kernel": "attention_kernel<%d> (decode, T=1)" % hd,
             "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK / 1e9, "unit": "GB/s",
             "frac": achieved * 1e9 / HBM_PEAK,
-            "traffic": ab * ATTN_TRAFFIC_RATIO if args.config == "6.7b" else None,
+            "traffic": (ab * ATTN_TRAFFIC_RATIO
+                        if args.config == "6.7b" and (B, P) == CONFIGS["6.7b"][1:3] else None),
             "bytes_per_launch": ab, "avg_launch_us": attn_s * 1e6, "context": S_probe,
             "plain_stream_read_GBps": stream_read,
         },

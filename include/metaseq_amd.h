@@ -38,8 +38,8 @@ typedef enum {
 
 /* flags */
 #define MSA_EPI_RELU 1u   /* y = max(y, 0) after the bias add                                  */
-#define MSA_IN_PACKED 2u  /* the input activation is in the packed layout (M <= 64, see below) */
-#define MSA_OUT_PACKED 4u /* write the output activation in the packed layout (M <= 64)        */
+#define MSA_IN_PACKED 2u  /* the input activation is in the packed layout (M <= 128, see below)*/
+#define MSA_OUT_PACKED 4u /* write the output activation in the packed layout (M <= 128)       */
 #define MSA_EMBED_COL_FROM_LEN 8u /* msa_embed_f16: the new token sits in column len_dev[b]      */
 /* per-row bits of the optional `row_mode` array of the selection entry points */
 #define MSA_ROW_BAN_EARLY 1u /* eos_idx and the stop ids are not eligible for this row (the row
@@ -61,8 +61,9 @@ int msa_version(void);
  *         0..7 = W[16t+r][64ks8 + 8g ..+7], 8..15 = W[16t+r][64ks8 + 32 + 8g ..+7], each byte
  *         stored biased (q + 128, unsigned).                                     K % 64 == 0.
  * The pack / unpack calls convert from / to row-major [N,K] (src != dst).
- * Activations of at most 64 rows may be PACKED the same way (the MFMA B operand in lane order):
- * with MB = ceil(M/16), element (m,k) sits at half offset
+ * Activations of at most 128 rows may be PACKED the same way (the MFMA B operand in lane order):
+ * with MB = ceil(M/16) row blocks up to 64 rows and MB = 8 for 65 .. 128 rows, element (m,k) sits
+ * at half offset
  *   ((k/32*MB + m/16)*64 + 16*((k%32)/8) + m%16)*8 + k%8;   the buffer holds MB*16*K halves.
  * No reference counterpart: the reference keeps torch's row-major tensors
  * (metaseq/modules/megatron/mpu/layers.py:290). */
@@ -145,7 +146,7 @@ int msa_embed_f16(const int64_t* tokens, int64_t tok_stride, int B, int n, int T
 /* y[M,N] = epilogue(x[M,K] . W[N,K]^T) with W tile-packed:
  *   t = round(acc); if bias: t = round(t + bias[n]); if RELU: t = max(t,0);
  *   if residual: t = round(t + residual[m,n]);  y[m,n] = t.
- * N % 16 == 0, K % 32 == 0.  With MSA_IN_PACKED (M <= 64) the HBM-bound weight-streaming kernel
+ * N % 16 == 0, K % 32 == 0.  With MSA_IN_PACKED (M <= 128) the HBM-bound weight-streaming kernel
  * runs; otherwise (any M, row-major x) an MFMA kernel tiled for the product's size: 256 x 256
  * tiles with weights read straight from the packed layout once they fill the chip (K % 128 == 0;
  * a ragged bottom block of at most 128 rows is streamed instead), 128 x 128 LDS tiles for the
@@ -168,7 +169,7 @@ int msa_linear_w8a16(const void* x, const int8_t* Wq, const void* scales, const 
                      const void* residual, void* y, int64_t M, int N, int K, unsigned flags,
                      void* stream);
 
-/* Split-K form for the decode step (1 <= M <= 64, MSA_IN_PACKED required): K is cut into S
+/* Split-K form for the decode step (1 <= M <= 128, MSA_IN_PACKED required): K is cut into S
  * ranges and part[s][m][n] (fp32, [S, M, N]) receives the exact fp32 partial sums of range s;
  * the consumer adds them in slice order (msa_residual_layernorm_f16).  Used where N alone gives
  * the chip too few weight tiles (out_proj, fc2).  msa_linear_default_splits suggests S.  The
@@ -202,7 +203,7 @@ int msa_qkv_proj_w8a16(const void* x, const int8_t* Wq, const void* scales, cons
  *   p = round(softmax_fp32(s));  out[b*T+t, h*hd:(h+1)*hd] = round(sum_key p * v).
  * key_pad_mask (optional) is uint8 [B, mask_stride].  hd in {64, 128}.  T == 1 is the
  * bandwidth-bound decode kernel; T > 1 the prefill kernel.  q is row-major; flags:
- * MSA_OUT_PACKED (T == 1, B <= 64).  With len_dev (T == 1) row b attends its own
+ * MSA_OUT_PACKED (T == 1, B <= 128).  With len_dev (T == 1) row b attends its own
  * len_dev[b] + 1 positions and S0 only has to bound them.
  * Replaces metaseq/modules/multihead_attention.py:492 (bmm q k^T), :516-531 (causal and
  * padding masks), :533-534 (fp32 softmax, cast back), :543-552 (bmm p v, transpose). */
@@ -349,12 +350,13 @@ int msa_lm_head_greedy_select_noalloc_f16(const void* x, const void* Ep, void* l
 /* ---- one decode step of the whole decoder in one call ------------------------------------------
  * msa_decoder_create copies a table of device pointers (it allocates host memory only and
  * touches no GPU); msa_decoder_step then launches, on `stream`, exactly the sequence a caller
- * would issue entry point by entry point for T == 1 and at most 64 rows: msa_embed_f16,
+ * would issue entry point by entry point for T == 1 and at most 128 rows: msa_embed_f16,
  * msa_layernorm_f16, per layer msa_qkv_proj_* / msa_attention_f16 / msa_linear_partial_* /
  * msa_residual_layernorm_f16 / msa_linear_* (ReLU) / msa_linear_partial_* /
  * msa_residual_layernorm_f16, then msa_lm_head_greedy_select_f16 (if `tok` is given; `logits`
- * optional) or msa_linear_f16 into `logits` - same arguments, same order, so bit-identical
- * results.  Every linear weight is in the packed layout, int8 with scales if cfg.int8 (the
+ * optional; beyond 64 rows msa_linear_f16 into `logits` or the workspace followed by
+ * msa_greedy_select_f16) or msa_linear_f16 into `logits` - same arguments, same order, so
+ * bit-identical results.  Every linear weight is in the packed layout, int8 with scales if cfg.int8 (the
  * embedding tables stay row-major fp16, lm_head_packed is the packed copy of embed_tokens).
  * With len_dev (per-row lengths, see above) the rows that took part are advanced by one at the
  * end of the step unless MSA_STEP_NO_ADVANCE; MSA_EMBED_COL_FROM_LEN as for msa_embed_f16.

@@ -362,9 +362,11 @@ extern "C" int msa_attention_f16(const void* q, const void* Kcache, const void* 
   MSA_REQUIRE(T <= 65535, MSA_ERR_INVALID_ARG, "msa_attention_f16: T=%d too large", T);
   MSA_REQUIRE((flags & ~MSA_OUT_PACKED) == 0, MSA_ERR_INVALID_ARG,
               "msa_attention_f16: unsupported flags 0x%x", flags);
-  MSA_REQUIRE(!(flags & MSA_OUT_PACKED) || (T == 1 && B <= 64), MSA_ERR_INVALID_ARG,
-              "msa_attention_f16: packed output needs T == 1 and B <= 64 (T=%d B=%d)", T, B);
-  const int out_mb = (flags & MSA_OUT_PACKED) ? (B + 15) / 16 : 0;
+  MSA_REQUIRE(!(flags & MSA_OUT_PACKED) || (T == 1 && B <= MSA_PACKED_MAX_ROWS),
+              MSA_ERR_INVALID_ARG,
+              "msa_attention_f16: packed output needs T == 1 and B <= %d (T=%d B=%d)",
+              MSA_PACKED_MAX_ROWS, T, B);
+  const int out_mb = (flags & MSA_OUT_PACKED) ? packed_row_blocks(B) : 0;
   MSA_REQUIRE(!len_dev || T == 1, MSA_ERR_INVALID_ARG,
               "msa_attention_f16: a device-side length needs T == 1");
   MSA_REQUIRE(!len_dev || S_cap <= 8192, MSA_ERR_CAPACITY,
@@ -426,11 +428,11 @@ extern "C" int msa_attention_split_f16(const void* q, const void* Kcache, const 
               "%s: mask_stride %lld shorter than %d keys", name, (long long)mask_stride, S0 + 1);
   MSA_REQUIRE((flags & ~MSA_OUT_PACKED) == 0, MSA_ERR_INVALID_ARG, "%s: unsupported flags 0x%x",
               name, flags);
-  MSA_REQUIRE(!(flags & MSA_OUT_PACKED) || B <= 64, MSA_ERR_INVALID_ARG,
-              "%s: packed output needs B <= 64 (B=%d)", name, B);
+  MSA_REQUIRE(!(flags & MSA_OUT_PACKED) || B <= MSA_PACKED_MAX_ROWS, MSA_ERR_INVALID_ARG,
+              "%s: packed output needs B <= %d (B=%d)", name, MSA_PACKED_MAX_ROWS, B);
   const int64_t BH = (int64_t)B * H;
   MSA_REQUIRE(BH * SPLIT_NS <= 0x7fffffff, MSA_ERR_INVALID_ARG, "%s: B*H too large", name);
-  const int out_mb = (flags & MSA_OUT_PACKED) ? (B + 15) / 16 : 0;
+  const int out_mb = (flags & MSA_OUT_PACKED) ? packed_row_blocks(B) : 0;
   const size_t lds = (size_t)(len_dev ? S_cap : S0 + 1) * sizeof(float);
   hipStream_t s = (hipStream_t)stream;
   const dim3 g1((unsigned)(BH * SPLIT_NS));

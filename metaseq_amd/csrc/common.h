@@ -61,9 +61,14 @@ int msa_launch_select_combine(const SelectPartial* partials, int n_parts, int B,
                               int64_t tok_stride, float* score, int64_t score_stride,
                               const int32_t* len_dev, hipStream_t stream);
 
-// Packed activation layout for M <= 64 rows (the B operand of v_mfma_f32_16x16x32_f16, stored
-// in lane order): element (m, k) of a [M, K] activation with MB = ceil(M/16) row blocks lives
-// at half offset ((k/32 * MB + m/16) * 64 + 16*((k%32)/8) + m%16) * 8 + k%8.
+// Packed activation layout for M <= 128 rows (the B operand of v_mfma_f32_16x16x32_f16, stored
+// in lane order): element (m, k) of a [M, K] activation with MB row blocks lives at half offset
+// ((k/32 * MB + m/16) * 64 + 16*((k%32)/8) + m%16) * 8 + k%8.  MB = ceil(M/16) up to 64 rows and
+// 8 for 65 .. 128 rows (one kernel shape serves them all; the rows past M are never read back).
+constexpr int MSA_PACKED_MAX_ROWS = 128;
+__host__ __device__ __forceinline__ int packed_row_blocks(int64_t M) {
+  return M <= 64 ? (int)((M + 15) / 16) : 8;
+}
 __host__ __device__ __forceinline__ int64_t packed_act_offset(int m, int k, int MB) {
   return ((((int64_t)(k >> 5) * MB + (m >> 4)) * 64 + (((k & 31) >> 3) << 4) + (m & 15)) << 3) +
          (k & 7);

@@ -27,7 +27,7 @@ int64_t align256(int64_t n) { return (n + 255) & ~(int64_t)255; }
 
 // workspace layout for B rows
 struct StepBuffers {
-  char *x, *q, *h, *o, *u, *part, *positions, *step_len, *select_ws, *attn_ws;
+  char *x, *q, *h, *o, *u, *part, *positions, *step_len, *select_ws, *attn_ws, *logits;
   int64_t attn_keys;  // key positions per (b, h) that attn_ws holds scores for (0: none)
   int64_t bytes;
 };
@@ -57,7 +57,7 @@ Splits pick_splits(const msa_decoder* d, int B) {
 }
 
 StepBuffers carve(const msa_decoder* d, int B, const Splits& sp, char* base) {
-  const int64_t D = d->cfg.d_model, F = d->cfg.ffn, MP = ((B + 15) / 16) * 16;
+  const int64_t D = d->cfg.d_model, F = d->cfg.ffn, MP = packed_row_blocks(B) * 16;
   const int64_t S = sp.out > sp.fc2 ? sp.out : sp.fc2;
   StepBuffers w{};
   int64_t off = 0;
@@ -74,7 +74,10 @@ StepBuffers carve(const msa_decoder* d, int B, const Splits& sp, char* base) {
   w.part = take(S * B * D * 4);
   w.positions = take(B * 8);
   w.step_len = take(B * 4);
-  w.select_ws = take(msa_lm_head_select_workspace_bytes(B));
+  // up to 64 rows the selection runs inside the vocabulary projection (partials per workgroup);
+  // beyond, the projection stores its logits and a second kernel selects from them
+  w.select_ws = take(B <= 64 ? msa_lm_head_select_workspace_bytes(B) : 0);
+  w.logits = take(B <= 64 ? 0 : (int64_t)B * d->cfg.vocab * 2);
   w.attn_keys = split_attention_keys(d, B);
   w.attn_ws = take(msa_attention_split_workspace_bytes(B, d->cfg.heads, (int)w.attn_keys));
   w.bytes = off;
@@ -135,7 +138,7 @@ extern "C" void msa_decoder_destroy(msa_decoder* d) {
 }
 
 extern "C" int64_t msa_decoder_step_workspace_bytes(msa_decoder* d, int B) {
-  if (!d || B < 1 || B > 64) return 0;
+  if (!d || B < 1 || B > MSA_PACKED_MAX_ROWS) return 0;
   return carve(d, B, pick_splits(d, B), nullptr).bytes;
 }
 
@@ -145,7 +148,8 @@ extern "C" int msa_decoder_step(msa_decoder* d, const msa_step_args* a, void* st
   MSA_REQUIRE(a->tokens && a->k_cache && a->v_cache && a->workspace, MSA_ERR_INVALID_ARG,
               "%s: null pointer in the step's arguments", name);
   const int B = a->B;
-  MSA_REQUIRE(B >= 1 && B <= 64, MSA_ERR_INVALID_ARG, "%s: B=%d outside 1..64", name, B);
+  MSA_REQUIRE(B >= 1 && B <= MSA_PACKED_MAX_ROWS, MSA_ERR_INVALID_ARG, "%s: B=%d outside 1..%d",
+              name, B, MSA_PACKED_MAX_ROWS);
   MSA_REQUIRE(a->logits || a->tok, MSA_ERR_INVALID_ARG,
               "%s: neither logits nor a token output was asked for", name);
   MSA_REQUIRE(!a->tok || a->score, MSA_ERR_INVALID_ARG, "%s: tok needs score", name);
@@ -229,6 +233,15 @@ extern "C" int msa_decoder_step(msa_decoder* d, const msa_step_args* a, void* st
   if (gate && !(a->flags & MSA_STEP_NO_ADVANCE)) {
     rc = msa_advance_len(a->len_dev, step_len, B, 1, stream);
     if (rc) return rc;
+  }
+  if (a->tok && B > 64) {
+    void* logits = a->logits ? a->logits : (void*)w.logits;
+    rc = msa_linear_f16(w.h, d->lm_head, nullptr, nullptr, logits, B, V, D, IN, stream);
+    if (rc) return rc;
+    return msa_greedy_select_f16(logits, V, B, V, a->temperature, a->banned, a->n_banned, a->stop,
+                                 a->n_stop, a->finished, a->row_mode, a->force_eos_all,
+                                 a->eos_idx, a->tok, a->tok_stride_out, a->score,
+                                 a->score_stride, a->col_dev, stream);
   }
   if (a->tok)
     return msa_lm_head_greedy_select_f16(w.h, d->lm_head, a->logits, w.select_ws, B, V, D,

@@ -513,9 +513,14 @@ struct ShareCfg {
   static constexpr int XH = SK * MB * 512;  // halves of activations per stage
   static constexpr int PIECES = XH / 8;     // 16-byte pieces per stage
   static constexpr int XP = (PIECES + THREADS - 1) / THREADS;  // pieces per thread and stage
-  // activations double buffered, then one tile slot's partial sums of the other K lanes
-  static constexpr int LDS_BYTES = 2 * XH * 2 + (KL - 1) * NG * MB * 1024;
+  // activations double buffered, then one tile slot's partial sums of the other K lanes; where
+  // both do not fit the 160 KB of a compute unit the partial sums take the place of the stage
+  // that has just been consumed
+  static constexpr int RED_BYTES = (KL - 1) * NG * MB * 1024;
+  static constexpr bool RED_ALIAS = 2 * XH * 2 + RED_BYTES > 160 * 1024;
+  static constexpr int LDS_BYTES = 2 * XH * 2 + (RED_ALIAS ? 0 : RED_BYTES);
   static_assert(U % 2 == 0, "a stage holds whole int8 blocks");
+  static_assert(!RED_ALIAS || RED_BYTES <= XH * 2, "the partial sums must fit one stage");
 };
 
 template <int MB, bool W8, int MODE, int KL, int NG, int NT, int U, int PF>
@@ -528,7 +533,7 @@ __global__ __launch_bounds__(KL * NG * 64) void linear_share_kernel(
   constexpr int SK = C::SK, UA = C::UA, XH = C::XH, XP = C::XP, THREADS = C::THREADS;
   constexpr int PIECES = C::PIECES;
   extern __shared__ __attribute__((aligned(16))) half_t lx_share[];  // [2][XH], then red
-  float4_t* red = reinterpret_cast<float4_t*>(lx_share + 2 * XH);    // [KL-1][NG][MB][64]
+  float4_t* red_own = reinterpret_cast<float4_t*>(lx_share + 2 * XH);  // [KL-1][NG][MB][64]
   const int lane = threadIdx.x & 63;
   // the wave number as a scalar: everything derived from it stays out of the vector registers
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -653,6 +658,11 @@ __global__ __launch_bounds__(KL * NG * 64) void linear_share_kernel(
   };
   auto finish = [&](int idx) {  // after the last stage of a tile group
     const int grp = idx / nstages;
+    float4_t* red = red_own;
+    if constexpr (C::RED_ALIAS) {  // the stage just consumed, once every wave is done reading it
+      red = reinterpret_cast<float4_t*>(lx_share + (idx & 1) * XH);
+      __syncthreads();
+    }
 #pragma unroll
     for (int j = 0; j < NT; ++j) {  // one tile slot per round through the reduction buffer
       if (kl > 0) {
@@ -1533,9 +1543,39 @@ void launch_share(const void* xp, const void* W, const void* scales, float* part
                                                ks_per_split, epi, s);
 }
 
+// 65 .. 128 packed rows (eight row blocks): the shared-activation kernel as 2 K lanes x 4 tile
+// lanes with stages of four K steps (32 KB of activations per stage; two stages and the
+// reduction buffer make 96 KB of LDS).  With so many rows per weight fragment the tiles of a
+// workgroup are few per wave, so more weight stages are kept in flight instead (PF).  Measured
+// at 128 x 12288 x 4096 (38.6 us as built): four K lanes x two tile lanes x two tiles 45.8 us,
+// stages of eight K steps 43.0, six weight stages in flight instead of four 44.3.
+template <bool W8, int MODE>
+void launch_wide(const void* xp, const void* W, const void* scales, float* part, int S, int M,
+                 int N, int K, const Epilogue& epi, hipStream_t s) {
+  const int ntiles = N / 16, nks = K / 32;
+  int G = num_cus() / S;
+  if (G < 1) G = 1;
+  const int tiles_per_wg = (ntiles + G - 1) / G;
+  const int gx = (ntiles + tiles_per_wg - 1) / tiles_per_wg;
+  int ks_per_split = (nks + S - 1) / S;
+  if (W8) ks_per_split = (ks_per_split + 1) & ~1;  // int8 blocks cover two steps
+  if (tiles_per_wg <= 4)
+    launch_share_cfg<8, W8, MODE, 2, 4, 1, 2, 4>(xp, W, scales, part, S, M, N, K, tiles_per_wg, gx,
+                                                 ks_per_split, epi, s);
+  else if (tiles_per_wg <= 8)
+    launch_share_cfg<8, W8, MODE, 2, 4, 2, 2, 3>(xp, W, scales, part, S, M, N, K, tiles_per_wg, gx,
+                                                 ks_per_split, epi, s);
+  else
+    launch_share_cfg<8, W8, MODE, 2, 4, 3, 2, 2>(xp, W, scales, part, S, M, N, K, tiles_per_wg, gx,
+                                                 ks_per_split, epi, s);
+}
+
 template <bool W8, int MODE, bool XR = false>
 void launch_stream(const void* xp, const void* W, const void* scales, float* part, int S, int M,
                    int N, int K, const Epilogue& epi, hipStream_t s, int64_t m_off = 0) {
+  if constexpr (!XR && MODE != MODE_SELECT) {
+    if (M > 64) return launch_wide<W8, MODE>(xp, W, scales, part, S, M, N, K, epi, s);
+  }
   if (!XR && MODE != MODE_SELECT && M > 32 && share_fits(N, S, W8)) {
     constexpr int PM = MODE == MODE_SELECT ? MODE_PLAIN : MODE;
     if (M > 48)
@@ -1664,8 +1704,9 @@ int check_linear_args(const char* name, const void* x, const void* W, const void
               (long long)M);
   MSA_REQUIRE((flags & ~allowed) == 0, MSA_ERR_INVALID_ARG, "%s: unsupported flags 0x%x", name,
               flags);
-  MSA_REQUIRE(!(flags & (MSA_IN_PACKED | MSA_OUT_PACKED)) || M <= 64, MSA_ERR_INVALID_ARG,
-              "%s: packed activations exist only for M <= 64 (M=%lld)", name, (long long)M);
+  MSA_REQUIRE(!(flags & (MSA_IN_PACKED | MSA_OUT_PACKED)) || M <= MSA_PACKED_MAX_ROWS,
+              MSA_ERR_INVALID_ARG, "%s: packed activations exist only for M <= %d (M=%lld)", name,
+              MSA_PACKED_MAX_ROWS, (long long)M);
   return MSA_OK;
 }
 
@@ -1686,7 +1727,7 @@ int linear_entry(const char* name, const void* x, const void* W, const void* sca
   e.y = (half_t*)y;
   e.N = N;
   e.flags = flags & MSA_EPI_RELU;
-  e.out_mb = (flags & MSA_OUT_PACKED) ? (int)((M + 15) / 16) : 0;
+  e.out_mb = (flags & MSA_OUT_PACKED) ? packed_row_blocks(M) : 0;
   if (flags & MSA_IN_PACKED)
     launch_stream<W8, MODE_PLAIN>(x, W, scales, nullptr, 1, (int)M, N, K, e, (hipStream_t)stream);
   else
@@ -1701,8 +1742,9 @@ int partial_entry(const char* name, const void* x, const void* W, const void* sc
   int rc = check_linear_args(name, x, W, part, M, N, K, W8, flags, MSA_IN_PACKED);
   if (rc) return rc;
   MSA_REQUIRE(!W8 || scales, MSA_ERR_INVALID_ARG, "%s: null scales", name);
-  MSA_REQUIRE((flags & MSA_IN_PACKED) && M >= 1 && M <= 64, MSA_ERR_INVALID_ARG,
-              "%s: needs packed activations and 1 <= M <= 64 (M=%lld)", name, (long long)M);
+  MSA_REQUIRE((flags & MSA_IN_PACKED) && M >= 1 && M <= MSA_PACKED_MAX_ROWS, MSA_ERR_INVALID_ARG,
+              "%s: needs packed activations and 1 <= M <= %d (M=%lld)", name, MSA_PACKED_MAX_ROWS,
+              (long long)M);
   MSA_REQUIRE(S >= 1 && S <= K / (W8 ? 64 : 32), MSA_ERR_INVALID_ARG,
               "%s: S=%d outside 1..%d", name, S, K / (W8 ? 64 : 32));
   {
@@ -1938,11 +1980,11 @@ namespace {
 // partial sums (written here, read back by the LayerNorm tail).  More splits mean more tiles
 // per workgroup over a shorter K range, i.e. fewer activation bytes per weight byte.
 int pick_splits(int64_t M, int N, int K, int wbytes) {
-  if (M < 1 || M > 64 || N % 16 || K % 64) return 1;
-  const int MB = (int)((M + 15) / 16), ntiles = N / 16, nks = K / 32;
+  if (M < 1 || M > MSA_PACKED_MAX_ROWS || N % 16 || K % 64) return 1;
+  const int MB = packed_row_blocks(M), ntiles = N / 16, nks = K / 32;
   // tiles that share one sweep over the activations (int8 has a 2 x 6 x 3 shape of the
   // shared-activation kernel for up to 18), and K steps per stage of the workgroup
-  const int NT = MB > 2 ? (wbytes == 1 ? SH_GROUP_W8 : SH_GROUP) : ST_NT;
+  const int NT = MB > 2 ? (wbytes == 1 && MB <= 4 ? SH_GROUP_W8 : SH_GROUP) : ST_NT;
   const int stage = MB > 2 ? 16 : ST_KG * 4;
   int best = 1;
   double best_cost = 0;

@@ -198,9 +198,10 @@ int check(const char* name, int64_t rows, int D, unsigned flags) {
               LN_THREADS * 8 * LN_MAX_CHUNKS);
   MSA_REQUIRE((flags & ~MSA_OUT_PACKED) == 0, MSA_ERR_INVALID_ARG, "%s: unsupported flags 0x%x",
               name, flags);
-  MSA_REQUIRE(!(flags & MSA_OUT_PACKED) || (rows <= 64 && D % 32 == 0), MSA_ERR_INVALID_ARG,
-              "%s: packed output needs rows <= 64 and D %% 32 == 0 (rows=%lld D=%d)", name,
-              (long long)rows, D);
+  MSA_REQUIRE(!(flags & MSA_OUT_PACKED) || (rows <= MSA_PACKED_MAX_ROWS && D % 32 == 0),
+              MSA_ERR_INVALID_ARG,
+              "%s: packed output needs rows <= %d and D %% 32 == 0 (rows=%lld D=%d)", name,
+              MSA_PACKED_MAX_ROWS, (long long)rows, D);
   return MSA_OK;
 }
 
@@ -212,7 +213,7 @@ extern "C" int msa_layernorm_f16(const void* x, const void* gamma, const void* b
   int rc = check("msa_layernorm_f16", rows, D, flags);
   if (rc) return rc;
   if (rows == 0) return MSA_OK;
-  const int out_mb = (flags & MSA_OUT_PACKED) ? (int)((rows + 15) / 16) : 0;
+  const int out_mb = (flags & MSA_OUT_PACKED) ? packed_row_blocks(rows) : 0;
   // many rows: the narrowest workgroup that covers the row
   const int threads = rows <= 64 || D > 256 * 8 * LN_MAX_CHUNKS ? LN_THREADS
                       : D > 128 * 8 * LN_MAX_CHUNKS             ? 256
@@ -257,7 +258,7 @@ extern "C" int msa_residual_layernorm_f16(const float* part, int S, const void* 
   int rc = check("msa_residual_layernorm_f16", rows, D, flags);
   if (rc) return rc;
   if (rows == 0) return MSA_OK;
-  const int out_mb = (flags & MSA_OUT_PACKED) ? (int)((rows + 15) / 16) : 0;
+  const int out_mb = (flags & MSA_OUT_PACKED) ? packed_row_blocks(rows) : 0;
   auto kernel = S == 1   ? layernorm_f16_kernel<1>
                 : S == 2 ? layernorm_f16_kernel<2>
                 : S == 4 ? layernorm_f16_kernel<4>

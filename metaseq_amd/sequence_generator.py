@@ -233,7 +233,7 @@ class SequenceGenerator(nn.Module):
             if (self.use_graph and all_lprobs is None and cache is not None and BB <= 64
                     and not cache.has_pads and not general):
                 st = self.static_state(decoder, cache, tokens, scores, finished, step_logits)
-            fused = (not general and all_lprobs is None and st is None and BB <= 64
+            fused = (not general and all_lprobs is None and st is None and BB <= 128
                      and hasattr(decoder, "forward_select"))
             if fused:
                 # the first token comes from the prefill logits; every later one is chosen inside

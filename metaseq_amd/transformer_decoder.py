@@ -128,7 +128,7 @@ class TransformerDecoder(nn.Module):
         # layer i of a pass over row-major activations (prefill); the tensor is overwritten by
         # the next layer, so a probe that keeps it must copy
         self.layer_probe = None
-        # decode steps of at most 64 rows go through msa_decoder_step (one C call per token);
+        # decode steps of at most 128 rows go through msa_decoder_step (one C call per token);
         # False drives the same kernels entry point by entry point from Python
         self.native_step = True
         self._native = None  # (handle, keep-alive references)
@@ -419,14 +419,23 @@ class TransformerDecoder(nn.Module):
         check(lib.msa_decoder_step(handle, ctypes.byref(a), stream))
         del keep
 
+    # most rows of a decode step on packed activations (the library's MSA_PACKED_MAX_ROWS)
+    PACKED_MAX_ROWS = 128
+
+    @staticmethod
+    def _packed_rows(B):
+        """Rows the packed activation buffers of a B-row step hold: whole blocks of 16 up to 64
+        rows, 128 beyond (one kernel shape serves 65 .. 128 rows)."""
+        return ((B + 15) // 16) * 16 if B <= 64 else 128
+
     def _step_buffers(self, cache, B):
-        """Work buffers of a decode step (<= 64 rows), allocated once per KV cache so that their
+        """Work buffers of a decode step (<= 128 rows), allocated once per KV cache so that their
         addresses stay fixed (a captured graph replays against them)."""
         bufs = getattr(cache, "step_bufs", None)
         if bufs is None:
             cfg, dev = self.cfg, cache.device
             D, F = cfg.decoder_embed_dim, cfg.decoder_ffn_embed_dim
-            MP = ((B + 15) // 16) * 16
+            MP = self._packed_rows(B)
             lib = self._lib
             int8 = self.layers[0].fc2.qweight is not None
             splits = lib.msa_linear_default_splits_w8a16 if int8 else lib.msa_linear_default_splits
@@ -446,7 +455,7 @@ class TransformerDecoder(nn.Module):
 
     def _decode_core(self, lib, stream, tokens, n, B, cache, mask, bufs, len_dev, S0,
                      want_packed, col_from_len=False):
-        """One decode step for at most 64 rows: packed activations, weight-streaming kernels,
+        """One decode step for at most 128 rows: packed activations, weight-streaming kernels,
         split-K tails fused into the LayerNorm that follows.  With ``len_dev`` (int32 [B] device
         tensor: positions of each row already in the cache, negative = inactive row) every row
         appends at and attends up to its own length, and nothing in the launch arguments
@@ -528,8 +537,8 @@ class TransformerDecoder(nn.Module):
         lib = self.prepare_()
         stream = _capi.stream_ptr()
         B = tokens.shape[0]
-        if B > 64 or cache.has_pads:
-            raise ValueError("static decode steps need at most 64 rows and no padding")
+        if B > self.PACKED_MAX_ROWS or cache.has_pads:
+            raise ValueError("static decode steps need at most 128 rows and no padding")
         if self.native_step and not self.return_inner_states:
             self._native_step(lib, stream, tokens, tokens.shape[1], B, cache, None, len_dev, 0,
                               {"logits": logits_out}, col_from_len=True, advance=False)
@@ -605,8 +614,10 @@ class TransformerDecoder(nn.Module):
             any_pad, all_trailing = torch.stack([m.any(), trailing.all()]).tolist()
             if any_pad:
                 mask = m
-                ragged = bool(all_trailing) and B <= 64
-                lens = counts.to(torch.int32)
+                # (a one-column prompt takes the single-token kernels, where per-row lengths
+                # mean positions already in the cache: it keeps the masked layout)
+                ragged = bool(all_trailing) and B <= self.PACKED_MAX_ROWS and n > 1
+                lens = counts.to(torch.int32) if ragged else None
         elif cache.ragged:
             lens = cache.lens
         elif cache.has_pads:
@@ -629,7 +640,8 @@ class TransformerDecoder(nn.Module):
             cache.grow(min(max(self.max_positions(), S0 + 1), int(cache.capacity * 1.5) + 64))
 
         M = B * T
-        if (T == 1 and M <= 64 and native_out is not None and self.native_step
+        PM = self.PACKED_MAX_ROWS
+        if (T == 1 and M <= PM and native_out is not None and self.native_step
                 and not self.return_inner_states):
             # the whole step (vocabulary projection / selection included) in one C call
             self._native_step(lib, stream, tokens, n, B, cache, mask, lens, S0, native_out)
@@ -638,7 +650,7 @@ class TransformerDecoder(nn.Module):
                 incremental_state[self._state_key] = cache
             return None, True, (B, T), {"inner_states": [{"tok": None, "pos": None, "emb": None},
                                                          None]}
-        if T == 1 and M <= 64:
+        if T == 1 and M <= PM:
             bufs = self._step_buffers(cache, B)
             feat, x_last = self._decode_core(lib, stream, tokens, n, B, cache, mask, bufs, lens,
                                              S0, want_packed)
@@ -726,9 +738,9 @@ class TransformerDecoder(nn.Module):
     # decode steps over all slots at once.  No reference counterpart: the reference's service
     # runs every batch to completion (metaseq/cli/interactive_hosted.py:66-175).
     def new_slot_cache(self, slots: int, capacity: int, device=None) -> KVCache:
-        """An empty cache of ``slots`` rows (at most 64) and ``capacity`` positions each."""
-        if not 1 <= slots <= 64:
-            raise ValueError("a slot cache holds 1..64 rows")
+        """An empty cache of ``slots`` rows (at most 128) and ``capacity`` positions each."""
+        if not 1 <= slots <= self.PACKED_MAX_ROWS:
+            raise ValueError("a slot cache holds 1..128 rows")
         cfg = self.cfg
         capacity = int(capacity)
         if not 1 <= capacity <= self.max_positions():
@@ -894,7 +906,8 @@ class TransformerDecoder(nn.Module):
         """metaseq/models/transformer_decoder.py:494-537."""
         native_out = None
         if (not features_only and self.native_step and incremental_state
-                and prev_output_tokens.dim() == 2 and prev_output_tokens.shape[0] <= 64
+                and prev_output_tokens.dim() == 2
+                and prev_output_tokens.shape[0] <= self.PACKED_MAX_ROWS
                 and prev_output_tokens.is_cuda):
             native_out = {"logits": torch.empty(prev_output_tokens.shape[0], self.cfg.vocab_size,
                                                 dtype=torch.float16,
@@ -911,7 +924,7 @@ class TransformerDecoder(nn.Module):
     def forward_select(self, prev_output_tokens, incremental_state, *, temperature, banned, stop,
                        finished, force_eos, eos, tok_out, tok_stride, score_out, score_stride,
                        logits_out=None, row_mode=None):
-        """One decode step (at most 64 rows) whose vocabulary projection is fused with the greedy
+        """One decode step (at most 128 rows) whose vocabulary projection is fused with the greedy
         selection of the next token (metaseq/models/transformer_decoder.py:494-537 followed by
         metaseq/sequence_generator.py:272-308,319-323): the logits are reduced inside the
         projection's epilogue and never stored unless ``logits_out`` ([B, V] fp16) is given.
@@ -927,7 +940,7 @@ class TransformerDecoder(nn.Module):
             prev_output_tokens, incremental_state, None, None, want_packed=True,
             native_out={"logits": logits_out, "select": select})
         if not packed:
-            raise ValueError("forward_select needs at most 64 rows")
+            raise ValueError("forward_select needs at most 128 rows")
         if f is None:
             return  # the native step selected
         self._select_from(self._lib, f, B, temperature, banned, stop, finished, row_mode,
@@ -935,8 +948,23 @@ class TransformerDecoder(nn.Module):
 
     def _select_from(self, lib, f, B, temperature, banned, stop, finished, row_mode, force_eos,
                      eos, tok_out, tok_stride, score_out, score_stride, logits_out):
-        """Vocabulary projection of the packed features ``f`` fused with the greedy selection."""
+        """Vocabulary projection of the packed features ``f`` fused with the greedy selection
+        (beyond 64 rows: the projection stores its logits and a second kernel selects)."""
         D, V = self.cfg.decoder_embed_dim, self.cfg.vocab_size
+        if B > 64:
+            banned, stop = list(banned), list(stop)
+            ba = (ctypes.c_int32 * max(1, len(banned)))(*banned)
+            sa = (ctypes.c_int32 * max(1, len(stop)))(*stop)
+            logits = logits_out if logits_out is not None else torch.empty(
+                B, V, dtype=torch.float16, device=f.device)
+            stream = _capi.stream_ptr()
+            check(lib.msa_linear_f16(ptr(f), ptr(self._lm_head), None, None, ptr(logits), B, V, D,
+                                     MSA_IN_PACKED, stream))
+            check(lib.msa_greedy_select_f16(
+                ptr(logits), V, B, V, float(temperature), ba, len(banned), sa, len(stop),
+                ptr(finished), ptr(row_mode), int(force_eos), int(eos), ptr(tok_out), tok_stride,
+                ptr(score_out), score_stride, None, stream))
+            return
         need = lib.msa_lm_head_select_workspace_bytes(B)
         ws = getattr(self, "_select_ws", None)
         if ws is None or ws.numel() < need or ws.device != f.device:

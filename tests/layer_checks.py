@@ -24,14 +24,14 @@ def pack_rows(x):
     """[M, K] row-major -> the packed activation layout of include/metaseq_amd.h (M <= 64), on
     x's device."""
     M, K = x.shape
-    MB = (M + 15) // 16
+    MB = (M + 15) // 16 if M <= 64 else 8   # 65 .. 128 rows: always eight row blocks
     xp = torch.zeros(MB * 16, K, dtype=x.dtype, device=x.device)
     xp[:M] = x
     return xp.view(MB, 16, K // 32, 4, 8).permute(2, 0, 3, 1, 4).contiguous().view(-1)
 
 
 def unpack_rows(xp, M, K):
-    MB = (M + 15) // 16
+    MB = (M + 15) // 16 if M <= 64 else 8   # 65 .. 128 rows: always eight row blocks
     x = xp.view(K // 32, MB, 4, 16, 8).permute(1, 3, 0, 2, 4).contiguous().view(MB * 16, K)
     return x[:M]
 

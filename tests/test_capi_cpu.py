@@ -84,7 +84,8 @@ def test_decoder_handle_is_host_only_bookkeeping():
     assert lib.msa_decoder_create(ctypes.byref(conf), one, one, one, one, one, table,
                                   ctypes.byref(h)) == 0
     w8, w40 = (lib.msa_decoder_step_workspace_bytes(h, b) for b in (8, 40))
-    assert 0 < w8 < w40 and lib.msa_decoder_step_workspace_bytes(h, 65) == 0
+    w100 = lib.msa_decoder_step_workspace_bytes(h, 100)
+    assert 0 < w8 < w40 and w100 > 0 and lib.msa_decoder_step_workspace_bytes(h, 129) == 0
     args = _capi.StepArgs()
     assert lib.msa_decoder_step(h, ctypes.byref(args), None) == -1     # nothing filled in
     lib.msa_decoder_destroy(h)

@@ -78,14 +78,14 @@ def pack_w8(lib, q):
 def pack_act(x):
     """[M, K] -> packed activation layout (host-side restatement of the documented formula)."""
     M, K = x.shape
-    MB = (M + 15) // 16
+    MB = (M + 15) // 16 if M <= 64 else 8   # 65 .. 128 rows: always eight row blocks
     xp = torch.zeros(MB * 16, K, dtype=x.dtype)
     xp[:M] = x
     return xp.view(MB, 16, K // 32, 4, 8).permute(2, 0, 3, 1, 4).contiguous().view(-1)
 
 
 def unpack_act(xp, M, K):
-    MB = (M + 15) // 16
+    MB = (M + 15) // 16 if M <= 64 else 8   # 65 .. 128 rows: always eight row blocks
     x = xp.view(K // 32, MB, 4, 16, 8).permute(1, 3, 0, 2, 4).contiguous().view(MB * 16, K)
     return x[:M]
 
@@ -112,8 +112,8 @@ def test_layernorm(lib, rows, D):
        lib)
     torch.cuda.synchronize()
     assert_fp16_close(y, want, what="layernorm")
-    if rows <= 64 and D % 32 == 0:
-        MB = (rows + 15) // 16
+    if rows <= 128 and D % 32 == 0:
+        MB = (rows + 15) // 16 if rows <= 64 else 8
         yp = torch.zeros(MB * 16 * D, dtype=torch.float16, device=DEV)
         ok(lib.msa_layernorm_f16(P(G(x)), P(G(g)), P(G(b)), P(yp), rows, D, 1e-5, OUT_PACKED,
                                  None), lib)
@@ -369,6 +369,9 @@ LINEAR_SHAPES = [
     # few rows under a wide output: one row tile of the four-wave kernel plus a bottom block for
     # the streaming kernel; two row tiles, the second moved up over most of the first
     (300, 32768, 128), (420, 32768, 128),
+    # 65 .. 128 packed rows: the shared-activation kernel with eight row blocks and 1, 2 and 3
+    # tiles per wave, several passes over a workgroup's tiles, a K range of one stage
+    (128, 4096, 128), (70, 8192, 256), (96, 24576, 128), (128, 50272, 128), (127, 1008, 96),
     # 64 and 44 bottom rows with few tiles per workgroup: the streaming kernel's four-tile groups
     (4160, 4096, 256), (4140, 8192, 128),
     # exactly one full round of 256 x 256 tiles, also with a moved-up bottom tile
@@ -423,7 +426,7 @@ def test_linear_f16(lib, M, N, K, epi):
     ok(lib.msa_linear_f16(P(G(x)), P(Wp), P(G(b)), P(G(res)), P(y), M, N, K, flags, None), lib)
     torch.cuda.synchronize()
     assert_fp16_close(y, want, atol=atol, what="linear %s (tiled)" % epi)
-    if M <= 64:
+    if M <= 128:
         xp = G(pack_act(x))
         y2 = torch.full((M, N), float("nan"), dtype=torch.float16, device=DEV)
         ok(lib.msa_linear_f16(P(xp), P(Wp), P(G(b)), P(G(res)), P(y2), M, N, K,
@@ -431,7 +434,7 @@ def test_linear_f16(lib, M, N, K, epi):
         torch.cuda.synchronize()
         assert_fp16_close(y2, want, atol=atol, what="linear %s (stream)" % epi)
         if N % 32 == 0:
-            MB = (M + 15) // 16
+            MB = (M + 15) // 16 if M <= 64 else 8
             y3 = torch.zeros(MB * 16 * N, dtype=torch.float16, device=DEV)
             ok(lib.msa_linear_f16(P(xp), P(Wp), P(G(b)), P(G(res)), P(y3), M, N, K,
                                   flags | IN_PACKED | OUT_PACKED, None), lib)
@@ -461,7 +464,7 @@ def test_linear_rejects_bad_shapes(lib):
     assert lib.msa_linear_f16(P(x), P(x), None, None, P(y), 4, 8, 32, 0, None) == -1    # N % 16
     assert lib.msa_linear_f16(None, P(x), None, None, P(y), 4, 16, 32, 0, None) == -1
     assert lib.msa_linear_f16(P(x), P(x), None, None, P(y), 4, 16, 32, 64, None) == -1  # flags
-    assert lib.msa_linear_f16(P(x), P(x), None, None, P(y), 65, 16, 32, IN_PACKED, None) == -1
+    assert lib.msa_linear_f16(P(x), P(x), None, None, P(y), 129, 16, 32, IN_PACKED, None) == -1
     assert lib.msa_linear_partial_f16(P(x), P(x), P(y), 4, 16, 64, 1, 0, None) == -1    # not packed
     assert lib.msa_linear_partial_f16(P(x), P(x), P(y), 4, 16, 64, 3, IN_PACKED, None) == -1
 
@@ -472,6 +475,8 @@ def test_linear_rejects_bad_shapes(lib):
                                    # 9 tiles per workgroup (12 waves as 4 x 3), the last
                                    # workgroup short of tiles and a K range of 1.5 stages
                                    (64, 36864, 256), (50, 36784, 192), (40, 36864, 256),
+                                   # 65 .. 128 packed rows
+                                   (100, 3072, 768), (128, 36864, 256), (70, 1008, 192),
                                    (1000, 16400, 128), (1124, 16400, 128)])   # large tiled kernel
 def test_linear_w8a16(lib, M, N, K):
     print("w8a16", M, N, K, flush=True)
@@ -485,7 +490,7 @@ def test_linear_w8a16(lib, M, N, K):
     ok(lib.msa_linear_w8a16(P(G(x)), P(qp), P(G(s)), P(G(b)), None, P(y), M, N, K, 0, None), lib)
     torch.cuda.synchronize()
     assert_fp16_close(y, want, atol=atol, what="w8a16 (tiled)")
-    if M <= 64:
+    if M <= 128:
         y2 = torch.empty(M, N, dtype=torch.float16, device=DEV)
         ok(lib.msa_linear_w8a16(P(G(pack_act(x))), P(qp), P(G(s)), P(G(b)), None, P(y2), M, N, K,
                                 IN_PACKED, None), lib)
@@ -498,7 +503,9 @@ def test_linear_w8a16(lib, M, N, K):
                                      (48, 4608, 2048, 4),
                                      # int8: 18 and 9 tiles per workgroup (12 waves as 2 x 6
                                      # and 4 x 3), the second with a ragged last K slice
-                                     (64, 9216, 1024, 8), (64, 9216, 1152, 4)])
+                                     (64, 9216, 1024, 8), (64, 9216, 1152, 4),
+                                     # 65 .. 128 rows
+                                     (70, 4096, 4096, 4), (128, 768, 3072, 4), (100, 2048, 1024, 2)])
 @pytest.mark.parametrize("w8", [False, True])
 def test_split_k_partials_and_fused_layernorm(lib, M, N, K, S, w8):
     """msa_linear_partial_* followed by msa_residual_layernorm_f16 equals the oracle's
@@ -522,7 +529,7 @@ def test_split_k_partials_and_fused_layernorm(lib, M, N, K, S, w8):
         ok(lib.msa_linear_partial_f16(P(xp), P(pack_w(lib, G(W))), P(part), M, N, K, S, IN_PACKED,
                                       None), lib)
     xd = G(res).clone()
-    MB = (M + 15) // 16
+    MB = (M + 15) // 16 if M <= 64 else 8   # 65 .. 128 rows: always eight row blocks
     hp = torch.zeros(MB * 16 * N, dtype=torch.float16, device=DEV)
     ok(lib.msa_residual_layernorm_f16(P(part), S, P(G(b)), P(xd), P(G(g)), P(G(be)), P(hp), M, N,
                                       1e-5, OUT_PACKED, None), lib)
@@ -552,7 +559,8 @@ def test_default_splits_are_valid(lib):
 
 
 @pytest.mark.parametrize("B,T,H,hd,S0", [(3, 1, 2, 64, 5), (2, 7, 4, 128, 0), (32, 1, 12, 64, 40),
-                                         (2, 70, 2, 64, 0), (64, 1, 4, 128, 3)])
+                                         (2, 70, 2, 64, 0), (64, 1, 4, 128, 3),
+                                         (100, 1, 4, 64, 9), (128, 1, 2, 128, 0)])
 @pytest.mark.parametrize("w8", [False, True])
 def test_qkv_proj_scatter(lib, B, T, H, hd, S0, w8):
     print("qkv", B, T, H, hd, S0, w8, flush=True)
@@ -570,7 +578,7 @@ def test_qkv_proj_scatter(lib, B, T, H, hd, S0, w8):
     want_k = k.view(B, T, H, hd).permute(0, 2, 1, 3)
     want_v = v.view(B, T, H, hd).permute(0, 2, 1, 3)
     atol = float(kvq.abs().max()) * 2 ** -10
-    modes = [0] + ([IN_PACKED] if B * T <= 64 else [])
+    modes = [0] + ([IN_PACKED] if B * T <= 128 else [])
     for flags in modes:
         Kc = torch.zeros(B, H, S_cap, hd, dtype=torch.float16, device=DEV)
         Vc = torch.zeros_like(Kc)
@@ -691,6 +699,7 @@ def _oracle_core(dtype=torch.float16):
 @pytest.mark.parametrize("B,H,hd,T,S0,masked", [
     (2, 2, 64, 1, 0, False), (3, 2, 64, 1, 37, False), (2, 3, 128, 1, 300, True),
     (32, 12, 64, 1, 65, False), (2, 2, 128, 9, 0, False), (2, 2, 64, 33, 0, True),
+    (100, 3, 64, 1, 40, True), (128, 2, 128, 1, 17, False),     # 65 .. 128 rows, packed output
     (1, 4, 128, 130, 0, False), (8, 32, 64, 1, 513, False), (2, 2, 64, 5, 11, False),
     (2, 3, 128, 257, 0, True), (1, 2, 64, 200, 56, False), (3, 1, 128, 129, 127, True),
     # query tiles are aligned to the end: exact multiples, one query over, one query short
@@ -725,8 +734,8 @@ def test_attention(lib, B, H, hd, T, S0, masked):
                              0 if dm is None else dm.stride(0), P(out), B, H, hd, T, S0, S_cap,
                              0, None, None), lib)
     torch.cuda.synchronize()
-    if T == 1 and B <= 64:
-        MB = (B + 15) // 16
+    if T == 1 and B <= 128:
+        MB = (B + 15) // 16 if B <= 64 else 8
         op = torch.zeros(MB * 16 * D, dtype=torch.float16, device=DEV)
         ok(lib.msa_attention_f16(P(G(q)), P(G(Kc)), P(G(Vc)), P(dm),
                                  0 if dm is None else dm.stride(0), P(op), B, H, hd, T, S0, S_cap,

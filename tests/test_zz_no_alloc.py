@@ -18,7 +18,7 @@ DEV = "cuda"
 
 def _pack_act(x):
     M, K = x.shape
-    MB = (M + 15) // 16
+    MB = (M + 15) // 16 if M <= 64 else 8   # 65 .. 128 rows: always eight row blocks
     xp = torch.zeros(MB * 16, K, dtype=x.dtype)
     xp[:M] = x
     return xp.view(MB, 16, K // 32, 4, 8).permute(2, 0, 3, 1, 4).contiguous().view(-1)
