@@ -41,6 +41,7 @@ typedef enum {
 #define MSA_IN_PACKED 2u  /* the input activation is in the packed layout (M <= 128, see below)*/
 #define MSA_OUT_PACKED 4u /* write the output activation in the packed layout (M <= 128)       */
 #define MSA_EMBED_COL_FROM_LEN 8u /* msa_embed_f16: the new token sits in column len_dev[b]      */
+#define MSA_EMBED_ROWS_GIVEN 32u /* msa_embed_f16: E holds the B*T_out token embeddings themselves */
 /* per-row bits of the optional `row_mode` array of the selection entry points */
 #define MSA_ROW_BAN_EARLY 1u /* eos_idx and the stop ids are not eligible for this row (the row
                                 has not reached its minimum length)                             */
@@ -133,7 +134,10 @@ int msa_residual_layernorm_f16(const float* part, int S, const void* bias, void*
  *   x[b*T_out + j, :] = round(E[tokens[b,t], :] + P[pos(b,t), :]),  t = n - T_out + j
  * tokens are int64 with row stride `tok_stride` elements.  positions_out (optional, int64
  * [B, T_out]) receives pos.  Ids outside [0,V) or positions >= n_pos_rows set *status_dev
- * (optional int32) to 1 and are clamped.  flags: MSA_EMBED_COL_FROM_LEN (with len_dev).
+ * (optional int32) to 1 and are clamped.  flags: MSA_EMBED_COL_FROM_LEN (with len_dev);
+ * MSA_EMBED_ROWS_GIVEN: E is not the table but fp16 [B*T_out, D], the token embeddings of the
+ * embedded columns as the caller computed them (the reference's `token_embeddings` argument);
+ * `tokens` then only says where the pads are.
  * Replaces TransformerDecoder.forward_embedding (metaseq/models/transformer_decoder.py:263-346),
  * utils.make_positions (metaseq/utils.py:83-93), LearnedPositionalEmbedding.forward
  * (metaseq/modules/learned_positional_embedding.py:30-54) and VocabParallelEmbedding.forward
@@ -212,7 +216,9 @@ int msa_attention_f16(const void* q, const void* Kcache, const void* Vcache,
                       int hd, int T, int S0, int S_cap, unsigned flags, const int32_t* len_dev,
                       void* stream);
 
-/* The decode step's attention (T == 1) in two launches, for few (batch row, head) pairs over long
+/* EXPERIMENTAL: pays only beyond OPT's 2048 positions (no benchmark configuration selects it;
+ * msa_decoder_step takes it for a single request over more than 4096 keys at head_dim 128).
+ * The decode step's attention (T == 1) in two launches, for few (batch row, head) pairs over long
  * histories (batch-1 serving, a nearly empty slot cache): one workgroup per pair leaves most
  * CUs idle and pulls the pair's K and V rows through a single CU.  Launch 1 writes the rounded
  * scores of 8 key ranges per pair to `workspace` (fp32 [B*H, S_cap],

@@ -16,6 +16,7 @@ MSA_EPI_RELU = 1
 MSA_IN_PACKED = 2
 MSA_OUT_PACKED = 4
 MSA_EMBED_COL_FROM_LEN = 8
+MSA_EMBED_ROWS_GIVEN = 32
 MSA_ROW_BAN_EARLY = 1
 MSA_ROW_ONLY_EOS = 2
 MSA_ROW_SKIP = 4

@@ -46,7 +46,7 @@ __global__ __launch_bounds__(EMB_THREADS) void embed_last_kernel(
     const int64_t* __restrict__ tokens, int64_t tok_stride, int n, const half_t* __restrict__ E,
     int V, const half_t* __restrict__ P, int n_pos_rows, int pad, int D, half_t* __restrict__ x,
     int64_t* __restrict__ positions_out, int32_t* status, const int32_t* __restrict__ len_dev,
-    int32_t* __restrict__ step_len_out, bool col_from_len) {
+    int32_t* __restrict__ step_len_out, bool col_from_len, bool rows_given) {
   __shared__ float red[16];
   const int b = blockIdx.x;
   const int64_t* row = tokens + b * tok_stride;
@@ -64,9 +64,10 @@ __global__ __launch_bounds__(EMB_THREADS) void embed_last_kernel(
     const int cnt = count_nonpad(row, n, pad, red);
     if (tok != pad) pos = pad + cnt;
   }
+  if (rows_given) tok = 0;  // E holds this row's token embedding itself: nothing to look up
   clamp_ids(tok, pos, V, n_pos_rows, status);
   if (positions_out && threadIdx.x == 0) positions_out[b] = pos;
-  gather_row(E, P, tok, pos, x + (int64_t)b * D, D);
+  gather_row(E, P, rows_given ? (int64_t)b : tok, pos, x + (int64_t)b * D, D);
 }
 
 // prefill: positions for the last T_out columns of every row (one block per row)
@@ -95,13 +96,14 @@ __global__ __launch_bounds__(EMB_THREADS) void positions_kernel(
 __global__ __launch_bounds__(EMB_THREADS) void embed_rows_kernel(
     const int64_t* __restrict__ tokens, int64_t tok_stride, int n, int T_out,
     const half_t* __restrict__ E, int V, const half_t* __restrict__ P, int n_pos_rows, int D,
-    half_t* __restrict__ x, const int64_t* __restrict__ positions, int32_t* status) {
+    half_t* __restrict__ x, const int64_t* __restrict__ positions, int32_t* status,
+    bool rows_given) {
   const int64_t r = blockIdx.x;  // b * T_out + j
   const int b = (int)(r / T_out), j = (int)(r % T_out);
-  int64_t tok = tokens[b * tok_stride + (n - T_out + j)];
+  int64_t tok = rows_given ? 0 : tokens[b * tok_stride + (n - T_out + j)];
   int pos = (int)positions[r];
   clamp_ids(tok, pos, V, n_pos_rows, status);
-  gather_row(E, P, tok, pos, x + r * D, D);
+  gather_row(E, P, rows_given ? r : tok, pos, x + r * D, D);
 }
 
 }  // namespace
@@ -120,9 +122,12 @@ extern "C" int msa_embed_f16(const int64_t* tokens, int64_t tok_stride, int B, i
               n_pos_rows, pad_idx);
   MSA_REQUIRE(!len_dev || T_out == 1, MSA_ERR_INVALID_ARG,
               "msa_embed_f16: device-side lengths need T_out == 1");
-  MSA_REQUIRE((flags & ~MSA_EMBED_COL_FROM_LEN) == 0 && (!flags || len_dev), MSA_ERR_INVALID_ARG,
+  MSA_REQUIRE((flags & ~(MSA_EMBED_COL_FROM_LEN | MSA_EMBED_ROWS_GIVEN)) == 0 &&
+                  (!(flags & MSA_EMBED_COL_FROM_LEN) || len_dev),
+              MSA_ERR_INVALID_ARG,
               "msa_embed_f16: unsupported flags 0x%x (MSA_EMBED_COL_FROM_LEN needs len_dev)",
               flags);
+  const bool rows_given = (flags & MSA_EMBED_ROWS_GIVEN) != 0;
   MSA_REQUIRE(!step_len_out || len_dev, MSA_ERR_INVALID_ARG,
               "msa_embed_f16: step_len_out needs len_dev");
   hipStream_t s = (hipStream_t)stream;
@@ -130,7 +135,7 @@ extern "C" int msa_embed_f16(const int64_t* tokens, int64_t tok_stride, int B, i
     hipLaunchKernelGGL(embed_last_kernel, dim3(B), dim3(EMB_THREADS), 0, s, tokens, tok_stride, n,
                        (const half_t*)E, V, (const half_t*)P, n_pos_rows, pad_idx, D, (half_t*)x,
                        positions_out, status_dev, len_dev, step_len_out,
-                       (flags & MSA_EMBED_COL_FROM_LEN) != 0);
+                       (flags & MSA_EMBED_COL_FROM_LEN) != 0, rows_given);
   } else {
     MSA_REQUIRE(positions_out, MSA_ERR_INVALID_ARG,
                 "msa_embed_f16: positions_out is required when T_out > 1");
@@ -138,7 +143,7 @@ extern "C" int msa_embed_f16(const int64_t* tokens, int64_t tok_stride, int B, i
                        T_out, pad_idx, positions_out);
     hipLaunchKernelGGL(embed_rows_kernel, dim3((unsigned)((int64_t)B * T_out)), dim3(EMB_THREADS),
                        0, s, tokens, tok_stride, n, T_out, (const half_t*)E, V, (const half_t*)P,
-                       n_pos_rows, D, (half_t*)x, positions_out, status_dev);
+                       n_pos_rows, D, (half_t*)x, positions_out, status_dev, rows_given);
   }
   MSA_CHECK_LAUNCH("msa_embed_f16");
   return MSA_OK;

@@ -15,8 +15,8 @@ import torch
 from torch import nn
 
 from . import _capi
-from ._capi import (MSA_EMBED_COL_FROM_LEN, MSA_EPI_RELU, MSA_IN_PACKED, MSA_OUT_PACKED, check,
-                    ptr)
+from ._capi import (MSA_EMBED_COL_FROM_LEN, MSA_EMBED_ROWS_GIVEN, MSA_EPI_RELU, MSA_IN_PACKED,
+                    MSA_OUT_PACKED, check, ptr)
 from .config import OPTConfig
 from .kv_cache import KVCache
 
@@ -454,7 +454,7 @@ class TransformerDecoder(nn.Module):
         return bufs
 
     def _decode_core(self, lib, stream, tokens, n, B, cache, mask, bufs, len_dev, S0,
-                     want_packed, col_from_len=False):
+                     want_packed, col_from_len=False, token_embeddings=None):
         """One decode step for at most 128 rows: packed activations, weight-streaming kernels,
         split-K tails fused into the LayerNorm that follows.  With ``len_dev`` (int32 [B] device
         tensor: positions of each row already in the cache, negative = inactive row) every row
@@ -468,12 +468,14 @@ class TransformerDecoder(nn.Module):
         # a row whose new token is a pad sits this step out (step_len = -1), as does an
         # inactive row; under graph replay there are no pads and the lengths are used as is
         step_len = bufs["step_len"] if (len_dev is not None and not col_from_len) else None
-        check(lib.msa_embed_f16(ptr(tokens), tokens.stride(0), B, n, 1,
-                                ptr(self.embed_tokens.weight), cfg.vocab_size,
-                                ptr(self.embed_positions.weight),
+        table = self.embed_tokens.weight if token_embeddings is None else token_embeddings
+        check(lib.msa_embed_f16(ptr(tokens), tokens.stride(0), B, n, 1, ptr(table),
+                                cfg.vocab_size, ptr(self.embed_positions.weight),
                                 self.embed_positions.weight.shape[0], self.padding_idx, D,
                                 ptr(x), ptr(bufs["positions"]), None, ptr(len_dev), ptr(step_len),
-                                MSA_EMBED_COL_FROM_LEN if col_from_len else 0, stream))
+                                (MSA_EMBED_COL_FROM_LEN if col_from_len else 0)
+                                | (MSA_EMBED_ROWS_GIVEN if token_embeddings is not None else 0),
+                                stream))
         if step_len is not None:
             len_dev = step_len
         self._layernorm(lib, stream, x, self.layers[0].self_attn_layer_norm, M, D, h, OUT)
@@ -563,8 +565,6 @@ class TransformerDecoder(nn.Module):
         extra): features are ``[B, T, D]`` row-major, or - for a decode step of at most 64 rows
         when ``want_packed`` - the packed activation buffer the vocabulary projection reads."""
         cfg = self.cfg
-        if token_embeddings is not None:
-            raise NotImplementedError("precomputed token_embeddings are not supported")
         tokens = prev_output_tokens
         if tokens.dim() != 2:
             raise AssertionError("prev_output_tokens must be [batch, tgt_len]")
@@ -640,9 +640,17 @@ class TransformerDecoder(nn.Module):
             cache.grow(min(max(self.max_positions(), S0 + 1), int(cache.capacity * 1.5) + 64))
 
         M = B * T
+        if token_embeddings is not None:
+            # the reference adds the positions to whatever embedding it is handed, one row per
+            # embedded column (the last column only on a decode step,
+            # metaseq/models/transformer_decoder.py:324-335)
+            if tuple(token_embeddings.shape) != (B, T, D) or not token_embeddings.is_cuda:
+                raise AssertionError("token_embeddings must be a device tensor [%d, %d, %d]"
+                                     % (B, T, D))
+            token_embeddings = token_embeddings.to(torch.float16).contiguous()
         PM = self.PACKED_MAX_ROWS
         if (T == 1 and M <= PM and native_out is not None and self.native_step
-                and not self.return_inner_states):
+                and not self.return_inner_states and token_embeddings is None):
             # the whole step (vocabulary projection / selection included) in one C call
             self._native_step(lib, stream, tokens, n, B, cache, mask, lens, S0, native_out)
             cache.length = S0 + T
@@ -653,7 +661,7 @@ class TransformerDecoder(nn.Module):
         if T == 1 and M <= PM:
             bufs = self._step_buffers(cache, B)
             feat, x_last = self._decode_core(lib, stream, tokens, n, B, cache, mask, bufs, lens,
-                                             S0, want_packed)
+                                             S0, want_packed, token_embeddings=token_embeddings)
             if lens is not None:
                 check(lib.msa_advance_len(ptr(lens), ptr(bufs["step_len"]), B, 1, stream))
             inner_states = [{"tok": None, "pos": bufs["positions"], "emb": None}, x_last]
@@ -663,7 +671,8 @@ class TransformerDecoder(nn.Module):
             if incremental_state is not None:
                 incremental_state[self._state_key] = cache
             return features, packed, (B, T), {"inner_states": inner_states}
-        h, inner_states = self._rows_core(lib, stream, tokens, B, n, T, S0, cache, mask)
+        h, inner_states = self._rows_core(lib, stream, tokens, B, n, T, S0, cache, mask,
+                                          token_embeddings)
         packed = False
         features = h.view(B, T, D)
         cache.length = S0 + T
@@ -671,7 +680,7 @@ class TransformerDecoder(nn.Module):
             incremental_state[self._state_key] = cache
         return features, packed, (B, T), {"inner_states": inner_states}
 
-    def _rows_core(self, lib, stream, tokens, B, n, T, S0, kv, mask):
+    def _rows_core(self, lib, stream, tokens, B, n, T, S0, kv, mask, token_embeddings=None):
         """Prefill (or a decode batch above 64 rows): the last T columns of ``tokens[B, n]``
         through embedding, L layers and the final LayerNorm on row-major activations and the
         tiled MFMA kernels, keys and values written at positions S0 .. S0 + T - 1 of ``kv``
@@ -683,11 +692,13 @@ class TransformerDecoder(nn.Module):
         M = B * T
         x = torch.empty(M, D, dtype=torch.float16, device=dev)
         positions = torch.empty(B, T, dtype=torch.long, device=dev)
-        check(lib.msa_embed_f16(ptr(tokens), tokens.stride(0), B, n, T,
-                                ptr(self.embed_tokens.weight), cfg.vocab_size,
-                                ptr(self.embed_positions.weight),
+        table = self.embed_tokens.weight if token_embeddings is None else token_embeddings
+        check(lib.msa_embed_f16(ptr(tokens), tokens.stride(0), B, n, T, ptr(table),
+                                cfg.vocab_size, ptr(self.embed_positions.weight),
                                 self.embed_positions.weight.shape[0], self.padding_idx, D,
-                                ptr(x), ptr(positions), None, None, None, 0, stream))
+                                ptr(x), ptr(positions), None, None, None,
+                                MSA_EMBED_ROWS_GIVEN if token_embeddings is not None else 0,
+                                stream))
         inner_states = [{"tok": None, "pos": positions, "emb": None}]
         if self.return_inner_states:
             inner_states[0]["emb"] = x.view(B, T, D).transpose(0, 1).clone()

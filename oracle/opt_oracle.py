@@ -325,8 +325,9 @@ class OracleDecoder:
         return x
 
     def extract_features(self, prev_output_tokens, incremental_state=None,
-                         self_attn_padding_mask=None):
-        """transformer_decoder.py:348-396 with forward_embedding :263-346."""
+                         self_attn_padding_mask=None, token_embeddings=None):
+        """transformer_decoder.py:348-396 with forward_embedding :263-346.  ``token_embeddings``
+        ([B, T, D]; T = 1 on a decode step) replaces the embedding lookup (:329-330)."""
         cfg = self.cfg
         tokens = prev_output_tokens.to(self.device)
         if self_attn_padding_mask is None and bool(tokens.eq(cfg.padding_idx).any()):
@@ -336,7 +337,10 @@ class OracleDecoder:
         if incremental_state:  # non-empty dict == decode step (:324-327)
             tokens = tokens[:, -1:]
             pos_emb = pos_emb[:, -1:]
-        emb = F.embedding(tokens, self.w.raw("decoder.embed_tokens.weight")).float()
+        if token_embeddings is None:
+            emb = F.embedding(tokens, self.w.raw("decoder.embed_tokens.weight")).float()
+        else:
+            emb = self._r(token_embeddings.to(self.device).float())
         x = self._r(emb + pos_emb)  # embed_scale == 1.0 (:89, :329-335)
         x = x.transpose(0, 1).contiguous()  # [T, B, D] (:341)
         T = x.shape[0]
@@ -358,9 +362,9 @@ class OracleDecoder:
         return self._linear(features, "decoder.embed_tokens.weight")
 
     def forward(self, prev_output_tokens, incremental_state=None, features_only=False,
-                self_attn_padding_mask=None):
+                self_attn_padding_mask=None, token_embeddings=None):
         x, extra = self.extract_features(prev_output_tokens, incremental_state,
-                                         self_attn_padding_mask)
+                                         self_attn_padding_mask, token_embeddings)
         if not features_only:
             x = self.output_layer(x)
         return x.transpose(0, 1).contiguous(), extra  # :536

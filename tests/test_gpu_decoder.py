@@ -377,3 +377,35 @@ def test_one_call_step_with_split_attention_equals_the_one_launch_form():
     dec.native_step = True
     for x, y in zip(*outs):
         assert torch.equal(x, y)
+
+
+def test_given_token_embeddings_replace_the_lookup():
+    """``token_embeddings=`` (metaseq/models/transformer_decoder.py:329-330): the decoder adds
+    the positions to the rows it is handed instead of looking the tokens up; prefill and decode
+    step against the oracle, with padded rows."""
+    cfg = tiny_cfg(layers=2, dim=128, heads=2, vocab=128, max_pos=64)
+    model, sd = build(cfg, seed=7)
+    oracle = make_oracle(cfg, sd, torch.float16)
+    toks = random_prompts(cfg, 3, 12, seed=5)
+    toks[2, 9:] = 1
+    g = torch.Generator().manual_seed(2)
+    emb = (torch.randn(3, 13, 128, generator=g) * 0.05).half()
+    inc_o, inc_h = {}, {}
+    want = oracle(toks[:, :10], incremental_state=inc_o, token_embeddings=emb[:, :10])[0]
+    got = model(toks[:, :10].to(DEV), incremental_state=inc_h,
+                token_embeddings=emb[:, :10].to(DEV))[0]
+    valid = toks[:, :10].ne(1)
+    check_logits(got.cpu()[valid], want[valid], "prefill from given embeddings")
+    for t in range(10, 13):
+        want = oracle(toks[:, :t + 1], incremental_state=inc_o,
+                      token_embeddings=emb[:, t:t + 1])[0]
+        got = model.decoder(toks[:, :t + 1].to(DEV), incremental_state=inc_h,
+                            token_embeddings=emb[:, t:t + 1].to(DEV))[0]
+        check_logits(got[:2], want[:2], "decode step %d from given embeddings" % t)
+    # the looked-up rows give the plain forward, bit for bit
+    E = model.decoder.embed_tokens.weight
+    a = model(toks[:, :10].to(DEV), incremental_state={})[0]
+    b = model(toks[:, :10].to(DEV), incremental_state={}, token_embeddings=E[toks[:, :10].to(DEV)])[0]
+    assert torch.equal(a[valid.to(DEV)], b[valid.to(DEV)])
+    with pytest.raises(AssertionError):
+        model(toks[:, :10].to(DEV), token_embeddings=emb[:, :4].to(DEV))

@@ -252,3 +252,31 @@ def test_lean_mode_changes_no_value():
     for x, y in zip(a["step_logits"], b["step_logits"]):
         assert torch.equal(x, y)
     assert torch.equal(plain(toks)[0], lean(toks)[0])
+
+
+def test_given_token_embeddings_replace_the_lookup():
+    """Handing the oracle the looked-up embeddings changes nothing (prefill and decode step);
+    handing it other rows changes exactly what a changed embedding table would."""
+    cfg = tiny_cfg(layers=2, dim=32, heads=2, vocab=40, max_pos=16)
+    sd = random_state_dict(cfg, seed=4, dtype=torch.float32)
+    dec = make_oracle(cfg, sd)
+    toks = torch.tensor([[2, 7, 9, 11], [2, 5, 1, 1]])
+    E = sd["decoder.embed_tokens.weight"]
+    a_inc, b_inc = {}, {}
+    a = dec(toks[:, :3], incremental_state=a_inc)[0]
+    b = dec(toks[:, :3], incremental_state=b_inc, token_embeddings=E[toks[:, :3]])[0]
+    assert torch.equal(a, b)
+    a = dec(toks, incremental_state=a_inc)[0]
+    b = dec(toks, incremental_state=b_inc, token_embeddings=E[toks[:, -1:]])[0]
+    assert torch.equal(a, b)
+    # other rows: the same as a table whose rows for these ids were replaced
+    other = torch.randn(2, 3, 32, generator=torch.Generator().manual_seed(1)) * 0.02
+    sd2 = dict(sd)
+    E2 = E.clone()
+    ids = torch.tensor([[30, 31, 32], [33, 34, 35]])          # unused ids stand for the new rows
+    E2[ids] = other
+    sd2["decoder.embed_tokens.weight"] = E2
+    t2 = torch.cat([toks[:, :1] * 0 + ids[:, :1], ids[:, 1:]], 1)
+    want = make_oracle(cfg, sd2).extract_features(t2)[0]
+    got = dec.extract_features(t2, token_embeddings=other)[0]
+    assert torch.allclose(got, want, atol=1e-6)
