@@ -227,7 +227,7 @@ def _run_config(size, B, P, G=32, max_pos=None, layers=None, int8=False, sequent
                   for t in traces.pop(i)[:max(decode_checks) + 1]]
         check_prefill_layer(dec, i, passes[0], B, n0, tag)
         for j in decode_checks:
-            if B <= 64 and j < len(passes):
+            if B <= 128 and j < len(passes):   # the packed decode path
                 check_decode_layer(dec, i, passes, j, B, n0, tag)
         del passes
     _free()
@@ -440,6 +440,16 @@ def test_config4_shape_opt30b_two_layers():
 def test_config5_shape_opt66b_int8_two_layers():
     """Config 5's shape with two layers; the oracle runs on the dequantised fp16 weights."""
     _run_config("66b", 64, 48, G=16, layers=2, int8=True)
+    _free()
+
+
+@pytest.mark.parametrize("rows", [70, 128, 200])
+def test_wide_decode_batches_at_the_6p7b_layer_shapes(rows):
+    """Service-sized decode batches (replicas, many short requests) at OPT-6.7B's real layer
+    shapes, two layers deep: 70 and 128 rows decode on the packed path with eight row blocks
+    (checked op by op against the oracle's own intermediates, then end to end), 200 rows on
+    row-major activations through the tiled kernels."""
+    _run_config("6.7b", rows, 40, G=8, layers=2)
     _free()
 
 
