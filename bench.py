@@ -65,6 +65,66 @@ def attn_bytes(cfg, B, S):
     return 2 * B * S * D * 2 + 2 * B * D * 2
 
 
+def counter_traffic(fetch_glob, write_glob, run_json, cfg, B):
+    """HBM bytes per decode-attention launch over its algorithmic bytes, from the counter files
+    of two earlier runs of this program under the profiler:
+
+        rocprofv3 --pmc FETCH_SIZE --output-format csv -d DIR_F -o b -- python3 bench.py \
+            --steps 4 --warmup 1 --repeats 1 --no-cpu-baseline --pmc-calibration > RUN.json
+        rocprofv3 --pmc WRITE_SIZE ... (the same command)
+
+    ``fetch_glob`` / ``write_glob`` match their ``*counter_collection.csv``; ``run_json`` holds
+    the line either of them printed (its steps, warm-up steps, repeats and context say which
+    contexts the traced launches attended).  Each counter is scaled by what it reads for the
+    1 GiB device copy --pmc-calibration adds (1 048 576 KiB read and as much written)."""
+    import csv
+    import glob
+
+    def readings(pattern, counter):
+        attn, copy = [], 0.0
+        paths = glob.glob(pattern, recursive=True)
+        if not paths:
+            raise SystemExit("bench.py: no counter file matches %r" % pattern)
+        for path in paths:
+            for r in csv.DictReader(open(path)):
+                if r["Counter_Name"] != counter:
+                    continue
+                name, v = r["Kernel_Name"], float(r["Counter_Value"])
+                if "attention_kernel" in name and "prefill" not in name:
+                    attn.append(v)
+                elif "copyBuffer" in name:
+                    copy = max(copy, v)
+        if not attn or copy <= 0:
+            raise SystemExit("bench.py: %r holds no %s readings of the decode attention kernel "
+                             "and the calibration copy" % (pattern, counter))
+        return attn, copy
+
+    run = None
+    for line in open(run_json):
+        if line.startswith("{"):
+            run = json.loads(line)
+    if run is None:
+        raise SystemExit("bench.py: no result line in %r" % run_json)
+    K, W, R = run["steps"], run["warmup"], run.get("repeats", 1)
+    S_end, L = run["roofline"]["context"], cfg.decoder_layers
+    # the contexts of every traced launch: warm-up steps once, the timed window R times, then
+    # the timing loop of the attention kernel (one untimed + four timed passes over the layers)
+    contexts = [S_end - K - W + 1 + j for j in range(W)]
+    contexts += [S_end - K + 1 + j for j in range(K)] * R
+    contexts += [S_end] * 5
+    algorithmic = sum(attn_bytes(cfg, B, S) for S in contexts) / len(contexts)
+    fetch, fcopy = readings(fetch_glob, "FETCH_SIZE")
+    write, wcopy = readings(write_glob, "WRITE_SIZE")
+    if len(fetch) != len(contexts) * L or len(write) != len(fetch):
+        raise SystemExit("bench.py: %d / %d traced attention launches, %d expected from %r"
+                         % (len(fetch), len(write), len(contexts) * L, run_json))
+    kib = float(1 << 20)
+    measured = (sum(fetch) / len(fetch) * kib / fcopy + sum(write) / len(write) * kib / wcopy) * 1024
+    return {"ratio": measured / algorithmic, "launches": len(fetch),
+            "fetch_scale": kib / fcopy, "write_scale": kib / wcopy,
+            "measured_bytes_per_launch": measured, "algorithmic_bytes_per_launch": algorithmic}
+
+
 def _host_cores():
     """Threads to use on this host: its CPU share, not what the machine reports in total."""
     n = os.cpu_count() or 1
@@ -290,6 +350,11 @@ def main():
     ap.add_argument("--pmc-calibration", action="store_true",
                     help="also run a plain 1 GiB device copy, the known-size kernel that "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE readings are scaled by")
+    ap.add_argument("--traffic-from", nargs=3, metavar=("FETCH_CSV", "WRITE_CSV", "RUN_JSON"),
+                    help="take roofline.traffic from the counter files of two earlier "
+                         "--pmc-calibration runs under rocprofv3 (--pmc FETCH_SIZE, --pmc "
+                         "WRITE_SIZE; glob patterns of their counter_collection.csv) and the "
+                         "result line one of them printed, instead of the ratio on record")
     ap.add_argument("--torch-eager", action="store_true",
                     help="also time the same decode steps written with stock PyTorch fp16 "
                          "operators on this GPU (reported as torch_eager_same_gpu)")
@@ -541,6 +606,17 @@ def main():
         kernels["sum_of_kernels_ms_per_step"] = (L * per_layer + t_lm + t_ln) * 1e3
     del probe
 
+    if args.traffic_from:
+        counters = counter_traffic(*args.traffic_from, cfg, B)
+        traffic = ab * counters["ratio"]
+        traffic_source = dict(counters, files=list(args.traffic_from))
+    elif args.config == "6.7b" and (B, P) == CONFIGS["6.7b"][1:3]:
+        traffic = ab * ATTN_TRAFFIC_RATIO
+        traffic_source = ("ratio %.4f on record in profiles/decode_attention_opt6.7b_bs32_pmc_"
+                          "traffic.txt; --traffic-from re-derives it from fresh counter files"
+                          % ATTN_TRAFFIC_RATIO)
+    else:
+        traffic = traffic_source = None
     result = {
         "metric": ("decode tokens/sec + % HBM roofline, OPT-6.7B-shape fp16 bs32, 1xMI355X"
                    if args.config == "6.7b" and (B, P) == CONFIGS["6.7b"][1:3] else
@@ -581,8 +657,7 @@ def main():
             "kernel": "attention_kernel<%d> (decode, T=1)" % hd,
             "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK / 1e9, "unit": "GB/s",
             "frac": achieved * 1e9 / HBM_PEAK,
-            "traffic": (ab * ATTN_TRAFFIC_RATIO
-                        if args.config == "6.7b" and (B, P) == CONFIGS["6.7b"][1:3] else None),
+            "traffic": traffic, "traffic_source": traffic_source,
             "bytes_per_launch": ab, "avg_launch_us": attn_s * 1e6, "context": S_probe,
             "plain_stream_read_GBps": stream_read,
         },

@@ -47,6 +47,46 @@ def test_attention_bytes_and_prefill_flops():
     assert abs(4.0 * 32 * 32 * 1025 * 1025 * 4096 - 17.6e12) < 0.1e12
 
 
+def test_counter_traffic_scales_the_readings_by_the_calibration_copy(tmp_path):
+    """Counter files as the profiler writes them (one row per dispatch and counter), made up so
+    that the answer is known: a FETCH_SIZE unit of 2 KiB, a WRITE_SIZE unit of 1 KiB, and
+    attention launches that move exactly their algorithmic bytes plus 1 %."""
+    import csv
+    import json
+    cfg = opt_config("6.7b")
+    B, K, W, L = 32, 2, 1, cfg.decoder_layers
+    S_end = 1030
+    contexts = [S_end - 2, S_end - 1, S_end] + [S_end] * 5  # warm-up, two timed steps, timing loop
+    rows_f = [("__amd_rocclr_copyBuffer", 524288.0), ("prefill_attention_kernelILi128EE", 9e9),
+              ("__amd_rocclr_copyBuffer", 16.0)]
+    rows_w = [("__amd_rocclr_copyBuffer", 1048576.0)]
+    for S in contexts:
+        read = 2 * B * S * 4096 * 2 + B * 4096 * 2
+        for _ in range(L):
+            rows_f.append(("attention_kernelILi128EEEvPKDF16_", 1.01 * read / 1024 / 2))
+            rows_w.append(("attention_kernelILi128EEEvPKDF16_", 1.01 * B * 4096 * 2 / 1024))
+    for name, rows, counter in (("f", rows_f, "FETCH_SIZE"), ("w", rows_w, "WRITE_SIZE")):
+        os.makedirs(tmp_path / name)
+        with open(tmp_path / name / "b_counter_collection.csv", "w", newline="") as fh:
+            wr = csv.writer(fh)
+            wr.writerow(["Kernel_Name", "Counter_Name", "Counter_Value"])
+            for kernel, v in rows:
+                wr.writerow([kernel, counter, v])
+    run = tmp_path / "run.json"
+    run.write_text("noise\n" + json.dumps({"steps": K, "warmup": W, "repeats": 1,
+                                           "roofline": {"context": S_end}}) + "\n")
+    r = bench.counter_traffic(str(tmp_path / "f" / "*.csv"), str(tmp_path / "w" / "*.csv"),
+                              str(run), cfg, B)
+    assert r["launches"] == len(contexts) * L
+    assert abs(r["fetch_scale"] - 2.0) < 1e-12 and abs(r["write_scale"] - 1.0) < 1e-12
+    assert abs(r["ratio"] - 1.01) < 1e-9
+    with pytest.raises(SystemExit):  # a launch count that does not fit the run is refused
+        run.write_text(json.dumps({"steps": K + 1, "warmup": W, "repeats": 1,
+                                   "roofline": {"context": S_end}}))
+        bench.counter_traffic(str(tmp_path / "f" / "*.csv"), str(tmp_path / "w" / "*.csv"),
+                              str(run), cfg, B)
+
+
 def test_more_than_one_gpu_is_refused_with_a_message():
     r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"],
                        capture_output=True, text=True, timeout=120)
