@@ -173,18 +173,23 @@ int msa_linear_w8a16(const void* x, const int8_t* Wq, const void* scales, const 
                      const void* residual, void* y, int64_t M, int N, int K, unsigned flags,
                      void* stream);
 
-/* Split-K form for the decode step (1 <= M <= 128, MSA_IN_PACKED required): K is cut into S
+/* Split-K form for the decode step (packed activations, MSA_IN_PACKED: 1 <= M <= 128): K is cut into S
  * ranges and part[s][m][n] (fp32, [S, M, N]) receives the exact fp32 partial sums of range s;
  * the consumer adds them in slice order (msa_residual_layernorm_f16).  Used where N alone gives
  * the chip too few weight tiles (out_proj, fc2).  msa_linear_default_splits suggests S.  The
  * ranges hold ceil(K/32 / S) 32-wide steps (rounded up to an even count for int8); an S that would
- * leave the last range(s) empty is rejected. */
+ * leave the last range(s) empty is rejected.
+ * Without MSA_IN_PACKED (msa_linear_partial_f16 only): x is row-major [M, K], any M >= 1, and the
+ * MFMA tile kernel sums over S equal ranges (K % (64 S) == 0, K / S >= 128): for decode batches
+ * above 128 rows, whose 256-row tiles against d_model output features occupy a quarter of the
+ * chip; msa_linear_default_splits_rows suggests S (1: one pass of msa_linear_f16 is as good). */
 int msa_linear_partial_f16(const void* x, const void* Wp, float* part, int64_t M, int N, int K,
                            int S, unsigned flags, void* stream);
 int msa_linear_partial_w8a16(const void* x, const int8_t* Wq, const void* scales, float* part,
                              int64_t M, int N, int K, int S, unsigned flags, void* stream);
 int msa_linear_default_splits(int64_t M, int N, int K);
 int msa_linear_default_splits_w8a16(int64_t M, int N, int K);
+int msa_linear_default_splits_rows(int64_t M, int N, int K);
 
 /* Fused QKV projection: kvq = round(round(x . Wqkv^T) + bqkv) with rows of Wqkv ordered
  * K | V | Q; then for row m = b*T + t and head h:

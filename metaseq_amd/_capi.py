@@ -73,6 +73,7 @@ SIGNATURES = {
     "msa_linear_partial_w8a16": [_P, _P, _P, _P, c_int64, c_int, c_int, c_int, c_uint, _P],
     "msa_linear_default_splits": [c_int64, c_int, c_int],
     "msa_linear_default_splits_w8a16": [c_int64, c_int, c_int],
+    "msa_linear_default_splits_rows": [c_int64, c_int, c_int],
     "msa_qkv_proj_f16": [_P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
                          c_uint, _P, _P],
     "msa_qkv_proj_w8a16": [_P, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int,

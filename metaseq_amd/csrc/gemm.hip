@@ -1126,10 +1126,13 @@ __device__ __forceinline__ void epilogue8(const Epilogue& e, int64_t m, int n, h
   }
 }
 
-template <int MODE, int WF>
+// PART: split-K.  Workgroup (bx, by, z) sums over the K range of ``part_stages`` 64-wide stages
+// that starts at stage z * part_stages and stores its fp32 sums, with no epilogue, as slice z of
+// ``part`` ([gridDim.z][M][N]); a later launch adds the slices in slice order.
+template <int MODE, int WF, bool PART = false>
 __global__ __launch_bounds__(TQ_THREADS) void linear_quad_kernel(
     const half_t* __restrict__ x, const void* __restrict__ Wp, int64_t M, int N, int K,
-    int rm_a, int rm_b, int rm_r, Epilogue epi) {
+    int rm_a, int rm_b, int rm_r, Epilogue epi, float* __restrict__ part, int part_stages) {
   extern __shared__ __attribute__((aligned(16))) char tq_lds[];
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lr = lane & 15, lg = lane >> 4;
@@ -1151,7 +1154,10 @@ __global__ __launch_bounds__(TQ_THREADS) void linear_quad_kernel(
   const int64_t m_own = (int64_t)by * TQ_BM;  // first row this tile owns
   const int64_t m0 = !CLAMP && m_own + TQ_BM > M ? M - TQ_BM : m_own;
   const int n0 = bx * TQ_BN;
-  const int nst = K / 64, nks = K / 32;
+  // the stages this workgroup sums over: all of K, or its slice (the operand bases below move
+  // to the slice's first stage, so that stage and step numbers count from 0 either way)
+  const int st_first = PART ? (int)blockIdx.z * part_stages : 0;
+  const int nst = PART ? part_stages : K / 64, nks = 2 * nst;
   const int ntiles = N / 16;
 
   // direct loads.  Activations, per stage: instruction i (0..7) of the wave fills rows
@@ -1164,12 +1170,13 @@ __global__ __launch_bounds__(TQ_THREADS) void linear_quad_kernel(
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
     const int64_t r = m0 + wave * 64 + i * 8;
-    xb[i] = (const char*)(x + (CLAMP ? min(r, M - 1) : r) * K) - (i - 4) * 1024;
+    xb[i] = (const char*)(x + (CLAMP ? min(r, M - 1) : r) * K + (int64_t)st_first * 64) -
+            (i - 4) * 1024;
   }
 #pragma unroll
   for (int j = 0; j < WL; ++j) {
     const int tt = min(n0 / 16 + wave * WL + j, ntiles - 1);
-    wb[j] = (const char*)Wp + (int64_t)tt * K * 32 - j * 1024;
+    wb[j] = (const char*)Wp + (int64_t)tt * K * 32 + (int64_t)st_first * 2048 - j * 1024;
   }
   const uint32_t xrow = (uint32_t)(lane >> 3) * (uint32_t)K * 2;
   const uint32_t xlane0 = xrow + (((lane & 7) ^ (lane >> 4)) * 16);
@@ -1342,6 +1349,23 @@ __global__ __launch_bounds__(TQ_THREADS) void linear_quad_kernel(
 #pragma unroll
     for (int j = 0; j < WF; ++j) asm volatile("" : "+a"(acc[i][j]));
   __syncthreads();  // every wave is done with the operand rings
+
+  if constexpr (PART) {
+    // the sums as the lanes hold them: D tile (i, j) = activation row 16 * i + lr of the wave's
+    // 128, features 16 * j + 4 * lg .. + 3 of the wave's 16 WF (16 bytes per lane, 64 per row)
+    float* slice = part + (int64_t)blockIdx.z * M * N;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int64_t m = m0 + wm * 128 + i * 16 + lr;
+#pragma unroll
+      for (int j = 0; j < WF; ++j) {
+        const int n = n0 + wn * (16 * WF) + 16 * j + 4 * lg;
+        if (m >= m_own && m < M && n < N)
+          *reinterpret_cast<float4_t*>(slice + m * N + n) = acc[i][j];
+      }
+    }
+    return;
+  }
 
   // D tile (i, j): the lane holds activation row 16 * i + lr of the wave's 128 and the 4 features
   // 16 * j + 4 * lg ...  Per i the wave's 16 rows x 16 WF features (4 or 2 KB, two buffers per wave)
@@ -1623,10 +1647,37 @@ void launch_quad(const void* x, const void* W, const void* scales, int64_t M, in
     }
   }
   hipLaunchKernelGGL((linear_quad_kernel<MODE, WF>), dim3(ncol, nrow), dim3(TQ_THREADS),
-                     tq_lds_bytes(WF), s, (const half_t*)x, W, M_main, N, K, rm_a, rm_b, rm_r, epi);
+                     tq_lds_bytes(WF), s, (const half_t*)x, W, M_main, N, K, rm_a, rm_b, rm_r, epi,
+                     (float*)nullptr, 0);
   for (int64_t m0 = M_main; m0 < M; m0 += 64)
     launch_stream<false, MODE, true>(x, W, scales, nullptr, 1, (int)min((int64_t)64, M - m0), N,
                                      K, epi, s, m0);
+}
+
+// Split-K launch of the narrowest four-wave form on row-major activations: S slices of K, each
+// a whole number of 64-wide stages (at least two), fp32 sums into part[S][M][N].
+void launch_quad_partial(const void* x, const void* W, float* part, int64_t M, int N, int K, int S,
+                         hipStream_t s) {
+  static std::atomic<uint64_t> lds_allowed_p{0};
+  auto kernel = linear_quad_kernel<MODE_PLAIN, 2, true>;
+  if (!allow_lds((const void*)kernel, tq_lds_bytes(2), lds_allowed_p)) return;
+  const int ncol = (N + tq_bn(2) - 1) / tq_bn(2);
+  const int nrow = (int)((M + TQ_BM - 1) / TQ_BM);
+  Epilogue e{};
+  hipLaunchKernelGGL(kernel, dim3(ncol, nrow, S), dim3(TQ_THREADS), tq_lds_bytes(2), s,
+                     (const half_t*)x, W, M, N, K, 0, 0, 0, e, part, K / 64 / S);
+}
+
+// Slices for a product of M row-major rows whose tiles alone leave most of the chip idle (a
+// decode batch of a few hundred rows against d_model output features): the most of 2, 4, 8 that
+// keep the workgroups within the chip, the K range of a slice at 512 or more, and whole stages.
+int pick_row_splits(int64_t M, int N, int K) {
+  if (M < 1 || N % 16 || K % 64) return 1;
+  const int64_t tiles = ((M + TQ_BM - 1) / TQ_BM) * ((N + tq_bn(2) - 1) / tq_bn(2));
+  int best = 1;
+  for (int S = 2; S <= 8; S *= 2)
+    if (tiles * S <= num_cus() && K % (64 * S) == 0 && K / S >= 512) best = S;
+  return best;
 }
 
 template <bool W8, int MODE>
@@ -1742,8 +1793,21 @@ int partial_entry(const char* name, const void* x, const void* W, const void* sc
   int rc = check_linear_args(name, x, W, part, M, N, K, W8, flags, MSA_IN_PACKED);
   if (rc) return rc;
   MSA_REQUIRE(!W8 || scales, MSA_ERR_INVALID_ARG, "%s: null scales", name);
-  MSA_REQUIRE((flags & MSA_IN_PACKED) && M >= 1 && M <= MSA_PACKED_MAX_ROWS, MSA_ERR_INVALID_ARG,
-              "%s: needs packed activations and 1 <= M <= %d (M=%lld)", name, MSA_PACKED_MAX_ROWS,
+  if (!(flags & MSA_IN_PACKED)) {
+    // row-major activations: the MFMA tile kernel over S equal K ranges
+    MSA_REQUIRE(!W8, MSA_ERR_INVALID_ARG,
+                "%s: partial sums of row-major activations exist for fp16 weights only (expand "
+                "the int8 matrix with msa_expand_weight_w8_f16 first)", name);
+    MSA_REQUIRE(M >= 1, MSA_ERR_INVALID_ARG, "%s: M=%lld", name, (long long)M);
+    MSA_REQUIRE(S >= 1 && K % (64 * S) == 0 && K / S >= 128, MSA_ERR_INVALID_ARG,
+                "%s: row-major activations need K=%d cut by S=%d into ranges that are multiples "
+                "of 64 and at least 128", name, K, S);
+    launch_quad_partial(x, W, part, M, N, K, S, (hipStream_t)stream);
+    MSA_CHECK_LAUNCH(name);
+    return MSA_OK;
+  }
+  MSA_REQUIRE(M >= 1 && M <= MSA_PACKED_MAX_ROWS, MSA_ERR_INVALID_ARG,
+              "%s: packed activations need 1 <= M <= %d (M=%lld)", name, MSA_PACKED_MAX_ROWS,
               (long long)M);
   MSA_REQUIRE(S >= 1 && S <= K / (W8 ? 64 : 32), MSA_ERR_INVALID_ARG,
               "%s: S=%d outside 1..%d", name, S, K / (W8 ? 64 : 32));
@@ -2011,6 +2075,10 @@ extern "C" int msa_linear_default_splits(int64_t M, int N, int K) {
 
 extern "C" int msa_linear_default_splits_w8a16(int64_t M, int N, int K) {
   return pick_splits(M, N, K, 1);
+}
+
+extern "C" int msa_linear_default_splits_rows(int64_t M, int N, int K) {
+  return pick_row_splits(M, N, K);
 }
 
 extern "C" int msa_linear_f16(const void* x, const void* Wp, const void* bias,

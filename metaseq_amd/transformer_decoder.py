@@ -738,10 +738,36 @@ class TransformerDecoder(nn.Module):
         check(lib.msa_attention_f16(ptr(q), ptr(kc), ptr(vc), ptr(mask), mask_stride, ptr(o), B,
                                     H, hd, T, S0, cap, 0, None, stream))
         # x = round(round(o Wo^T + bo) + x)   (transformer_decoder_layer.py:222-230)
-        self._linear(lib, stream, o, layer.self_attn.out_proj, M, D, D, residual=x, out=x)
-        self._layernorm(lib, stream, x, layer.final_layer_norm, M, D, h)
+        ln2 = layer.final_layer_norm
+        if not self._linear_split(lib, stream, o, layer.self_attn.out_proj, x, work, M, D, D,
+                                  ln=ln2, ln_out=h):
+            self._linear(lib, stream, o, layer.self_attn.out_proj, M, D, D, residual=x, out=x)
+            self._layernorm(lib, stream, x, ln2, M, D, h)
         self._linear(lib, stream, h, layer.fc1, M, F, D, relu=True, out=u)
-        self._linear(lib, stream, u, layer.fc2, M, D, F, residual=x, out=x)
+        if not self._linear_split(lib, stream, u, layer.fc2, x, work, M, D, F):
+            self._linear(lib, stream, u, layer.fc2, M, D, F, residual=x, out=x)
+
+    def _linear_split(self, lib, stream, a, lin, x, work, M, N, K, ln=None, ln_out=None):
+        """``x = round(round(a W^T + b) + x)`` as split-K partial sums + the fused tail, where M
+        row-major rows against N output features leave most of the chip without a tile (a decode
+        batch above 128 rows: 64 workgroups for d_model 4096); with ``ln``, the LayerNorm of the
+        new ``x`` goes to ``ln_out`` in the same launch.  False (nothing done) where one pass of
+        the tile kernel is as good, or for int8 weights below the row count from which they run
+        expanded to fp16."""
+        if lin.qweight is not None and M < self.W8_EXPAND_ROWS:
+            return False
+        S = lib.msa_linear_default_splits_rows(M, N, K)
+        if S <= 1:
+            return False
+        part = work.get("part")
+        if part is None or part.numel() < S * M * N:
+            part = work["part"] = torch.empty(S * M * N, dtype=torch.float32, device=a.device)
+        w = self._expanded(lib, stream, lin) if lin.qweight is not None else ptr(lin.weight)
+        check(lib.msa_linear_partial_f16(ptr(a), w, ptr(part), M, N, K, S, 0, stream))
+        g, b = (ln.weight, ln.bias) if ln is not None else (None, None)
+        check(lib.msa_residual_layernorm_f16(ptr(part), S, ptr(lin.bias), ptr(x), ptr(g), ptr(b),
+                                             ptr(ln_out), M, N, 1e-5, 0, stream))
+        return True
 
     # ------------------------------------------------------------------ slot interface
     # A running batch whose rows belong to different requests (continuous batching): a fixed

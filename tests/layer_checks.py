@@ -266,3 +266,58 @@ def check_decode_layer(dec, i, trace, j, B, n0, tag):
     rep.cmp_chained(x, t["x_out"], t["x_in"])
     torch.cuda.synchronize()
     return rep
+
+
+def check_rows_decode_layer(dec, i, trace, j, B, n0, tag):
+    """As check_decode_layer for a decode batch above 128 rows: row-major activations through
+    ``_rows_layer`` (tile kernels; split-K partial sums + the fused tail where the library
+    suggests slices)."""
+    lib = dec.prepare_()
+    stream = _capi.stream_ptr()
+    cfg = dec.cfg
+    D, H, hd, F = (cfg.decoder_embed_dim, cfg.decoder_attention_heads, cfg.head_dim,
+                   cfg.decoder_ffn_embed_dim)
+    layer = dec.layers[i]
+    t = trace[j]
+    dev = t["x_in"].device
+    S0 = n0 + j - 1
+    cap = S0 + 8
+    rep = Report("%s layer %d decode step %d (row-major)" % (tag, i, j))
+    cache = KVCache(1, B, H, hd, cap, dev)
+    kc, vc = cache.k(0), cache.v(0)
+    kc[:, :, :n0].copy_(_heads(trace[0]["k"], B, n0, H, hd))
+    vc[:, :, :n0].copy_(_heads(trace[0]["v"], B, n0, H, hd))
+    for s in range(1, j):
+        kc[:, :, n0 + s - 1].copy_(trace[s]["k"].view(B, H, hd))
+        vc[:, :, n0 + s - 1].copy_(trace[s]["v"].view(B, H, hd))
+    work = dec._rows_buffers(B, dev)
+    h, u = work["h"], work["u"]
+    op, ln = layer.self_attn.out_proj, layer.final_layer_norm
+    x = t["x_in"].clone()
+    o = t["o"].clone()
+    split = dec._linear_split(lib, stream, o, op, x, work, B, D, D, ln=ln, ln_out=h)
+    if not split:
+        dec._linear(lib, stream, o, op, B, D, D, residual=x, out=x)
+        dec._layernorm(lib, stream, x, ln, B, D, h)
+    rep.cmp("out_proj + residual" + (" (split-K)" if split else ""), x, t["x_mid"], stages=3,
+            also=t["x_in"].abs() + op.bias.abs().view(1, D),
+            acc=(D, t["x_mid"].float() - t["x_in"].float()))
+    rep.cmp("... LayerNorm 2", h, t["h2"], stages=2,
+            also=ln_also(t["x_mid"], t["x_mid"].abs() + t["x_in"].abs() + op.bias.abs().view(1, D),
+                         ln, 3))
+    dec._linear(lib, stream, t["h2"].clone(), layer.fc1, B, F, D, relu=True, out=u)
+    rep.cmp("fc1 + ReLU", u, t["u"], stages=2, also=layer.fc1.bias.view(1, F), acc=(D, t["u"]))
+    x = t["x_mid"].clone()
+    uu = t["u"].clone()
+    split = dec._linear_split(lib, stream, uu, layer.fc2, x, work, B, D, F)
+    if not split:
+        dec._linear(lib, stream, uu, layer.fc2, B, D, F, residual=x, out=x)
+    rep.cmp("fc2 + residual" + (" (split-K)" if split else ""), x, t["x_out"], stages=3,
+            also=t["x_mid"].abs() + layer.fc2.bias.abs().view(1, D),
+            acc=(F, t["x_out"].float() - t["x_mid"].float()))
+    # chained, from the layer's input
+    x = t["x_in"].clone()
+    dec._rows_layer(lib, stream, layer, x, work, B, 1, S0, kc, vc, cap, None)
+    rep.cmp_chained(x, t["x_out"], t["x_in"])
+    torch.cuda.synchronize()
+    return rep

@@ -34,7 +34,8 @@ from metaseq_amd import (Dictionary, SequenceGenerator, TransformerLanguageModel
                          iter_random_state_dict, opt_config, random_prompts, random_state_dict)
 from oracle.opt_oracle import dequantize_int8, greedy_generate, layer_norm, quantize_int8
 from tests.common import make_oracle
-from tests.layer_checks import check_decode_layer, check_prefill_layer
+from tests.layer_checks import (check_decode_layer, check_prefill_layer,
+                                check_rows_decode_layer)
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda"
@@ -227,8 +228,9 @@ def _run_config(size, B, P, G=32, max_pos=None, layers=None, int8=False, sequent
                   for t in traces.pop(i)[:max(decode_checks) + 1]]
         check_prefill_layer(dec, i, passes[0], B, n0, tag)
         for j in decode_checks:
-            if B <= 128 and j < len(passes):   # the packed decode path
-                check_decode_layer(dec, i, passes, j, B, n0, tag)
+            if j < len(passes):   # the packed decode path up to 128 rows, row-major above
+                (check_decode_layer if B <= 128 else check_rows_decode_layer)(
+                    dec, i, passes, j, B, n0, tag)
         del passes
     _free()
     gen = SequenceGenerator([model], Dictionary(cfg.vocab_size), max_len_b=max_len_b,

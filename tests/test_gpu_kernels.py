@@ -550,6 +550,54 @@ def test_split_k_partials_and_fused_layernorm(lib, M, N, K, S, w8):
     assert torch.equal(xd2, xd)
 
 
+@pytest.mark.parametrize("M,N,K,S", [(129, 4096, 4096, 4), (200, 1024, 8192, 8),
+                                     (256, 4096, 1024, 2), (256, 2064, 512, 4),
+                                     (300, 768, 3072, 1), (1, 64, 128, 1), (77, 4096, 2048, 4)])
+def test_split_k_partials_of_row_major_rows(lib, M, N, K, S):
+    """msa_linear_partial_f16 without MSA_IN_PACKED (decode batches above 128 rows): slice s of
+    the output holds the fp32 sums over K range s and nothing else, for row counts that are not
+    multiples of the 256-row tile and an N that is not a multiple of the 64-wide tile; followed
+    by msa_residual_layernorm_f16 on row-major rows it equals the oracle's linear + bias,
+    residual add and LayerNorm."""
+    print("row-major splitk", M, N, K, S, flush=True)
+    x, W, b = rnd(M, K, seed=7), rnd(N, K, seed=8, std=0.03), rnd(N, seed=9, std=0.1)
+    res, g, be = rnd(M, N, seed=10), (1 + rnd(N, seed=11, std=0.1).float()).half(), rnd(N, seed=12)
+    part = torch.full((S + 1, M, N), float("nan"), dtype=torch.float32, device=DEV)
+    ok(lib.msa_linear_partial_f16(P(G(x)), P(pack_w(lib, G(W))), P(part), M, N, K, S, 0, None), lib)
+    torch.cuda.synchronize()
+    assert bool(torch.isnan(part[S]).all()), "wrote past the last slice"
+    per = K // S
+    for s_ in range(S):
+        want = x[:, s_ * per:(s_ + 1) * per].double() @ W[:, s_ * per:(s_ + 1) * per].double().t()
+        err = float((part[s_].cpu().double() - want).abs().max())
+        assert err < 2e-4, "slice %d off by %.3g" % (s_, err)
+    xo = r16(O.linear(x.float(), W.float(), b.float(), r16) + res.float())
+    want_h = O.layer_norm(xo, g, be).half()
+    xd = G(res).clone()
+    h = torch.zeros(M, N, dtype=torch.float16, device=DEV)
+    ok(lib.msa_residual_layernorm_f16(P(part), S, P(G(b)), P(xd), P(G(g)), P(G(be)), P(h), M, N,
+                                      1e-5, 0, None), lib)
+    torch.cuda.synchronize()
+    atol = float(xo.abs().max()) * 2 ** -10
+    assert_fp16_close(xd, xo.half(), atol=atol, what="residual stream")
+    assert_fp16_close(h, want_h, max_ulp=2, max_frac=2e-2, atol=4 * atol, what="fused LN")
+
+
+def test_split_k_of_row_major_rows_rejects_and_suggestion(lib):
+    x = torch.zeros(256, 4096, dtype=torch.float16, device=DEV)
+    part = torch.zeros(8 * 256 * 64, dtype=torch.float32, device=DEV)
+    f = lib.msa_linear_partial_f16
+    assert f(P(x), P(x), P(part), 256, 64, 4096, 3, 0, None) == -1    # 4096 / 3 is no whole range
+    assert f(P(x), P(x), P(part), 256, 64, 256, 4, 0, None) == -1     # ranges of one stage
+    assert lib.msa_linear_partial_w8a16(P(x), P(x), P(x), P(part), 256, 64, 4096, 4, 0, None) == -1
+    # a few hundred rows against d_model output features: split; enough tiles already: not
+    assert lib.msa_linear_default_splits_rows(256, 4096, 16384) == 4
+    assert lib.msa_linear_default_splits_rows(200, 4096, 4096) == 4
+    assert lib.msa_linear_default_splits_rows(512, 4096, 4096) == 2
+    assert lib.msa_linear_default_splits_rows(256, 16384, 4096) == 1
+    assert lib.msa_linear_default_splits_rows(4096, 4096, 4096) == 1
+
+
 def test_default_splits_are_valid(lib):
     for M, N, K in [(32, 4096, 4096), (32, 4096, 16384), (32, 12288, 4096), (1, 768, 768),
                     (8, 2048, 8192), (64, 9216, 36864), (200, 4096, 4096)]:
