@@ -1654,29 +1654,45 @@ void launch_quad(const void* x, const void* W, const void* scales, int64_t M, in
                                      K, epi, s, m0);
 }
 
-// Split-K launch of the narrowest four-wave form on row-major activations: S slices of K, each
-// a whole number of 64-wide stages (at least two), fp32 sums into part[S][M][N].
-void launch_quad_partial(const void* x, const void* W, float* part, int64_t M, int N, int K, int S,
-                         hipStream_t s) {
+// Split-K launch of a narrow four-wave form (WF = 2: 256 x 64 tiles, WF = 4: 256 x 128) on
+// row-major activations: S slices of K, each a whole number of 64-wide stages (at least two),
+// fp32 sums into part[S][M][N].
+template <int WF>
+void launch_quad_partial_w(const void* x, const void* W, float* part, int64_t M, int N, int K,
+                           int S, hipStream_t s) {
   static std::atomic<uint64_t> lds_allowed_p{0};
-  auto kernel = linear_quad_kernel<MODE_PLAIN, 2, true>;
-  if (!allow_lds((const void*)kernel, tq_lds_bytes(2), lds_allowed_p)) return;
-  const int ncol = (N + tq_bn(2) - 1) / tq_bn(2);
+  auto kernel = linear_quad_kernel<MODE_PLAIN, WF, true>;
+  if (!allow_lds((const void*)kernel, tq_lds_bytes(WF), lds_allowed_p)) return;
+  const int ncol = (N + tq_bn(WF) - 1) / tq_bn(WF);
   const int nrow = (int)((M + TQ_BM - 1) / TQ_BM);
   Epilogue e{};
-  hipLaunchKernelGGL(kernel, dim3(ncol, nrow, S), dim3(TQ_THREADS), tq_lds_bytes(2), s,
+  hipLaunchKernelGGL(kernel, dim3(ncol, nrow, S), dim3(TQ_THREADS), tq_lds_bytes(WF), s,
                      (const half_t*)x, W, M, N, K, 0, 0, 0, e, part, K / 64 / S);
+}
+
+// 256 x 64 tiles while their S slices fit the chip in one round; an S beyond that (given M >= 256,
+// which the wider form needs to move a ragged tile up) means 256 x 128 tiles.
+void launch_quad_partial(const void* x, const void* W, float* part, int64_t M, int N, int K, int S,
+                         hipStream_t s) {
+  const int64_t tiles2 = ((M + TQ_BM - 1) / TQ_BM) * ((N + tq_bn(2) - 1) / tq_bn(2));
+  if (M >= TQ_BM && tiles2 * S > num_cus())
+    return launch_quad_partial_w<4>(x, W, part, M, N, K, S, s);
+  launch_quad_partial_w<2>(x, W, part, M, N, K, S, s);
 }
 
 // Slices for a product of M row-major rows whose tiles alone leave most of the chip idle (a
 // decode batch of a few hundred rows against d_model output features): the most of 2, 4, 8 that
-// keep the workgroups within the chip, the K range of a slice at 512 or more, and whole stages.
+// keep the 256 x 64 tiles within the chip, the K range of a slice at 512 or more, and whole
+// stages.  Where a slice would still span 4096 or more of K, twice the slices over 256 x 128
+// tiles measured faster (half the activation bytes per workgroup and weight byte: M = 256,
+// N = 4096, K = 16384: 51.8 against 55.4 us; M = 512: 78.0 against 93.6).
 int pick_row_splits(int64_t M, int N, int K) {
   if (M < 1 || N % 16 || K % 64) return 1;
   const int64_t tiles = ((M + TQ_BM - 1) / TQ_BM) * ((N + tq_bn(2) - 1) / tq_bn(2));
   int best = 1;
   for (int S = 2; S <= 8; S *= 2)
     if (tiles * S <= num_cus() && K % (64 * S) == 0 && K / S >= 512) best = S;
+  if (best > 1 && best < 8 && M >= TQ_BM && K / best >= 4096 && K % (128 * best) == 0) best *= 2;
   return best;
 }
 
