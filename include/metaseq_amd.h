@@ -273,6 +273,9 @@ int msa_greedy_select_f16(const void* logits, int64_t ld_logits, int B, int V, f
  *   score -inf, as does a row with no eligible id);
  *   banned / early / only-eos ids -> -inf;  lp[v] -= counts[b,v] * alpha_frequency +
  *   (counts[b,v] > 0) * alpha_presence, likewise counts_src (int64 [B, V] device, optional);
+ *   penalty_rows (optional, fp32 [B, 4] device: presence, frequency, presence_src, frequency_src)
+ *   gives every row its own four weights in place of the scalar arguments (rows of one batch
+ *   that belong to different requests);
  *   lprobs_out (optional, fp32, row stride ld_lprobs) receives that masked, penalised row: what
  *   the reference stores as the step's distribution;
  *   p = softmax(lp);  with the ids in order of decreasing p (ties: increasing id), id k belongs
@@ -298,9 +301,9 @@ int msa_sample_topp_f16(const void* logits, int64_t ld_logits, int B, int V, flo
                         const float* topp_rows, float topp_all, const float* noise,
                         int64_t* counts, const int64_t* counts_src, float alpha_presence,
                         float alpha_frequency, float alpha_presence_src,
-                        float alpha_frequency_src, float* lprobs_out, int64_t ld_lprobs,
-                        int64_t* tok, int64_t tok_stride, float* score, int64_t score_stride,
-                        void* stream);
+                        float alpha_frequency_src, const float* penalty_rows,
+                        float* lprobs_out, int64_t ld_lprobs, int64_t* tok, int64_t tok_stride,
+                        float* score, int64_t score_stride, void* stream);
 
 /* fp32 log-softmax of n_outer x n_inner fp16 logits rows of V ids:
  *   out[o*out_outer_stride + i*ld_out + v] = z[v] - max z - log(sum(exp(z - max z))),

@@ -87,7 +87,7 @@ SIGNATURES = {
                               c_int, c_int, _P, c_int64, _P, c_int64, _P, _P],
     "msa_sample_topp_f16": [_P, c_int64, c_int, c_int, c_float, _P, _P, c_int, _P, c_int, _P, _P,
                             c_int, c_int, _P, c_float, _P, _P, _P, c_float, c_float, c_float,
-                            c_float, _P, c_int64, _P, c_int64, _P, c_int64, _P],
+                            c_float, _P, _P, c_int64, _P, c_int64, _P, c_int64, _P],
     "msa_log_softmax_f16": [_P, c_int64, c_int64, c_int, c_int, c_int, c_float, _P, c_int64,
                             c_int64, _P],
     "msa_target_logprob_f16": [_P, c_int64, c_int64, c_int, c_float, _P, _P, _P],

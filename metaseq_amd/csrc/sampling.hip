@@ -298,6 +298,7 @@ struct Penalties {
   int64_t* counts;            // [B, V] generated-token counts (updated) or NULL
   const int64_t* counts_src;  // [B, V] prompt-token counts or NULL
   float presence, frequency, presence_src, frequency_src;
+  const float* rows;  // [B, 4] per-row presence, frequency, presence_src, frequency_src, or NULL
 };
 
 __device__ __forceinline__ void argbest(float& v, int& i, float ov, int oi) {
@@ -315,6 +316,10 @@ __global__ __launch_bounds__(SP_THREADS) void sample_topp_kernel(
     const float* __restrict__ noise, Penalties pen, float* __restrict__ lprobs_out,
     int64_t ld_lprobs, int64_t* __restrict__ tok, int64_t tok_stride,
     float* __restrict__ score, int64_t score_stride) {
+  if (pen.rows) {  // this row's own penalty weights (rows of a batch from different requests)
+    const float* w = pen.rows + 4 * (int64_t)blockIdx.x;
+    pen.presence = w[0], pen.frequency = w[1], pen.presence_src = w[2], pen.frequency_src = w[3];
+  }
   __shared__ float red[16];
   __shared__ float rbest[16], rprob[16];
   __shared__ int ridx[16];
@@ -618,7 +623,8 @@ extern "C" int msa_sample_topp_f16(const void* logits, int64_t ld_logits, int B,
                                    int64_t* counts, const int64_t* counts_src,
                                    float alpha_presence, float alpha_frequency,
                                    float alpha_presence_src, float alpha_frequency_src,
-                                   float* lprobs_out, int64_t ld_lprobs, int64_t* tok,
+                                   const float* penalty_rows, float* lprobs_out,
+                                   int64_t ld_lprobs, int64_t* tok,
                                    int64_t tok_stride, float* score, int64_t score_stride,
                                    void* stream) {
   const char* name = "msa_sample_topp_f16";
@@ -646,6 +652,7 @@ extern "C" int msa_sample_topp_f16(const void* logits, int64_t ld_logits, int B,
   pen.frequency = alpha_frequency;
   pen.presence_src = alpha_presence_src;
   pen.frequency_src = alpha_frequency_src;
+  pen.rows = penalty_rows;
   hipLaunchKernelGGL(sample_topp_kernel, dim3(B), dim3(SP_THREADS), 0, (hipStream_t)stream,
                      (const half_t*)logits, ld_logits, V, temperature, temperature_rows, banned,
                      stop, finished, row_mode, force_eos_all, eos_idx, topp_rows, topp_all, noise,

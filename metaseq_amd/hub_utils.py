@@ -23,6 +23,30 @@ import torch
 from .sequence_generator import SequenceGenerator
 
 
+class TopRows:
+    """What is kept of a row's per-position distributions when only the best entries are
+    reported: ``values`` / ``ids`` [positions, k], most likely first.  Indexable by position
+    like the dense [positions, vocab] array it stands for."""
+
+    def __init__(self, values, ids):
+        self.values, self.ids = np.asarray(values, dtype=np.float64), np.asarray(ids, np.int64)
+        self.shape = self.values.shape
+
+    @classmethod
+    def from_pairs(cls, pairs, k):
+        """``pairs``: per position (values, ids) lists of k entries, or empty lists for a
+        position without a prediction (stored as -inf / id 0)."""
+        values = np.full((len(pairs), k), -np.inf)
+        ids = np.zeros((len(pairs), k), dtype=np.int64)
+        for i, (v, t) in enumerate(pairs):
+            if len(v):
+                values[i], ids[i] = v, t
+        return cls(values, ids)
+
+    def __getitem__(self, sel):
+        return TopRows(self.values[sel], self.ids[sel])
+
+
 class _IdTokenizer:
     """Stand-in tokenizer: a token is its decimal id, a text is ids joined by single spaces."""
 
@@ -185,7 +209,10 @@ class GeneratorInterface:
         """Per position, the k most likely tokens as {token string: log-probability}."""
         if rows.shape[0] == 0:
             return []
-        values, ids = torch.as_tensor(rows).topk(k, dim=-1)
+        if isinstance(rows, TopRows):
+            values, ids = rows.values[:, :k], rows.ids[:, :k]
+        else:
+            values, ids = torch.as_tensor(rows).topk(k, dim=-1)
         return [{self.bpe.decode([i]): v for i, v in zip(id_row, value_row)}
                 for id_row, value_row in zip(ids.tolist(), values.tolist())]
 

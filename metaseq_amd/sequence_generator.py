@@ -340,7 +340,8 @@ class SequenceGenerator(nn.Module):
             self.eos, ptr(topp_rows), float(self.sampling_topp) if self.sampling else 0.0,
             ptr(noise), ptr(gs["count_tokens"]), ptr(gs["count_tokens_src"]),
             float(self.alpha_presence), float(self.alpha_frequency),
-            float(self.alpha_presence_src), float(self.alpha_frequency_src), ptr(lprobs_out),
+            float(self.alpha_presence_src), float(self.alpha_frequency_src), None,
+            ptr(lprobs_out),
             lprobs_out.stride(0) if lprobs_out is not None else 0, ptr(tok), tokens.stride(0),
             ptr(sc), scores.stride(0), _capi.stream_ptr()))
         if self.sampling and self.lambda_decay > 0:

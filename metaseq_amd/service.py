@@ -12,9 +12,10 @@ thread that drives the GPU, results delivered through a per-request queue):
 * ``ContinuousBatcher`` - no reference counterpart: a fixed set of slots over one KV cache with
   per-row lengths; a request is prefilled into a free slot whenever one exists and leaves it the
   moment it ends, while the other rows keep decoding.  Greedy and sampled requests share the
-  batch; each row follows its own temperature, nucleus and ``min_tokens`` / ``max_tokens`` /
-  end-of-sequence rules, and gets the record a single-request ``GeneratorInterface.generate``
-  call would give it.
+  batch; each row follows its own temperature, nucleus (fixed or decaying), repetition
+  penalties and ``min_tokens`` / ``max_tokens`` / end-of-sequence rules, and gets the record a
+  single-request ``GeneratorInterface.generate`` call would give it, alternatives per position
+  (``logprobs``) included.
 """
 import heapq
 import itertools
@@ -246,7 +247,7 @@ class _Row:
     """One replica of a request while it occupies a slot."""
 
     __slots__ = ("group", "replica", "tokens", "scores", "n_new", "min_new", "max_new", "last",
-                 "done")
+                 "done", "top")
 
     def __init__(self, group: "_Group", replica: int, tokens: List[int], scores: List[float]):
         req = group.req
@@ -257,6 +258,9 @@ class _Row:
         self.max_new = group.max_new
         self.last = tokens[-1]
         self.done = False
+        # with ``logprobs``: per position of ``tokens``, the most likely ids and their
+        # log-probabilities ((values, ids) lists; empty lists where nothing was predicted)
+        self.top: Optional[List[tuple]] = None
 
     def mode(self) -> int:
         """Selection regime of this row's next token: end-of-sequence and stop tokens are barred
@@ -297,9 +301,26 @@ class _Group:
         if temperature == 0:
             temperature, top_p = 1.0, 0.0
         self.temperature, self.topp = temperature, top_p
+
+        def weight(key):
+            return max(0.0, float(o.get(key, 0.0) or 0.0))
+        # repetition penalties (metaseq/sequence_generator.py:118-123, 478-534): presence,
+        # frequency, and the same two for the prompt's tokens
+        self.alphas = (weight("alpha_presence"), weight("alpha_frequency"),
+                       weight("alpha_presence_src"), weight("alpha_frequency_src"))
+        self.src_end = int(o.get("alpha_src_penalty_end_idx", -1) or -1)
+        self.penalised = max(self.alphas) > 0
+        # factual nucleus (:107-116, 443-476): only a sampled row has a nucleus to decay
+        decay = o.get("lambda_decay", -1)
+        self.decay = float(decay) if (decay is not None and decay > 0 and top_p > 0) else -1.0
+        omega = o.get("omega_bound", 0.3)
+        self.omega = float(0.3 if omega is None else omega)
+        self.logprobs = int(o.get("logprobs", 0) or 0)
         # rows chosen inside the vocabulary projection (greedy on the unscaled logits) or by the
-        # sampling kernel on the stored logits (any other temperature, nucleus sampling)
-        self.plain = temperature == 1.0 and top_p == 0.0
+        # sampling kernel on the stored logits (any other temperature, nucleus sampling,
+        # penalties, recorded distributions)
+        self.plain = (temperature == 1.0 and top_p == 0.0 and not self.penalised
+                      and self.logprobs == 0)
         self.finished: Dict[int, "_Row"] = {}
 
 
@@ -341,17 +362,15 @@ class ContinuousBatcher(_Front):
     ``capacity`` is the number of positions a slot can hold (prompt + continuation).  Greedy and
     sampled requests (``temperature``, ``top_p``) share the running batch, each row under its own
     temperature, nucleus and length rules; ``n`` / ``best_of`` replicas of a request are rows of
-    their own that share one prefill.  Requests that need penalties, the factual-nucleus decay
-    or ``logprobs`` are refused with a ValueError delivered to the caller (serve them through
-    ``BatchingService``).
+    their own that share one prefill.  Repetition penalties and the factual-nucleus decay are
+    per-row state of the sampling kernel's call; with ``logprobs`` the kernel also stores the
+    step's masked log-probabilities, of which the requested number of best entries is kept per
+    position.
 
     ``noise_fn(request, replica, position, vocab)`` -> fp32 [vocab] device tensor, if given,
     supplies the Exp(1) numbers of the draw that chooses the token at ``position`` of that
     replica (tests hand both engines the same numbers); otherwise they come from torch's device
     generator.  A request that has waited ``patience`` steps is served before cheaper ones."""
-
-    UNSUPPORTED = ("lambda_decay", "alpha_presence", "alpha_frequency", "alpha_presence_src",
-                   "alpha_frequency_src")
 
     def __init__(self, interface, slots: int = 32, capacity: int = MAX_SEQ_LEN,
                  idle_ms: float = 2.0, noise_fn=None, patience: int = 64):
@@ -378,6 +397,12 @@ class ContinuousBatcher(_Front):
         self._score = torch.zeros(slots, dtype=torch.float32, device=dev)
         # state of the rows the sampling kernel chooses (allocated with the first such request)
         self._smode = self._temp = self._topp = self._logits = self._noise = None
+        # [slots, 1] fp32: initial nucleus, decay factor (<= 0: none), floor, tokens since the
+        # last full stop; [slots, 4] penalty weights; [slots, V] token counts and log-prob rows
+        self._initp = self._lam = self._omega = self._since = self._pen = None
+        self._counts = self._counts_src = self._lprobs = None
+        self._full_stop = torch.tensor([self.dict.index(w) for w in (".", "?", "!")],
+                                       dtype=torch.long, device=dev)
         self._clock = 0         # step() calls so far; a request's arrival is stamped with it
         self._arrived: Dict[int, int] = {}
         self.steps = 0          # decode steps run
@@ -405,11 +430,13 @@ class ContinuousBatcher(_Front):
         if max(n, best_of) > len(self.batch.rows):
             return ("%d replicas do not fit the %d slots of the running batch"
                     % (max(n, best_of), len(self.batch.rows)))
-        if (o.get("logprobs", 0) or 0) > 0:
-            return "continuous batching does not record distributions (logprobs > 0)"
-        for k in self.UNSUPPORTED:
-            if (o.get(k, 0) or 0) > 0:
-                return "continuous batching does not apply %s" % k
+        if (o.get("logprobs", 0) or 0) > len(self.dict):
+            return "logprobs asks for more alternatives than the vocabulary has"
+        decay = o.get("lambda_decay", -1)
+        if (decay is not None and decay > 0 and (o.get("top_p") or 0) > 0
+                and all(int(i) == self.dict.unk() for i in self._full_stop.tolist())):
+            return ("factual-nucleus sampling (lambda_decay > 0) needs a dictionary that "
+                    "resolves '.', '?' and '!' to token ids")
         if len(o.get("stop") or []) > 14:
             return "at most 14 stop tokens are supported"
         if self.batch.room_for(req) == 0:
@@ -428,6 +455,40 @@ class ContinuousBatcher(_Front):
             self._topp = torch.zeros(slots, dtype=torch.float32, device=dev)
             self._logits = torch.empty(slots, V, dtype=torch.float16, device=dev)
             self._noise = torch.empty(slots, V, dtype=torch.float32, device=dev)
+            self._initp = torch.zeros(slots, 1, dtype=torch.float32, device=dev)
+            self._lam = torch.full((slots, 1), -1.0, dtype=torch.float32, device=dev)
+            self._omega = torch.zeros(slots, 1, dtype=torch.float32, device=dev)
+            self._since = torch.zeros(slots, 1, dtype=torch.float32, device=dev)
+            self._pen = torch.zeros(slots, 4, dtype=torch.float32, device=dev)
+
+    def _penalty_state(self):
+        if self._counts is None:
+            torch, slots, V = self._torch, len(self.batch.rows), len(self.dict)
+            self._counts = torch.zeros(slots, V, dtype=torch.long, device=self.device)
+            self._counts_src = torch.zeros(slots, V, dtype=torch.long, device=self.device)
+
+    def _logprob_state(self):
+        if self._lprobs is None:
+            self._lprobs = self._torch.empty(len(self.batch.rows), len(self.dict),
+                                             dtype=self._torch.float32, device=self.device)
+
+    def _nucleus_now(self):
+        """Every slot's nucleus for the next draw: the request's top-p, decayed by its factor
+        per token since the last full stop and never below its floor (the arithmetic of
+        metaseq/sequence_generator.py:443-476, in fp32 on the device)."""
+        torch = self._torch
+        decay = (self._since - 1).clamp_(min=0)
+        decayed = torch.maximum(self._initp * self._lam ** decay, self._omega)
+        return torch.where(self._lam > 0, decayed, self._initp).view(-1)
+
+    def _count_chosen(self, slots: List[int], tokens):
+        """After a draw: a full stop restarts the decay of a row's nucleus, any other token
+        extends it (``tokens``: int64 device tensor, one per listed slot)."""
+        torch = self._torch
+        idx = torch.tensor(slots, dtype=torch.long, device=self.device)
+        hit = (tokens.view(-1, 1) == self._full_stop.view(1, -1)).any(dim=1, keepdim=True)
+        self._since[idx] = torch.where(hit, torch.zeros_like(self._since[idx]),
+                                       self._since[idx] + 1)
 
     def _draw_noise(self, out, rows):
         """Exp(1) numbers for the draws of ``rows`` ((index into ``out``, row) pairs)."""
@@ -452,7 +513,7 @@ class ContinuousBatcher(_Front):
         R = len(rows)
         tok = torch.zeros(R, dtype=torch.long, device=self.device)
         score = torch.zeros(R, dtype=torch.float32, device=self.device)
-        extra = {}
+        extra, detail, lp = {}, {}, None
         if not group.plain:
             self._sampling_state()
             noise = None
@@ -460,15 +521,58 @@ class ContinuousBatcher(_Front):
                 noise = self._noise[:R]
                 self._draw_noise(noise, list(enumerate(rows)))
             extra = dict(temperature=group.temperature, topp=group.topp, noise=noise)
+            V = len(self.dict)
+            if group.penalised:
+                self._penalty_state()
+                # the prompt's token counts, leading end-of-sequence token included, up to
+                # alpha_src_penalty_end_idx if given (metaseq/sequence_generator.py:380-389)
+                src = torch.tensor(ids if group.src_end <= 0 else ids[:group.src_end],
+                                   dtype=torch.long, device=self.device)
+                counts_src = torch.zeros(R, V, dtype=torch.long, device=self.device)
+                counts_src[0].scatter_add_(0, src.clamp(0, V - 1), torch.ones_like(src))
+                counts_src[1:] = counts_src[0]
+                extra["penalties"] = dict(
+                    alphas=group.alphas, counts_src=counts_src,
+                    counts=torch.zeros(R, V, dtype=torch.long, device=self.device))
+            if group.logprobs > 0:
+                self._logprob_state()
+                lp = extra["lprobs_out"] = torch.empty(R, V, dtype=torch.float32,
+                                                       device=self.device)
+                if req.options.get("echo", False):
+                    extra.update(prompt_topk=group.logprobs, detail=detail)
         if R > 1:
             extra["replicas"] = slots[1:]
         prompt_scores = self.decoder.admit_slot(
             self.cache, slots[0], torch.tensor(ids, dtype=torch.long, device=self.device),
             banned=[pad], stop=self._stop, eos=eos, mode=rows[0].mode(), tok_out=tok,
             score_out=score, **extra)
+        if not group.plain:
+            idx = torch.tensor(slots, dtype=torch.long, device=self.device)
+            self._initp[idx] = group.topp
+            self._lam[idx] = group.decay
+            self._omega[idx] = group.omega
+            self._since[idx] = 0.0
+            self._pen[idx] = torch.tensor(group.alphas, dtype=torch.float32, device=self.device)
+            if group.decay > 0:
+                self._count_chosen(slots, tok)
+            if group.penalised:
+                self._counts[idx] = extra["penalties"]["counts"]
+                self._counts_src[idx] = extra["penalties"]["counts_src"]
+        first_top = prompt_top = None
+        if group.logprobs > 0:
+            values, top_ids = lp.topk(group.logprobs, dim=-1)
+            first_top = list(zip(values.tolist(), top_ids.tolist()))
+            # nothing is predicted for the leading token; the prompt's alternatives are kept
+            # only where they can be shown (echo)
+            prompt_top = [([], [])] * len(ids)
+            if "prompt_top" in detail:
+                values, top_ids = detail["prompt_top"]
+                prompt_top = [([], [])] + list(zip(values.tolist(), top_ids.tolist()))
         toks, scs = tok.tolist(), score.tolist()
         for j, (slot, row) in enumerate(zip(slots, rows)):
             row.scores = list(prompt_scores)
+            if first_top is not None:
+                row.top = list(prompt_top) + [first_top[j]]
             self.batch.rows[slot] = row
             if row.take(toks[j], scs[j], eos, self._stop):
                 self._retire(slot)
@@ -483,18 +587,23 @@ class ContinuousBatcher(_Front):
             return
         req = group.req
         try:
+            from .hub_utils import TopRows
             # replicas best cumulative score first (metaseq/sequence_generator.py:325-333), each
             # as the generation loop would return it: tokens up to the end, then eos
             ranked = sorted(group.finished.values(), key=lambda r: (-sum(r.scores), r.replica))
             records = []
             for r in ranked[:group.n]:
                 toks, scs = list(r.tokens), list(r.scores)
+                top = list(r.top) if r.top is not None else None
                 if toks[-1] != self.dict.eos():
                     toks.append(self.dict.eos())
                     scs.append(0.0)
+                    if top is not None:
+                        top.append(([], []))
                 records.append(self.interface._record(
-                    toks, scs, None, len(req.prompt), group.max_new,
-                    bool(req.options.get("echo", False)), 0))
+                    toks, scs, TopRows.from_pairs(top, group.logprobs) if top else None,
+                    len(req.prompt), group.max_new, bool(req.options.get("echo", False)),
+                    group.logprobs))
             req.answer(records)
         except Exception as e:  # noqa: BLE001 - delivered to the caller
             req.answer(e)
@@ -551,22 +660,38 @@ class ContinuousBatcher(_Front):
         self._mode.copy_(torch.tensor(mode, dtype=torch.uint8))
         extra = {}
         if general:
-            smode, temp, topp = [4] * slots, [1.0] * slots, [0.0] * slots  # 4 = MSA_ROW_SKIP
+            smode, temp = [4] * slots, [1.0] * slots  # 4 = MSA_ROW_SKIP
             for i, row in general:
-                smode[i], temp[i], topp[i] = mode[i], row.group.temperature, row.group.topp
+                smode[i], temp[i] = mode[i], row.group.temperature
             self._smode.copy_(torch.tensor(smode, dtype=torch.uint8))
             self._temp.copy_(torch.tensor(temp, dtype=torch.float32))
-            self._topp.copy_(torch.tensor(topp, dtype=torch.float32))
+            self._topp.copy_(self._nucleus_now())
             noise = None
-            if any(t > 0 for t in topp):
+            drawn = [(i, row) for i, row in general if row.group.topp > 0]
+            if drawn:
                 noise = self._noise
-                self._draw_noise(noise, [(i, row) for i, row in general if row.group.topp > 0])
-            extra = dict(logits_out=self._logits,
-                         sampled=dict(row_mode=self._smode, temperature=self._temp,
-                                      topp=self._topp, noise=noise))
+                self._draw_noise(noise, drawn)
+            sampled = dict(row_mode=self._smode, temperature=self._temp, topp=self._topp,
+                           noise=noise)
+            if any(row.group.penalised for _, row in general):
+                sampled.update(penalty_rows=self._pen, counts=self._counts,
+                               counts_src=self._counts_src)
+            if any(row.group.logprobs > 0 for _, row in general):
+                sampled["lprobs_out"] = self._lprobs
+            extra = dict(logits_out=self._logits, sampled=sampled)
         self.decoder.decode_slots(self.cache, self._last, temperature=1.0, banned=[pad],
                                   stop=self._stop, eos=eos, row_mode=self._mode,
                                   tok_out=self._tok, score_out=self._score, **extra)
+        decaying = [i for i, row in general if row.group.decay > 0]
+        if decaying:
+            self._count_chosen(decaying, self._tok[torch.tensor(decaying, device=self.device)])
+        watched = [(i, row) for i, row in general if row.group.logprobs > 0]
+        if watched:
+            k = max(row.group.logprobs for _, row in watched)
+            picked = self._lprobs[torch.tensor([i for i, _ in watched], device=self.device)]
+            values, top_ids = picked.topk(k, dim=-1)
+            for (i, row), v, t in zip(watched, values.tolist(), top_ids.tolist()):
+                row.top.append((v[:row.group.logprobs], t[:row.group.logprobs]))
         toks, scs = self._tok.tolist(), self._score.tolist()
         self.steps += 1
         self.rows_stepped += len(active)

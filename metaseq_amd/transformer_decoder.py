@@ -810,7 +810,8 @@ class TransformerDecoder(nn.Module):
 
     def admit_slot(self, cache: KVCache, slot: int, tokens: torch.Tensor, *, banned=(), stop=(),
                    eos=2, mode=0, tok_out=None, score_out=None, temperature=1.0, topp=0.0,
-                   noise=None, replicas=()):
+                   noise=None, replicas=(), penalties=None, lprobs_out=None, prompt_topk=0,
+                   detail=None):
         """``prefill_slot`` plus what a request needs from its prompt: the log-probability of
         every prompt token given its prefix (returned as a list, 0.0 for the first token) and
         the choice of the first new token from the last position, written to ``tok_out`` /
@@ -821,7 +822,16 @@ class TransformerDecoder(nn.Module):
         the logits (prompt scores included, as the reference's loop does); ``topp`` > 0 with
         ``noise`` (fp32 [1 + len(replicas), V], independent Exp(1) numbers) draws from the
         nucleus.  ``replicas``: further slots that receive a copy of the prompt's keys and values
-        and make their own choice (row r of ``noise``, element r of the outputs)."""
+        and make their own choice (row r of ``noise``, element r of the outputs).
+
+        ``penalties``: dict with ``alphas`` (presence, frequency, presence_src, frequency_src),
+        ``counts`` (int64 [R, V], updated with the chosen tokens) and ``counts_src`` (int64
+        [R, V] prompt-token counts), R = 1 + len(replicas): the reference's repetition penalties
+        on the first choice.  ``lprobs_out`` (fp32 [R, V]) receives the masked, penalised
+        log-probabilities the choice was made from.  ``prompt_topk`` > 0 with a dict ``detail``:
+        ``detail["prompt_top"]`` = (values, ids), CPU tensors [T - 1, k], the k most likely
+        tokens at every prompt position after the first (log-softmax of logits / temperature,
+        what the reference records for the prompt with ``need_logprobs``)."""
         lib = self.prepare_()
         logits = self.prefill_slot(cache, slot, tokens)
         T, V = logits.shape
@@ -833,10 +843,18 @@ class TransformerDecoder(nn.Module):
             check(lib.msa_target_logprob_f16(ptr(logits), logits.stride(0), T - 1, V,
                                              float(temperature), ptr(target), ptr(lp), stream))
             scores[1:] = lp.tolist()
+            if prompt_topk > 0 and detail is not None:
+                dist = torch.empty(T - 1, V, dtype=torch.float32, device=logits.device)
+                check(lib.msa_log_softmax_f16(ptr(logits), 0, logits.stride(0), 1, T - 1, V,
+                                              float(temperature), ptr(dist), 0, V, stream))
+                values, ids = dist.topk(min(int(prompt_topk), V), dim=-1)
+                detail["prompt_top"] = (values.cpu(), ids.cpu())
+                del dist
         for dst in replicas:
             self.copy_slot(cache, slot, dst)
         R = 1 + len(replicas)
-        plain = float(temperature) == 1.0 and not topp > 0 and noise is None
+        plain = (float(temperature) == 1.0 and not topp > 0 and noise is None
+                 and penalties is None and lprobs_out is None)
         banned, stop = list(banned), list(stop)
         ba = (ctypes.c_int32 * max(1, len(banned)))(*banned)
         sa = (ctypes.c_int32 * max(1, len(stop)))(*stop)
@@ -849,10 +867,24 @@ class TransformerDecoder(nn.Module):
                                             sa, len(stop), None, ptr(row_mode), 0, int(eos),
                                             ptr(tok_out), 1, ptr(score_out), 1, None, stream))
         else:
+            pen = penalties or {}
+            alphas = [float(a) for a in pen.get("alphas", (0.0, 0.0, 0.0, 0.0))]
+            for name in ("counts", "counts_src"):
+                t = pen.get(name)
+                if t is not None and (t.shape != (R, V) or t.dtype != torch.long
+                                      or not t.is_contiguous()):
+                    raise AssertionError("%s must be contiguous int64 [%d, %d]" % (name, R, V))
+            if lprobs_out is not None and (lprobs_out.shape != (R, V)
+                                           or lprobs_out.dtype != torch.float32
+                                           or lprobs_out.stride(1) != 1):
+                raise AssertionError("lprobs_out must be fp32 [%d, %d]" % (R, V))
             check(lib.msa_sample_topp_f16(
                 ptr(last), last.stride(0), R, V, float(temperature), None, ba, len(banned), sa,
-                len(stop), None, ptr(row_mode), 0, int(eos), None, float(topp), ptr(noise), None,
-                None, 0.0, 0.0, 0.0, 0.0, None, 0, ptr(tok_out), 1, ptr(score_out), 1, stream))
+                len(stop), None, ptr(row_mode), 0, int(eos), None, float(topp), ptr(noise),
+                ptr(pen.get("counts")), ptr(pen.get("counts_src")), alphas[0], alphas[1],
+                alphas[2], alphas[3], None, ptr(lprobs_out),
+                lprobs_out.stride(0) if lprobs_out is not None else 0, ptr(tok_out), 1,
+                ptr(score_out), 1, stream))
         return scores
 
     def copy_slot(self, cache: KVCache, src: int, dst: int):
@@ -881,7 +913,11 @@ class TransformerDecoder(nn.Module):
         all others), ``temperature`` and ``topp`` (fp32 [slots]; top-p 0 = greedy at that
         temperature) and ``noise`` (fp32 [slots, V] Exp(1) numbers, or None).  The step then
         also stores its logits (``logits_out``, [slots, V] fp16, required) and
-        msa_sample_topp_f16 overwrites the outputs of those rows."""
+        msa_sample_topp_f16 overwrites the outputs of those rows.  Optional entries:
+        ``penalty_rows`` (fp32 [slots, 4]: presence, frequency, presence_src, frequency_src of
+        every row) with ``counts`` / ``counts_src`` (int64 [slots, V]; the former is updated
+        with the chosen tokens), and ``lprobs_out`` (fp32 [slots, V]): the masked, penalised
+        log-probabilities of those rows."""
         lib = self.prepare_()
         stream = _capi.stream_ptr()
         B = cache.batch
@@ -907,11 +943,25 @@ class TransformerDecoder(nn.Module):
             ba = (ctypes.c_int32 * max(1, len(banned)))(*banned)
             sa = (ctypes.c_int32 * max(1, len(stop)))(*stop)
             V = self.cfg.vocab_size
+            lp = sampled.get("lprobs_out")
+            for name, dtype in (("counts", torch.long), ("counts_src", torch.long),
+                                ("lprobs_out", torch.float32)):
+                t = sampled.get(name)
+                if t is not None and (t.shape != (B, V) or t.dtype != dtype
+                                      or not t.is_contiguous()):
+                    raise AssertionError("%s must be contiguous [%d, %d]" % (name, B, V))
+            pr = sampled.get("penalty_rows")
+            if pr is not None and (pr.shape != (B, 4) or pr.dtype != torch.float32
+                                   or not pr.is_contiguous()):
+                raise AssertionError("penalty_rows must be contiguous fp32 [%d, 4]" % B)
             check(lib.msa_sample_topp_f16(
                 ptr(logits_out), logits_out.stride(0), B, V, 1.0, ptr(sampled["temperature"]), ba,
                 len(banned), sa, len(stop), ptr(finished), ptr(sampled["row_mode"]), 0, int(eos),
-                ptr(sampled["topp"]), 0.0, ptr(sampled.get("noise")), None, None, 0.0, 0.0, 0.0,
-                0.0, None, 0, ptr(tok_out), 1, ptr(score_out), 1, stream))
+                ptr(sampled["topp"]), 0.0, ptr(sampled.get("noise")),
+                ptr(sampled.get("counts")) if pr is not None else None,
+                ptr(sampled.get("counts_src")) if pr is not None else None, 0.0, 0.0, 0.0, 0.0,
+                ptr(pr), ptr(lp), V if lp is not None else 0, ptr(tok_out), 1, ptr(score_out), 1,
+                stream))
 
     def extract_features(self, prev_output_tokens, incremental_state=None,
                          token_embeddings=None, self_attn_padding_mask=None):

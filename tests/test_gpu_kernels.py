@@ -1036,7 +1036,8 @@ def test_stream_read_probe_runs_and_validates(lib):
 # ---- nucleus sampling kernel ------------------------------------------------------------------
 def _sample(lib, logits, *, temperature=1.0, banned=(1,), stop=(), finished=None, row_mode=None,
             force=0, eos=2, topp_rows=None, topp_all=0.0, noise=None, counts=None,
-            counts_src=None, alphas=(0.0, 0.0, 0.0, 0.0), temperature_rows=None, lprobs=None):
+            counts_src=None, alphas=(0.0, 0.0, 0.0, 0.0), temperature_rows=None, lprobs=None,
+            penalty_rows=None):
     B, V = logits.shape
     ba = (ctypes.c_int32 * max(1, len(banned)))(*banned)
     sa = (ctypes.c_int32 * max(1, len(stop)))(*stop)
@@ -1045,7 +1046,8 @@ def _sample(lib, logits, *, temperature=1.0, banned=(1,), stop=(), finished=None
     ok(lib.msa_sample_topp_f16(P(logits), logits.stride(0), B, V, temperature, P(temperature_rows),
                                ba, len(banned), sa, len(stop), P(finished), P(row_mode), force,
                                eos, P(topp_rows), topp_all, P(noise), P(counts), P(counts_src),
-                               alphas[0], alphas[1], alphas[2], alphas[3], P(lprobs),
+                               alphas[0], alphas[1], alphas[2], alphas[3], P(penalty_rows),
+                               P(lprobs),
                                0 if lprobs is None else lprobs.stride(0), P(tok), 1, P(sc), 1,
                                None), lib)
     torch.cuda.synchronize()
@@ -1133,7 +1135,7 @@ def test_sampling_kernel_per_row_temperature_and_skipped_rows(lib):
     sc = torch.full((B,), 5.0, dtype=torch.float32, device=DEV)
     ok(lib.msa_sample_topp_f16(P(ld), V, B, V, 1.0, P(G(temps)), ba, 1, sa, 1, None, P(G(modes)),
                                0, 2, P(G(topp)), 0.0, P(nd), None, None, 0.0, 0.0, 0.0, 0.0, None,
-                               0, P(tok), 1, P(sc), 1, None), lib)
+                               None, 0, P(tok), 1, P(sc), 1, None), lib)
     torch.cuda.synchronize()
     assert int(tok[2]) == -7 and float(sc[2]) == 5.0
     for r in (0, 1, 3, 4, 5):
@@ -1210,6 +1212,26 @@ def test_nucleus_sampling_kernel_closed_forms(lib):
     assert int(tok[0]) == int(lp.argmax()) == b2 and bool((tok == b2).all())
     assert abs(float(sc[0]) - float(lp[b2])) < 2e-5
     assert int(cd[0, b2]) == 1
+    # the same weights given per row (and none for the odd rows, which keep the best id), with
+    # scalar arguments that must be ignored
+    cd = G(counts.clone())
+    rows = torch.zeros(N, 4)
+    rows[0::2] = torch.tensor([0.3, 0.2, 0.0, 0.0])
+    tok, sc = _sample(lib, G(logits), banned=[], counts=cd, alphas=(9.0, 9.0, 9.0, 9.0),
+                      penalty_rows=G(rows))
+    assert bool((tok[0::2] == b2).all()) and bool((tok[1::2] == a).all())
+    assert abs(float(sc[0]) - float(lp[b2])) < 2e-5
+    assert abs(float(sc[1]) - float(torch.log_softmax(logits[1].float(), -1)[a])) < 2e-5
+    # prompt counts with per-row weights: frequency_src 0.5 on a count of 4 and presence_src 0.1
+    cs = torch.zeros(N, V, dtype=torch.long)
+    cs[:, a] = 4
+    rows = torch.zeros(N, 4)
+    rows[0] = torch.tensor([0.0, 0.0, 0.1, 0.5])
+    tok, sc = _sample(lib, G(logits), banned=[], counts_src=G(cs), penalty_rows=G(rows))
+    lp = torch.log_softmax(logits[0].float(), -1)
+    lp[a] -= 4 * 0.5 + 0.1
+    assert int(tok[0]) == int(lp.argmax()) and abs(float(sc[0]) - float(lp.max())) < 2e-5
+    assert bool((tok[1:] == a).all())
     # a NaN logit: token 0 with score -inf, whatever the mode
     bad = logits[:2].clone()
     bad[0, 3] = float("nan")

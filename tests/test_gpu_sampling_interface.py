@@ -332,3 +332,73 @@ def test_continuous_batcher_sampled_rows_equal_single_request_generation():
             greedy = gi.generate([prompt], max_tokens=[9], min_tokens=[0])[0][0]
             assert greedy["tokens"] != got[0]["tokens"]
     assert cb.cache.lens.tolist() == [-1] * 5
+
+
+def test_continuous_batcher_penalties_decaying_nucleus_and_logprobs_equal_single_requests():
+    """Requests with repetition penalties (generated and prompt tokens, the prompt counts cut at
+    alpha_src_penalty_end_idx), with the factual-nucleus decay, with ``logprobs`` (with and
+    without ``echo``) and plain ones share the slots of one running batch.  Given the same noise
+    per (request, replica, position), each gets the tokens, the scores and the per-position
+    alternatives of a generation of its own through SequenceGenerator's general path."""
+    from metaseq_amd.service import ContinuousBatcher
+    cfg = tiny_cfg(layers=2, dim=128, heads=2, vocab=64, max_pos=48)
+    sd = random_state_dict(cfg, seed=21, dtype=torch.float16)
+    model = TransformerLanguageModel.build_model(cfg, sd, device=DEV)
+    stops = {".": 13, "?": 29, "!": 41}
+    gi = GeneratorInterface(model, Dictionary(cfg.vocab_size, symbols=stops))
+    specs = [dict(prompt=[5, 9, 5, 5, 7], max_tokens=12, alpha_presence=0.8, alpha_frequency=0.6),
+             dict(prompt=[8, 8, 8, 21], max_tokens=14, temperature=0.9, top_p=0.9,
+                  lambda_decay=0.6, omega_bound=0.2),
+             dict(prompt=[40, 41], max_tokens=6, logprobs=3),
+             dict(prompt=[17, 4, 17, 17], max_tokens=9, alpha_presence_src=0.7,
+                  alpha_frequency_src=0.5, alpha_src_penalty_end_idx=3, top_p=0.7, logprobs=2,
+                  echo=True),
+             dict(prompt=[30, 31, 32], max_tokens=7),
+             dict(prompt=[33, 13, 11], max_tokens=12, min_tokens=3, top_p=0.8, lambda_decay=0.5,
+                  alpha_frequency=0.4, n=2, best_of=2, logprobs=1)]
+    cb = ContinuousBatcher(gi, slots=4, capacity=40,
+                           noise_fn=lambda req, j, pos, V: _noise_for(req.prompt, j, pos, V))
+    replies = [cb.submit(s["prompt"], **{k: v for k, v in s.items() if k != "prompt"})
+               for s in specs]
+    n = 0
+    while cb.step():
+        n += 1
+        assert n < 300
+    assert cb.rows_stepped > cb.steps > 0
+    extras = ("lambda_decay", "omega_bound", "alpha_presence", "alpha_frequency",
+              "alpha_presence_src", "alpha_frequency_src", "alpha_src_penalty_end_idx", "logprobs")
+    for s, r in zip(specs, replies):
+        _, got = r.get_nowait()
+        assert not isinstance(got, Exception), (s, got)
+        prompt = s["prompt"]
+        gi.noise_fn = lambda step, BB, V: torch.stack(
+            [_noise_for(prompt, j, step, V) for j in range(BB)])
+        want = gi.generate([prompt], max_tokens=[s["max_tokens"]],
+                           min_tokens=[s.get("min_tokens", 0)], echo=s.get("echo", False),
+                           temperature=s.get("temperature", 1.0), top_p=s.get("top_p", -1.0),
+                           n=s.get("n", 1), best_of=s.get("best_of"),
+                           **{k: s[k] for k in extras if k in s})[0]
+        gi.noise_fn = None
+        assert len(got) == len(want) == s.get("n", 1)
+        for g_rec, w_rec in zip(got, want):
+            assert g_rec["tokens"] == w_rec["tokens"], (s, g_rec["tokens"], w_rec["tokens"])
+            assert g_rec["token_scores"] == w_rec["token_scores"], s
+            if not s.get("logprobs"):
+                assert g_rec["top_logprobs"] is None and w_rec["top_logprobs"] is None
+                continue
+            assert len(g_rec["top_logprobs"]) == len(w_rec["top_logprobs"])
+            for pos, (g_top, w_top) in enumerate(zip(g_rec["top_logprobs"], w_rec["top_logprobs"])):
+                if w_top is None:
+                    assert g_top is None
+                    continue
+                # the same values; the same ids wherever a value is not tied with the next one
+                # (the two sides rank ties by different routines)
+                gv, wv = sorted(g_top.values()), sorted(w_top.values())
+                assert gv == wv, (s, pos, g_top, w_top)
+                if len(set(wv)) == len(wv) and len(w_top) == s["logprobs"]:
+                    assert g_top == w_top, (s, pos, g_top, w_top)
+        if s is specs[0]:
+            # the penalties acted: the continuation is not the request's unpenalised one
+            base = gi.generate([prompt], max_tokens=[12], min_tokens=[0])[0][0]
+            assert base["tokens"] != got[0]["tokens"]
+    assert cb.cache.lens.tolist() == [-1] * 4

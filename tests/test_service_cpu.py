@@ -128,19 +128,36 @@ def _rule(last, length):
     return EOS if t % 9 == 0 else max(t, 4)
 
 
-def _choose(last, length, mode, stop, temperature=1.0, topp=0.0, noise=None):
+def _choose(last, length, mode, stop, temperature=1.0, topp=0.0, noise=None, penalty=0):
     """A row of the scripted model.  Rows that are not plainly greedy shift the rule's token by
-    a function of their temperature and, when they sample, of the largest noise entry: what
-    matters to these tests is that every parameter reaches the row it belongs to."""
+    a function of their temperature, of their nucleus and, when they sample, of the largest
+    noise entry, and by ``penalty``: what matters to these tests is that every parameter
+    reaches the row it belongs to."""
     t = _rule(last, length)
-    if temperature != 1.0 or topp > 0:
-        shift = int(round(temperature * 10)) + (int(noise.argmax()) if topp > 0 else 0)
+    if temperature != 1.0 or topp > 0 or penalty:
+        shift = int(round(temperature * 10)) + penalty
+        if topp > 0:
+            shift += int(noise.argmax()) + int(round(topp * 100))
         t = max((t + shift) % V, 4)
     if mode & 2:
         return EOS
     if mode & 1 and (t == EOS or t in stop):
         return ALT
     return t
+
+
+def _penalty(alphas, counts, counts_src, last):
+    """The scripted model's use of the penalty state of a row: its four weights, how many
+    tokens it has generated, and how often its last token occurs in the prompt."""
+    if max(alphas) <= 0:
+        return 0
+    return (int(round(sum(a * w for a, w in zip(alphas, (10, 20, 30, 40)))))
+            + int(counts.sum()) + 3 * int(counts_src[last]))
+
+
+def _lprob_row(tok):
+    """The scripted model's log-probabilities of a step that chose ``tok``: no two alike."""
+    return -((torch.arange(V) * 7 + tok) % V).float()
 
 
 class FakeSlotDecoder:
@@ -161,16 +178,31 @@ class FakeSlotDecoder:
         return self.Cache(slots)
 
     def admit_slot(self, cache, slot, tokens, *, banned, stop, eos, mode, tok_out, score_out,
-                   temperature=1.0, topp=0.0, noise=None, replicas=()):
+                   temperature=1.0, topp=0.0, noise=None, replicas=(), penalties=None,
+                   lprobs_out=None, prompt_topk=0, detail=None):
         assert banned == [PAD] and eos == EOS
         ids = tokens.tolist()
         self.prefills.append((slot, ids))
         for r, s in enumerate([slot] + list(replicas)):
             assert cache.lens[s] == -1
             cache.lens[s] = len(ids)
-            tok_out[r] = _choose(ids[-1], len(ids), mode, stop, temperature, topp,
-                                 None if noise is None else noise[r])
+            pen = 0
+            if penalties is not None:
+                assert int(penalties["counts"][r].sum()) == 0
+                pen = _penalty(penalties["alphas"], penalties["counts"][r],
+                               penalties["counts_src"][r], ids[-1])
+            t = _choose(ids[-1], len(ids), mode, stop, temperature, topp,
+                        None if noise is None else noise[r], pen)
+            tok_out[r] = t
             score_out[r] = -0.5 - 0.01 * r
+            if penalties is not None:
+                penalties["counts"][r, t] += 1
+            if lprobs_out is not None:
+                lprobs_out[r] = _lprob_row(t)
+        if prompt_topk:
+            rows = torch.stack([_lprob_row(t) for t in ids[1:]])
+            values, top = rows.topk(prompt_topk, dim=-1)
+            detail["prompt_top"] = (values, top)
         return [0.0] + [-1.0] * (len(ids) - 1)
 
     def decode_slots(self, cache, last_tokens, *, temperature, banned, stop, eos, row_mode,
@@ -189,40 +221,65 @@ class FakeSlotDecoder:
                 if m & 4:
                     continue
                 topp = float(sampled["topp"][i])
-                tok_out[i] = _choose(int(last_tokens[i]), cache.lens[i], m, stop,
-                                     round(float(sampled["temperature"][i]), 4), topp,
-                                     sampled["noise"][i] if topp > 0 else None)
+                pen = 0
+                if sampled.get("penalty_rows") is not None:
+                    pen = _penalty([round(float(a), 4) for a in sampled["penalty_rows"][i]],
+                                   sampled["counts"][i], sampled["counts_src"][i],
+                                   int(last_tokens[i]))
+                t = _choose(int(last_tokens[i]), cache.lens[i], m, stop,
+                            round(float(sampled["temperature"][i]), 4), round(topp, 4),
+                            sampled["noise"][i] if topp > 0 else None, pen)
+                tok_out[i] = t
                 score_out[i] = -0.125 * (i + 1)
+                if sampled.get("penalty_rows") is not None:
+                    sampled["counts"][i, t] += 1
+                if sampled.get("lprobs_out") is not None:
+                    sampled["lprobs_out"][i] = _lprob_row(t)
 
     def release_slot(self, cache, slot):
         cache.lens[slot] = -1
 
 
 def _expected(prompt, min_tokens=0, max_tokens=0, stop=(), capacity=64, temperature=1.0,
-              topp=0.0, noise=None):
+              topp=0.0, noise=None, alphas=(0.0, 0.0, 0.0, 0.0), src_end=-1, decay=-1.0,
+              omega=0.3, full_stop=(), top=None):
     """What one request generates on its own: the loop written out.  ``noise(position)`` gives
-    the row's Exp(1) numbers for the draw of the token at that position."""
+    the row's Exp(1) numbers for the draw of the token at that position; ``top`` (a list)
+    receives the scripted log-probability row of every step."""
     ids = [EOS] + list(prompt)
     room = capacity - len(ids)
     max_new = max(1, min(max_tokens or room, room))
-    out = []
+    counts = torch.zeros(V, dtype=torch.long)
+    counts_src = torch.zeros(V, dtype=torch.long)
+    for t in (ids if src_end <= 0 else ids[:src_end]):
+        counts_src[t] += 1
+    since, out = 0, []
     while True:
         mode = (1 if len(out) < min_tokens else 0) | (2 if len(out) >= max_new - 1 else 0)
-        t = _choose(ids[-1], len(ids), mode, stop, temperature, topp,
-                    noise(len(ids)) if (noise and topp > 0) else None)
+        p = topp
+        if decay > 0 and topp > 0:   # fp32, as the generation loop computes it
+            p = float(torch.clamp(torch.tensor(topp) * torch.tensor(decay) ** max(since - 1, 0),
+                                  min=omega))
+        t = _choose(ids[-1], len(ids), mode, stop, temperature, round(p, 4),
+                    noise(len(ids)) if (noise and topp > 0) else None,
+                    _penalty(alphas, counts, counts_src, ids[-1]))
+        counts[t] += 1
+        since = 0 if t in full_stop else since + 1
+        if top is not None:
+            top.append(_lprob_row(t))
         out.append(t)
         if t == EOS or t in stop or len(out) >= max_new:
             return out
         ids.append(t)
 
 
-def _batcher(slots=3, capacity=64, **kw):
+def _batcher(slots=3, capacity=64, symbols=None, **kw):
     class Model:
         pass
     model = Model()
     model.decoder = FakeSlotDecoder()
     model.max_positions = model.decoder.max_positions
-    gi = GeneratorInterface(model, Dictionary(V), device="cpu")
+    gi = GeneratorInterface(model, Dictionary(V, symbols=symbols), device="cpu")
     return ContinuousBatcher(gi, slots=slots, capacity=capacity, **kw), model.decoder
 
 
@@ -290,8 +347,8 @@ def test_continuous_batcher_echo_stop_lists_and_refusals():
         str(t) for t in _expected([8, 8, 8], max_tokens=5) if t != EOS]
     assert all(len(act) == 1 for act in dec.steps[-8:])   # the two never shared a step
     # what the engine does not serve is answered with an error, not queued
-    for bad in (dict(logprobs=3), dict(alpha_presence=0.5), dict(lambda_decay=0.9), dict(n=3),
-                dict(n=2, best_of=1), dict(temperature=-1)):
+    for bad in (dict(logprobs=V + 1), dict(lambda_decay=0.9, top_p=0.5), dict(n=3),
+                dict(n=2, best_of=1), dict(temperature=-1)):   # no "." in this dictionary
         res = cb.submit([5], **bad).get_nowait()[1]
         assert isinstance(res, ValueError), bad
     assert isinstance(cb.submit([5] * 70).get_nowait()[1], ValueError)    # longer than a slot
@@ -397,3 +454,60 @@ def test_continuous_batcher_serving_thread():
     for n in out:
         want = [str(x) for x in _expected([9] * n, max_tokens=6) if x != EOS]
         assert out[n][0]["tokens"] == want
+
+
+FULL_STOPS = {".": 13, "?": 29, "!": 41}
+
+
+def test_continuous_batcher_penalties_decaying_nucleus_and_alternatives_per_row():
+    """Requests with repetition penalties (own weights, prompt counts cut at
+    alpha_src_penalty_end_idx), with a decaying nucleus, with ``logprobs`` and with none of
+    these share the running batch; slots are reused by requests of another kind.  Every answer
+    equals the request's own loop, and the alternatives reported per position are those of the
+    step that chose the token there."""
+    cb, dec = _batcher(slots=3, symbols=FULL_STOPS, noise_fn=_noise)
+    specs = [
+        dict(prompt=[5, 9, 5, 5], max_tokens=10, alpha_presence=0.5, alpha_frequency=0.2),
+        dict(prompt=[8, 8, 8], max_tokens=12, temperature=0.8, top_p=0.9, lambda_decay=0.7,
+             omega_bound=0.4),
+        dict(prompt=[6] * 5, max_tokens=9, logprobs=3),
+        dict(prompt=[17, 4, 17, 17], max_tokens=8, alpha_presence_src=0.3,
+             alpha_frequency_src=0.1, alpha_src_penalty_end_idx=3, top_p=0.6, logprobs=2,
+             echo=True),
+        dict(prompt=[21, 30], max_tokens=10),
+        dict(prompt=[33, 13, 2 + 9], max_tokens=14, top_p=0.8, lambda_decay=0.5, min_tokens=3,
+             alpha_frequency=0.4),
+    ]
+    replies = [cb.submit(s["prompt"], **{k: v for k, v in s.items() if k != "prompt"})
+               for s in specs]
+    _drain(cb)
+    assert max(len(a) for a in dec.steps) == 3 and len({slot for slot, _ in dec.prefills}) == 3
+    for s, r in zip(specs, replies):
+        res = r.get_nowait()[1]
+        assert not isinstance(res, Exception), (s, res)
+        req = Request(0, s["prompt"], {})
+        top = []
+        want = _expected(
+            s["prompt"], s.get("min_tokens", 0), s["max_tokens"],
+            temperature=s.get("temperature", 1.0), topp=max(s.get("top_p", 0.0), 0.0),
+            noise=lambda pos: _noise(req, 0, pos, V),
+            alphas=tuple(s.get(k, 0.0) for k in ("alpha_presence", "alpha_frequency",
+                                                 "alpha_presence_src", "alpha_frequency_src")),
+            src_end=s.get("alpha_src_penalty_end_idx", -1), decay=s.get("lambda_decay", -1.0),
+            omega=s.get("omega_bound", 0.3), full_stop=tuple(FULL_STOPS.values()), top=top)
+        shown = [t for t in want if t != EOS]
+        lead = [str(t) for t in [EOS] + s["prompt"]] if s.get("echo") else []
+        assert res[0]["tokens"] == lead + [str(t) for t in shown], (s, res[0]["tokens"], want)
+        k = s.get("logprobs", 0)
+        if not k:
+            assert res[0]["top_logprobs"] is None
+            continue
+        rows = top[:len(shown)]
+        if s.get("echo"):   # the prompt's positions: nothing for the leading token
+            assert res[0]["top_logprobs"][0] is None
+            rows = [_lprob_row(t) for t in s["prompt"]] + rows
+        got = res[0]["top_logprobs"][1:] if s.get("echo") else res[0]["top_logprobs"]
+        assert len(got) == len(rows)
+        for g, row in zip(got, rows):
+            values, ids = row.topk(k)
+            assert g == {str(i): v for i, v in zip(ids.tolist(), values.tolist())}
