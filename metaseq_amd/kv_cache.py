@@ -34,6 +34,14 @@ class KVCache:
     def v(self, i):
         return self.layers[i][1]
 
+    def rows_view(self, b0, b1):
+        """Rows b0 .. b1 - 1 as a cache of their own (a decode step taken in row chunks); the
+        same object for the same range, so that work buffers kept on it persist."""
+        views = self.__dict__.setdefault("_row_views", {})
+        if (b0, b1) not in views:
+            views[(b0, b1)] = _RowsView(self, b0, b1)
+        return views[(b0, b1)]
+
     def grow(self, new_capacity):
         """Reallocates every layer to ``new_capacity`` positions, keeping the valid prefix."""
         new_capacity = int(new_capacity)
@@ -48,3 +56,22 @@ class KVCache:
 
     def bytes(self):
         return sum(t.numel() * 2 for t in self.layers)
+
+
+class _RowsView:
+    """Rows b0 .. b1 - 1 of a ``KVCache`` with what a decode step reads of a cache: ``k(i)``,
+    ``v(i)`` (contiguous slices of the parent's current tensors), ``capacity``, ``device``."""
+
+    def __init__(self, cache, b0, b1):
+        self._cache, self._b0, self._b1 = cache, b0, b1
+        self.device = cache.device
+
+    @property
+    def capacity(self):
+        return self._cache.capacity
+
+    def k(self, i):
+        return self._cache.layers[i][0][self._b0:self._b1]
+
+    def v(self, i):
+        return self._cache.layers[i][1][self._b0:self._b1]

@@ -278,6 +278,8 @@ class TransformerDecoder(nn.Module):
     # fp16 matrix (3 bytes moved per weight) and multiplied by the fp16 kernel, which is faster
     # than dequantising every fragment in every workgroup; the values are the same.
     W8_EXPAND_ROWS = 4096
+    # decode steps of int8 weights above 128 rows run in chunks of <= 128 rows up to here
+    W8_CHUNKED_ROWS = 512
 
     def _expanded(self, lib, stream, lin):
         """Pointer to the scratch matrix holding ``lin``'s int8 weights expanded to packed fp16."""
@@ -671,6 +673,33 @@ class TransformerDecoder(nn.Module):
             if incremental_state is not None:
                 incremental_state[self._state_key] = cache
             return features, packed, (B, T), {"inner_states": inner_states}
+        int8 = self.layers[0].fc2.qweight is not None
+        if T == 1 and int8 and M <= self.W8_CHUNKED_ROWS:
+            # int8 weights have no MFMA tile kernel that fills the chip at a few hundred rows
+            # (66B shape, 200 rows: 162 ms per step): the batch runs as chunks of at most 128
+            # rows through the packed path, one sweep over the weights per chunk
+            chunks = (B + PM - 1) // PM
+            size = (B + chunks - 1) // chunks
+            features = torch.empty(B, T, D, dtype=torch.float16, device=dev)
+            x_last, positions = [], []
+            for b0 in range(0, B, size):
+                b1 = min(B, b0 + size)
+                view = cache.rows_view(b0, b1)
+                bufs = self._step_buffers(view, b1 - b0)
+                feat, xl = self._decode_core(
+                    lib, stream, tokens[b0:b1], n, b1 - b0, view,
+                    None if mask is None else mask[b0:b1].contiguous(), bufs, None, S0, False,
+                    token_embeddings=None if token_embeddings is None
+                    else token_embeddings[b0:b1].contiguous())
+                features[b0:b1] = feat.view(b1 - b0, T, D)
+                x_last.append(xl)
+                positions.append(bufs["positions"])
+            cache.length = S0 + T
+            if incremental_state is not None:
+                incremental_state[self._state_key] = cache
+            inner = [{"tok": None, "pos": torch.cat(positions), "emb": None},
+                     torch.cat(x_last, dim=1) if self.return_inner_states else None]
+            return features, False, (B, T), {"inner_states": inner}
         h, inner_states = self._rows_core(lib, stream, tokens, B, n, T, S0, cache, mask,
                                           token_embeddings)
         packed = False

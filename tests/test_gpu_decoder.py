@@ -299,6 +299,50 @@ def test_batch_above_64_rows_generates_like_the_oracle(rows):
     assert int(same.sum()) >= rows - 3  # tiny random models have near-tied logits now and then
 
 
+@pytest.mark.parametrize("rows", [140, 300])
+def test_int8_decode_above_128_rows_runs_in_row_chunks(rows):
+    """int8 weights, more than 128 rows: the step is taken in chunks of at most 128 rows through
+    the packed path.  Logits match the oracle on the dequantised weights, every chunk's rows
+    equal, bit for bit, what the same rows give as a batch of their own from the same keys and
+    values (same kernels, same summation order), and generation agrees with the oracle's."""
+    cfg = tiny_cfg(layers=2, dim=128, heads=2, vocab=96, max_pos=40)
+    model, sd = build(cfg, seed=21, int8=True)
+    src = random_prompts(cfg, rows, 6, seed=9)
+    oracle = make_oracle(cfg, sd, torch.float16)
+    want = greedy_generate(oracle, src, max_len_b=16, min_len=15, return_step_logits=True)
+    hist = want["tokens"][:, 0, :src.shape[1] + 2].to(DEV)
+    n0 = src.shape[1]
+    inc = {}
+    logits = model(src.to(DEV), incremental_state=inc)[0]
+    check_logits(logits, want["step_logits"][0], "prefill, %d rows" % rows)
+    dec = model.decoder
+    step1 = dec.extract_features(hist[:, :n0 + 1], incremental_state=inc)[0]
+    check_logits(dec.output_layer(step1), want["step_logits"][1], "decode step 1, %d rows" % rows)
+    step2 = dec.extract_features(hist[:, :n0 + 2], incremental_state=inc)[0]
+    check_logits(dec.output_layer(step2), want["step_logits"][2], "decode step 2, %d rows" % rows)
+    chunks = (rows + 127) // 128
+    size = (rows + chunks - 1) // chunks
+    for b0 in range(0, rows, size):
+        b1 = min(rows, b0 + size)
+        inc_c = {}
+        model(src[b0:b1].to(DEV), incremental_state=inc_c)
+        # the prompt's keys and values as the whole batch's prefill wrote them (a prefill of
+        # fewer rows may take other tile shapes and differ in the last bit)
+        whole, own = model.decoder.get_cache(inc), model.decoder.get_cache(inc_c)
+        for big, small in zip(whole.layers, own.layers):
+            small[:, :, :, :n0].copy_(big[:, b0:b1, :, :n0])
+        # (the features: the vocabulary projection of 140 rows takes another kernel than that
+        # of 70)
+        alone1 = dec.extract_features(hist[b0:b1, :n0 + 1], incremental_state=inc_c)[0]
+        alone2 = dec.extract_features(hist[b0:b1, :n0 + 2], incremental_state=inc_c)[0]
+        assert torch.equal(step1[b0:b1], alone1) and torch.equal(step2[b0:b1], alone2), (b0, b1)
+    got = run_generate(model, cfg, src, 16, 15)
+    same = (got["tokens"].cpu() == want["tokens"]).all(dim=-1).flatten()
+    print("%d-row int8 generation: %d / %d rows identical" % (rows, int(same.sum()), rows),
+          flush=True)
+    assert int(same.sum()) >= rows - 4
+
+
 @pytest.mark.parametrize("B", [5, 100])
 @pytest.mark.parametrize("int8", [False, True])
 def test_one_call_decode_step_equals_the_step_driven_entry_point_by_entry_point(int8, B):
