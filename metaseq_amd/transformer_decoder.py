@@ -504,7 +504,7 @@ class TransformerDecoder(nn.Module):
 
     def _decode_layer(self, lib, stream, layer, kc, vc, cap, bufs, B, S0, mask, len_dev, tail_ln,
                       tail_out, tail_flags):
-        """One layer of a decode step of at most 64 rows (transformer_decoder_layer.py:233-284).
+        """One layer of a decode step of at most 128 rows (transformer_decoder_layer.py:233-284).
         In: the residual stream ``bufs["x"]`` (row-major) and its LayerNorm ``bufs["h"]``
         (packed).  Out: ``x`` updated in place and, through the tail fused behind fc2,
         ``tail_out = LayerNorm(x; tail_ln)`` - the next layer's input or the decoder's final
@@ -564,7 +564,7 @@ class TransformerDecoder(nn.Module):
     def _forward_features(self, prev_output_tokens, incremental_state, token_embeddings,
                           self_attn_padding_mask, want_packed, native_out=None):
         """Embedding, L pre-LN layers and the final LayerNorm.  Returns (features, packed,
-        extra): features are ``[B, T, D]`` row-major, or - for a decode step of at most 64 rows
+        extra): features are ``[B, T, D]`` row-major, or - for a decode step of at most 128 rows
         when ``want_packed`` - the packed activation buffer the vocabulary projection reads."""
         cfg = self.cfg
         tokens = prev_output_tokens
@@ -710,7 +710,7 @@ class TransformerDecoder(nn.Module):
         return features, packed, (B, T), {"inner_states": inner_states}
 
     def _rows_core(self, lib, stream, tokens, B, n, T, S0, kv, mask, token_embeddings=None):
-        """Prefill (or a decode batch above 64 rows): the last T columns of ``tokens[B, n]``
+        """Prefill (or a decode batch above 128 rows): the last T columns of ``tokens[B, n]``
         through embedding, L layers and the final LayerNorm on row-major activations and the
         tiled MFMA kernels, keys and values written at positions S0 .. S0 + T - 1 of ``kv``
         (anything with ``k(i)``, ``v(i)`` and ``capacity``).  Returns the normalised features

@@ -21,7 +21,7 @@ from tests.fp16util import fp16_stats
 
 
 def pack_rows(x):
-    """[M, K] row-major -> the packed activation layout of include/metaseq_amd.h (M <= 64), on
+    """[M, K] row-major -> the packed activation layout of include/metaseq_amd.h (M <= 128), on
     x's device."""
     M, K = x.shape
     MB = (M + 15) // 16 if M <= 64 else 8   # 65 .. 128 rows: always eight row blocks
@@ -192,7 +192,7 @@ def check_prefill_layer(dec, i, tr, B, T, tag):
 def check_decode_layer(dec, i, trace, j, B, n0, tag):
     """Layer ``i`` of ``dec`` for the decode step that the oracle made as its pass ``j`` >= 1
     (``trace``: the list of that layer's recorded passes; pass 0 is the prefill of n0
-    positions), on the packed <= 64-row path."""
+    positions), on the packed <= 128-row path."""
     lib = dec.prepare_()
     stream = _capi.stream_ptr()
     cfg = dec.cfg
