@@ -423,6 +423,7 @@ class TransformerDecoder(nn.Module):
 
     # most rows of a decode step on packed activations (the library's MSA_PACKED_MAX_ROWS)
     PACKED_MAX_ROWS = 128
+    SLOT_MAX_ROWS = 256     # rows of a slot cache (continuous batching)
 
     @staticmethod
     def _packed_rows(B):
@@ -675,31 +676,13 @@ class TransformerDecoder(nn.Module):
             return features, packed, (B, T), {"inner_states": inner_states}
         int8 = self.layers[0].fc2.qweight is not None
         if T == 1 and int8 and M <= self.W8_CHUNKED_ROWS:
-            # int8 weights have no MFMA tile kernel that fills the chip at a few hundred rows
-            # (66B shape, 200 rows: 162 ms per step): the batch runs as chunks of at most 128
-            # rows through the packed path, one sweep over the weights per chunk
-            chunks = (B + PM - 1) // PM
-            size = (B + chunks - 1) // chunks
-            features = torch.empty(B, T, D, dtype=torch.float16, device=dev)
-            x_last, positions = [], []
-            for b0 in range(0, B, size):
-                b1 = min(B, b0 + size)
-                view = cache.rows_view(b0, b1)
-                bufs = self._step_buffers(view, b1 - b0)
-                feat, xl = self._decode_core(
-                    lib, stream, tokens[b0:b1], n, b1 - b0, view,
-                    None if mask is None else mask[b0:b1].contiguous(), bufs, None, S0, False,
-                    token_embeddings=None if token_embeddings is None
-                    else token_embeddings[b0:b1].contiguous())
-                features[b0:b1] = feat.view(b1 - b0, T, D)
-                x_last.append(xl)
-                positions.append(bufs["positions"])
+            feat, x_last, positions = self._decode_chunks(lib, stream, tokens, n, B, cache, mask,
+                                                          None, S0, token_embeddings)
             cache.length = S0 + T
             if incremental_state is not None:
                 incremental_state[self._state_key] = cache
-            inner = [{"tok": None, "pos": torch.cat(positions), "emb": None},
-                     torch.cat(x_last, dim=1) if self.return_inner_states else None]
-            return features, False, (B, T), {"inner_states": inner}
+            inner = [{"tok": None, "pos": positions, "emb": None}, x_last]
+            return feat.view(B, T, D), False, (B, T), {"inner_states": inner}
         h, inner_states = self._rows_core(lib, stream, tokens, B, n, T, S0, cache, mask,
                                           token_embeddings)
         packed = False
@@ -709,12 +692,16 @@ class TransformerDecoder(nn.Module):
             incremental_state[self._state_key] = cache
         return features, packed, (B, T), {"inner_states": inner_states}
 
-    def _rows_core(self, lib, stream, tokens, B, n, T, S0, kv, mask, token_embeddings=None):
+    def _rows_core(self, lib, stream, tokens, B, n, T, S0, kv, mask, token_embeddings=None,
+                   len_dev=None, step_len=None):
         """Prefill (or a decode batch above 128 rows): the last T columns of ``tokens[B, n]``
         through embedding, L layers and the final LayerNorm on row-major activations and the
         tiled MFMA kernels, keys and values written at positions S0 .. S0 + T - 1 of ``kv``
         (anything with ``k(i)``, ``v(i)`` and ``capacity``).  Returns the normalised features
-        [B * T, D] and the inner-states list."""
+        [B * T, D] and the inner-states list.  With ``len_dev`` (T == 1; int32 [B] device
+        tensor: positions each row already holds, negative = inactive row) every row appends at
+        and attends up to its own length; ``step_len`` (int32 [B]) receives the lengths the
+        step used (-1 for the rows that sat it out)."""
         cfg = self.cfg
         D = cfg.decoder_embed_dim
         dev = tokens.device
@@ -725,16 +712,18 @@ class TransformerDecoder(nn.Module):
         check(lib.msa_embed_f16(ptr(tokens), tokens.stride(0), B, n, T, ptr(table),
                                 cfg.vocab_size, ptr(self.embed_positions.weight),
                                 self.embed_positions.weight.shape[0], self.padding_idx, D,
-                                ptr(x), ptr(positions), None, None, None,
+                                ptr(x), ptr(positions), None, ptr(len_dev), ptr(step_len),
                                 MSA_EMBED_ROWS_GIVEN if token_embeddings is not None else 0,
                                 stream))
+        if step_len is not None:
+            len_dev = step_len
         inner_states = [{"tok": None, "pos": positions, "emb": None}]
         if self.return_inner_states:
             inner_states[0]["emb"] = x.view(B, T, D).transpose(0, 1).clone()
         work = self._rows_buffers(M, dev)
         for i, layer in enumerate(self.layers):
             self._rows_layer(lib, stream, layer, x, work, B, T, S0, kv.k(i), kv.v(i),
-                             kv.capacity, mask)
+                             kv.capacity, mask, len_dev)
             if self.layer_probe is not None:
                 self.layer_probe(i, x)
         if self.return_inner_states:
@@ -745,6 +734,38 @@ class TransformerDecoder(nn.Module):
         self._layernorm(lib, stream, x, self.layer_norm, M, D, h)
         return h, inner_states
 
+    def _decode_chunks(self, lib, stream, tokens, n, B, cache, mask, lens, S0,
+                       token_embeddings=None):
+        """A decode step of more than 128 rows over int8 weights, which have no MFMA tile kernel
+        that fills the chip at a few hundred rows (66B shape, 200 rows: 162 ms per step): the
+        batch runs as chunks of at most 128 rows through the packed path, one sweep over the
+        weights per chunk.  ``lens``: per-row lengths (advanced here), or None.  Returns the
+        features [B, D], the last layer's residual stream (if inner states are kept) and the
+        positions."""
+        PM = self.PACKED_MAX_ROWS
+        D = self.cfg.decoder_embed_dim
+        chunks = (B + PM - 1) // PM
+        size = (B + chunks - 1) // chunks
+        features = torch.empty(B, D, dtype=torch.float16, device=tokens.device)
+        x_last, positions = [], []
+        for b0 in range(0, B, size):
+            b1 = min(B, b0 + size)
+            view = cache.rows_view(b0, b1)
+            bufs = self._step_buffers(view, b1 - b0)
+            rows = None if lens is None else lens[b0:b1]
+            feat, xl = self._decode_core(
+                lib, stream, tokens[b0:b1], n, b1 - b0, view,
+                None if mask is None else mask[b0:b1].contiguous(), bufs, rows, S0, False,
+                token_embeddings=None if token_embeddings is None
+                else token_embeddings[b0:b1].contiguous())
+            if rows is not None:
+                check(lib.msa_advance_len(ptr(rows), ptr(bufs["step_len"]), b1 - b0, 1, stream))
+            features[b0:b1] = feat
+            x_last.append(xl)
+            positions.append(bufs["positions"])
+        return (features, torch.cat(x_last, dim=1) if self.return_inner_states else None,
+                torch.cat(positions))
+
     def _rows_buffers(self, M, dev):
         """Work buffers of ``_rows_layer`` for M row-major activation rows."""
         D, F = self.cfg.decoder_embed_dim, self.cfg.decoder_ffn_embed_dim
@@ -752,7 +773,7 @@ class TransformerDecoder(nn.Module):
         return {"q": torch.empty(M, D, **f16), "h": torch.empty(M, D, **f16),
                 "o": torch.empty(M, D, **f16), "u": torch.empty(M, F, **f16)}
 
-    def _rows_layer(self, lib, stream, layer, x, work, B, T, S0, kc, vc, cap, mask):
+    def _rows_layer(self, lib, stream, layer, x, work, B, T, S0, kc, vc, cap, mask, len_dev=None):
         """One layer over B * T row-major rows (transformer_decoder_layer.py:233-284): ``x`` is
         the residual stream, updated in place; keys and values of the T new positions of every
         row go to positions S0 .. S0 + T - 1 of ``kc`` / ``vc``."""
@@ -763,9 +784,10 @@ class TransformerDecoder(nn.Module):
         q, h, o, u = work["q"], work["h"], work["o"], work["u"]
         mask_stride = mask.stride(0) if mask is not None else 0
         self._layernorm(lib, stream, x, layer.self_attn_layer_norm, M, D, h)
-        self._qkv(lib, stream, h, layer.self_attn.qkv_proj, q, kc, vc, B, T, H, hd, S0, cap, D, 0)
+        self._qkv(lib, stream, h, layer.self_attn.qkv_proj, q, kc, vc, B, T, H, hd, S0, cap, D, 0,
+                  len_dev)
         check(lib.msa_attention_f16(ptr(q), ptr(kc), ptr(vc), ptr(mask), mask_stride, ptr(o), B,
-                                    H, hd, T, S0, cap, 0, None, stream))
+                                    H, hd, T, S0, cap, 0, ptr(len_dev), stream))
         # x = round(round(o Wo^T + bo) + x)   (transformer_decoder_layer.py:222-230)
         ln2 = layer.final_layer_norm
         if not self._linear_split(lib, stream, o, layer.self_attn.out_proj, x, work, M, D, D,
@@ -804,9 +826,9 @@ class TransformerDecoder(nn.Module):
     # decode steps over all slots at once.  No reference counterpart: the reference's service
     # runs every batch to completion (metaseq/cli/interactive_hosted.py:66-175).
     def new_slot_cache(self, slots: int, capacity: int, device=None) -> KVCache:
-        """An empty cache of ``slots`` rows (at most 128) and ``capacity`` positions each."""
-        if not 1 <= slots <= self.PACKED_MAX_ROWS:
-            raise ValueError("a slot cache holds 1..128 rows")
+        """An empty cache of ``slots`` rows (at most 256) and ``capacity`` positions each."""
+        if not 1 <= slots <= self.SLOT_MAX_ROWS:
+            raise ValueError("a slot cache holds 1..%d rows" % self.SLOT_MAX_ROWS)
         cfg = self.cfg
         capacity = int(capacity)
         if not 1 <= capacity <= self.max_positions():
@@ -954,7 +976,24 @@ class TransformerDecoder(nn.Module):
             raise AssertionError("last_tokens must be int64 [%d]" % B)
         if sampled is not None and logits_out is None:
             raise AssertionError("sampled rows need logits_out")
-        if self.native_step and not self.return_inner_states:
+        if B > self.PACKED_MAX_ROWS:
+            # row-major activations through the tile kernels (int8 weights: chunks of <= 128
+            # rows through the packed path), stored logits, stand-alone selection
+            tokens = last_tokens.view(B, 1)
+            if self.layers[0].fc2.qweight is not None:
+                feat, _, _ = self._decode_chunks(lib, stream, tokens, 1, B, cache, None,
+                                                 cache.lens, 0)
+            else:
+                step_len = getattr(cache, "step_len", None)
+                if step_len is None:
+                    step_len = cache.step_len = torch.empty(B, dtype=torch.int32,
+                                                            device=cache.device)
+                feat, _ = self._rows_core(lib, stream, tokens, B, 1, 1, 0, cache, None,
+                                          len_dev=cache.lens, step_len=step_len)
+                check(lib.msa_advance_len(ptr(cache.lens), ptr(step_len), B, 1, stream))
+            self._select_from(lib, feat, B, temperature, banned, stop, finished, row_mode, False,
+                              eos, tok_out, 1, score_out, 1, logits_out, packed=False)
+        elif self.native_step and not self.return_inner_states:
             select = dict(temperature=temperature, banned=banned, stop=stop, finished=finished,
                           row_mode=row_mode, force_eos=False, eos=eos, tok_out=tok_out,
                           tok_stride=1, score_out=score_out, score_stride=1)
@@ -1063,11 +1102,12 @@ class TransformerDecoder(nn.Module):
                           force_eos, eos, tok_out, tok_stride, score_out, score_stride, logits_out)
 
     def _select_from(self, lib, f, B, temperature, banned, stop, finished, row_mode, force_eos,
-                     eos, tok_out, tok_stride, score_out, score_stride, logits_out):
+                     eos, tok_out, tok_stride, score_out, score_stride, logits_out, packed=True):
         """Vocabulary projection of the packed features ``f`` fused with the greedy selection
-        (beyond 64 rows: the projection stores its logits and a second kernel selects)."""
+        (beyond 64 rows, or for row-major features: the projection stores its logits and a
+        second kernel selects)."""
         D, V = self.cfg.decoder_embed_dim, self.cfg.vocab_size
-        if B > 64:
+        if B > 64 or not packed:
             banned, stop = list(banned), list(stop)
             ba = (ctypes.c_int32 * max(1, len(banned)))(*banned)
             sa = (ctypes.c_int32 * max(1, len(stop)))(*stop)
@@ -1075,7 +1115,7 @@ class TransformerDecoder(nn.Module):
                 B, V, dtype=torch.float16, device=f.device)
             stream = _capi.stream_ptr()
             check(lib.msa_linear_f16(ptr(f), ptr(self._lm_head), None, None, ptr(logits), B, V, D,
-                                     MSA_IN_PACKED, stream))
+                                     MSA_IN_PACKED if packed else 0, stream))
             check(lib.msa_greedy_select_f16(
                 ptr(logits), V, B, V, float(temperature), ba, len(banned), sa, len(stop),
                 ptr(finished), ptr(row_mode), int(force_eos), int(eos), ptr(tok_out), tok_stride,

@@ -402,3 +402,60 @@ def test_continuous_batcher_penalties_decaying_nucleus_and_logprobs_equal_single
             base = gi.generate([prompt], max_tokens=[12], min_tokens=[0])[0][0]
             assert base["tokens"] != got[0]["tokens"]
     assert cb.cache.lens.tolist() == [-1] * 4
+
+
+@pytest.mark.parametrize("int8", [False, True])
+def test_continuous_batcher_with_more_than_128_slots(int8):
+    """150 slots: the running batch leaves the packed path (row-major activations through the
+    tile kernels with per-row lengths; int8 weights: chunks of at most 128 rows through the
+    packed path).  Requests of different lengths, some sampled, join and leave; each gets what
+    a generation of its own gives - the logits now come from other kernels than a single
+    request's, so a near-tie may be decided the other way in a few requests, and scores agree
+    to the kernels' tolerance rather than to the bit."""
+    from metaseq_amd.service import ContinuousBatcher
+    cfg = tiny_cfg(layers=2, dim=128, heads=2, vocab=64, max_pos=48)
+    sd = random_state_dict(cfg, seed=21, dtype=torch.float16)
+    model = TransformerLanguageModel.build_model(cfg, sd, device=DEV)
+    if int8:
+        model.decoder.quantize_int8_()
+    gi = GeneratorInterface(model, Dictionary(cfg.vocab_size))
+    g = torch.Generator().manual_seed(5)
+    specs = []
+    for i in range(190):
+        n = int(torch.randint(1, 9, (1,), generator=g))
+        spec = dict(prompt=torch.randint(4, 64, (n,), generator=g).tolist(),
+                    max_tokens=int(torch.randint(6, 20, (1,), generator=g)))
+        if i % 7 == 0:
+            spec.update(temperature=0.8, top_p=0.9)
+        if i % 11 == 0:
+            spec.update(min_tokens=min(3, spec["max_tokens"]))
+        specs.append(spec)
+    cb = ContinuousBatcher(gi, slots=150, capacity=32,
+                           noise_fn=lambda req, j, pos, V: _noise_for(req.prompt, j, pos, V))
+    replies = [cb.submit(s["prompt"], **{k: v for k, v in s.items() if k != "prompt"})
+               for s in specs]
+    n = widest = 0
+    while cb.step():
+        n += 1
+        assert n < 400
+        widest = max(widest, int((cb.cache.lens >= 0).sum()))
+    assert widest > 128      # steps really ran with more rows than the packed path takes
+    same = 0
+    for s, r in zip(specs, replies):
+        _, got = r.get_nowait()
+        assert not isinstance(got, Exception), (s, got)
+        prompt = s["prompt"]
+        gi.noise_fn = lambda step, BB, V: torch.stack(
+            [_noise_for(prompt, j, step, V) for j in range(BB)])
+        want = gi.generate([prompt], max_tokens=[s["max_tokens"]],
+                           min_tokens=[s.get("min_tokens", 0)],
+                           temperature=s.get("temperature", 1.0), top_p=s.get("top_p", -1.0))[0]
+        gi.noise_fn = None
+        if got[0]["tokens"] == want[0]["tokens"]:
+            same += 1
+            assert all(abs(a - b) < 2e-2 for a, b in zip(got[0]["token_scores"],
+                                                         want[0]["token_scores"])), s
+    print("more than 128 slots, int8=%s: %d / %d requests identical to their own generation"
+          % (int8, same, len(specs)), flush=True)
+    assert same >= len(specs) - 6
+    assert cb.cache.lens.tolist() == [-1] * 150
