@@ -10,6 +10,8 @@ slot).  The object lives inside the caller-owned
 ``incremental_state`` dict, as the reference's per-module buffers do
 (metaseq/incremental_decoding_utils.py:30-69), and is freed with it.
 """
+import weakref
+
 import torch
 
 
@@ -63,7 +65,9 @@ class _RowsView:
     ``v(i)`` (contiguous slices of the parent's current tensors), ``capacity``, ``device``."""
 
     def __init__(self, cache, b0, b1):
-        self._cache, self._b0, self._b1 = cache, b0, b1
+        # a weak reference: the cache keeps its views, and must still be freed by its last
+        # outside reference going away, not by a later garbage-collection pass
+        self._cache, self._b0, self._b1 = weakref.proxy(cache), b0, b1
         self.device = cache.device
 
     @property

@@ -278,6 +278,15 @@ class TransformerDecoder(nn.Module):
     # fp16 matrix (3 bytes moved per weight) and multiplied by the fp16 kernel, which is faster
     # than dequantising every fragment in every workgroup; the values are the same.
     W8_EXPAND_ROWS = 4096
+
+    def _expands(self, M, N):
+        """Whether a product of M row-major rows with an int8 [N, K] matrix runs on the matrix
+        expanded to fp16: from 4096 rows on (the expansion is small beside the product), and
+        for the few hundred rows whose 256 x 256 int8 tiles would leave CUs idle, where only
+        the slow 128 x 128 int8 kernel remains."""
+        if M >= self.W8_EXPAND_ROWS:
+            return True
+        return M > self.PACKED_MAX_ROWS and ((M + 255) // 256) * ((N + 255) // 256) < 256
     # decode steps of int8 weights above 128 rows run in chunks of <= 128 rows up to here
     W8_CHUNKED_ROWS = 512
 
@@ -296,7 +305,7 @@ class TransformerDecoder(nn.Module):
         y = out if out is not None else torch.empty(M, N, dtype=torch.float16, device=x.device)
         flags |= MSA_EPI_RELU if relu else 0
         b = lin.bias if bias else None
-        if lin.qweight is not None and M >= self.W8_EXPAND_ROWS:
+        if lin.qweight is not None and self._expands(M, N):
             check(lib.msa_linear_f16(ptr(x), self._expanded(lib, stream, lin), ptr(b),
                                      ptr(residual), ptr(y), M, N, K, flags, stream))
         elif lin.qweight is not None:
@@ -316,7 +325,7 @@ class TransformerDecoder(nn.Module):
                                              MSA_IN_PACKED, stream))
 
     def _qkv(self, lib, stream, h, qkv, q, kc, vc, B, T, H, hd, S0, cap, D, flags, len_dev=None):
-        if qkv.qweight is not None and B * T >= self.W8_EXPAND_ROWS:
+        if qkv.qweight is not None and self._expands(B * T, 3 * D):
             check(lib.msa_qkv_proj_f16(ptr(h), self._expanded(lib, stream, qkv), ptr(qkv.bias),
                                        ptr(q), ptr(kc), ptr(vc), B, T, H, hd, S0, cap, D, flags,
                                        ptr(len_dev), stream))
@@ -805,7 +814,7 @@ class TransformerDecoder(nn.Module):
         new ``x`` goes to ``ln_out`` in the same launch.  False (nothing done) where one pass of
         the tile kernel is as good, or for int8 weights below the row count from which they run
         expanded to fp16."""
-        if lin.qweight is not None and M < self.W8_EXPAND_ROWS:
+        if lin.qweight is not None and not self._expands(M, N):
             return False
         S = lib.msa_linear_default_splits_rows(M, N, K)
         if S <= 1:

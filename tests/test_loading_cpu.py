@@ -38,3 +38,32 @@ def test_unsupported_head_size_is_refused_before_anything_is_allocated():
     assert cfg.head_dim == 80
     with pytest.raises(NotImplementedError, match="head_dim 80"):
         TransformerDecoder(cfg, None, device="meta")
+
+
+def test_kv_cache_row_views_follow_growth_and_keep_nothing_alive():
+    """A view of rows b0 .. b1 - 1 reads the cache's current tensors (also after growth), is
+    the same object for the same range (work buffers kept on it persist), and does not keep
+    the cache alive: dropping the last outside reference frees it at once."""
+    import gc
+    import weakref
+
+    import torch
+
+    from metaseq_amd.kv_cache import KVCache
+    cache = KVCache(2, 6, 2, 8, 16, "cpu")
+    cache.layers[1][1].copy_(torch.arange(6).view(6, 1, 1, 1).expand(6, 2, 16, 8))
+    view = cache.rows_view(2, 5)
+    assert view is cache.rows_view(2, 5) and view is not cache.rows_view(0, 2)
+    assert view.k(0).shape == (3, 2, 16, 8) and view.v(1).is_contiguous()
+    assert view.v(1)[:, 0, 0, 0].tolist() == [2.0, 3.0, 4.0]
+    cache.length = 16
+    cache.grow(40)
+    assert view.capacity == 40 and view.v(1).shape == (3, 2, 40, 8)
+    assert view.v(1)[:, 1, 15, 7].tolist() == [2.0, 3.0, 4.0]
+    gc.disable()
+    try:
+        ref = weakref.ref(cache)
+        del cache, view
+        assert ref() is None
+    finally:
+        gc.enable()
