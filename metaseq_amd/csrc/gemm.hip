@@ -1699,6 +1699,11 @@ int pick_row_splits(int64_t M, int N, int K) {
 template <bool W8, int MODE>
 void launch_tiled(const void* x, const void* W, const void* scales, int64_t M, int N, int K,
                   const Epilogue& epi, hipStream_t s) {
+  // Up to 64 rows (a short prompt, a small batch held row-major): one sweep of the
+  // weight-streaming kernel, which reads its activation fragments from the row-major matrix.
+  // No tile kernel comes near it there (64 x 12288 x 4096, fp16: 101 us on 128 x 128 tiles).
+  if (M <= 64)
+    return launch_stream<W8, MODE, true>(x, W, scales, nullptr, 1, (int)M, N, K, epi, s, 0);
   // the 256 x 256 kernel once it fills the chip; the 128 x 128 one for the shapes in between
   const int64_t big_tiles = ((M + TB_BM - 1) / TB_BM) * ((N + TB_BN - 1) / TB_BN);
   if constexpr (!W8) {
