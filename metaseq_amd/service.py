@@ -370,10 +370,19 @@ class ContinuousBatcher(_Front):
     ``noise_fn(request, replica, position, vocab)`` -> fp32 [vocab] device tensor, if given,
     supplies the Exp(1) numbers of the draw that chooses the token at ``position`` of that
     replica (tests hand both engines the same numbers); otherwise they come from torch's device
-    generator.  A request that has waited ``patience`` steps is served before cheaper ones."""
+    generator.  A request that has waited ``patience`` steps is served before cheaper ones.
+
+    ``prefill_batch`` > 1 lets up to that many waiting requests share one prefill (the weights
+    are read once for all their prompts; a lone prompt's prefill costs about as much as three
+    decode steps of a full batch), and ``prefill_wait`` holds fewer waiting requests back for up
+    to that many steps while rows are decoding, for company.  With the default (1, 0) every
+    request is prefilled alone and its result does not depend on its neighbours to the last
+    bit; a shared prefill runs on other tile shapes, so results can then differ in the last bit
+    of a logit, as they do between batches of the reference's own service."""
 
     def __init__(self, interface, slots: int = 32, capacity: int = MAX_SEQ_LEN,
-                 idle_ms: float = 2.0, noise_fn=None, patience: int = 64):
+                 idle_ms: float = 2.0, noise_fn=None, patience: int = 64,
+                 prefill_batch: int = 1, prefill_wait: int = 0):
         super().__init__(idle_ms / 1000.0)
         import torch
 
@@ -390,6 +399,8 @@ class ContinuousBatcher(_Front):
         self.cache = None  # allocated with the first request
         self._stop: tuple = ()  # stop ids of the running batch
         self.noise_fn, self.patience = noise_fn, int(patience)
+        self.prefill_batch, self.prefill_wait = max(1, int(prefill_batch)), int(prefill_wait)
+        self._held = 0          # steps the waiting requests have been held back for company
         dev = self.device
         self._last = torch.full((slots,), self.dict.pad(), dtype=torch.long, device=dev)
         self._mode = torch.zeros(slots, dtype=torch.uint8, device=dev)
@@ -499,14 +510,12 @@ class ContinuousBatcher(_Front):
         for i, row in rows:
             out[i].copy_(self.noise_fn(row.group.req, row.replica, len(row.tokens), V))
 
-    def _admit(self, slots: List[int], req: Request):
-        """One prefill for the request, its keys and values copied to every replica's slot, and
-        each replica's first token chosen from the prompt's last position."""
+    def _prepare(self, slots: List[int], req: Request, noise_at: int):
+        """What the admission of ``req`` into ``slots`` (its replicas' rows) hands to the
+        decoder: rows, output tensors and the keyword arguments of ``admit_slot``.  The
+        request's draws use rows ``noise_at`` .. of the shared noise buffer."""
         torch = self._torch
         eos, pad = self.dict.eos(), self.dict.pad()
-        if self.cache is None:
-            self.cache = self.decoder.new_slot_cache(len(self.batch.rows), self.batch.capacity,
-                                                     self.device)
         ids = [eos] + req.prompt
         group = _Group(req, self.batch.room_for(req))
         rows = [_Row(group, j, list(ids), []) for j in range(group.replicas)]
@@ -518,7 +527,7 @@ class ContinuousBatcher(_Front):
             self._sampling_state()
             noise = None
             if group.topp > 0:
-                noise = self._noise[:R]
+                noise = self._noise[noise_at:noise_at + R]
                 self._draw_noise(noise, list(enumerate(rows)))
             extra = dict(temperature=group.temperature, topp=group.topp, noise=noise)
             V = len(self.dict)
@@ -542,10 +551,18 @@ class ContinuousBatcher(_Front):
                     extra.update(prompt_topk=group.logprobs, detail=detail)
         if R > 1:
             extra["replicas"] = slots[1:]
-        prompt_scores = self.decoder.admit_slot(
-            self.cache, slots[0], torch.tensor(ids, dtype=torch.long, device=self.device),
-            banned=[pad], stop=self._stop, eos=eos, mode=rows[0].mode(), tok_out=tok,
-            score_out=score, **extra)
+        call = dict(slot=slots[0], tokens=torch.tensor(ids, dtype=torch.long, device=self.device),
+                    banned=[pad], stop=self._stop, eos=eos, mode=rows[0].mode(), tok_out=tok,
+                    score_out=score, **extra)
+        return dict(slots=slots, req=req, group=group, rows=rows, ids=ids, tok=tok, score=score,
+                    extra=extra, detail=detail, lp=lp, call=call)
+
+    def _finish(self, p, prompt_scores):
+        """Book-keeping after the decoder has admitted a prepared request: per-slot sampling
+        state, the alternatives of the first choice and of the prompt, the rows themselves."""
+        torch = self._torch
+        slots, group, rows, tok, extra = p["slots"], p["group"], p["rows"], p["tok"], p["extra"]
+        eos = self.dict.eos()
         if not group.plain:
             idx = torch.tensor(slots, dtype=torch.long, device=self.device)
             self._initp[idx] = group.topp
@@ -560,15 +577,15 @@ class ContinuousBatcher(_Front):
                 self._counts_src[idx] = extra["penalties"]["counts_src"]
         first_top = prompt_top = None
         if group.logprobs > 0:
-            values, top_ids = lp.topk(group.logprobs, dim=-1)
+            values, top_ids = p["lp"].topk(group.logprobs, dim=-1)
             first_top = list(zip(values.tolist(), top_ids.tolist()))
             # nothing is predicted for the leading token; the prompt's alternatives are kept
             # only where they can be shown (echo)
-            prompt_top = [([], [])] * len(ids)
-            if "prompt_top" in detail:
-                values, top_ids = detail["prompt_top"]
+            prompt_top = [([], [])] * len(p["ids"])
+            if "prompt_top" in p["detail"]:
+                values, top_ids = p["detail"]["prompt_top"]
                 prompt_top = [([], [])] + list(zip(values.tolist(), top_ids.tolist()))
-        toks, scs = tok.tolist(), score.tolist()
+        toks, scs = tok.tolist(), p["score"].tolist()
         for j, (slot, row) in enumerate(zip(slots, rows)):
             row.scores = list(prompt_scores)
             if first_top is not None:
@@ -576,6 +593,39 @@ class ContinuousBatcher(_Front):
             self.batch.rows[slot] = row
             if row.take(toks[j], scs[j], eos, self._stop):
                 self._retire(slot)
+
+    def _admit_many(self, items):
+        """Admits ``items`` ((slots, request) pairs): a prefill per request or, with
+        ``prefill_batch`` > 1, one shared prefill for all of them; every request's keys and
+        values are copied to its replicas' slots and each replica's first token is chosen from
+        the prompt's last position.  An error is the answer of every request it concerns."""
+        if self.cache is None:
+            self.cache = self.decoder.new_slot_cache(len(self.batch.rows), self.batch.capacity,
+                                                     self.device)
+        at, prepared = 0, []
+        for slots, req in items:
+            prepared.append(self._prepare(slots, req, at))
+            at += len(slots)
+        n = self.prefill_batch
+        groups = [prepared[i:i + n] for i in range(0, len(prepared), n)]
+        for members in groups:
+            try:
+                if len(members) == 1:
+                    call = dict(members[0]["call"])
+                    scores = [self.decoder.admit_slot(self.cache, call.pop("slot"),
+                                                      call.pop("tokens"), **call)]
+                else:
+                    scores = self.decoder.admit_slots(self.cache, [p["call"] for p in members])
+                for p, sc in zip(members, scores):
+                    self._finish(p, sc)
+            except RuntimeError:
+                raise
+            except Exception as e:  # noqa: BLE001 - these requests' own answer
+                for p in members:
+                    for slot in p["slots"]:
+                        self.batch.rows[slot] = None
+                        self.decoder.release_slot(self.cache, slot)
+                    p["req"].answer(e)
 
     def _retire(self, slot: int):
         row = self.batch.rows[slot]
@@ -622,31 +672,35 @@ class ContinuousBatcher(_Front):
         torch = self._torch
         self._clock += 1
         served = 0
-        while True:
-            free = self.batch.free_slots()
-            if not free:
-                break
+        free = self.batch.free_slots()
+        taken: List[tuple] = []
+        while free:
             req = self._next_request()
             if req is None:
                 break
             need = int(req.options.get("best_of") or req.options.get("n", 1) or 1)
             stop = tuple(sorted(req.options.get("stop") or ()))
-            if (self.batch.active() and stop != self._stop) or need > len(free):
+            if ((self.batch.active() or taken) and stop != self._stop) or need > len(free):
                 self.backlog.put(req, signature="")
                 break
             self._stop = stop
-            self._arrived.pop(req.uid, None)
-            try:
-                self._admit(free[:need], req)
-            except RuntimeError:
-                raise
-            except Exception as e:  # noqa: BLE001 - this request's own answer
-                for slot in free[:need]:
-                    self.batch.rows[slot] = None
-                    if self.cache is not None:
-                        self.decoder.release_slot(self.cache, slot)
-                req.answer(e)
-            served += need
+            taken.append((free[:need], req))
+            free = free[need:]
+        # a shared prefill is worth waiting for: while rows are decoding, fewer admissible
+        # requests than prefill_batch (few free slots, or few waiting) are held back for up to
+        # prefill_wait steps
+        if (taken and len(taken) < self.prefill_batch and self.prefill_wait > 0
+                and self.batch.active() and self._held < self.prefill_wait):
+            self._held += 1
+            for _, req in reversed(taken):
+                self.backlog.put(req, signature="")
+            taken = []
+        if taken:
+            self._held = 0
+            for _, req in taken:
+                self._arrived.pop(req.uid, None)
+            self._admit_many(taken)
+            served += sum(len(slots) for slots, _ in taken)
         active = self.batch.active()
         if not active:
             return served

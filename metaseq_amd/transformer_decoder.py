@@ -868,10 +868,64 @@ class TransformerDecoder(nn.Module):
         cache.lens[slot] = T
         return self._project(h, False, 1, T)[0]
 
+    def prefill_slots(self, cache: KVCache, slots, prompts):
+        """One prefill for several prompts (1-D id tensors on the device, as for
+        ``prefill_slot``) into the rows ``slots`` of ``cache``: the prompts run as one
+        right-padded batch, so the weights are read once for all of them - under the causal
+        mask no real position sees a pad, and the pads' own rows are dropped - and every
+        prompt's keys and values are then copied to its slot.  Returns the logits of every
+        prompt's positions, a list of ``[T_i, V]`` fp16 tensors.  The products run on other
+        tile shapes than a prompt's own prefill would, so results can differ from
+        ``prefill_slot``'s in the last bit."""
+        if len(slots) != len(prompts) or not prompts:
+            raise AssertionError("one slot per prompt")
+        if len(prompts) == 1:
+            return [self.prefill_slot(cache, slots[0], prompts[0])]
+        lib = self.prepare_()
+        cfg = self.cfg
+        lens = [int(t.numel()) for t in prompts]
+        for slot, t, T in zip(slots, prompts, lens):
+            if t.dim() != 1 or T == 0 or not t.is_cuda:
+                raise AssertionError("tokens must be non-empty 1-D device tensors")
+            if T >= cache.capacity:
+                raise ValueError("a prompt of %d tokens leaves no room in a cache of %d "
+                                 "positions" % (T, cache.capacity))
+            if not (cache.ragged and 0 <= slot < cache.batch):
+                raise ValueError("not a slot cache, or slot %d outside 0..%d"
+                                 % (slot, cache.batch - 1))
+        if len(set(slots)) != len(slots):
+            raise ValueError("a slot is named twice")
+        k, Tmax = len(prompts), max(lens)
+        dev = prompts[0].device
+        toks = torch.full((k, Tmax), self.padding_idx, dtype=torch.long, device=dev)
+        for r, t in enumerate(prompts):
+            toks[r, :lens[r]] = t
+        tmp = KVCache(cfg.decoder_layers, k, cfg.decoder_attention_heads, cfg.head_dim, Tmax, dev)
+        h, _ = self._rows_core(lib, _capi.stream_ptr(), toks, k, Tmax, Tmax, 0, tmp, None)
+        # one copy per layer: whole padded rows (what lies past a prompt's length is never read)
+        where = torch.tensor(slots, device=dev)
+        for mine, theirs in zip(cache.layers, tmp.layers):
+            mine[:, :, :, :Tmax].index_copy_(1, where, theirs)
+        cache.lens[where] = torch.tensor(lens, dtype=torch.int32, device=dev)
+        logits = self._project(h, False, k, Tmax)
+        return [logits[r, :lens[r]] for r in range(k)]
+
+    def admit_slots(self, cache: KVCache, requests):
+        """``admit_slot`` for several requests with one shared prefill (``prefill_slots``).
+        ``requests``: dicts with ``slot``, ``tokens`` and the keyword arguments of
+        ``admit_slot``; returns the list of their prompt scores."""
+        logits = self.prefill_slots(cache, [r["slot"] for r in requests],
+                                    [r["tokens"] for r in requests])
+        out = []
+        for r, lg in zip(requests, logits):
+            kw = {k: v for k, v in r.items() if k not in ("slot", "tokens")}
+            out.append(self.admit_slot(cache, r["slot"], r["tokens"], _logits=lg, **kw))
+        return out
+
     def admit_slot(self, cache: KVCache, slot: int, tokens: torch.Tensor, *, banned=(), stop=(),
                    eos=2, mode=0, tok_out=None, score_out=None, temperature=1.0, topp=0.0,
                    noise=None, replicas=(), penalties=None, lprobs_out=None, prompt_topk=0,
-                   detail=None):
+                   detail=None, _logits=None):
         """``prefill_slot`` plus what a request needs from its prompt: the log-probability of
         every prompt token given its prefix (returned as a list, 0.0 for the first token) and
         the choice of the first new token from the last position, written to ``tok_out`` /
@@ -893,7 +947,8 @@ class TransformerDecoder(nn.Module):
         tokens at every prompt position after the first (log-softmax of logits / temperature,
         what the reference records for the prompt with ``need_logprobs``)."""
         lib = self.prepare_()
-        logits = self.prefill_slot(cache, slot, tokens)
+        # (_logits: the prompt was already prefilled into the slot, by prefill_slots)
+        logits = _logits if _logits is not None else self.prefill_slot(cache, slot, tokens)
         T, V = logits.shape
         stream = _capi.stream_ptr()
         scores = [0.0] * T

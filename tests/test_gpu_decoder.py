@@ -453,3 +453,47 @@ def test_given_token_embeddings_replace_the_lookup():
     assert torch.equal(a[valid.to(DEV)], b[valid.to(DEV)])
     with pytest.raises(AssertionError):
         model(toks[:, :10].to(DEV), token_embeddings=emb[:, :4].to(DEV))
+
+
+@pytest.mark.parametrize("int8", [False, True])
+def test_shared_prefill_of_several_prompts_matches_their_own_prefills(int8):
+    """prefill_slots: prompts of different lengths run as one right-padded batch (no real
+    position sees a pad under the causal mask) and land in their slots.  Logits, keys and
+    values agree with each prompt's own prefill to the kernels' tolerance (other tile shapes:
+    not to the bit), the lengths are the prompts' own, other slots stay empty, and a decode
+    step over the slots agrees likewise."""
+    cfg = tiny_cfg(layers=2, dim=128, heads=2, vocab=96, max_pos=40)
+    model, _ = build(cfg, seed=21, int8=int8)
+    dec = model.decoder
+    g = torch.Generator().manual_seed(3)
+    lens, slots = [5, 1, 9, 3], [3, 0, 5, 1]
+    prompts = [torch.cat([torch.tensor([2]), torch.randint(4, 96, (n - 1,), generator=g)]).to(DEV)
+               for n in lens]
+    shared = dec.new_slot_cache(6, 24)
+    got = dec.prefill_slots(shared, slots, prompts)
+    alone = dec.new_slot_cache(6, 24)
+    want = [dec.prefill_slot(alone, s, p) for s, p in zip(slots, prompts)]
+    torch.cuda.synchronize()
+    assert shared.lens.tolist() == alone.lens.tolist() == [1, 3, -1, 5, -1, 9]
+    for g_l, w_l, n in zip(got, want, lens):
+        assert g_l.shape == w_l.shape == (n, 96)
+        check_logits(g_l, w_l, "shared prefill, %d positions" % n)
+    for a, b in zip(shared.layers, alone.layers):
+        for s, n in zip(slots, lens):
+            d = (a[:, s, :, :n].float() - b[:, s, :, :n].float()).abs()
+            assert float(d.max()) < 2e-2
+    last = torch.tensor([7, 30, 1, 41, 1, 52], device=DEV)
+    outs = []
+    for cache in (shared, alone):
+        logits = torch.empty(6, 96, dtype=torch.float16, device=DEV)
+        tok = torch.zeros(6, dtype=torch.long, device=DEV)
+        sc = torch.zeros(6, dtype=torch.float32, device=DEV)
+        dec.decode_slots(cache, last, banned=[1], eos=2, tok_out=tok, score_out=sc,
+                         logits_out=logits)
+        outs.append(logits)
+    torch.cuda.synchronize()
+    rows = torch.tensor(slots, device=DEV)
+    check_logits(outs[0][rows], outs[1][rows], "decode step after a shared prefill")
+    assert shared.lens.tolist() == [2, 4, -1, 6, -1, 10]
+    with pytest.raises(ValueError):
+        dec.prefill_slots(shared, [2, 2], prompts[:2])

@@ -168,7 +168,15 @@ class FakeSlotDecoder:
             self.lens = [-1] * slots
 
     def __init__(self):
-        self.prefills, self.steps = [], []
+        self.prefills, self.steps, self.shared = [], [], []
+
+    def admit_slots(self, cache, requests):
+        self.shared.append(len(requests))
+        out = []
+        for r in requests:
+            kw = {k: v for k, v in r.items() if k not in ("slot", "tokens")}
+            out.append(self.admit_slot(cache, r["slot"], r["tokens"], **kw))
+        return out
 
     def max_positions(self):
         return 64
@@ -511,3 +519,43 @@ def test_continuous_batcher_penalties_decaying_nucleus_and_alternatives_per_row(
         for g, row in zip(got, rows):
             values, ids = row.topk(k)
             assert g == {str(i): v for i, v in zip(ids.tolist(), values.tolist())}
+
+
+def test_continuous_batcher_shares_prefills_and_waits_for_company():
+    """prefill_batch > 1: the requests admitted in one step share one prefill; with
+    prefill_wait a lone admissible request is held back, while rows are decoding, until others
+    can join it or the wait is over.  Every answer still equals the request's own loop."""
+    cb, dec = _batcher(slots=4, noise_fn=_noise, prefill_batch=3, prefill_wait=2)
+    specs = [dict(prompt=[5, 9, 4], max_tokens=12), dict(prompt=[8], max_tokens=3),
+             dict(prompt=[6] * 10, min_tokens=6, max_tokens=20, temperature=0.7, top_p=0.9),
+             dict(prompt=[17, 4], max_tokens=2), dict(prompt=[21, 30, 12, 9], max_tokens=9),
+             dict(prompt=[33], max_tokens=30, top_p=0.5), dict(prompt=[4, 4, 4, 4], max_tokens=7),
+             dict(prompt=[40, 41], max_tokens=5), dict(prompt=[44], max_tokens=11)]
+    replies = [cb.submit(s["prompt"], **{k: v for k, v in s.items() if k != "prompt"})
+               for s in specs]
+    _drain(cb)
+    for s, r in zip(specs, replies):
+        res = r.get_nowait()[1]
+        assert not isinstance(res, Exception), res
+        req = Request(0, s["prompt"], {})
+        want = _expected(s["prompt"], s.get("min_tokens", 0), s["max_tokens"],
+                         temperature=s.get("temperature", 1.0), topp=max(s.get("top_p", 0.0), 0.0),
+                         noise=lambda pos: _noise(req, 0, pos, V))
+        assert res[0]["tokens"] == [str(t) for t in want if t != EOS], (s, res[0]["tokens"])
+    assert len(dec.prefills) == len(specs)
+    assert dec.shared[0] == 3                       # the first three at once
+    assert sum(dec.shared) + (len(dec.prefills) - sum(dec.shared)) == len(specs)
+    assert len(dec.shared) >= 2 and max(dec.shared) <= 3
+    # a request arriving while rows decode waits at most prefill_wait steps for company
+    cb, dec = _batcher(slots=4, prefill_batch=3, prefill_wait=2)
+    first = cb.submit([6] * 5, max_tokens=30, min_tokens=30)
+    cb.step()
+    late = cb.submit([7, 7], max_tokens=4)
+    cb.step(), cb.step()
+    assert len(dec.prefills) == 1                   # held back twice
+    cb.step()
+    assert len(dec.prefills) == 2                   # then admitted alone
+    _drain(cb)
+    assert not isinstance(first.get_nowait()[1], Exception)
+    assert late.get_nowait()[1][0]["tokens"] == [
+        str(t) for t in _expected([7, 7], max_tokens=4) if t != EOS]
