@@ -151,10 +151,12 @@ int msa_embed_f16(const int64_t* tokens, int64_t tok_stride, int B, int n, int T
  *   t = round(acc); if bias: t = round(t + bias[n]); if RELU: t = max(t,0);
  *   if residual: t = round(t + residual[m,n]);  y[m,n] = t.
  * N % 16 == 0, K % 32 == 0.  With MSA_IN_PACKED (M <= 128) the HBM-bound weight-streaming kernel
- * runs; otherwise (any M, row-major x) an MFMA kernel tiled for the product's size: 256 x 256
- * tiles with weights read straight from the packed layout once they fill the chip (K % 128 == 0;
- * a ragged bottom block of at most 128 rows is streamed instead), 128 x 128 LDS tiles for the
- * shapes in between.  All variants round at the same points.  residual is row-major and may
+ * runs; otherwise (any M, row-major x) a kernel chosen for the product's size: up to 64 rows
+ * (int8 weights: 256) sweeps of the weight-streaming kernel over row-major activations, 64 rows
+ * each; above that MFMA tiles, 256 rows by 256, 128 or 64 features with weights read straight
+ * from the packed layout (K % 64 == 0; a ragged bottom block of at most 128 rows may be
+ * streamed instead), and 128 x 128 LDS tiles for what is left.  All variants round at the same
+ * points.  residual is row-major and may
  * alias a row-major y.  flags: MSA_EPI_RELU | MSA_IN_PACKED | MSA_OUT_PACKED.
  * Replaces LinearWithGradAccumulationAndAsyncCommunication.forward
  * (metaseq/modules/megatron/mpu/layers.py:290-292) as used by out_proj
