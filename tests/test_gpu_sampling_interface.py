@@ -514,3 +514,76 @@ def test_continuous_batcher_with_shared_prefills():
           % (shared, same, len(specs)), flush=True)
     assert same >= len(specs) - 3
     assert cb.cache.lens.tolist() == [-1] * 12
+
+
+def test_continuous_batcher_random_request_mix_equals_single_requests():
+    """Forty requests with options drawn at random from everything the engine serves
+    (temperature, top-p, decaying nucleus, the four penalty weights, logprobs, echo, replicas,
+    minimum / maximum lengths, stop lists) over six slots that are reused many times: whatever
+    a slot's previous occupant left behind, each request gets the tokens and scores of a
+    generation of its own (lone prefills: to the last bit)."""
+    from metaseq_amd.service import ContinuousBatcher
+    cfg = tiny_cfg(layers=2, dim=128, heads=2, vocab=64, max_pos=48)
+    sd = random_state_dict(cfg, seed=33, dtype=torch.float16)
+    model = TransformerLanguageModel.build_model(cfg, sd, device=DEV)
+    gi = GeneratorInterface(model, Dictionary(cfg.vocab_size, symbols={".": 13, "?": 29, "!": 41}))
+    g = torch.Generator().manual_seed(77)
+
+    def coin(p):
+        return float(torch.rand(1, generator=g)) < p
+
+    def pick(values):
+        return values[int(torch.randint(0, len(values), (1,), generator=g))]
+    specs = []
+    for i in range(40):
+        n = int(torch.randint(1, 10, (1,), generator=g))
+        s = dict(prompt=torch.randint(4, 64, (n,), generator=g).tolist(),
+                 max_tokens=int(torch.randint(2, 14, (1,), generator=g)))
+        if coin(0.5):
+            s.update(top_p=pick([0.3, 0.7, 0.95]), temperature=pick([0.7, 1.0, 1.3]))
+            if coin(0.4):
+                s.update(lambda_decay=pick([0.5, 0.8]), omega_bound=pick([0.1, 0.3]))
+        elif coin(0.3):
+            s.update(temperature=pick([0.0, 0.6]))
+        if coin(0.3):
+            s.update(alpha_presence=pick([0.0, 0.6]), alpha_frequency=pick([0.2, 0.5]))
+        if coin(0.2):
+            s.update(alpha_presence_src=0.5, alpha_frequency_src=pick([0.0, 0.3]),
+                     alpha_src_penalty_end_idx=pick([-1, 2]))
+        if coin(0.3):
+            s.update(logprobs=pick([1, 4]), echo=coin(0.5))
+        if coin(0.2):
+            s.update(n=2, best_of=pick([2, 3]))
+        if coin(0.3):
+            s.update(min_tokens=min(3, s["max_tokens"]))
+        if coin(0.15):
+            s.update(stop=[pick([20, 33])])
+        specs.append(s)
+    cb = ContinuousBatcher(gi, slots=6, capacity=30,
+                           noise_fn=lambda req, j, pos, V: _noise_for(req.prompt, j, pos, V))
+    replies = [cb.submit(s["prompt"], **{k: v for k, v in s.items() if k != "prompt"})
+               for s in specs]
+    n = 0
+    while cb.step():
+        n += 1
+        assert n < 1000
+    for s, r in zip(specs, replies):
+        _, got = r.get_nowait()
+        assert not isinstance(got, Exception), (s, got)
+        prompt = s["prompt"]
+        gi.noise_fn = lambda step, BB, V: torch.stack(
+            [_noise_for(prompt, j, step, V) for j in range(BB)])
+        kw = {k: v for k, v in s.items() if k not in ("prompt", "max_tokens", "min_tokens")}
+        want = gi.generate([prompt], max_tokens=[s["max_tokens"]],
+                           min_tokens=[s.get("min_tokens", 0)], **kw)[0]
+        gi.noise_fn = None
+        assert len(got) == len(want)
+        for g_rec, w_rec in zip(got, want):
+            assert g_rec["tokens"] == w_rec["tokens"], (s, g_rec["tokens"], w_rec["tokens"])
+            assert g_rec["token_scores"] == w_rec["token_scores"], s
+            if s.get("logprobs"):
+                for g_top, w_top in zip(g_rec["top_logprobs"], w_rec["top_logprobs"]):
+                    assert (g_top is None) == (w_top is None)
+                    if w_top is not None:
+                        assert sorted(g_top.values()) == sorted(w_top.values()), s
+    assert cb.cache.lens.tolist() == [-1] * 6
