@@ -373,8 +373,8 @@ class ContinuousBatcher(_Front):
     generator.  A request that has waited ``patience`` steps is served before cheaper ones.
 
     ``prefill_batch`` > 1 lets up to that many waiting requests share one prefill (the weights
-    are read once for all their prompts; a lone prompt's prefill costs about as much as three
-    decode steps of a full batch), and ``prefill_wait`` holds fewer waiting requests back for up
+    are read once for all their prompts; a lone short prompt's prefill costs a third to a half
+    of a full batch's decode step), and ``prefill_wait`` holds fewer waiting requests back for up
     to that many steps while rows are decoding, for company.  With the default (1, 0) every
     request is prefilled alone and its result does not depend on its neighbours to the last
     bit; a shared prefill runs on other tile shapes, so results can then differ in the last bit
