@@ -318,6 +318,63 @@ def torch_eager_steps(cfg, sd, B, S_first, K, warmup, dev):
                     "%d..%d positions" % (K, S_first, S_first + K - 1)}
 
 
+def service_throughput(config, slots, prefill_batch, prefill_wait, seed=1):
+    """A request-level run beside the headline: ``ContinuousBatcher`` with ``slots`` rows over
+    the configuration's model shape (random weights), three requests per slot with prompts of
+    16-95 random ids and 32-127 new tokens, every other one sampled (temperature 0.8, top-p
+    0.9).  Times everything from the first admission to the last answer, host work included."""
+    import torch
+
+    from metaseq_amd import (Dictionary, GeneratorInterface, TransformerLanguageModel, opt_config,
+                             random_state_dict)
+    from metaseq_amd.service import ContinuousBatcher
+    size = CONFIGS[config][0]
+    int8 = config.endswith("int8")
+    cfg = opt_config(size, max_target_positions=2048)
+    dev = torch.device("cuda:0")
+    sd = random_state_dict(cfg, seed=1234, dtype=torch.float16, device=dev)
+    model = TransformerLanguageModel.build_model(cfg, sd, device=dev)
+    del sd
+    if int8:
+        model.decoder.quantize_int8_()
+    torch.cuda.empty_cache()
+    engine = ContinuousBatcher(GeneratorInterface(model, Dictionary(cfg.vocab_size)), slots=slots,
+                               capacity=256, prefill_batch=prefill_batch,
+                               prefill_wait=prefill_wait)
+    g = torch.Generator().manual_seed(seed)
+    replies = []
+    for i in range(3 * slots):
+        n = int(torch.randint(16, 96, (1,), generator=g))
+        options = dict(max_tokens=int(torch.randint(32, 128, (1,), generator=g)), min_tokens=32)
+        if i % 2:
+            options.update(temperature=0.8, top_p=0.9)
+        prompt = torch.randint(4, cfg.vocab_size, (n,), generator=g).tolist()
+        replies.append(engine.submit(prompt, **options))
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    while engine.step():
+        pass
+    torch.cuda.synchronize()
+    seconds = time.perf_counter() - t0
+    new = 0
+    for r in replies:
+        result = r.get_nowait()[1]
+        if isinstance(result, Exception):
+            raise result
+        new += len(result[0]["tokens"])
+    return {
+        "metric": "continuous batching, new tokens/s end to end, OPT-%s shape, 1xMI355X" % size,
+        "value": new / seconds, "unit": "tokens/s", "n_gpus": 1, "higher_is_better": True,
+        "dtype": "f16" if not int8 else "int8-weights/f16", "data": "synthetic",
+        "config": {"workload": "%d requests (prompts of 16-95 ids, 32-127 new tokens, half of "
+                               "them sampled) through %d slots" % (3 * slots, slots),
+                   "slots": slots, "prefill_batch": prefill_batch, "prefill_wait": prefill_wait},
+        "seconds": seconds, "new_tokens": new, "decode_steps": engine.steps,
+        "rows_per_step": engine.rows_stepped / max(1, engine.steps),
+        "ms_per_step_overall": seconds / max(1, engine.steps) * 1e3,
+    }
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -355,6 +412,13 @@ def main():
                          "--pmc-calibration runs under rocprofv3 (--pmc FETCH_SIZE, --pmc "
                          "WRITE_SIZE; glob patterns of their counter_collection.csv) and the "
                          "result line one of them printed, instead of the ratio on record")
+    ap.add_argument("--service", type=int, default=0, metavar="SLOTS",
+                    help="instead of the headline run: requests through the continuous "
+                         "batching engine with this many slots, one JSON line of its own")
+    ap.add_argument("--prefill-batch", type=int, default=1,
+                    help="--service: requests that may share one prefill")
+    ap.add_argument("--prefill-wait", type=int, default=0,
+                    help="--service: steps admissible requests may be held back for company")
     ap.add_argument("--torch-eager", action="store_true",
                     help="also time the same decode steps written with stock PyTorch fp16 "
                          "operators on this GPU (reported as torch_eager_same_gpu)")
@@ -372,6 +436,10 @@ def main():
     if not os.path.exists(_capi.LIB_PATH):
         from metaseq_amd.csrc.build import build
         build(force=True)
+    if args.service:
+        print(json.dumps(service_throughput(args.config, args.service, args.prefill_batch,
+                                            args.prefill_wait)))
+        return
 
     size, B, P, G = CONFIGS[args.config]
     B, P = args.batch or B, args.prompt or P
