@@ -790,6 +790,9 @@ class TransformerDecoder(nn.Module):
         D, H, hd, F = (cfg.decoder_embed_dim, cfg.decoder_attention_heads, cfg.head_dim,
                        cfg.decoder_ffn_embed_dim)
         M = B * T
+        if M <= self.PACKED_MAX_ROWS:
+            return self._rows_layer_short(lib, stream, layer, x, work, B, T, S0, kc, vc, cap, mask,
+                                          len_dev)
         q, h, o, u = work["q"], work["h"], work["o"], work["u"]
         mask_stride = mask.stride(0) if mask is not None else 0
         self._layernorm(lib, stream, x, layer.self_attn_layer_norm, M, D, h)
@@ -807,7 +810,55 @@ class TransformerDecoder(nn.Module):
         if not self._linear_split(lib, stream, u, layer.fc2, x, work, M, D, F):
             self._linear(lib, stream, u, layer.fc2, M, D, F, residual=x, out=x)
 
-    def _linear_split(self, lib, stream, a, lin, x, work, M, N, K, ln=None, ln_out=None):
+    def _rows_layer_short(self, lib, stream, layer, x, work, B, T, S0, kc, vc, cap, mask,
+                          len_dev=None):
+        """``_rows_layer`` for at most 128 rows (a short prompt): the layer's GEMM inputs are
+        produced in the packed activation layout by the kernels in front of them, so that qkv,
+        fc1 and fc2 run on the weight-streaming kernels of the decode step (56 rows, OPT-6.7B
+        shapes: 25 / 30 / 30 us against 32 / 45 / 52 on row-major rows).  The attention output
+        stays row-major (the prefill attention kernel writes no packed rows), so out_proj runs
+        as in ``_rows_layer``."""
+        cfg = self.cfg
+        D, H, hd, F = (cfg.decoder_embed_dim, cfg.decoder_attention_heads, cfg.head_dim,
+                       cfg.decoder_ffn_embed_dim)
+        M = B * T
+        IN, OUT = MSA_IN_PACKED, MSA_OUT_PACKED
+        q, o = work["q"], work["o"]
+        if "hp" not in work:
+            MP = self._packed_rows(M)
+            work["hp"] = torch.empty(MP * D, dtype=torch.float16, device=x.device)
+            work["up"] = torch.empty(MP * F, dtype=torch.float16, device=x.device)
+            int8 = layer.fc2.qweight is not None
+            splits = lib.msa_linear_default_splits_w8a16 if int8 else lib.msa_linear_default_splits
+            work["S_f"] = splits(M, D, F)
+        hp, up, S_f = work["hp"], work["up"], work["S_f"]
+        mask_stride = mask.stride(0) if mask is not None else 0
+        self._layernorm(lib, stream, x, layer.self_attn_layer_norm, M, D, hp, OUT)
+        self._qkv(lib, stream, hp, layer.self_attn.qkv_proj, q, kc, vc, B, T, H, hd, S0, cap, D, IN,
+                  len_dev)
+        check(lib.msa_attention_f16(ptr(q), ptr(kc), ptr(vc), ptr(mask), mask_stride, ptr(o), B,
+                                    H, hd, T, S0, cap, 0, ptr(len_dev), stream))
+        ln2 = layer.final_layer_norm
+        if not self._linear_split(lib, stream, o, layer.self_attn.out_proj, x, work, M, D, D,
+                                  ln=ln2, ln_out=hp, ln_flags=OUT):
+            self._linear(lib, stream, o, layer.self_attn.out_proj, M, D, D, residual=x, out=x)
+            self._layernorm(lib, stream, x, ln2, M, D, hp, OUT)
+        self._linear(lib, stream, hp, layer.fc1, M, F, D, relu=True, out=up, flags=IN | OUT)
+        part = self._part(work, S_f * M * D, x.device)
+        self._linear_partial(lib, stream, up, layer.fc2, part, M, D, F, S_f)
+        check(lib.msa_residual_layernorm_f16(ptr(part), S_f, ptr(layer.fc2.bias), ptr(x), None,
+                                             None, None, M, D, 1e-5, 0, stream))
+
+    @staticmethod
+    def _part(work, n, dev):
+        """The fp32 partial-sum buffer of a layer's work buffers, at least ``n`` elements."""
+        part = work.get("part")
+        if part is None or part.numel() < n:
+            part = work["part"] = torch.empty(n, dtype=torch.float32, device=dev)
+        return part
+
+    def _linear_split(self, lib, stream, a, lin, x, work, M, N, K, ln=None, ln_out=None,
+                      ln_flags=0):
         """``x = round(round(a W^T + b) + x)`` as split-K partial sums + the fused tail, where M
         row-major rows against N output features leave most of the chip without a tile (a decode
         batch above 128 rows: 64 workgroups for d_model 4096); with ``ln``, the LayerNorm of the
@@ -819,14 +870,12 @@ class TransformerDecoder(nn.Module):
         S = lib.msa_linear_default_splits_rows(M, N, K)
         if S <= 1:
             return False
-        part = work.get("part")
-        if part is None or part.numel() < S * M * N:
-            part = work["part"] = torch.empty(S * M * N, dtype=torch.float32, device=a.device)
+        part = self._part(work, S * M * N, a.device)
         w = self._expanded(lib, stream, lin) if lin.qweight is not None else ptr(lin.weight)
         check(lib.msa_linear_partial_f16(ptr(a), w, ptr(part), M, N, K, S, 0, stream))
         g, b = (ln.weight, ln.bias) if ln is not None else (None, None)
         check(lib.msa_residual_layernorm_f16(ptr(part), S, ptr(lin.bias), ptr(x), ptr(g), ptr(b),
-                                             ptr(ln_out), M, N, 1e-5, 0, stream))
+                                             ptr(ln_out), M, N, 1e-5, ln_flags, stream))
         return True
 
     # ------------------------------------------------------------------ slot interface
