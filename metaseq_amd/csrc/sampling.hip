@@ -292,6 +292,7 @@ __global__ __launch_bounds__(SM_THREADS) void log_softmax_kernel(
 // The draw is an exponential race: arg-max of p / noise over the nucleus, noise ~ Exp(1) per id,
 // which picks id v with probability p[v] / mass(nucleus).
 constexpr int SP_THREADS = 1024;
+constexpr int SP_TIE_BLOCKS = 64;  // rounds of SP_THREADS ids the one-pass tie search covers
 constexpr float SP_FIXED = 281474976710656.f;  // 2^48
 
 struct Penalties {
@@ -300,6 +301,27 @@ struct Penalties {
   float presence, frequency, presence_src, frequency_src;
   const float* rows;  // [B, 4] per-row presence, frequency, presence_src, frequency_src, or NULL
 };
+
+// Adds `mass` to hist[bucket] for the active lanes of a wave: the wave first sums the masses of
+// the lanes that name the same bucket (up to four buckets, lowest lane first), so that one LDS
+// atomic per bucket remains; what four buckets do not cover is added per lane.
+__device__ __forceinline__ void hist_add_wave(unsigned long long* hist, bool active,
+                                              unsigned bucket, unsigned long long mass) {
+  const int lane = threadIdx.x & 63;
+  unsigned long long todo = __ballot(active);
+  for (int trip = 0; todo != 0 && trip < 4; ++trip) {
+    const int leader = __builtin_ctzll(todo);
+    const unsigned lb = (unsigned)__shfl((int)bucket, leader, MSA_WAVE);
+    const bool mine = active && bucket == lb;
+    unsigned long long m = mine ? mass : 0ull;
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) m += __shfl_xor(m, o, MSA_WAVE);
+    if (lane == leader) atomicAdd(&hist[lb], m);
+    active = active && !mine;
+    todo = __ballot(active);
+  }
+  if (active) atomicAdd(&hist[bucket], mass);
+}
 
 __device__ __forceinline__ void argbest(float& v, int& i, float ov, int oi) {
   if (ov > v || (ov == v && oi < i)) {
@@ -326,6 +348,10 @@ __global__ __launch_bounds__(SP_THREADS) void sample_topp_kernel(
   __shared__ unsigned long long hist[256];
   __shared__ unsigned sh_bucket;
   __shared__ unsigned long long sh_above;
+  __shared__ unsigned long long wsum[4];
+  __shared__ int sh_found, sh_limit;
+  __shared__ unsigned tcnt[SP_TIE_BLOCKS];
+  __shared__ unsigned long long tmask[SP_THREADS / 64];
   const int b = blockIdx.x;
   const half_t* row = logits + (int64_t)b * ld;
   const unsigned rm = row_mode ? row_mode[b] : 0u;
@@ -364,6 +390,7 @@ __global__ __launch_bounds__(SP_THREADS) void sample_topp_kernel(
   // raw z for the log-softmax that the greedy branch's score is taken from ----
   bool nan = false;
   float mx = -INFINITY, mx_all = -INFINITY;
+  #pragma unroll 8
   for (int id = threadIdx.x; id < V; id += SP_THREADS) {
     mx = fmaxf(mx, e_of(id, nan));
     float z = (float)row[id];
@@ -376,6 +403,7 @@ __global__ __launch_bounds__(SP_THREADS) void sample_topp_kernel(
   float s = 0.f, s_all = 0.f;
   if (!dead) {
     bool unused = false;
+    #pragma unroll 8
     for (int id = threadIdx.x; id < V; id += SP_THREADS) {
       const float e = e_of(id, unused);
       s += e > -INFINITY ? expf(e - mx) : 0.f;
@@ -408,28 +436,62 @@ __global__ __launch_bounds__(SP_THREADS) void sample_topp_kernel(
       const int shift = 24 - 8 * level;
       if (threadIdx.x < 256) hist[threadIdx.x] = 0;
       __syncthreads();
+      // At level 0 (sign and seven exponent bits) nearly all ids fall into two or three
+      // buckets: a thread first adds up its own ids' masses in a table of four buckets, a wave
+      // then those of its lanes, and one LDS atomic per wave and bucket remains (1024 lanes
+      // adding 64-bit masses to the same few LDS words cost more than everything else here).
+      unsigned tb[4] = {~0u, ~0u, ~0u, ~0u};
+      unsigned long long tm[4] = {0ull, 0ull, 0ull, 0ull};
+      #pragma unroll 8
       for (int id = threadIdx.x; id < V; id += SP_THREADS) {
         const float pv = p_of(id);
         const unsigned u = __float_as_uint(pv);
-        if (pv > 0.f && (level == 0 || (u >> (shift + 8)) == prefix))
-          atomicAdd(&hist[(u >> shift) & 255u], (unsigned long long)(pv * SP_FIXED));
+        if (pv > 0.f && (level == 0 || (u >> (shift + 8)) == prefix)) {
+          const unsigned bucket = (u >> shift) & 255u;
+          const unsigned long long mass = (unsigned long long)(pv * SP_FIXED);
+          bool done = false;
+#pragma unroll
+          for (int j = 0; j < 4; ++j)
+            if (!done && (tb[j] == bucket || tb[j] == ~0u)) {
+              tb[j] = bucket;
+              tm[j] += mass;
+              done = true;
+            }
+          if (!done) atomicAdd(&hist[bucket], mass);
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j) hist_add_wave(hist, tb[j] != ~0u, tb[j], tm[j]);
+      __syncthreads();
+      // the lowest non-empty bucket that still has less than topp above it: thread j < 256
+      // looks at bucket 255 - j, with the mass of the buckets above it in front of it
+      if (threadIdx.x == 0) sh_found = -1;
+      unsigned long long h = 0, before = 0;
+      if (threadIdx.x < 256) {
+        h = hist[255 - threadIdx.x];
+        unsigned long long inc = h;
+#pragma unroll
+        for (int o = 1; o < 64; o <<= 1) {
+          const unsigned long long up = __shfl_up(inc, o, MSA_WAVE);
+          if ((int)(threadIdx.x & 63) >= o) inc += up;
+        }
+        if ((threadIdx.x & 63) == 63) wsum[threadIdx.x >> 6] = inc;
+        before = inc - h;
       }
       __syncthreads();
-      if (threadIdx.x == 0) {
-        // the lowest non-empty bucket that still has less than topp above it
-        unsigned long long cum = above, found_above = above;
-        unsigned found = 255;
-        bool any = false;
-        for (int d = 255; d >= 0; --d) {
-          if (hist[d] != 0 && cum < P) {
-            found = (unsigned)d;
-            found_above = cum;
-            any = true;
-          }
-          cum += hist[d];
-        }
-        sh_bucket = any ? found : 0u;
-        sh_above = any ? found_above : above;
+      if (threadIdx.x < 256) {
+        for (int w = 0; w < (int)(threadIdx.x >> 6); ++w) before += wsum[w];
+        before += above;
+        if (h != 0 && before < P) atomicMax(&sh_found, (int)threadIdx.x);
+      }
+      __syncthreads();
+      if (threadIdx.x < 256 && (int)threadIdx.x == sh_found) {
+        sh_bucket = 255u - threadIdx.x;
+        sh_above = before;
+      }
+      if (threadIdx.x == 0 && sh_found < 0) {
+        sh_bucket = 0u;
+        sh_above = above;
       }
       __syncthreads();
       prefix = (prefix << 8) | sh_bucket;
@@ -444,7 +506,60 @@ __global__ __launch_bounds__(SP_THREADS) void sample_topp_kernel(
     // the i-th tied id (from 0) has above + i * T before it
     long long n_in = n_ties;
     if (Tfx && P != ~0ull && above < P) n_in = min(n_ties, (long long)((P - above + Tfx - 1) / Tfx));
-    if (n_in < n_ties) {  // the smallest id bound below which exactly n_in tied ids lie
+    if (n_in < n_ties && V <= SP_TIE_BLOCKS * SP_THREADS) {
+      // The smallest id bound below which exactly n_in tied ids lie.  Ids in increasing order
+      // are (round k of the loop, wave, lane) in lexicographic order: count the tied ids of
+      // every round, find the round that holds the n_in-th, then its wave and lane.  (fp16
+      // logits make ties at the boundary the rule, not the exception.)
+      if (threadIdx.x < SP_TIE_BLOCKS) tcnt[threadIdx.x] = 0;
+      __syncthreads();
+      for (int id = threadIdx.x, k = 0; id - (int)threadIdx.x < V; id += SP_THREADS, ++k) {
+        const bool tied = id < V && __float_as_uint(p_of(min(id, V - 1))) == tbits;
+        const unsigned long long m = __ballot(tied);
+        if ((threadIdx.x & 63) == 0 && m) atomicAdd(&tcnt[k], (unsigned)__popcll(m));
+      }
+      __syncthreads();
+      if (threadIdx.x == 0) {
+        long long cum = 0;
+        int kk = -1;
+        if (n_in > 0)
+          for (int k = 0; k < SP_TIE_BLOCKS; ++k) {
+            if (cum + tcnt[k] >= n_in) {
+              kk = k;
+              break;
+            }
+            cum += tcnt[k];
+          }
+        sh_found = kk;
+        sh_above = (unsigned long long)(n_in - cum);  // which of that round's tied ids (from 1)
+        sh_limit = 0;                                  // n_in == 0: no tied id is in
+      }
+      __syncthreads();
+      const int kk = sh_found;
+      if (kk >= 0) {
+        const int id = kk * SP_THREADS + (int)threadIdx.x;
+        const bool tied = id < V && __float_as_uint(p_of(min(id, V - 1))) == tbits;
+        const unsigned long long m = __ballot(tied);
+        if ((threadIdx.x & 63) == 0) tmask[threadIdx.x >> 6] = m;
+        __syncthreads();
+        if (threadIdx.x == 0) {
+          long long need = (long long)sh_above;
+          for (int w = 0; w < SP_THREADS / 64; ++w) {
+            unsigned long long mw = tmask[w];
+            const int c = __popcll(mw);
+            if (need > c) {
+              need -= c;
+              continue;
+            }
+            for (; need > 1; --need) mw &= mw - 1;  // drop the lowest set bits
+            sh_limit = kk * SP_THREADS + w * 64 + __builtin_ctzll(mw) + 1;
+            break;
+          }
+        }
+      }
+      __syncthreads();
+      tie_limit = sh_limit;
+    } else if (n_in < n_ties) {  // larger vocabularies: bisection, a pass over the row per step
       int lo = 0, hi = V;
       while (lo < hi) {
         const int mid = lo + ((hi - lo) >> 1);
@@ -492,6 +607,7 @@ __global__ __launch_bounds__(SP_THREADS) void sample_topp_kernel(
   float best = -INFINITY, bestp = 0.f;
   int bidx = 0x7fffffff;
   if (!dead) {
+    #pragma unroll 8
     for (int id = threadIdx.x; id < V; id += SP_THREADS) {
       bool unused = false;
       const float e = e_of(id, unused);

@@ -1198,6 +1198,19 @@ def test_nucleus_sampling_kernel_closed_forms(lib):
     assert set(tok.tolist()) == {0, 1, 2}
     for t in (0, 1, 2):
         assert abs(float((tok == t).float().mean()) - 1 / 3) < 0.03
+    # the same cut among tied ids for ties that lie in different rounds of the kernel's loop
+    # (ids 5, 1100, 2500, 40000 and 51000 tied at the top, top-p 0.5: the first three), and in a
+    # vocabulary beyond 65 536 ids, where the search among tied ids is a bisection
+    for big in (51200, 70000):
+        M = 256
+        wide = torch.full((M, big), -20.0, dtype=torch.float16)
+        tied = [5, 1100, 2500, 40000, big - 200]
+        wide[:, tied] = 3.0
+        nz = torch.empty(M, big).exponential_(generator=torch.Generator().manual_seed(6))
+        tok, sc = _sample(lib, G(wide), banned=[], topp_all=0.5, noise=G(nz))
+        assert set(tok.tolist()) == set(tied[:3]), (big, set(tok.tolist()))
+        want = torch.log_softmax(wide[0].float(), -1)[5]
+        assert torch.allclose(sc, want.expand(M), atol=1e-4)
     # (iii) the whole distribution
     tok, _ = _sample(lib, G(logits), banned=[], topp_all=1.0, noise=G(noise))
     freq = torch.bincount(tok, minlength=V).float() / N
