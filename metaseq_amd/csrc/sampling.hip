@@ -1,6 +1,7 @@
 // Per-row vocabulary reductions of the greedy generation loop: fp32 log-sum-exp over fp16
 // logits, masked arg-max with lowest-index tie-break, and target log-probability gather.
 // One workgroup per logits row; the row (V * 2 bytes) is read twice from cache/HBM.
+#include <atomic>
 #include <math.h>
 
 #include "common.h"
@@ -292,6 +293,7 @@ __global__ __launch_bounds__(SM_THREADS) void log_softmax_kernel(
 // The draw is an exponential race: arg-max of p / noise over the nucleus, noise ~ Exp(1) per id,
 // which picks id v with probability p[v] / mass(nucleus).
 constexpr int SP_THREADS = 1024;
+constexpr int SP_CACHE_IDS = 40000;  // ids whose values stay in LDS between the passes
 constexpr int SP_TIE_BLOCKS = 64;  // rounds of SP_THREADS ids the one-pass tie search covers
 constexpr float SP_FIXED = 281474976710656.f;  // 2^48
 
@@ -337,7 +339,12 @@ __global__ __launch_bounds__(SP_THREADS) void sample_topp_kernel(
     int eos, const float* __restrict__ topp_rows, float topp_all,
     const float* __restrict__ noise, Penalties pen, float* __restrict__ lprobs_out,
     int64_t ld_lprobs, int64_t* __restrict__ tok, int64_t tok_stride,
-    float* __restrict__ score, int64_t score_stride) {
+    float* __restrict__ score, int64_t score_stride, int cap) {
+  // e(id) of the first `cap` ids, kept from the first pass for the six that follow (dynamic
+  // LDS, 4 * cap bytes): an LDS read in place of the load, the exact division by the
+  // temperature, the masks and the penalties.  Every pass walks the ids in the same
+  // thread-to-id mapping, so a thread only ever reads back what it wrote itself.
+  extern __shared__ __attribute__((aligned(16))) float e_cache[];
   if (pen.rows) {  // this row's own penalty weights (rows of a batch from different requests)
     const float* w = pen.rows + 4 * (int64_t)blockIdx.x;
     pen.presence = w[0], pen.frequency = w[1], pen.presence_src = w[2], pen.frequency_src = w[3];
@@ -392,39 +399,47 @@ __global__ __launch_bounds__(SP_THREADS) void sample_topp_kernel(
   float mx = -INFINITY, mx_all = -INFINITY;
   #pragma unroll 8
   for (int id = threadIdx.x; id < V; id += SP_THREADS) {
-    mx = fmaxf(mx, e_of(id, nan));
+    const float e = e_of(id, nan);
+    if (id < cap) e_cache[id] = e;
+    mx = fmaxf(mx, e);
     float z = (float)row[id];
     if (scale) z = z / temperature;
     mx_all = fmaxf(mx_all, z);
   }
+  auto e_at = [&](int id) {
+    bool unused = false;
+    return id < cap ? e_cache[id] : e_of(id, unused);
+  };
   mx = block_max(mx, red);
   mx_all = block_max(mx_all, red);
   const bool dead = block_max(nan ? 1.f : 0.f, red) > 0.f || !(mx > -INFINITY);
+  const bool sampling = noise != nullptr && topp > 0.f && temperature > 0.f && !dead;
+  // the log-softmax over all ids of the raw values: the greedy score and the stored row
+  const bool need_all = lprobs_out != nullptr || !sampling;
   float s = 0.f, s_all = 0.f;
   if (!dead) {
-    bool unused = false;
     #pragma unroll 8
     for (int id = threadIdx.x; id < V; id += SP_THREADS) {
-      const float e = e_of(id, unused);
+      const float e = e_at(id);
       s += e > -INFINITY ? expf(e - mx) : 0.f;
-      float z = (float)row[id];
-      if (scale) z = z / temperature;
-      s_all += expf(z - mx_all);
+      if (need_all) {
+        float z = (float)row[id];
+        if (scale) z = z / temperature;
+        s_all += expf(z - mx_all);
+      }
     }
   }
   s = block_sum(s, red);
   s_all = block_sum(s_all, red);
   const float inv = dead ? 0.f : 1.f / s;
   auto p_of = [&](int id) {
-    bool unused = false;
-    const float e = e_of(id, unused);
+    const float e = e_at(id);
     return e > -INFINITY ? expf(e - mx) * inv : 0.f;
   };
 
   // ---- nucleus: ids in order of decreasing p (ties: increasing id) belong while the mass
   // before them is < topp.  T = the smallest probability whose strictly-greater mass is below
   // topp: everything above T is in, of the ids equal to T those below tie_limit.
-  const bool sampling = noise != nullptr && topp > 0.f && temperature > 0.f && !dead;
   unsigned tbits = 0;
   int tie_limit = V;
   if (sampling) {
@@ -609,8 +624,7 @@ __global__ __launch_bounds__(SP_THREADS) void sample_topp_kernel(
   if (!dead) {
     #pragma unroll 8
     for (int id = threadIdx.x; id < V; id += SP_THREADS) {
-      bool unused = false;
-      const float e = e_of(id, unused);
+      const float e = e_at(id);
       if (!(e > -INFINITY)) continue;
       const float pv = expf(e - mx) * inv;
       float key = e;
@@ -670,6 +684,22 @@ __global__ __launch_bounds__(SP_THREADS) void sample_topp_kernel(
       if (f) finished[b] = 1;
     }
   }
+}
+
+// Raises sample_topp_kernel's dynamic LDS limit, once per device.
+bool allow_cache_lds(int bytes) {
+  static std::atomic<uint64_t> done{0};
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return false;
+  const uint64_t bit = 1ull << dev;
+  if (done.load(std::memory_order_acquire) & bit) return true;
+  if (hipFuncSetAttribute((const void*)sample_topp_kernel,
+                          hipFuncAttributeMaxDynamicSharedMemorySize, bytes) != hipSuccess) {
+    (void)hipGetLastError();
+    return false;
+  }
+  done.fetch_or(bit, std::memory_order_release);
+  return true;
 }
 
 }  // namespace
@@ -769,10 +799,15 @@ extern "C" int msa_sample_topp_f16(const void* logits, int64_t ld_logits, int B,
   pen.presence_src = alpha_presence_src;
   pen.frequency_src = alpha_frequency_src;
   pen.rows = penalty_rows;
-  hipLaunchKernelGGL(sample_topp_kernel, dim3(B), dim3(SP_THREADS), 0, (hipStream_t)stream,
-                     (const half_t*)logits, ld_logits, V, temperature, temperature_rows, banned,
-                     stop, finished, row_mode, force_eos_all, eos_idx, topp_rows, topp_all, noise,
-                     pen, lprobs_out, ld_lprobs, tok, tok_stride, score, score_stride);
+  // as many ids' values as the CU's LDS holds beside the kernel's own 3 KB stay in LDS
+  // between the passes (none if the limit cannot be raised)
+  int cap = min(V, SP_CACHE_IDS);
+  if (cap * 4 > 48 * 1024 && !allow_cache_lds(SP_CACHE_IDS * 4)) cap = 48 * 1024 / 4;
+  hipLaunchKernelGGL(sample_topp_kernel, dim3(B), dim3(SP_THREADS), (size_t)cap * 4,
+                     (hipStream_t)stream, (const half_t*)logits, ld_logits, V, temperature,
+                     temperature_rows, banned, stop, finished, row_mode, force_eos_all, eos_idx,
+                     topp_rows, topp_all, noise, pen, lprobs_out, ld_lprobs, tok, tok_stride,
+                     score, score_stride, cap);
   MSA_CHECK_LAUNCH(name);
   return MSA_OK;
 }
