@@ -291,7 +291,9 @@ int msa_greedy_select_f16(const void* logits, int64_t ld_logits, int B, int V, f
  *   A row whose row_mode has MSA_ROW_SKIP is left alone (no output is written for it): a batch
  *   whose other rows were chosen by another entry point.
  * The nucleus is found without sorting (radix descent over the bit patterns of p with exact
- * fixed-point masses), so the result does not depend on the order of any summation.
+ * fixed-point masses), so the result does not depend on the order of any summation.  The first
+ * call on a device raises the kernel's dynamic LDS limit (it keeps 160 KB of per-id values between
+ * its passes): make one call outside any stream capture.
  * Replaces SequenceGenerator._sample_topp and _apply_repetition_penalties
  * (metaseq/sequence_generator.py:399-441, :478-534), the masking in front of them (:272-293)
  * and the copy of the step's distribution (:301-303); the reference draws with
