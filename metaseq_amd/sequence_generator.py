@@ -25,6 +25,30 @@ from . import _capi
 from ._capi import check, ptr
 
 
+class _FinishWatch:
+    """"Have all rows finished?", asked of the device without making it wait: ``post`` queues
+    the test of the flags as they stand and its copy to pinned host memory; ``all_finished``
+    waits for that copy alone (not for work queued after it) and returns the answer."""
+
+    def __init__(self, finished: torch.Tensor):
+        self.finished = finished
+        self.host = torch.zeros(1, dtype=torch.bool, pin_memory=True)
+        self.event = torch.cuda.Event()
+        self.posted = False
+
+    def post(self):
+        self.host.copy_(self.finished.all().view(1), non_blocking=True)
+        self.event.record()
+        self.posted = True
+
+    def all_finished(self) -> bool:
+        if not self.posted:
+            return False
+        self.event.synchronize()
+        self.posted = False
+        return bool(self.host[0])
+
+
 class SequenceGenerator(nn.Module):
     def __init__(self, models, tgt_dict, beam_size: int = 1, max_len_a: int = 0,
                  max_len_b: int = 200, min_len: int = 1, temperature: float = 1.0,
@@ -235,16 +259,30 @@ class SequenceGenerator(nn.Module):
                 st = self.static_state(decoder, cache, tokens, scores, finished, step_logits)
             fused = (not general and all_lprobs is None and st is None and BB <= 128
                      and hasattr(decoder, "forward_select"))
+            # Whether every row has finished is learnt one step late: the flag of a step is
+            # copied to the host without waiting, the next step is launched, and only then does
+            # the host wait for the flag - with work queued behind it, so the GPU never idles
+            # for the host (a wait per step costs 0.15 ms: 2.5 % of a step at the OPT-6.7B
+            # shape, 11 % at OPT-1.3B's).  If the flag says yes, what the extra step wrote is
+            # wiped.  Rows can only finish once eos / stop tokens are allowed or forced.
+            watch = _FinishWatch(finished)
+
+            def can_end(at):
+                return at >= min_len or at >= max_len - 1
+
+            def wipe(col):
+                tokens[:, col] = self.pad
+                scores[:, col] = 0
+                if all_lprobs is not None:
+                    all_lprobs[:, col] = 0
             if fused:
                 # the first token comes from the prefill logits; every later one is chosen inside
                 # the decode step's vocabulary projection, so logits are never materialised
                 step = start_step
                 self._select(lib, step_logits, step, min_len, max_len, finished, tokens, scores)
-                while True:
-                    if (step >= min_len or step >= max_len - 1) and bool(finished.all()):
-                        break
-                    if step + 1 >= max_len:
-                        break
+                while step + 1 < max_len:
+                    if can_end(step):
+                        watch.post()
                     nxt = step + 1
                     decoder.forward_select(
                         tokens[:, :nxt], incremental_states, temperature=self.temperature,
@@ -252,6 +290,9 @@ class SequenceGenerator(nn.Module):
                         force_eos=nxt >= max_len - 1, eos=self.eos, tok_out=tokens[:, nxt],
                         tok_stride=tokens.stride(0), score_out=scores[:, nxt],
                         score_stride=scores.stride(0))
+                    if can_end(step) and watch.all_finished():
+                        wipe(nxt)
+                        break
                     step = nxt
             for step in range(start_step, max_len if not fused else start_step):
                 if general:
@@ -259,8 +300,13 @@ class SequenceGenerator(nn.Module):
                     self._sample_step(lib, step_logits, step, min_len, max_len, finished, gs,
                                       tokens, scores,
                                       all_lprobs[:, step] if all_lprobs is not None else None)
-                    if bool(finished.all()) or step + 1 >= max_len:
+                    if step > start_step and can_end(step - 1) and watch.all_finished():
+                        wipe(step)  # every row had finished a step ago
                         break
+                    if step + 1 >= max_len:
+                        break
+                    if can_end(step):
+                        watch.post()
                     out = decoder(tokens[:, :step + 1], incremental_state=incremental_states)[0]
                     step_logits = out.view(BB, V)
                     continue

@@ -8,6 +8,7 @@ import torch
 
 from metaseq_amd import (Dictionary, OPTConfig, SequenceGenerator, TransformerLanguageModel,
                          opt_config, random_prompts, random_state_dict)
+from oracle import opt_oracle as O
 from oracle.opt_oracle import greedy_generate
 from tests.common import assert_tokens_match_up_to_ties, make_oracle, tiny_cfg
 from tests.scripted import CASES, ScriptedDecoder
@@ -497,3 +498,33 @@ def test_shared_prefill_of_several_prompts_matches_their_own_prefills(int8):
     assert shared.lens.tolist() == [2, 4, -1, 6, -1, 10]
     with pytest.raises(ValueError):
         dec.prefill_slots(shared, [2, 2], prompts[:2])
+
+
+@pytest.mark.parametrize("kw", [dict(), dict(temperature=0.7), dict(need_logprobs=True),
+                                dict(alpha_presence=0.4, alpha_frequency=0.1)],
+                         ids=["fused greedy", "fused, scaled", "distributions kept",
+                              "general path"])
+def test_generation_that_ends_early_leaves_nothing_behind(kw):
+    """All rows end well before max_len (stop tokens).  The generator learns it one step late -
+    it never makes the GPU wait for the host - and must then return exactly what a loop that
+    stops at once returns: the oracle's tokens and scores, pads and zeros after the last step."""
+    cfg = tiny_cfg(layers=2, dim=128, heads=2, vocab=96, max_pos=48)
+    model, sd = build(cfg, seed=11)
+    src = random_prompts(cfg, 3, 5, seed=2)
+    n0 = src.shape[1]
+    oracle = make_oracle(cfg, sd, torch.float16)
+    okw = {k: v for k, v in kw.items() if k != "need_logprobs"}
+    free = O.generate(oracle, src, max_len_b=40, min_len=30, **okw)
+    # stop ids: what each row writes at its third / fifth / fourth new position
+    stop = sorted({int(free["tokens"][0, 0, n0 + 2]), int(free["tokens"][1, 0, n0 + 4]),
+                   int(free["tokens"][2, 0, n0 + 3])})
+    want = O.generate(oracle, src, max_len_b=40, min_len=1, stop=stop, **kw)
+    got = run_generate(model, cfg, src, 40, 1, stop=stop, **kw)
+    ended = int((want["tokens"][:, 0] != 1).sum(dim=1).max())
+    assert ended < 40 - 2, "the rows did not end early: nothing is tested"
+    assert torch.equal(got["tokens"].cpu(), want["tokens"])
+    assert torch.allclose(got["scores"].cpu(), want["scores"], atol=5e-2)
+    assert bool((got["tokens"][:, 0, ended:] == 1).all())
+    assert float(got["scores"][:, 0, ended:].abs().max()) == 0.0
+    if kw.get("need_logprobs"):
+        assert float(got["distributions"][:, 0, ended:].abs().max()) == 0.0
