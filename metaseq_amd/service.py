@@ -594,6 +594,23 @@ class ContinuousBatcher(_Front):
             if row.take(toks[j], scs[j], eos, self._stop):
                 self._retire(slot)
 
+    def _prefill_groups(self, prepared):
+        """Which prepared requests share a prefill: at most ``prefill_batch`` of them, of
+        similar lengths - a shared prefill pads every prompt to its longest, so a group is
+        closed when the padded rows would exceed the real ones by more than half."""
+        groups, current, real = [], [], 0
+        for p in sorted(prepared, key=lambda p: len(p["ids"])):
+            n = len(p["ids"])
+            if current and (len(current) >= self.prefill_batch
+                            or (len(current) + 1) * n > 1.5 * (real + n)):
+                groups.append(current)
+                current, real = [], 0
+            current.append(p)
+            real += n
+        if current:
+            groups.append(current)
+        return groups
+
     def _admit_many(self, items):
         """Admits ``items`` ((slots, request) pairs): a prefill per request or, with
         ``prefill_batch`` > 1, one shared prefill for all of them; every request's keys and
@@ -606,8 +623,7 @@ class ContinuousBatcher(_Front):
         for slots, req in items:
             prepared.append(self._prepare(slots, req, at))
             at += len(slots)
-        n = self.prefill_batch
-        groups = [prepared[i:i + n] for i in range(0, len(prepared), n)]
+        groups = self._prefill_groups(prepared)
         for members in groups:
             try:
                 if len(members) == 1:

@@ -559,3 +559,17 @@ def test_continuous_batcher_shares_prefills_and_waits_for_company():
     assert not isinstance(first.get_nowait()[1], Exception)
     assert late.get_nowait()[1][0]["tokens"] == [
         str(t) for t in _expected([7, 7], max_tokens=4) if t != EOS]
+
+
+def test_shared_prefills_group_prompts_of_similar_length():
+    """A shared prefill pads every prompt to its longest: groups are closed at prefill_batch
+    members or when padding would exceed half of the real rows."""
+    class Knobs:
+        prefill_batch = 4
+    groups = ContinuousBatcher._prefill_groups(
+        Knobs(), [dict(ids=[0] * n) for n in (5, 6, 7, 100, 8, 120, 110, 9, 300)])
+    assert [[len(p["ids"]) for p in g] for g in groups] == [[5, 6, 7, 8], [9], [100, 110, 120],
+                                                            [300]]
+    Knobs.prefill_batch = 1
+    groups = ContinuousBatcher._prefill_groups(Knobs(), [dict(ids=[0] * n) for n in (3, 3, 3)])
+    assert [len(g) for g in groups] == [1, 1, 1]
