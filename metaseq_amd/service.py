@@ -181,9 +181,15 @@ class _Front:
         return result
 
     def serve_forever(self):
-        while not self._halt.is_set():
-            if self.step() == 0:
-                self._halt.wait(self._idle_wait)
+        try:
+            while not self._halt.is_set():
+                if self.step() == 0:
+                    self._halt.wait(self._idle_wait)
+        finally:
+            self._flush()   # answers an engine may hold back until its next step
+
+    def _flush(self):
+        pass
 
     def stop(self):
         self._halt.set()
@@ -401,6 +407,7 @@ class ContinuousBatcher(_Front):
         self.noise_fn, self.patience = noise_fn, int(patience)
         self.prefill_batch, self.prefill_wait = max(1, int(prefill_batch)), int(prefill_wait)
         self._held = 0          # steps the waiting requests have been held back for company
+        self._done: List[_Group] = []   # ended requests whose records are not built yet
         dev = self.device
         self._last = torch.full((slots,), self.dict.pad(), dtype=torch.long, device=dev)
         self._mode = torch.zeros(slots, dtype=torch.uint8, device=dev)
@@ -651,6 +658,11 @@ class ContinuousBatcher(_Front):
         group.finished[row.replica] = row
         if len(group.finished) < group.replicas:
             return
+        # the records are built (token strings, offsets, alternatives) while the GPU runs the
+        # next decode step, not between two steps
+        self._done.append(group)
+
+    def _answer(self, group: "_Group"):
         req = group.req
         try:
             from .hub_utils import TopRows
@@ -674,6 +686,12 @@ class ContinuousBatcher(_Front):
         except Exception as e:  # noqa: BLE001 - delivered to the caller
             req.answer(e)
 
+    def _flush(self):
+        """Answers the requests whose last replica has ended."""
+        done, self._done = self._done, []
+        for group in done:
+            self._answer(group)
+
     def _next_request(self) -> Optional[Request]:
         """The cheapest waiting request, unless the oldest one has waited ``patience`` steps."""
         old = self.backlog.take_oldest(
@@ -684,7 +702,9 @@ class ContinuousBatcher(_Front):
         """Takes waiting requests into free slots, then runs one decode step over the occupied
         slots.  Returns the number of rows that were served (admitted or stepped).  The rows of
         the running batch share one stop list: a request with another one waits until the batch
-        has drained, and nothing is admitted past it while it waits."""
+        has drained, and nothing is admitted past it while it waits.  A request whose last row
+        ends in this call is answered in the next one, once that call's decode step is queued
+        (at once if no row is left)."""
         torch = self._torch
         self._clock += 1
         served = 0
@@ -719,6 +739,7 @@ class ContinuousBatcher(_Front):
             served += sum(len(slots) for slots, _ in taken)
         active = self.batch.active()
         if not active:
+            self._flush()
             return served
         eos, pad = self.dict.eos(), self.dict.pad()
         slots = len(self.batch.rows)
@@ -752,6 +773,7 @@ class ContinuousBatcher(_Front):
         self.decoder.decode_slots(self.cache, self._last, temperature=1.0, banned=[pad],
                                   stop=self._stop, eos=eos, row_mode=self._mode,
                                   tok_out=self._tok, score_out=self._score, **extra)
+        self._flush()   # the step is queued: the GPU works while the host writes records
         decaying = [i for i, row in general if row.group.decay > 0]
         if decaying:
             self._count_chosen(decaying, self._tok[torch.tensor(decaying, device=self.device)])
