@@ -409,15 +409,38 @@ class ContinuousBatcher(_Front):
         self._held = 0          # steps the waiting requests have been held back for company
         self._done: List[_Group] = []   # ended requests whose records are not built yet
         dev = self.device
-        self._last = torch.full((slots,), self.dict.pad(), dtype=torch.long, device=dev)
-        self._mode = torch.zeros(slots, dtype=torch.uint8, device=dev)
+        # What a step uploads - every slot's last token (int64), temperature (fp32), row mode
+        # and row mode for the sampling kernel (uint8) - lies in one pinned staging buffer and
+        # goes to the device in one copy that nothing waits for (four tensors built from lists
+        # cost four blocking copies, 0.2 ms each, while the GPU sits idle between two steps).
+        n = slots
+        on_gpu = torch.device(dev).type == "cuda"
+        self._stage_host = torch.zeros(14 * n + 8, dtype=torch.uint8, pin_memory=on_gpu)
+        self._stage_dev = torch.zeros(14 * n + 8, dtype=torch.uint8, device=dev)
+        view = lambda buf: (buf[:8 * n].view(torch.long), buf[8 * n:12 * n].view(torch.float32),
+                            buf[12 * n:13 * n], buf[13 * n:14 * n])
+        self._h_last, self._h_temp, self._h_mode, self._h_smode = (
+            t.numpy() for t in view(self._stage_host))
+        self._last, self._temp, self._mode, self._smode = view(self._stage_dev)
         self._tok = torch.zeros(slots, dtype=torch.long, device=dev)
         self._score = torch.zeros(slots, dtype=torch.float32, device=dev)
-        # state of the rows the sampling kernel chooses (allocated with the first such request)
-        self._smode = self._temp = self._topp = self._logits = self._noise = None
-        # [slots, 1] fp32: initial nucleus, decay factor (<= 0: none), floor, tokens since the
-        # last full stop; [slots, 4] penalty weights; [slots, V] token counts and log-prob rows
-        self._initp = self._lam = self._omega = self._since = self._pen = None
+        # Per-slot parameters of the rows the sampling kernel chooses, set at admission in a
+        # pinned mirror and uploaded, if anything changed, with the step's first copy: initial
+        # nucleus, decay factor (<= 0: none), floor ([slots, 3]) and the four penalty weights
+        # ([slots, 4], contiguous: the kernel's penalty_rows).
+        self._par_host = torch.zeros(7 * n, dtype=torch.float32, pin_memory=on_gpu)
+        self._par_dev = torch.zeros(7 * n, dtype=torch.float32, device=dev)
+        self._h_par = self._par_host[:3 * n].view(n, 3).numpy()
+        self._h_pen = self._par_host[3 * n:].view(n, 4).numpy()
+        self._h_par[:, 1] = -1.0
+        par = self._par_dev[:3 * n].view(n, 3)
+        self._initp, self._lam, self._omega = par[:, 0:1], par[:, 1:2], par[:, 2:3]
+        self._pen = self._par_dev[3 * n:].view(n, 4)
+        self._par_dirty = True
+        # state allocated with the first request that needs it: [slots] current nucleus,
+        # [slots, 1] tokens since the last full stop, [slots, V] logits, noise, token counts and
+        # log-probability rows
+        self._topp = self._logits = self._noise = self._since = None
         self._counts = self._counts_src = self._lprobs = None
         self._full_stop = torch.tensor([self.dict.index(w) for w in (".", "?", "!")],
                                        dtype=torch.long, device=dev)
@@ -465,19 +488,13 @@ class ContinuousBatcher(_Front):
     # -- consumer side ------------------------------------------------------------------
     def _sampling_state(self):
         """Per-slot state of the rows chosen by the sampling kernel, on first use."""
-        if self._smode is None:
+        if self._topp is None:
             torch, dev, slots = self._torch, self.device, len(self.batch.rows)
             V = len(self.dict)
-            self._smode = torch.zeros(slots, dtype=torch.uint8, device=dev)
-            self._temp = torch.ones(slots, dtype=torch.float32, device=dev)
             self._topp = torch.zeros(slots, dtype=torch.float32, device=dev)
             self._logits = torch.empty(slots, V, dtype=torch.float16, device=dev)
             self._noise = torch.empty(slots, V, dtype=torch.float32, device=dev)
-            self._initp = torch.zeros(slots, 1, dtype=torch.float32, device=dev)
-            self._lam = torch.full((slots, 1), -1.0, dtype=torch.float32, device=dev)
-            self._omega = torch.zeros(slots, 1, dtype=torch.float32, device=dev)
             self._since = torch.zeros(slots, 1, dtype=torch.float32, device=dev)
-            self._pen = torch.zeros(slots, 4, dtype=torch.float32, device=dev)
 
     def _penalty_state(self):
         if self._counts is None:
@@ -571,13 +588,13 @@ class ContinuousBatcher(_Front):
         slots, group, rows, tok, extra = p["slots"], p["group"], p["rows"], p["tok"], p["extra"]
         eos = self.dict.eos()
         if not group.plain:
-            idx = torch.tensor(slots, dtype=torch.long, device=self.device)
-            self._initp[idx] = group.topp
-            self._lam[idx] = group.decay
-            self._omega[idx] = group.omega
-            self._since[idx] = 0.0
-            self._pen[idx] = torch.tensor(group.alphas, dtype=torch.float32, device=self.device)
+            self._h_par[slots] = (group.topp, group.decay, group.omega)
+            self._h_pen[slots] = group.alphas
+            self._par_dirty = True
+            if group.decay > 0 or group.penalised:
+                idx = torch.tensor(slots, dtype=torch.long, device=self.device)
             if group.decay > 0:
+                self._since[idx] = 0.0
                 self._count_chosen(slots, tok)
             if group.penalised:
                 self._counts[idx] = extra["penalties"]["counts"]
@@ -747,15 +764,20 @@ class ContinuousBatcher(_Front):
         general = [(i, row) for i, row in active if not row.group.plain]
         for i, row in active:
             last[i], mode[i] = row.last, row.mode()
-        self._last.copy_(torch.tensor(last, dtype=torch.long))
-        self._mode.copy_(torch.tensor(mode, dtype=torch.uint8))
-        extra = {}
+        self._h_last[:] = last
+        self._h_mode[:] = mode
         if general:
             smode, temp = [4] * slots, [1.0] * slots  # 4 = MSA_ROW_SKIP
             for i, row in general:
                 smode[i], temp[i] = mode[i], row.group.temperature
-            self._smode.copy_(torch.tensor(smode, dtype=torch.uint8))
-            self._temp.copy_(torch.tensor(temp, dtype=torch.float32))
+            self._h_smode[:] = smode
+            self._h_temp[:] = temp
+        self._stage_dev.copy_(self._stage_host, non_blocking=True)
+        if self._par_dirty:
+            self._par_dev.copy_(self._par_host, non_blocking=True)
+            self._par_dirty = False
+        extra = {}
+        if general:
             self._topp.copy_(self._nucleus_now())
             noise = None
             drawn = [(i, row) for i, row in general if row.group.topp > 0]
