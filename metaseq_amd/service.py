@@ -253,7 +253,7 @@ class _Row:
     """One replica of a request while it occupies a slot."""
 
     __slots__ = ("group", "replica", "tokens", "scores", "n_new", "min_new", "max_new", "last",
-                 "done", "top")
+                 "done", "top", "released")
 
     def __init__(self, group: "_Group", replica: int, tokens: List[int], scores: List[float]):
         req = group.req
@@ -264,18 +264,20 @@ class _Row:
         self.max_new = group.max_new
         self.last = tokens[-1]
         self.done = False
+        self.released = False   # the device has been told to drop the row (its slot is still ours)
         # with ``logprobs``: per position of ``tokens``, the most likely ids and their
         # log-probabilities ((values, ids) lists; empty lists where nothing was predicted)
         self.top: Optional[List[tuple]] = None
 
-    def mode(self) -> int:
-        """Selection regime of this row's next token: end-of-sequence and stop tokens are barred
-        until ``min_tokens`` are out, and the last allowed token can only be end-of-sequence,
-        as in the generation loop (metaseq/sequence_generator.py:272-284)."""
-        m = 0
-        if self.n_new < self.min_new:
+    def mode(self, ahead: int = 0) -> int:
+        """Selection regime of this row's next token (``ahead``: tokens chosen on the device
+        that the host has not seen yet): end-of-sequence and stop tokens are barred until
+        ``min_tokens`` are out, and the last allowed token can only be end-of-sequence, as in
+        the generation loop (metaseq/sequence_generator.py:272-284)."""
+        n, m = self.n_new + ahead, 0
+        if n < self.min_new:
             m |= 1  # MSA_ROW_BAN_EARLY
-        if self.n_new >= self.max_new - 1:
+        if n >= self.max_new - 1:
             m |= 2  # MSA_ROW_ONLY_EOS
         return m
 
@@ -287,6 +289,15 @@ class _Row:
         self.last = token
         self.done = token == eos or token in stop or self.n_new >= self.max_new
         return self.done
+
+
+class _Launched:
+    """A decode step that has been queued: which result buffer it writes, the rows it steps
+    (by slot), and the alternatives of the rows that record them."""
+
+    def __init__(self, buf: int, rows: Dict[int, "_Row"]):
+        self.buf, self.rows = buf, rows
+        self.watched, self.top = None, None
 
 
 class _Group:
@@ -415,15 +426,21 @@ class ContinuousBatcher(_Front):
         # cost four blocking copies, 0.2 ms each, while the GPU sits idle between two steps).
         n = slots
         on_gpu = torch.device(dev).type == "cuda"
-        self._stage_host = torch.zeros(14 * n + 8, dtype=torch.uint8, pin_memory=on_gpu)
-        self._stage_dev = torch.zeros(14 * n + 8, dtype=torch.uint8, device=dev)
+        self._stage_host = torch.zeros(15 * n + 8, dtype=torch.uint8, pin_memory=on_gpu)
+        self._stage_dev = torch.zeros(15 * n + 8, dtype=torch.uint8, device=dev)
         view = lambda buf: (buf[:8 * n].view(torch.long), buf[8 * n:12 * n].view(torch.float32),
-                            buf[12 * n:13 * n], buf[13 * n:14 * n])
-        self._h_last, self._h_temp, self._h_mode, self._h_smode = (
+                            buf[12 * n:13 * n], buf[13 * n:14 * n], buf[14 * n:15 * n])
+        self._h_last, self._h_temp, self._h_mode, self._h_smode, self._h_fed = (
             t.numpy() for t in view(self._stage_host))
-        self._last, self._temp, self._mode, self._smode = view(self._stage_dev)
-        self._tok = torch.zeros(slots, dtype=torch.long, device=dev)
-        self._score = torch.zeros(slots, dtype=torch.float32, device=dev)
+        self._last, self._temp, self._mode, self._smode, self._fed = view(self._stage_dev)
+        # results of a step: two buffers (the step in flight and the one before it), each with
+        # a pinned host copy that is queued right behind the step and waited for by its own event
+        self._tok = torch.zeros(2, slots, dtype=torch.long, device=dev)
+        self._score = torch.zeros(2, slots, dtype=torch.float32, device=dev)
+        self._host_tok = torch.zeros(2, slots, dtype=torch.long, pin_memory=on_gpu)
+        self._host_score = torch.zeros(2, slots, dtype=torch.float32, pin_memory=on_gpu)
+        self._events = [torch.cuda.Event(), torch.cuda.Event()] if on_gpu else None
+        self._inflight: Optional[_Launched] = None
         # Per-slot parameters of the rows the sampling kernel chooses, set at admission in a
         # pinned mirror and uploaded, if anything changed, with the step's first copy: initial
         # nucleus, decay factor (<= 0: none), floor ([slots, 3]) and the four penalty weights
@@ -525,14 +542,16 @@ class ContinuousBatcher(_Front):
         self._since[idx] = torch.where(hit, torch.zeros_like(self._since[idx]),
                                        self._since[idx] + 1)
 
-    def _draw_noise(self, out, rows):
-        """Exp(1) numbers for the draws of ``rows`` ((index into ``out``, row) pairs)."""
+    def _draw_noise(self, out, rows, ahead=None):
+        """Exp(1) numbers for the draws of ``rows`` ((index into ``out``, row) pairs);
+        ``ahead[i]``: tokens of that row the host has not seen yet (its position counts them)."""
         if self.noise_fn is None:
             out.exponential_()
             return
         V = out.shape[1]
         for i, row in rows:
-            out[i].copy_(self.noise_fn(row.group.req, row.replica, len(row.tokens), V))
+            position = len(row.tokens) + (ahead.get(i, 0) if ahead else 0)
+            out[i].copy_(self.noise_fn(row.group.req, row.replica, position, V))
 
     def _prepare(self, slots: List[int], req: Request, noise_at: int):
         """What the admission of ``req`` into ``slots`` (its replicas' rows) hands to the
@@ -717,11 +736,11 @@ class ContinuousBatcher(_Front):
 
     def step(self) -> int:
         """Takes waiting requests into free slots, then runs one decode step over the occupied
-        slots.  Returns the number of rows that were served (admitted or stepped).  The rows of
+        slots.  Returns the number of rows that were served (admitted, stepped or read).  The rows of
         the running batch share one stop list: a request with another one waits until the batch
-        has drained, and nothing is admitted past it while it waits.  A request whose last row
-        ends in this call is answered in the next one, once that call's decode step is queued
-        (at once if no row is left)."""
+        has drained, and nothing is admitted past it while it waits.  The step queued by this
+        call is read by the next one (after that call has queued its own): a request's answer
+        follows the call that chose its last token by one or two calls."""
         torch = self._torch
         self._clock += 1
         served = 0
@@ -754,18 +773,52 @@ class ContinuousBatcher(_Front):
                 self._arrived.pop(req.uid, None)
             self._admit_many(taken)
             served += sum(len(slots) for slots, _ in taken)
-        active = self.batch.active()
-        if not active:
+        # The step launched by the previous call is still running, or its results are still
+        # unread: its rows' tokens are on the device only.  This call launches the next step
+        # first - the rows that step chose tokens for are fed from the device, their modes
+        # follow from the count of their tokens alone - and reads the previous step's results
+        # while the new one runs.  A row whose previous token turns out to have ended it has
+        # then been stepped once more: that output is dropped.  (Reading every step's tokens
+        # before launching the next leaves the GPU idle for all of the host's work between
+        # two steps: a fifth of the time at 128 slots.)
+        before = self._inflight
+        stepping = []
+        for i, row in self.batch.active():
+            ahead = 1 if (before is not None and before.rows.get(i) is row) else 0
+            if row.n_new + ahead >= row.max_new:
+                # its last token is in flight: nothing more to decode; the device may drop it
+                if ahead and not row.released:
+                    self.decoder.release_slot(self.cache, i)
+                    row.released = True
+                continue
+            stepping.append((i, row, ahead))
+        self._inflight = self._launch(stepping, before) if stepping else None
+        self._flush()   # a step is queued: the GPU works while the host writes records
+        if before is not None:
+            self._collect(before)
+            served += len(before.rows)
+        if self._inflight is None:
             self._flush()
-            return served
+        return served + len(stepping)
+
+    def _launch(self, stepping, before):
+        """Queues one decode step for ``stepping`` ((slot, row, tokens in flight) triples) and
+        the copy of its results to pinned host memory; returns what ``_collect`` needs."""
+        torch = self._torch
         eos, pad = self.dict.eos(), self.dict.pad()
         slots = len(self.batch.rows)
-        last, mode = [pad] * slots, [0] * slots
-        general = [(i, row) for i, row in active if not row.group.plain]
-        for i, row in active:
-            last[i], mode[i] = row.last, row.mode()
+        buf = 1 - before.buf if before is not None else 0
+        last, mode, fed = [pad] * slots, [0] * slots, [0] * slots
+        general = [(i, row) for i, row, _ in stepping if not row.group.plain]
+        for i, row, ahead in stepping:
+            mode[i] = row.mode(ahead)
+            if ahead:
+                fed[i] = 1          # its last token is what the previous step chose
+            else:
+                last[i] = row.last
         self._h_last[:] = last
         self._h_mode[:] = mode
+        self._h_fed[:] = fed
         if general:
             smode, temp = [4] * slots, [1.0] * slots  # 4 = MSA_ROW_SKIP
             for i, row in general:
@@ -776,6 +829,9 @@ class ContinuousBatcher(_Front):
         if self._par_dirty:
             self._par_dev.copy_(self._par_host, non_blocking=True)
             self._par_dirty = False
+        feed = self._last
+        if before is not None and any(fed):
+            feed = torch.where(self._fed.bool(), self._tok[before.buf], self._last)
         extra = {}
         if general:
             self._topp.copy_(self._nucleus_now())
@@ -783,7 +839,8 @@ class ContinuousBatcher(_Front):
             drawn = [(i, row) for i, row in general if row.group.topp > 0]
             if drawn:
                 noise = self._noise
-                self._draw_noise(noise, drawn)
+                ahead_of = {i: ahead for i, _, ahead in stepping}
+                self._draw_noise(noise, drawn, ahead_of)
             sampled = dict(row_mode=self._smode, temperature=self._temp, topp=self._topp,
                            noise=noise)
             if any(row.group.penalised for _, row in general):
@@ -792,24 +849,45 @@ class ContinuousBatcher(_Front):
             if any(row.group.logprobs > 0 for _, row in general):
                 sampled["lprobs_out"] = self._lprobs
             extra = dict(logits_out=self._logits, sampled=sampled)
-        self.decoder.decode_slots(self.cache, self._last, temperature=1.0, banned=[pad],
+        tok, score = self._tok[buf], self._score[buf]
+        self.decoder.decode_slots(self.cache, feed, temperature=1.0, banned=[pad],
                                   stop=self._stop, eos=eos, row_mode=self._mode,
-                                  tok_out=self._tok, score_out=self._score, **extra)
-        self._flush()   # the step is queued: the GPU works while the host writes records
+                                  tok_out=tok, score_out=score, **extra)
         decaying = [i for i, row in general if row.group.decay > 0]
         if decaying:
-            self._count_chosen(decaying, self._tok[torch.tensor(decaying, device=self.device)])
+            self._count_chosen(decaying, tok[torch.tensor(decaying, device=self.device)])
+        launched = _Launched(buf, {i: row for i, row, _ in stepping})
         watched = [(i, row) for i, row in general if row.group.logprobs > 0]
         if watched:
             k = max(row.group.logprobs for _, row in watched)
             picked = self._lprobs[torch.tensor([i for i, _ in watched], device=self.device)]
             values, top_ids = picked.topk(k, dim=-1)
-            for (i, row), v, t in zip(watched, values.tolist(), top_ids.tolist()):
-                row.top.append((v[:row.group.logprobs], t[:row.group.logprobs]))
-        toks, scs = self._tok.tolist(), self._score.tolist()
+            launched.watched = watched
+            launched.top = (values.to("cpu", non_blocking=True),
+                            top_ids.to("cpu", non_blocking=True))
+        self._host_tok[buf].copy_(tok, non_blocking=True)
+        self._host_score[buf].copy_(score, non_blocking=True)
+        if self._events is not None:
+            self._events[buf].record()
         self.steps += 1
-        self.rows_stepped += len(active)
-        for i, row in active:
+        self.rows_stepped += len(stepping)
+        return launched
+
+    def _collect(self, launched):
+        """Reads the results of a launched step (waiting for that step alone) and books them:
+        tokens, scores, alternatives; rows that have ended leave their slots."""
+        if self._events is not None:
+            self._events[launched.buf].synchronize()
+        toks = self._host_tok[launched.buf].tolist()
+        scs = self._host_score[launched.buf].tolist()
+        eos = self.dict.eos()
+        if launched.watched:
+            values, top_ids = (t.tolist() for t in launched.top)
+            for (i, row), v, t in zip(launched.watched, values, top_ids):
+                if not row.done:
+                    row.top.append((v[:row.group.logprobs], t[:row.group.logprobs]))
+        for i, row in launched.rows.items():
+            if row.done:
+                continue    # it had ended a step earlier: this output is not its
             if row.take(toks[i], scs[i], eos, self._stop):
                 self._retire(i)
-        return served + len(active)
