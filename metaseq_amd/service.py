@@ -863,8 +863,10 @@ class ContinuousBatcher(_Front):
             picked = self._lprobs[torch.tensor([i for i, _ in watched], device=self.device)]
             values, top_ids = picked.topk(k, dim=-1)
             launched.watched = watched
-            launched.top = (values.to("cpu", non_blocking=True),
-                            top_ids.to("cpu", non_blocking=True))
+            pinned = self._events is not None
+            launched.top = tuple(
+                torch.empty(t.shape, dtype=t.dtype, pin_memory=pinned).copy_(t, non_blocking=True)
+                for t in (values, top_ids))
         self._host_tok[buf].copy_(tok, non_blocking=True)
         self._host_score[buf].copy_(score, non_blocking=True)
         if self._events is not None:
