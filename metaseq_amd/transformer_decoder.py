@@ -968,13 +968,15 @@ class TransformerDecoder(nn.Module):
         out = []
         for r, lg in zip(requests, logits):
             kw = {k: v for k, v in r.items() if k not in ("slot", "tokens")}
-            out.append(self.admit_slot(cache, r["slot"], r["tokens"], _logits=lg, **kw))
-        return out
+            out.append(self.admit_slot(cache, r["slot"], r["tokens"], _logits=lg, _lazy=True,
+                                       **kw))
+        # every request's kernels are queued: one wait for the first list, none for the rest
+        return [[0.0] + lp.tolist() if lp is not None else [0.0] for lp in out]
 
     def admit_slot(self, cache: KVCache, slot: int, tokens: torch.Tensor, *, banned=(), stop=(),
                    eos=2, mode=0, tok_out=None, score_out=None, temperature=1.0, topp=0.0,
                    noise=None, replicas=(), penalties=None, lprobs_out=None, prompt_topk=0,
-                   detail=None, _logits=None):
+                   detail=None, _logits=None, _lazy=False):
         """``prefill_slot`` plus what a request needs from its prompt: the log-probability of
         every prompt token given its prefix (returned as a list, 0.0 for the first token) and
         the choice of the first new token from the last position, written to ``tok_out`` /
@@ -1000,13 +1002,14 @@ class TransformerDecoder(nn.Module):
         logits = _logits if _logits is not None else self.prefill_slot(cache, slot, tokens)
         T, V = logits.shape
         stream = _capi.stream_ptr()
-        scores = [0.0] * T
+        scores, lp = [0.0] * T, None
         if T > 1:
             lp = torch.empty(T - 1, dtype=torch.float32, device=logits.device)
             target = tokens.long()[1:].contiguous()
             check(lib.msa_target_logprob_f16(ptr(logits), logits.stride(0), T - 1, V,
                                              float(temperature), ptr(target), ptr(lp), stream))
-            scores[1:] = lp.tolist()
+            if not _lazy:   # (_lazy: the caller reads the device tensor once all is queued)
+                scores[1:] = lp.tolist()
             if prompt_topk > 0 and detail is not None:
                 dist = torch.empty(T - 1, V, dtype=torch.float32, device=logits.device)
                 check(lib.msa_log_softmax_f16(ptr(logits), 0, logits.stride(0), 1, T - 1, V,
@@ -1049,7 +1052,7 @@ class TransformerDecoder(nn.Module):
                 alphas[2], alphas[3], None, ptr(lprobs_out),
                 lprobs_out.stride(0) if lprobs_out is not None else 0, ptr(tok_out), 1,
                 ptr(score_out), 1, stream))
-        return scores
+        return lp if _lazy else scores
 
     def copy_slot(self, cache: KVCache, src: int, dst: int):
         """Makes slot ``dst`` a copy of slot ``src``: keys, values and length (a replica of a
