@@ -143,6 +143,73 @@ def test_prefill_gemm_random_shapes(lib):
         assert err <= float(want.abs().max()) * 2 ** -9 + 2e-3, (it, err)
 
 
+def test_few_row_major_rows_gemm_random_shapes(lib):
+    """Row-major activations of 1 .. 64 rows (fp16 and int8: one sweep of the streaming kernel)
+    and of 65 .. 256 rows over int8 weights (a sweep per 64 rows), with output widths that are
+    not multiples of a workgroup's tiles, every epilogue, y aliasing the residual; and the
+    split-K form on row-major rows with the slices the library suggests."""
+    rng = random.Random(31)
+    for it in range(24):
+        w8 = it % 2 == 1
+        M = rng.randint(65, 256) if (w8 and it % 4 == 3) else rng.randint(1, 64)
+        N = 16 * rng.choice([1, 3, 7, 20, 63, 64, 100, 257, 500, 768, 2304])
+        K = 64 * rng.choice([1, 2, 3, 5, 8, 12, 17, 32, 64])
+        relu, use_res = rng.random() < 0.4, rng.random() < 0.6
+        in_place = use_res and rng.random() < 0.5
+        print("few rows gemm case", it, M, N, K, "int8" if w8 else "fp16", relu, use_res,
+              in_place, flush=True)
+        g = torch.Generator(device=DEV).manual_seed(300 + it)
+        x = (torch.randn(M, K, generator=g, device=DEV) * 0.5).half()
+        b = (torch.randn(N, generator=g, device=DEV) * 0.1).half()
+        res = torch.randn(M, N, generator=g, device=DEV).half() if use_res else None
+        if w8:
+            q = torch.randint(-127, 128, (N, K), generator=g, device=DEV, dtype=torch.int8)
+            sc = (torch.rand(N, generator=g, device=DEV) * 0.01 + 0.001).half()
+            Wd = (q.float() * sc.float()[:, None]).half()
+            Wp = torch.empty_like(q)
+            assert lib.msa_pack_weight_i8(q.data_ptr(), Wp.data_ptr(), N, K, None) == 0
+        else:
+            Wd = (torch.randn(N, K, generator=g, device=DEV) * 0.05).half()
+            Wp = torch.empty_like(Wd)
+            assert lib.msa_pack_weight_f16(Wd.data_ptr(), Wp.data_ptr(), N, K, None) == 0
+        prod = x.float() @ Wd.float().t()
+        want = r16(r16(prod) + b.float())
+        if relu:
+            want = want.clamp_min(0)
+        if use_res:
+            want = r16(want + res.float())
+        y = res.clone() if in_place else torch.full((M, N), float("nan"), dtype=torch.float16,
+                                                    device=DEV)
+        rp = None if res is None else (y.data_ptr() if in_place else res.data_ptr())
+        flags = 1 if relu else 0
+        if w8:
+            rc = lib.msa_linear_w8a16(x.data_ptr(), Wp.data_ptr(), sc.data_ptr(), b.data_ptr(), rp,
+                                      y.data_ptr(), M, N, K, flags, None)
+        else:
+            rc = lib.msa_linear_f16(x.data_ptr(), Wp.data_ptr(), b.data_ptr(), rp, y.data_ptr(), M,
+                                    N, K, flags, None)
+        assert rc == 0, lib.msa_last_error()
+        torch.cuda.synchronize()
+        got = y.float()
+        assert torch.isfinite(got).all(), (it, "unwritten or non-finite output")
+        err = float((got - want).abs().max())
+        assert err <= float(want.abs().max()) * 2 ** -9 + 2e-3, (it, err)
+        if w8 or K < 256:
+            continue
+        # split-K partial sums of the same product on row-major rows
+        S = max(2, lib.msa_linear_default_splits_rows(M, N, K))
+        while K % (64 * S) or K // S < 128:
+            S //= 2
+        if S < 2:
+            continue
+        part = torch.full((S, M, N), float("nan"), dtype=torch.float32, device=DEV)
+        rc = lib.msa_linear_partial_f16(x.data_ptr(), Wp.data_ptr(), part.data_ptr(), M, N, K, S,
+                                        0, None)
+        assert rc == 0, lib.msa_last_error()
+        torch.cuda.synchronize()
+        assert float((part.sum(0) - prod).abs().max()) < 2e-3 * max(1.0, float(prod.abs().max()))
+
+
 def test_attention_random_shapes(lib):
     rng = random.Random(11)
     for it in range(48):
