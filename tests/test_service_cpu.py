@@ -2,6 +2,7 @@
 generator (cost model, per-signature backlogs, budget and overflow rules, result routing, error
 propagation) and the continuous batcher against a scripted fake decoder (slot bookkeeping,
 per-row minimum / maximum / stop rules, records)."""
+import random
 import threading
 
 import pytest
@@ -573,3 +574,66 @@ def test_shared_prefills_group_prompts_of_similar_length():
     Knobs.prefill_batch = 1
     groups = ContinuousBatcher._prefill_groups(Knobs(), [dict(ids=[0] * n) for n in (3, 3, 3)])
     assert [len(g) for g in groups] == [1, 1, 1]
+
+
+@pytest.mark.parametrize("seed,slots,prefill", [(1, 2, (1, 0)), (2, 3, (3, 2)), (3, 5, (4, 1)),
+                                                (4, 1, (1, 0)), (5, 7, (2, 5))])
+def test_continuous_batcher_random_traffic_against_the_scripted_model(seed, slots, prefill):
+    """150 requests with random prompts, length limits, temperatures, nuclei (fixed and
+    decaying), penalties, replicas and two stop lists, arriving in bursts while the engine
+    runs, over few slots: every answer equals the request's own loop.  The engine queues each
+    decode step before it reads the previous one, so rows that have just ended are stepped once
+    more, slots change hands between two reads, and requests with another stop list wait for
+    the batch to drain - none of which may show in a result."""
+    rng = random.Random(seed)
+    cb, dec = _batcher(slots=slots, symbols=FULL_STOPS, noise_fn=_noise,
+                       prefill_batch=prefill[0], prefill_wait=prefill[1], patience=20)
+    specs, replies = [], []
+    pending = 150
+    steps = 0
+    while True:
+        busy = cb.step()
+        if not (pending or busy or any(r.empty() for r in replies)):
+            break
+        steps += 1
+        assert steps < 20000
+        for _ in range(min(pending, rng.choice([0, 0, 0, 1, 2, 5]))):
+            pending -= 1
+            s = dict(prompt=[rng.randint(4, V - 1) for _ in range(rng.randint(1, 9))],
+                     max_tokens=rng.randint(1, 14))
+            if rng.random() < 0.5:
+                s.update(temperature=rng.choice([0.7, 1.3]), top_p=rng.choice([0.4, 0.9]))
+                if rng.random() < 0.4:
+                    s.update(lambda_decay=rng.choice([0.5, 0.8]), omega_bound=0.2)
+            elif rng.random() < 0.3:
+                s.update(temperature=0.5)
+            if rng.random() < 0.3:
+                s.update(alpha_presence=0.5, alpha_frequency=rng.choice([0.0, 0.3]))
+            if rng.random() < 0.2:
+                s.update(alpha_frequency_src=0.2, alpha_src_penalty_end_idx=rng.choice([-1, 2]))
+            if rng.random() < 0.3:
+                s.update(min_tokens=min(rng.randint(1, 4), s["max_tokens"]))
+            if rng.random() < 0.15:
+                s.update(stop=[17, 23])
+            if rng.random() < 0.15 and slots >= 2:
+                s.update(n=1, best_of=2)
+            specs.append(s)
+            replies.append(cb.submit(s["prompt"],
+                                     **{k: v for k, v in s.items() if k != "prompt"}))
+    for s, r in zip(specs, replies):
+        res = r.get_nowait()[1]
+        assert not isinstance(res, Exception), (s, res)
+        req = Request(0, s["prompt"], {})
+        runs = []
+        for j in range(s.get("best_of", 1)):
+            want = _expected(
+                s["prompt"], s.get("min_tokens", 0), s["max_tokens"], stop=s.get("stop", ()),
+                temperature=s.get("temperature", 1.0), topp=max(s.get("top_p", 0.0), 0.0),
+                noise=lambda pos, j=j: _noise(req, j, pos, V),
+                alphas=(s.get("alpha_presence", 0.0), s.get("alpha_frequency", 0.0), 0.0,
+                        s.get("alpha_frequency_src", 0.0)),
+                src_end=s.get("alpha_src_penalty_end_idx", -1), decay=s.get("lambda_decay", -1.0),
+                omega=s.get("omega_bound", 0.3), full_stop=tuple(FULL_STOPS.values()))
+            runs.append([str(t) for t in want if t != EOS])
+        assert res[0]["tokens"] in runs, (s, res[0]["tokens"], runs)
+    assert all(n < 0 for n in cb.cache.lens)
