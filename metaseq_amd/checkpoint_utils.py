@@ -249,6 +249,45 @@ def load_fsdp_checkpoint(paths: List[str]) -> "OrderedDict[str, torch.Tensor]":
     return normalize_state_dict(glue_model_parts(states) if len(states) > 1 else states[0])
 
 
+# ---------------------------------------------------------------- offline int8 weights
+_QUANTIZED = re.compile(r"^(decoder\.)?layers\.\d+\.(self_attn\.qkv_proj|self_attn\.out_proj|fc1|fc2)"
+                        r"\.weight$")
+
+
+def quantize_rows(w: torch.Tensor):
+    """Symmetric int8 per output row of a [out, in] matrix: scale_j = fp16(max_i |w_ji| / 127),
+    q_ji = clamp(rint(w_ji / scale_j), -127, 127) in fp32 arithmetic - the weight-only form the
+    reference asks of its serving backend for these matrices
+    (metaseq/scripts/convert_metaseq_ft.py:99-133).  Runs wherever ``w`` lives, with the same
+    result on the CPU and on the GPU (every step is one correctly rounded operation)."""
+    wf = w.float()
+    scales = (wf.abs().amax(dim=1) / 127.0).to(torch.float16)
+    s = scales.float().clamp_min(1e-30).unsqueeze(1)
+    q = torch.clamp(torch.round(wf / s), -127, 127).to(torch.int8)
+    return q.contiguous(), scales.contiguous()
+
+
+def quantize_state_dict(state: Dict[str, torch.Tensor]) -> "OrderedDict[str, torch.Tensor]":
+    """The offline step of int8 serving: every per-layer qkv_proj / out_proj / fc1 / fc2
+    ``<name>.weight`` of a reference-named state dict becomes ``<name>.qweight`` (int8 [out, in],
+    row-major) and ``<name>.scales`` (fp16 [out]); everything else is passed through.  The
+    result is what ``TransformerDecoder.load_state_dict`` / ``load_tensors`` take in place of
+    fp16 weights, so a served model never has to hold (or read) the fp16 matrices; it needs no
+    GPU and can be saved with ``torch.save``."""
+    out = OrderedDict()
+    for k, v in state.items():
+        if _QUANTIZED.match(k):
+            stem = k[:-len("weight")]
+            out[stem + "qweight"], out[stem + "scales"] = quantize_rows(v)
+        else:
+            out[k] = v
+    return out
+
+
+def is_quantized_state(state) -> bool:
+    return any(k.endswith(".qweight") for k in state)
+
+
 def find_model_parts(names: List[str]) -> List[str]:
     """Sorts file names of one checkpoint by their `-model_part-{r}` number
     (metaseq/distributed/stitch_fsdp_ckpt.py:342-352) and checks that no rank is missing."""

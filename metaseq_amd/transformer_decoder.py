@@ -17,6 +17,7 @@ from torch import nn
 from . import _capi
 from ._capi import (MSA_EMBED_COL_FROM_LEN, MSA_EMBED_ROWS_GIVEN, MSA_EPI_RELU, MSA_IN_PACKED,
                     MSA_OUT_PACKED, check, ptr)
+from .checkpoint_utils import quantize_rows
 from .config import OPTConfig
 from .kv_cache import KVCache
 
@@ -44,28 +45,44 @@ class _Affine(nn.Module):
         N, K = self.shape
         w = self.weight.data
         if int8:
-            wf = w.float()
-            scales = (wf.abs().amax(dim=1) / 127.0).to(torch.float16)
-            s = scales.float().clamp_min(1e-30).unsqueeze(1)
-            q = torch.clamp(torch.round(wf / s), -127, 127).to(torch.int8).contiguous()
-            del wf
-            qp = torch.empty_like(q)
-            check(lib.msa_pack_weight_i8(ptr(q), ptr(qp), N, K, _capi.stream_ptr()))
-            self.qweight, self.scales = qp, scales.contiguous()
-            self.weight.data = torch.empty(0, dtype=torch.float16, device=w.device)
+            self.adopt_int8_(lib, *quantize_rows(w))
         else:
             wp = torch.empty_like(w)
             check(lib.msa_pack_weight_f16(ptr(w), ptr(wp), N, K, _capi.stream_ptr()))
             self.weight.data = wp
             self.packed = True
 
+    def adopt_int8_(self, lib, q, scales):
+        """Takes already quantised weights (int8 [N, K] row-major, fp16 [N] scales), packs them
+        for the kernels and frees the fp16 matrix."""
+        N, K = self.shape
+        dev = self.bias.device
+        if tuple(q.shape) != (N, K) or q.dtype != torch.int8:
+            raise ValueError("int8 weight: expected int8 %s, got %s %s"
+                             % ((N, K), q.dtype, tuple(q.shape)))
+        if tuple(scales.shape) != (N,):
+            raise ValueError("int8 scales: expected %s, got %s" % ((N,), tuple(scales.shape)))
+        q = q.to(dev).contiguous()
+        qp = torch.empty_like(q)
+        check(lib.msa_pack_weight_i8(ptr(q), ptr(qp), N, K, _capi.stream_ptr()))
+        self.qweight = qp
+        self.scales = scales.to(device=dev, dtype=torch.float16).contiguous()
+        self.weight.data = torch.empty(0, dtype=torch.float16, device=dev)
+        self.packed = False
+
+    def row_major_int8(self, lib):
+        """(int8 [N, K] row-major, fp16 [N] scales) of a quantised matrix."""
+        N, K = self.shape
+        q = torch.empty_like(self.qweight)
+        check(lib.msa_unpack_weight_i8(ptr(self.qweight), ptr(q), N, K, _capi.stream_ptr()))
+        return q, self.scales
+
     def row_major_weight(self, lib):
         """fp16 [N, K] row-major weight (for int8: the dequantised round(q * scale))."""
         N, K = self.shape
         if self.qweight is not None:
-            q = torch.empty_like(self.qweight)
-            check(lib.msa_unpack_weight_i8(ptr(self.qweight), ptr(q), N, K, _capi.stream_ptr()))
-            return (q.float() * self.scales.float().unsqueeze(1)).to(torch.float16)
+            q, scales = self.row_major_int8(lib)
+            return (q.float() * scales.float().unsqueeze(1)).to(torch.float16)
         if not self.packed:
             return self.weight.data
         w = torch.empty_like(self.weight.data)
@@ -166,6 +183,9 @@ class TransformerDecoder(nn.Module):
                 lin.packed, lin.qweight, lin.scales = False, None, None
         self._lm_head = None
         self._drop_native()
+        if any(k.endswith(".qweight") for k in sd):
+            # weights quantised offline (checkpoint_utils.quantize_state_dict)
+            return self.load_tensors(sd.items())
         return super().load_state_dict(sd, strict=strict, **kw)
 
     def load_tensors(self, named_tensors, quantize_int8=False):
@@ -173,7 +193,10 @@ class TransformerDecoder(nn.Module):
         copy: ``named_tensors`` yields (reference parameter name, tensor) pairs, each is copied
         into place and may be freed by the producer right away.  With ``quantize_int8`` every
         linear layer is quantised and packed as soon as its weight has arrived, so the fp16
-        matrices never all exist at once.  Every parameter must arrive exactly once."""
+        matrices never all exist at once.  A linear layer quantised offline arrives as
+        ``<name>.qweight`` (int8 [out, in]) and ``<name>.scales`` (fp16 [out]) in place of
+        ``<name>.weight`` (``checkpoint_utils.quantize_state_dict``) and is packed as it is.
+        Every parameter must arrive exactly once."""
         lib = self._lib = self._lib or _capi.load()
         if quantize_int8:
             self.cfg.quantize_int8 = True
@@ -185,10 +208,25 @@ class TransformerDecoder(nn.Module):
         self._lm_head = None
         self._drop_native()
         seen = set()
+        halves = {}  # linear name -> {"qweight": ..., "scales": ...} until both have arrived
         for name, t in named_tensors:
             if name.startswith("decoder."):
                 name = name[len("decoder."):]
             if name in ("version", "output_projection.weight"):
+                continue
+            stem, _, kind = name.rpartition(".")
+            if kind in ("qweight", "scales"):
+                if stem not in linears:
+                    raise KeyError("unexpected parameter %r" % name)
+                got = halves.setdefault(stem, {})
+                if kind in got or stem + ".weight" in seen:
+                    raise KeyError("unexpected or repeated parameter %r" % name)
+                got[kind] = t
+                if len(got) == 2:
+                    linears[stem].adopt_int8_(lib, got["qweight"], got["scales"])
+                    halves[stem] = {"qweight": None, "scales": None}  # arrived; tensors released
+                    seen.add(stem + ".weight")
+                    self.cfg.quantize_int8 = True
                 continue
             if name not in own or name in seen:
                 raise KeyError("unexpected or repeated parameter %r" % name)
@@ -202,7 +240,31 @@ class TransformerDecoder(nn.Module):
         missing = sorted(set(own) - seen)
         if missing:
             raise KeyError("missing parameters: %s" % ", ".join(missing[:8]))
+        if halves:
+            for name, lin in linears.items():
+                if lin.qweight is None:
+                    raise KeyError("%s arrived in fp16 beside int8 layers; quantise all of the "
+                                   "per-layer matrices or none" % name)
         return self
+
+    def quantized_state_dict(self):
+        """The int8 model as ``checkpoint_utils.quantize_state_dict`` writes it (reference
+        names with a "decoder." prefix; ``.qweight`` int8 [out, in] row-major and ``.scales``
+        in place of the four per-layer ``.weight``): saved with ``torch.save``, it is loaded
+        again by ``load_state_dict`` / ``load_tensors`` without the fp16 matrices."""
+        if not self.cfg.quantize_int8:
+            raise RuntimeError("quantized_state_dict() needs an int8 model (quantize_int8_())")
+        lib = self.prepare_()
+        linears = dict(self._linears())
+        out = {}
+        for k, v in nn.Module.state_dict(self).items():
+            stem = k[:-len(".weight")] if k.endswith(".weight") else None
+            if stem in linears:
+                out["decoder." + stem + ".qweight"], out["decoder." + stem + ".scales"] = \
+                    linears[stem].row_major_int8(lib)
+            else:
+                out["decoder." + k] = v
+        return out
 
     def state_dict(self, *args, **kwargs):
         """Reference-layout (row-major, fp16) state dict; quantised matrices come back as their

@@ -61,3 +61,80 @@ def test_glued_parts_load_into_the_decoder_and_match_the_tensor_parallel_oracle(
     wrong[k] = torch.cat([p[k] for p in parts], 0)
     bad = TransformerLanguageModel.build_model(cfg, wrong, device="cuda")(tokens.cuda())[0]
     assert float((bad.float().cpu() - want).abs().max()) > 5e-2
+
+
+def _int8_models(tmp_path):
+    from metaseq_amd import random_state_dict
+    from tests.common import tiny_cfg
+    cfg = tiny_cfg(layers=2, dim=128, heads=2, vocab=96, max_pos=48)
+    sd = random_state_dict(cfg, seed=21, dtype=torch.float16)
+    online = TransformerLanguageModel.build_model(tiny_cfg(layers=2, dim=128, heads=2, vocab=96,
+                                                           max_pos=48), sd, device="cuda:0")
+    online.decoder.quantize_int8_()
+    return cfg, sd, online
+
+
+def _same_logits(a, b, cfg):
+    g = torch.Generator().manual_seed(3)
+    toks = torch.randint(4, cfg.vocab_size, (3, 17), generator=g).to("cuda:0")
+    toks[:, 0] = 2
+    ia, ib = {}, {}
+    assert torch.equal(a(toks[:, :12], incremental_state=ia)[0],
+                       b(toks[:, :12], incremental_state=ib)[0])
+    for t in range(12, 17):
+        assert torch.equal(a.decoder(toks[:, :t + 1], incremental_state=ia)[0],
+                           b.decoder(toks[:, :t + 1], incremental_state=ib)[0])
+
+
+def test_weights_quantised_offline_on_the_cpu_load_as_the_model_quantised_on_the_gpu(tmp_path):
+    """The offline step (``quantize_state_dict`` on CPU tensors, saved and read back with the
+    loader that executes nothing) gives, bit for bit, the model that ``quantize_int8_()`` makes
+    from the fp16 weights on the GPU: same packed int8 bytes and scales, same logits through
+    prefill and decode steps."""
+    print("offline int8", flush=True)
+    cfg, sd, online = _int8_models(tmp_path)
+    path = str(tmp_path / "int8.pt")
+    torch.save({"model": C.quantize_state_dict(sd)}, path)
+    state = torch.load(path, map_location="cpu", weights_only=True)["model"]
+    offline = TransformerLanguageModel.build_model(cfg, state, device="cuda:0")
+    assert cfg.quantize_int8
+    for (name, a), (_, b) in zip(online.decoder._linears(), offline.decoder._linears()):
+        assert b.weight.numel() == 0 and not b.packed
+        assert torch.equal(a.qweight, b.qweight) and torch.equal(a.scales, b.scales), name
+    _same_logits(online, offline, cfg)
+
+
+def test_quantised_state_dict_round_trip_and_streaming(tmp_path):
+    """``quantized_state_dict()`` of an int8 model equals the offline step's output, loads
+    again whole (``load_state_dict``, also over a model that already holds packed weights) and
+    streamed (``load_tensors``), and fp16 matrices beside int8 ones are refused."""
+    print("int8 state dict", flush=True)
+    from tests.common import tiny_cfg
+    cfg, sd, online = _int8_models(tmp_path)
+    qsd = online.decoder.quantized_state_dict()
+    want = C.quantize_state_dict(sd)
+    assert set(qsd) - {"decoder.version"} == set(want) - {"decoder.version"}
+    for k, v in want.items():
+        if k != "decoder.version":
+            assert torch.equal(qsd[k].cpu(), v), k
+    new = lambda: tiny_cfg(layers=2, dim=128, heads=2, vocab=96, max_pos=48)
+    again = TransformerLanguageModel.build_model(new(), sd, device="cuda:0")
+    again.decoder.prepare_()                       # packed fp16 weights, replaced below
+    again.load_state_dict(qsd)
+    _same_logits(online, again, cfg)
+    streamed = TransformerLanguageModel.build_model(new(), None, device="cuda:0")
+    streamed.decoder.load_tensors((k, v.cpu()) for k, v in qsd.items())
+    _same_logits(online, streamed, cfg)
+    mixed = dict(want)
+    k = "decoder.layers.1.fc2."
+    del mixed[k + "qweight"], mixed[k + "scales"]
+    mixed[k + "weight"] = sd[k + "weight"]
+    with pytest.raises(KeyError, match="layers.1.fc2 arrived in fp16 beside int8 layers"):
+        TransformerLanguageModel.build_model(new(), mixed, device="cuda:0")
+    with pytest.raises(ValueError, match="int8 weight: expected"):
+        bad = dict(want)
+        bad[k + "qweight"] = bad[k + "qweight"][:-1]
+        TransformerLanguageModel.build_model(new(), bad, device="cuda:0")
+    fp16 = TransformerLanguageModel.build_model(new(), sd, device="cuda:0")
+    with pytest.raises(RuntimeError, match="needs an int8 model"):
+        fp16.decoder.quantized_state_dict()

@@ -67,3 +67,47 @@ def test_kv_cache_row_views_follow_growth_and_keep_nothing_alive():
         assert ref() is None
     finally:
         gc.enable()
+
+
+def test_offline_quantisation_replaces_the_four_per_layer_matrices_and_nothing_else():
+    """``quantize_state_dict`` against the oracle's quantiser: qkv_proj / out_proj / fc1 / fc2
+    weights of every layer become (.qweight, .scales) with the oracle's values; embeddings,
+    biases and LayerNorms pass through untouched, with or without the "decoder." prefix."""
+    from metaseq_amd.checkpoint_utils import is_quantized_state, quantize_state_dict
+    from oracle.opt_oracle import quantize_int8
+    cfg = tiny_cfg(layers=2, dim=64, heads=1, vocab=64, max_pos=32)
+    sd = random_state_dict(cfg, seed=5)
+    sd["decoder.layers.1.fc1.weight"][3].zero_()  # an all-zero row: scale 0, q 0
+    for prefix in ("decoder.", ""):
+        src = {(k[len("decoder."):] if not prefix else k): v for k, v in sd.items()}
+        out = quantize_state_dict(src)
+        assert is_quantized_state(out) and not is_quantized_state(src)
+        changed = {k for k in src if k not in out}
+        want = {"%slayers.%d.%s.weight" % (prefix, i, m) for i in range(2)
+                for m in ("self_attn.qkv_proj", "self_attn.out_proj", "fc1", "fc2")}
+        assert changed == want
+        for k in want:
+            q, s = quantize_int8(src[k])
+            stem = k[:-len("weight")]
+            assert out[stem + "qweight"].dtype == torch.int8 and out[stem + "scales"].dtype == torch.float16
+            assert torch.equal(out[stem + "qweight"], q) and torch.equal(out[stem + "scales"], s)
+        for k in src:
+            if k not in want:
+                assert out[k] is src[k]
+        assert out[prefix + "layers.1.fc1.scales"][3] == 0
+        assert not out[prefix + "layers.1.fc1.qweight"][3].any()
+
+
+def test_load_tensors_refuses_int8_names_it_does_not_know():
+    from metaseq_amd.checkpoint_utils import quantize_state_dict
+    cfg = tiny_cfg(layers=1, dim=64, heads=1, vocab=64, max_pos=32)
+    items = list(quantize_state_dict(dict(iter_random_state_dict(cfg, seed=3))).items())
+    odd = [("layer_norm.qweight", torch.zeros(64, dtype=torch.int8))] + items
+    with pytest.raises(KeyError, match="unexpected parameter 'layer_norm.qweight'"):
+        TransformerDecoder(cfg, None, device="cpu").load_tensors(odd)
+    twice = [items[i] for i in range(len(items))]
+    name = next(n for n, _ in items if n.endswith("fc1.scales"))
+    twice.insert(0, (name, dict(items)[name]))
+    twice.insert(0, (name, dict(items)[name]))
+    with pytest.raises(KeyError, match="unexpected or repeated parameter"):
+        TransformerDecoder(cfg, None, device="cpu").load_tensors(twice)
