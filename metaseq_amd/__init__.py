@@ -1,6 +1,6 @@
 """MI355X-native OPT incremental-decoding forward path (drop-in for metaseq's
 TransformerDecoder.forward / SequenceGenerator on one gfx950 GPU)."""
-from .config import OPTConfig, opt_config
+from .config import OPTConfig, config_from_state_dict, opt_config
 from .dictionary import Dictionary
 from .hub_utils import GeneratorInterface
 from .kv_cache import KVCache
@@ -10,7 +10,7 @@ from .transformer_decoder import ModelParallelTransformerDecoder, TransformerDec
 from .transformer_lm import TransformerLanguageModel
 
 __all__ = [
-    "OPTConfig", "opt_config", "Dictionary", "GeneratorInterface", "KVCache", "SequenceGenerator", "random_prompts",
+    "OPTConfig", "opt_config", "config_from_state_dict", "Dictionary", "GeneratorInterface", "KVCache", "SequenceGenerator", "random_prompts",
     "random_state_dict", "iter_random_state_dict", "TransformerDecoder", "ModelParallelTransformerDecoder",
     "TransformerLanguageModel",
 ]

@@ -69,3 +69,35 @@ _OPT_SIZES = {
 def opt_config(name: str, **overrides) -> OPTConfig:
     layers, dim, heads = _OPT_SIZES[name.lower()]
     return replace(OPTConfig(layers, dim, heads), **overrides)
+
+
+def config_from_state_dict(state, heads: int = 0, **overrides) -> OPTConfig:
+    """The configuration a reference-named state dict (fp16, or quantised offline) implies:
+    layers, widths, vocabulary and position count are read off the tensor shapes.  The number
+    of heads is in no shape; it is taken from the OPT size table by (layers, width) unless
+    given.  For checkpoints whose own "cfg" entry cannot be read by a loader that executes
+    nothing (metaseq/checkpoint_utils.py:540-557 pickles an arbitrary namespace there)."""
+    def shape(name):
+        for k in (name, "decoder." + name):
+            if k in state:
+                return tuple(state[k].shape)
+        raise KeyError("state dict has no %r" % name)
+
+    layers = 1 + max(int(k.split("layers.")[1].split(".")[0]) for k in state if "layers." in k)
+    vocab, dim = shape("embed_tokens.weight")
+    positions = shape("embed_positions.weight")[0]
+    try:
+        ffn = shape("layers.0.fc1.weight")[0]
+    except KeyError:
+        ffn = shape("layers.0.fc1.qweight")[0]
+    if not heads:
+        known = {(l, d): h for l, d, h in _OPT_SIZES.values()}
+        if (layers, dim) not in known:
+            raise ValueError("%d layers of width %d are no OPT size: pass heads=" % (layers, dim))
+        heads = known[(layers, dim)]
+    padding_idx = overrides.pop("padding_idx", 1)
+    # the learned positional table holds padding_idx + 1 unused leading rows
+    # (metaseq/modules/learned_positional_embedding.py:23-28)
+    cfg = OPTConfig(layers, dim, heads, decoder_ffn_embed_dim=ffn, vocab_size=vocab,
+                    max_target_positions=positions - padding_idx - 1, padding_idx=padding_idx)
+    return replace(cfg, **overrides)

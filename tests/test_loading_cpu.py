@@ -111,3 +111,25 @@ def test_load_tensors_refuses_int8_names_it_does_not_know():
     twice.insert(0, (name, dict(items)[name]))
     with pytest.raises(KeyError, match="unexpected or repeated parameter"):
         TransformerDecoder(cfg, None, device="cpu").load_tensors(twice)
+
+
+def test_configuration_is_read_off_a_state_dicts_shapes():
+    """Layers, widths, vocabulary and position count come from tensor shapes (fp16 or
+    quantised offline, with or without the "decoder." prefix); heads from the OPT size table,
+    or from the caller where the shape pair is no OPT size."""
+    from metaseq_amd import config_from_state_dict, opt_config
+    from metaseq_amd.checkpoint_utils import quantize_state_dict
+    cfg = tiny_cfg(layers=3, dim=64, heads=1, vocab=72, max_pos=40, ffn=96)
+    sd = random_state_dict(cfg, seed=1)
+    with pytest.raises(ValueError, match="pass heads="):
+        config_from_state_dict(sd)
+    for state in (sd, quantize_state_dict(sd), {k[len("decoder."):]: v for k, v in sd.items()}):
+        got = config_from_state_dict(state, heads=1)
+        assert got == cfg
+        TransformerDecoder(got, None, device="meta")
+    # an OPT size: shapes alone (meta tensors stand in for OPT-125M's weights)
+    want = opt_config("125m")
+    dec = TransformerDecoder(want, None, device="meta")
+    assert config_from_state_dict(torch.nn.Module.state_dict(dec)) == want
+    assert config_from_state_dict(torch.nn.Module.state_dict(dec), max_target_positions=512
+                                  ).max_target_positions == 512
