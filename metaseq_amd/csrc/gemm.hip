@@ -1149,8 +1149,9 @@ __global__ __launch_bounds__(TQ_THREADS) void linear_quad_kernel(
     }
   }
   // The narrowest form (WF = 2) also serves fewer than 256 rows: it does not move a ragged tile up
-  // but repeats the last row in its loads and drops the rows past it in the epilogue.
-  constexpr bool CLAMP = WF == 2;
+  // but repeats the last row in its loads and drops the rows past it in the epilogue.  So does
+  // the split-K form of WF = 4 (decode batches of 129 .. 255 rows cut K eight ways over it).
+  constexpr bool CLAMP = WF == 2 || (WF == 4 && PART);
   const int64_t m_own = (int64_t)by * TQ_BM;  // first row this tile owns
   const int64_t m0 = !CLAMP && m_own + TQ_BM > M ? M - TQ_BM : m_own;
   const int n0 = bx * TQ_BN;
@@ -1670,12 +1671,12 @@ void launch_quad_partial_w(const void* x, const void* W, float* part, int64_t M,
                      (const half_t*)x, W, M, N, K, 0, 0, 0, e, part, K / 64 / S);
 }
 
-// 256 x 64 tiles while their S slices fit the chip in one round; an S beyond that (given M >= 256,
-// which the wider form needs to move a ragged tile up) means 256 x 128 tiles.
+// 256 x 64 tiles while their S slices fit the chip in one round; an S beyond that means 256 x 128
+// tiles.
 void launch_quad_partial(const void* x, const void* W, float* part, int64_t M, int N, int K, int S,
                          hipStream_t s) {
   const int64_t tiles2 = ((M + TQ_BM - 1) / TQ_BM) * ((N + tq_bn(2) - 1) / tq_bn(2));
-  if (M >= TQ_BM && tiles2 * S > num_cus())
+  if (tiles2 * S > num_cus())
     return launch_quad_partial_w<4>(x, W, part, M, N, K, S, s);
   launch_quad_partial_w<2>(x, W, part, M, N, K, S, s);
 }
@@ -1685,14 +1686,15 @@ void launch_quad_partial(const void* x, const void* W, float* part, int64_t M, i
 // keep the 256 x 64 tiles within the chip, the K range of a slice at 512 or more, and whole
 // stages.  Where a slice would still span 4096 or more of K, twice the slices over 256 x 128
 // tiles measured faster (half the activation bytes per workgroup and weight byte: M = 256,
-// N = 4096, K = 16384: 51.8 against 55.4 us; M = 512: 78.0 against 93.6).
+// N = 4096, K = 16384: 51.8 against 55.4 us; M = 512: 78.0 against 93.6; M = 200, inside a
+// decode step: 42.4 against 47.2).
 int pick_row_splits(int64_t M, int N, int K) {
   if (M < 1 || N % 16 || K % 64) return 1;
   const int64_t tiles = ((M + TQ_BM - 1) / TQ_BM) * ((N + tq_bn(2) - 1) / tq_bn(2));
   int best = 1;
   for (int S = 2; S <= 8; S *= 2)
     if (tiles * S <= num_cus() && K % (64 * S) == 0 && K / S >= 512) best = S;
-  if (best > 1 && best < 8 && M >= TQ_BM && K / best >= 4096 && K % (128 * best) == 0) best *= 2;
+  if (best > 1 && best < 8 && M > 128 && K / best >= 4096 && K % (128 * best) == 0) best *= 2;
   return best;
 }
 

@@ -556,7 +556,12 @@ def test_split_k_partials_and_fused_layernorm(lib, M, N, K, S, w8):
                                      # more slices than 256 x 64 tiles fit at once: 256 x 128
                                      # tiles (a ragged second row tile moved up, a ragged last
                                      # column tile)
-                                     (256, 4096, 4096, 8), (300, 2064, 1024, 8)])
+                                     (256, 4096, 4096, 8), (300, 2064, 1024, 8),
+                                     # the same form below 256 rows and with a ragged last row
+                                     # tile: the last row repeated in the loads, rows past it
+                                     # dropped
+                                     (129, 4096, 16384, 8), (200, 4096, 4096, 8), (1, 4096, 2048, 8),
+                                     (513, 4096, 1024, 2)])
 def test_split_k_partials_of_row_major_rows(lib, M, N, K, S):
     """msa_linear_partial_f16 without MSA_IN_PACKED (decode batches above 128 rows): slice s of
     the output holds the fp32 sums over K range s and nothing else, for row counts that are not
@@ -596,7 +601,8 @@ def test_split_k_of_row_major_rows_rejects_and_suggestion(lib):
     assert lib.msa_linear_partial_w8a16(P(x), P(x), P(x), P(part), 256, 64, 4096, 4, 0, None) == -1
     # a few hundred rows against d_model output features: split; enough tiles already: not
     assert lib.msa_linear_default_splits_rows(256, 4096, 16384) == 8   # over 256 x 128 tiles
-    assert lib.msa_linear_default_splits_rows(200, 4096, 16384) == 4
+    assert lib.msa_linear_default_splits_rows(200, 4096, 16384) == 8   # the same below 256 rows
+    assert lib.msa_linear_default_splits_rows(100, 4096, 16384) == 4   # up to 128: 256 x 64 tiles
     assert lib.msa_linear_default_splits_rows(200, 4096, 4096) == 4
     assert lib.msa_linear_default_splits_rows(512, 4096, 4096) == 2
     assert lib.msa_linear_default_splits_rows(256, 16384, 4096) == 1
