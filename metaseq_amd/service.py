@@ -25,6 +25,14 @@ import random
 import threading
 from typing import Any, Dict, List, Optional
 
+
+def upload(values, dtype, device):
+    """A short host list as a device tensor, stream-ordered through pinned memory (see
+    ``transformer_decoder.upload``): the serving loop must not wait for the step in flight
+    every time it hands the GPU a few indices."""
+    from .transformer_decoder import upload as _upload
+    return _upload(values, dtype, device)
+
 # options that must agree within a run-to-completion batch (metaseq/service/workers.py:13-23)
 SIGNATURE_OPTIONS = ("temperature", "top_p", "n", "lambda_decay", "omega_bound", "alpha_presence",
                      "alpha_frequency", "alpha_presence_src", "alpha_frequency_src")
@@ -417,6 +425,8 @@ class ContinuousBatcher(_Front):
         self._stop: tuple = ()  # stop ids of the running batch
         self.noise_fn, self.patience = noise_fn, int(patience)
         self.prefill_batch, self.prefill_wait = max(1, int(prefill_batch)), int(prefill_wait)
+        # with rows running, queue the decode step before the admissions of the same call
+        self.launch_before_admission = True
         self._held = 0          # steps the waiting requests have been held back for company
         self._done: List[_Group] = []   # ended requests whose records are not built yet
         dev = self.device
@@ -537,7 +547,7 @@ class ContinuousBatcher(_Front):
         """After a draw: a full stop restarts the decay of a row's nucleus, any other token
         extends it (``tokens``: int64 device tensor, one per listed slot)."""
         torch = self._torch
-        idx = torch.tensor(slots, dtype=torch.long, device=self.device)
+        idx = upload(slots, torch.long, self.device)
         hit = (tokens.view(-1, 1) == self._full_stop.view(1, -1)).any(dim=1, keepdim=True)
         self._since[idx] = torch.where(hit, torch.zeros_like(self._since[idx]),
                                        self._since[idx] + 1)
@@ -553,18 +563,18 @@ class ContinuousBatcher(_Front):
             position = len(row.tokens) + (ahead.get(i, 0) if ahead else 0)
             out[i].copy_(self.noise_fn(row.group.req, row.replica, position, V))
 
-    def _prepare(self, slots: List[int], req: Request, noise_at: int):
+    def _prepare(self, slots: List[int], req: Request, noise_at: int, tok_all, score_all):
         """What the admission of ``req`` into ``slots`` (its replicas' rows) hands to the
         decoder: rows, output tensors and the keyword arguments of ``admit_slot``.  The
-        request's draws use rows ``noise_at`` .. of the shared noise buffer."""
+        request's draws use rows ``noise_at`` .. of the shared noise buffer, its first tokens
+        and their scores go to the same rows of ``tok_all`` / ``score_all``."""
         torch = self._torch
         eos, pad = self.dict.eos(), self.dict.pad()
         ids = [eos] + req.prompt
         group = _Group(req, self.batch.room_for(req))
         rows = [_Row(group, j, list(ids), []) for j in range(group.replicas)]
         R = len(rows)
-        tok = torch.zeros(R, dtype=torch.long, device=self.device)
-        score = torch.zeros(R, dtype=torch.float32, device=self.device)
+        tok, score = tok_all[noise_at:noise_at + R], score_all[noise_at:noise_at + R]
         extra, detail, lp = {}, {}, None
         if not group.plain:
             self._sampling_state()
@@ -578,8 +588,8 @@ class ContinuousBatcher(_Front):
                 self._penalty_state()
                 # the prompt's token counts, leading end-of-sequence token included, up to
                 # alpha_src_penalty_end_idx if given (metaseq/sequence_generator.py:380-389)
-                src = torch.tensor(ids if group.src_end <= 0 else ids[:group.src_end],
-                                   dtype=torch.long, device=self.device)
+                src = upload(ids if group.src_end <= 0 else ids[:group.src_end], torch.long,
+                             self.device)
                 counts_src = torch.zeros(R, V, dtype=torch.long, device=self.device)
                 counts_src[0].scatter_add_(0, src.clamp(0, V - 1), torch.ones_like(src))
                 counts_src[1:] = counts_src[0]
@@ -594,15 +604,16 @@ class ContinuousBatcher(_Front):
                     extra.update(prompt_topk=group.logprobs, detail=detail)
         if R > 1:
             extra["replicas"] = slots[1:]
-        call = dict(slot=slots[0], tokens=torch.tensor(ids, dtype=torch.long, device=self.device),
+        call = dict(slot=slots[0], tokens=upload(ids, torch.long, self.device),
                     banned=[pad], stop=self._stop, eos=eos, mode=rows[0].mode(), tok_out=tok,
                     score_out=score, **extra)
         return dict(slots=slots, req=req, group=group, rows=rows, ids=ids, tok=tok, score=score,
-                    extra=extra, detail=detail, lp=lp, call=call)
+                    extra=extra, detail=detail, lp=lp, call=call, at=noise_at)
 
-    def _finish(self, p, prompt_scores):
+    def _finish(self, p, prompt_scores, toks, scs):
         """Book-keeping after the decoder has admitted a prepared request: per-slot sampling
-        state, the alternatives of the first choice and of the prompt, the rows themselves."""
+        state, the alternatives of the first choice and of the prompt, the rows themselves
+        (``toks`` / ``scs``: its replicas' first tokens and their scores, on the host)."""
         torch = self._torch
         slots, group, rows, tok, extra = p["slots"], p["group"], p["rows"], p["tok"], p["extra"]
         eos = self.dict.eos()
@@ -611,7 +622,7 @@ class ContinuousBatcher(_Front):
             self._h_pen[slots] = group.alphas
             self._par_dirty = True
             if group.decay > 0 or group.penalised:
-                idx = torch.tensor(slots, dtype=torch.long, device=self.device)
+                idx = upload(slots, torch.long, self.device)
             if group.decay > 0:
                 self._since[idx] = 0.0
                 self._count_chosen(slots, tok)
@@ -628,7 +639,6 @@ class ContinuousBatcher(_Front):
             if "prompt_top" in p["detail"]:
                 values, top_ids = p["detail"]["prompt_top"]
                 prompt_top = [([], [])] + list(zip(values.tolist(), top_ids.tolist()))
-        toks, scs = tok.tolist(), p["score"].tolist()
         for j, (slot, row) in enumerate(zip(slots, rows)):
             row.scores = list(prompt_scores)
             if first_top is not None:
@@ -662,25 +672,57 @@ class ContinuousBatcher(_Front):
         if self.cache is None:
             self.cache = self.decoder.new_slot_cache(len(self.batch.rows), self.batch.capacity,
                                                      self.device)
+        torch = self._torch
+        total = sum(len(slots) for slots, _ in items)
+        tok_all = torch.zeros(total, dtype=torch.long, device=self.device)
+        score_all = torch.zeros(total, dtype=torch.float32, device=self.device)
         at, prepared = 0, []
         for slots, req in items:
-            prepared.append(self._prepare(slots, req, at))
+            prepared.append(self._prepare(slots, req, at, tok_all, score_all))
             at += len(slots)
-        groups = self._prefill_groups(prepared)
-        for members in groups:
+        # every group's kernels are queued before anything is read back: the prompt scores of
+        # all of them, the first tokens and their scores then come in one copy each (a read per
+        # request left the GPU idle between them once the prefills were done)
+        lazy = {"lazy": True} if getattr(self.decoder, "lazy_admission", False) else {}
+        queued = []
+        for members in self._prefill_groups(prepared):
             try:
                 if len(members) == 1:
                     call = dict(members[0]["call"])
                     scores = [self.decoder.admit_slot(self.cache, call.pop("slot"),
-                                                      call.pop("tokens"), **call)]
+                                                      call.pop("tokens"), **call, **lazy)]
                 else:
-                    scores = self.decoder.admit_slots(self.cache, [p["call"] for p in members])
-                for p, sc in zip(members, scores):
-                    self._finish(p, sc)
+                    scores = self.decoder.admit_slots(self.cache, [p["call"] for p in members],
+                                                      **lazy)
+                queued.append((members, scores))
             except RuntimeError:
                 raise
             except Exception as e:  # noqa: BLE001 - these requests' own answer
                 for p in members:
+                    for slot in p["slots"]:
+                        self.batch.rows[slot] = None
+                        self.decoder.release_slot(self.cache, slot)
+                    p["req"].answer(e)
+        if not queued:
+            return
+        on_device = [sc for _, scores in queued for sc in scores if torch.is_tensor(sc)]
+        flat = torch.cat(on_device).tolist() if on_device else []
+        toks, scs = tok_all.tolist(), score_all.tolist()
+        cursor = 0
+        for members, scores in queued:
+            for p, sc in zip(members, scores):
+                if torch.is_tensor(sc):
+                    n = sc.numel()
+                    sc = [0.0] + flat[cursor:cursor + n]
+                    cursor += n
+                elif sc is None:
+                    sc = [0.0]
+                a, R = p["at"], len(p["slots"])
+                try:
+                    self._finish(p, sc, toks[a:a + R], scs[a:a + R])
+                except RuntimeError:
+                    raise
+                except Exception as e:  # noqa: BLE001 - this request's own answer
                     for slot in p["slots"]:
                         self.batch.rows[slot] = None
                         self.decoder.release_slot(self.cache, slot)
@@ -771,8 +813,14 @@ class ContinuousBatcher(_Front):
             self._held = 0
             for _, req in taken:
                 self._arrived.pop(req.uid, None)
-            self._admit_many(taken)
             served += sum(len(slots) for slots, _ in taken)
+        # With rows running, the decode step below is queued before the admissions: preparing
+        # a few dozen requests takes the host as long as a decode step takes the GPU, and the
+        # GPU would sit idle behind the step in flight (a tenth of the time at 256 slots).  The
+        # new rows then join the step after this one.  With nothing to step, admit first.
+        if taken and not (self.launch_before_admission and self.batch.active()):
+            self._admit_many(taken)
+            taken = []
         # The step launched by the previous call is still running, or its results are still
         # unread: its rows' tokens are on the device only.  This call launches the next step
         # first - the rows that step chose tokens for are fed from the device, their modes
@@ -793,6 +841,8 @@ class ContinuousBatcher(_Front):
                 continue
             stepping.append((i, row, ahead))
         self._inflight = self._launch(stepping, before) if stepping else None
+        if taken:
+            self._admit_many(taken)
         self._flush()   # a step is queued: the GPU works while the host writes records
         if before is not None:
             self._collect(before)
@@ -855,12 +905,12 @@ class ContinuousBatcher(_Front):
                                   tok_out=tok, score_out=score, **extra)
         decaying = [i for i, row in general if row.group.decay > 0]
         if decaying:
-            self._count_chosen(decaying, tok[torch.tensor(decaying, device=self.device)])
+            self._count_chosen(decaying, tok[upload(decaying, torch.long, self.device)])
         launched = _Launched(buf, {i: row for i, row, _ in stepping})
         watched = [(i, row) for i, row in general if row.group.logprobs > 0]
         if watched:
             k = max(row.group.logprobs for _, row in watched)
-            picked = self._lprobs[torch.tensor([i for i, _ in watched], device=self.device)]
+            picked = self._lprobs[upload([i for i, _ in watched], torch.long, self.device)]
             values, top_ids = picked.topk(k, dim=-1)
             launched.watched = watched
             pinned = self._events is not None

@@ -22,6 +22,16 @@ from .config import OPTConfig
 from .kv_cache import KVCache
 
 
+def upload(values, dtype, device):
+    """A short host list as a device tensor without a blocking copy: through pinned memory and
+    stream-ordered.  (A copy from pageable memory makes the host wait for everything queued
+    ahead of it - a whole decode step - and leaves the GPU idle while the host goes on.)"""
+    t = torch.tensor(values, dtype=dtype)
+    if torch.device(device).type != "cuda":
+        return t.to(device)
+    return t.pin_memory().to(device, non_blocking=True)
+
+
 class _Affine(nn.Module):
     """weight + bias holder (Linear or LayerNorm parameters under the reference's names).
 
@@ -976,7 +986,7 @@ class TransformerDecoder(nn.Module):
         toks = tokens.long().contiguous().view(1, T)
         h, _ = self._rows_core(lib, _capi.stream_ptr(), toks, 1, T, T, 0, _SlotView(cache, slot),
                                None)
-        cache.lens[slot] = T
+        cache.lens[slot:slot + 1].fill_(T)   # (an element assignment waits for the stream)
         return self._project(h, False, 1, T)[0]
 
     def prefill_slots(self, cache: KVCache, slots, prompts):
@@ -1014,17 +1024,22 @@ class TransformerDecoder(nn.Module):
         tmp = KVCache(cfg.decoder_layers, k, cfg.decoder_attention_heads, cfg.head_dim, Tmax, dev)
         h, _ = self._rows_core(lib, _capi.stream_ptr(), toks, k, Tmax, Tmax, 0, tmp, None)
         # one copy per layer: whole padded rows (what lies past a prompt's length is never read)
-        where = torch.tensor(slots, device=dev)
+        where = upload(slots, torch.long, dev)
         for mine, theirs in zip(cache.layers, tmp.layers):
             mine[:, :, :, :Tmax].index_copy_(1, where, theirs)
-        cache.lens[where] = torch.tensor(lens, dtype=torch.int32, device=dev)
+        cache.lens[where] = upload(lens, torch.int32, dev)
         logits = self._project(h, False, k, Tmax)
         return [logits[r, :lens[r]] for r in range(k)]
 
-    def admit_slots(self, cache: KVCache, requests):
+    # admit_slot / admit_slots take ``lazy=True``: the prompt scores come back as device tensors
+    # (None for a one-token prompt) for the caller to read together with everything else
+    lazy_admission = True
+
+    def admit_slots(self, cache: KVCache, requests, lazy=False):
         """``admit_slot`` for several requests with one shared prefill (``prefill_slots``).
         ``requests``: dicts with ``slot``, ``tokens`` and the keyword arguments of
-        ``admit_slot``; returns the list of their prompt scores."""
+        ``admit_slot``; returns the list of their prompt scores (``lazy``: as fp32 device
+        tensors without the leading 0.0, nothing read back yet)."""
         logits = self.prefill_slots(cache, [r["slot"] for r in requests],
                                     [r["tokens"] for r in requests])
         out = []
@@ -1032,13 +1047,22 @@ class TransformerDecoder(nn.Module):
             kw = {k: v for k, v in r.items() if k not in ("slot", "tokens")}
             out.append(self.admit_slot(cache, r["slot"], r["tokens"], _logits=lg, _lazy=True,
                                        **kw))
-        # every request's kernels are queued: one wait for the first list, none for the rest
-        return [[0.0] + lp.tolist() if lp is not None else [0.0] for lp in out]
+        if lazy:
+            return out
+        # every request's kernels are queued: one copy for all the scores
+        flat = torch.cat([lp for lp in out if lp is not None]).tolist() if any(
+            lp is not None for lp in out) else []
+        scores, at = [], 0
+        for lp in out:
+            n = lp.numel() if lp is not None else 0
+            scores.append([0.0] + flat[at:at + n])
+            at += n
+        return scores
 
     def admit_slot(self, cache: KVCache, slot: int, tokens: torch.Tensor, *, banned=(), stop=(),
                    eos=2, mode=0, tok_out=None, score_out=None, temperature=1.0, topp=0.0,
                    noise=None, replicas=(), penalties=None, lprobs_out=None, prompt_topk=0,
-                   detail=None, _logits=None, _lazy=False):
+                   detail=None, lazy=False, _logits=None, _lazy=False):
         """``prefill_slot`` plus what a request needs from its prompt: the log-probability of
         every prompt token given its prefix (returned as a list, 0.0 for the first token) and
         the choice of the first new token from the last position, written to ``tok_out`` /
@@ -1060,6 +1084,7 @@ class TransformerDecoder(nn.Module):
         tokens at every prompt position after the first (log-softmax of logits / temperature,
         what the reference records for the prompt with ``need_logprobs``)."""
         lib = self.prepare_()
+        _lazy = _lazy or lazy
         # (_logits: the prompt was already prefilled into the slot, by prefill_slots)
         logits = _logits if _logits is not None else self.prefill_slot(cache, slot, tokens)
         T, V = logits.shape
@@ -1080,7 +1105,7 @@ class TransformerDecoder(nn.Module):
                 detail["prompt_top"] = (values.cpu(), ids.cpu())
                 del dist
         for dst in replicas:
-            self.copy_slot(cache, slot, dst)
+            self.copy_slot(cache, slot, dst, length=T)
         R = 1 + len(replicas)
         plain = (float(temperature) == 1.0 and not topp > 0 and noise is None
                  and penalties is None and lprobs_out is None)
@@ -1116,16 +1141,19 @@ class TransformerDecoder(nn.Module):
                 ptr(score_out), 1, stream))
         return lp if _lazy else scores
 
-    def copy_slot(self, cache: KVCache, src: int, dst: int):
+    def copy_slot(self, cache: KVCache, src: int, dst: int, length: Optional[int] = None):
         """Makes slot ``dst`` a copy of slot ``src``: keys, values and length (a replica of a
-        request starts from the same prompt)."""
-        n = int(cache.lens[src])
+        request starts from the same prompt).  ``length``: the source's length where the caller
+        knows it (reading it from the device waits for everything queued)."""
+        n = int(cache.lens[src]) if length is None else int(length)
         for layer in cache.layers:
             layer[:, dst, :, :n].copy_(layer[:, src, :, :n])
-        cache.lens[dst] = n
+        cache.lens[dst:dst + 1].fill_(n)
 
     def release_slot(self, cache: KVCache, slot: int):
-        cache.lens[slot] = -1
+        # a fill kernel on a one-element view: ``lens[slot] = -1`` copies a host scalar to the
+        # device and makes the caller wait for the work queued ahead of it
+        cache.lens[slot:slot + 1].fill_(-1)
 
     def decode_slots(self, cache: KVCache, last_tokens: torch.Tensor, *, temperature=1.0,
                      banned=(), stop=(), eos=2, row_mode=None, tok_out=None, score_out=None,

@@ -483,7 +483,8 @@ def test_continuous_batcher_with_shared_prefills():
                            noise_fn=lambda req, j, pos, V: _noise_for(req.prompt, j, pos, V))
     shared = []
     inner = cb.decoder.admit_slots
-    cb.decoder.admit_slots = lambda cache, reqs: (shared.append(len(reqs)), inner(cache, reqs))[1]
+    cb.decoder.admit_slots = lambda cache, reqs, **kw: (shared.append(len(reqs)),
+                                                        inner(cache, reqs, **kw))[1]
     try:
         replies = [cb.submit(s["prompt"], **{k: v for k, v in s.items() if k != "prompt"})
                    for s in specs]
