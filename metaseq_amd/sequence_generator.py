@@ -271,10 +271,10 @@ class SequenceGenerator(nn.Module):
                 return at >= min_len or at >= max_len - 1
 
             def wipe(col):
-                tokens[:, col] = self.pad
-                scores[:, col] = 0
+                tokens[:, col].fill_(self.pad)
+                scores[:, col].fill_(0)
                 if all_lprobs is not None:
-                    all_lprobs[:, col] = 0
+                    all_lprobs[:, col].fill_(0)
             if fused:
                 # the first token comes from the prefill logits; every later one is chosen inside
                 # the decode step's vocabulary projection, so logits are never materialised

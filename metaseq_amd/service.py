@@ -624,7 +624,7 @@ class ContinuousBatcher(_Front):
             if group.decay > 0 or group.penalised:
                 idx = upload(slots, torch.long, self.device)
             if group.decay > 0:
-                self._since[idx] = 0.0
+                self._since.index_fill_(0, idx, 0.0)
                 self._count_chosen(slots, tok)
             if group.penalised:
                 self._counts[idx] = extra["penalties"]["counts"]
